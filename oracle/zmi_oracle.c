@@ -1,0 +1,526 @@
+/*
+ * zmi_oracle.c -- CPU restatement of the reference's LowOHA int8 matmul path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the product (the zendnn_amd package,
+ * libzmi_lowoha.so, the C++ adapter) may link, load or call this file; it is
+ * used by tests/, by __graft_entry__.smoke() and by bench.py's cpu_baseline
+ * leg, always as the checker or the timed CPU baseline.
+ *
+ * It takes the same flat structs as the C ABI (include/zmi_lowoha.h) but with
+ * HOST pointers, so one ctypes description drives both sides of a parity test.
+ *
+ * Each function cites the reference file:line whose arithmetic it follows
+ * (paths relative to zendnnl/src/ of the reference tree).  The reference's
+ * default backend for this path is AOCL-DLP (github.com/amd/aocl-dlp, pinned
+ * at b3db7f5800aca3ba3ce5bdfab10f557c5b896e5a), which is not vendored; its
+ * semantics are the ones the reference's own scalar kernel states
+ * (operators/matmul/matmul_ref_kernel.cpp), and that is what is restated.
+ *
+ * Parity status of each function (what pins it, see tests/test_oracle_*.py):
+ *   zo_f32_to_bf16_ctor / _rne   exhaustive hi-half table + torch bfloat16
+ *   zo_quant_per_token           closed forms (constant row, zero row, NaN/Inf,
+ *                                ties-to-even), |q|<=127, max|q|==127
+ *   zo_gemm_s32                  int64 brute force, all-ones closed form, the
+ *                                reference example's deterministic recipe
+ *   zp compensation              integer identity sum((a-zp)w) == sum(aw)-zp*sum(w)
+ *   dequant chain / bias         special cases (unit scales, equal per-channel
+ *                                scales == per-tensor), op order from source
+ *   post-ops                     libm double evaluation within 2 f32 ulp
+ *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
+ *   prepack layout, weight_prepack_size values: parity unpinned (opaque by the
+ *     reference's contract; only the round trip matmul(prepack(B)) == matmul(B)
+ *     is checkable) -- the oracle has no function for them.
+ *   AOCL-DLP's vectorised SWISH / GELU_TANH last-ulp behaviour: parity unpinned
+ *     (only a run of AOCL-DLP could pin it; the scalar reference defines the target).
+ *
+ * Build: gcc -O2 -ffp-contract=off -fopenmp -shared -fPIC (see oracle/build.py).
+ * -ffp-contract=off matters: the reference chain is a sequence of separately
+ * rounded f32 operations.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../include/zmi_lowoha.h"
+
+#define ZO_EXPORT __attribute__((visibility("default")))
+
+/* ---- bf16 ------------------------------------------------------------- */
+
+/* bfloat16_t::bfloat16_t(float), common/bfloat16.cpp:27-51: zero and subnormal
+ * inputs give a signed zero, NaN keeps the high half with the quiet bit set,
+ * normals round to nearest even.  Used by the matmul store
+ * (operators/matmul/matmul_ref_kernel.cpp:207-218) and the gated activation
+ * (lowoha_operators/matmul/group_matmul/group_matmul_moe_act.cpp:110-117). */
+ZO_EXPORT uint16_t zo_f32_to_bf16_ctor(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  uint32_t exp = u & 0x7f800000u, man = u & 0x007fffffu;
+  if (exp == 0) return (uint16_t)((u >> 16) & 0x8000u);
+  if (exp == 0x7f800000u) {
+    if (man == 0) return (uint16_t)(u >> 16);
+    return (uint16_t)((u >> 16) | 0x40u);
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+/* bfloat16_t::f32_to_bf16_val, common/bfloat16.cpp:69-79: the plain bit trick,
+ * no special cases.  Used by the MoE weighted reduce
+ * (group_matmul/group_matmul_moe_postop.cpp:85-88, 262-283). */
+ZO_EXPORT uint16_t zo_f32_to_bf16_rne(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+/* bfloat16_t::bf16_to_f32_val, common/bfloat16.cpp:60-66. */
+ZO_EXPORT float zo_bf16_to_f32(uint16_t h) {
+  uint32_t u = ((uint32_t)h) << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+ZO_EXPORT void zo_f32_to_bf16_buf(const float *src, uint16_t *dst, int64_t n, int ctor) {
+  for (int64_t i = 0; i < n; ++i)
+    dst[i] = ctor ? zo_f32_to_bf16_ctor(src[i]) : zo_f32_to_bf16_rne(src[i]);
+}
+
+/* ---- helpers ---------------------------------------------------------- */
+
+static int64_t zo_nelems(const zmi_quant_t *q) {
+  int64_t n = 1;
+  for (int i = 0; i < q->ndims; ++i) n *= q->dims[i];
+  return n;
+}
+
+/* read_and_cast<float> of the reference for the dtypes this path uses. */
+static float zo_read_f32(const void *p, int32_t dt, int64_t i) {
+  switch (dt) {
+  case ZMI_DT_F32: return ((const float *)p)[i];
+  case ZMI_DT_BF16: return zo_bf16_to_f32(((const uint16_t *)p)[i]);
+  case ZMI_DT_S32: return (float)((const int32_t *)p)[i];
+  case ZMI_DT_S8: return (float)((const int8_t *)p)[i];
+  case ZMI_DT_U8: return (float)((const uint8_t *)p)[i];
+  default: return 0.0f;
+  }
+}
+
+static int32_t zo_read_s32(const void *p, int32_t dt, int64_t i) {
+  switch (dt) {
+  case ZMI_DT_S32: return ((const int32_t *)p)[i];
+  case ZMI_DT_S8: return ((const int8_t *)p)[i];
+  case ZMI_DT_U8: return ((const uint8_t *)p)[i];
+  case ZMI_DT_F32: return (int32_t)((const float *)p)[i];
+  default: return 0;
+  }
+}
+
+/* ---- per-token dynamic quantization ------------------------------------ */
+
+/* dynamic_per_token_quant_{bf16,f32}_s8_ref,
+ * lowoha_operators/reorder/reorder_data_type/scalar_impl/dynamic_per_token_ref_kernel.cpp:31-36,70-96:
+ * absmax over finite values; scale = max(absmax,1e-10)/127 clamped to >= 1e-10;
+ * q = (int8) nearbyint(v / scale) (true division, ties to even, truncating
+ * narrow); non-finite -> 0. */
+ZO_EXPORT void zo_quant_per_token(const void *src, int32_t src_dt, int64_t M, int64_t K,
+                                  int64_t ld_src, int8_t *dst, int64_t ld_dst, float *scales) {
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float absmax = 0.0f;
+    for (int64_t j = 0; j < K; ++j) {
+      float v = zo_read_f32(src, src_dt, m * ld_src + j);
+      if (isfinite(v)) {
+        float a = fabsf(v);
+        if (a > absmax) absmax = a;
+      }
+    }
+    if (absmax < 1e-10f) absmax = 1e-10f;
+    float scale = absmax / 127.0f;
+    if (scale < 1e-10f) scale = 1e-10f;
+    scales[m] = scale;
+    if (!dst) continue;
+    for (int64_t j = 0; j < K; ++j) {
+      float v = zo_read_f32(src, src_dt, m * ld_src + j);
+      if (!isfinite(v)) { dst[m * ld_dst + j] = 0; continue; }
+      int32_t q = (int32_t)nearbyintf(v / scale);
+      dst[m * ld_dst + j] = (int8_t)q;
+    }
+  }
+}
+
+/* ---- exact integer GEMM -------------------------------------------------- */
+
+/* Accumulator of compute_quantized_matmul,
+ * operators/matmul/matmul_ref_kernel.cpp:1003-1030 (non-grouped branch):
+ * acc[m,n] = sum_k a[m,k] * w[k,n] in int32.  The sum is also carried in int64
+ * and the function returns the number of elements whose int64 value does not
+ * fit int32 (0 for every case the tests use), so "bit-exact s32" is checked
+ * against arithmetic that cannot wrap. */
+__attribute__((target_clones("default", "avx2", "arch=skylake-avx512")))
+static void zo_dot_rows_s8(const int8_t *a, const int8_t *bt, int64_t K, int64_t N,
+                           int64_t ldbt, int32_t *out) {
+  for (int64_t n = 0; n < N; ++n) {
+    const int8_t *b = bt + n * ldbt;
+    int32_t s = 0;
+    for (int64_t k = 0; k < K; ++k) s += (int32_t)a[k] * (int32_t)b[k];
+    out[n] = s;
+  }
+}
+
+__attribute__((target_clones("default", "avx2", "arch=skylake-avx512")))
+static void zo_dot_rows_u8(const uint8_t *a, const int8_t *bt, int64_t K, int64_t N,
+                           int64_t ldbt, int32_t *out) {
+  for (int64_t n = 0; n < N; ++n) {
+    const int8_t *b = bt + n * ldbt;
+    int32_t s = 0;
+    for (int64_t k = 0; k < K; ++k) s += (int32_t)a[k] * (int32_t)b[k];
+    out[n] = s;
+  }
+}
+
+/* Fast path used for large shapes and for the timed CPU baseline: weights are
+ * transposed once to [N,K] so the k loop is contiguous for both operands. */
+ZO_EXPORT void zo_transpose_s8(const int8_t *B, int64_t K, int64_t N, int64_t ldb, int8_t *Bt) {
+  #pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t k = 0; k < K; ++k) Bt[n * K + k] = B[k * ldb + n];
+}
+
+ZO_EXPORT void zo_gemm_s32_bt(const void *A, int32_t a_dt, int64_t lda, const int8_t *Bt,
+                              int64_t ldbt, int64_t M, int64_t N, int64_t K, int32_t *acc,
+                              int64_t ldacc) {
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    if (a_dt == ZMI_DT_U8)
+      zo_dot_rows_u8((const uint8_t *)A + m * lda, Bt, K, N, ldbt, acc + m * ldacc);
+    else
+      zo_dot_rows_s8((const int8_t *)A + m * lda, Bt, K, N, ldbt, acc + m * ldacc);
+  }
+}
+
+/* General (strided, optionally transposed) form with the int64 overflow check. */
+ZO_EXPORT int64_t zo_gemm_s32(const void *A, int32_t a_dt, int32_t transA, int64_t lda,
+                              const int8_t *B, int32_t transB, int64_t ldb, int64_t M, int64_t N,
+                              int64_t K, int32_t *acc, int64_t ldacc) {
+  int64_t overflow = 0;
+  #pragma omp parallel for schedule(static) reduction(+ : overflow)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      int64_t s = 0;
+      for (int64_t k = 0; k < K; ++k) {
+        int64_t ai = transA ? k * lda + m : m * lda + k;
+        int64_t bi = transB ? n * ldb + k : k * ldb + n;
+        int32_t a = (a_dt == ZMI_DT_U8) ? (int32_t)((const uint8_t *)A)[ai]
+                                        : (int32_t)((const int8_t *)A)[ai];
+        s += (int64_t)a * (int64_t)B[bi];
+      }
+      if (s > INT32_MAX || s < INT32_MIN) overflow++;
+      acc[m * ldacc + n] = (int32_t)s;
+    }
+  }
+  return overflow;
+}
+
+/* compute_zero_point_compensation, src_zp-only branch,
+ * operators/matmul/matmul_ref_kernel.cpp:71-91 (same as
+ * lowoha_operators/matmul/lru_cache/lowoha_cache.hpp:99-133):
+ * comp[n] = 0 - src_zp * sum_k w[k,n]. */
+ZO_EXPORT void zo_zp_comp(const int8_t *B, int32_t transB, int64_t ldb, int64_t K, int64_t N,
+                          int32_t src_zp, int32_t *comp) {
+  for (int64_t n = 0; n < N; ++n) {
+    int32_t s = 0;
+    for (int64_t k = 0; k < K; ++k) s += B[transB ? n * ldb + k : k * ldb + n];
+    comp[n] = 0 - src_zp * s;
+  }
+}
+
+/* ---- element-wise post-ops ---------------------------------------------- */
+
+/* Constants of operators/matmul/matmul_ref_kernel.hpp:31-33. */
+#define ZO_SQRT_2_OVER_PI 0.79788458347320556640625f
+#define ZO_SQRT_2_OVER_2 0.707106769084930419921875f
+#define ZO_FITTING_CONST 0.044715f
+
+/* operators/matmul/matmul_ref_kernel.cpp:694-761, same expressions and the
+ * same float/double promotion as the C++ source. */
+static float zo_gelu_tanh(float x) {
+  float v = tanhf(ZO_SQRT_2_OVER_PI * x * (1 + ZO_FITTING_CONST * x * x));
+  return (float)(0.5 * x * (1.0f + v));
+}
+static float zo_gelu_erf(float x) {
+  float v = x * ZO_SQRT_2_OVER_2;
+  return 0.5f * x * (1.0f + erff(v));
+}
+static float zo_sigmoid(float x) { return (float)(1.0 / (1.0 + expf(-x))); }
+static float zo_swish(float x, float scale) {
+  float sx = x * scale;
+  return (float)(x * (1.0 / (1.0 + expf(-sx))));
+}
+
+ZO_EXPORT float zo_eltwise(int32_t po, float x, float alpha, float beta) {
+  switch (po) {
+  case ZMI_PO_RELU: return x > 0 ? x : 0;
+  /* the AOCL wiring passes a fixed default slope, backends/aocl/aocl_postop.cpp:410 */
+  case ZMI_PO_LEAKY_RELU: return x > 0 ? x : 0.01f * x;
+  case ZMI_PO_GELU_TANH: return zo_gelu_tanh(x);
+  case ZMI_PO_GELU_ERF: return zo_gelu_erf(x);
+  case ZMI_PO_SIGMOID: return zo_sigmoid(x);
+  /* swish scale is the constant 1, backends/aocl/aocl_postop.cpp:421-423 */
+  case ZMI_PO_SWISH: return zo_swish(x, 1.0f);
+  case ZMI_PO_TANH: return tanhf(x);
+  case ZMI_PO_CLIP: { x = x > alpha ? x : alpha; return x > beta ? beta : x; }
+  default: return x;
+  }
+}
+
+/* ---- full quantized matmul ---------------------------------------------- */
+
+typedef struct zo_matmul_call {
+  char layout;
+  int32_t transA, transB, M, N, K;
+  float alpha;
+  const void *src; int32_t lda;
+  const void *weight; int32_t ldb;
+  const void *bias; float beta;
+  void *dst; int32_t ldc;
+  const zmi_matmul_params_t *params;
+  int32_t *acc_out;   /* optional [M,N]: the raw s32 accumulator (before compensation) */
+  float *scale_out;   /* optional [M]: the per-token scales a dynamic_quant call computed */
+} zo_matmul_call;
+
+static void zo_store(void *dst, int32_t dt, int64_t i, float val) {
+  /* store_output, operators/matmul/matmul_ref_kernel.cpp:154-254 */
+  switch (dt) {
+  case ZMI_DT_U8:
+    val = val < 0.0f ? 0.0f : (val > 255.0f ? 255.0f : val);
+    ((uint8_t *)dst)[i] = (uint8_t)nearbyintf(val);
+    break;
+  case ZMI_DT_S8:
+    val = val < -128.0f ? -128.0f : (val > 127.0f ? 127.0f : val);
+    ((int8_t *)dst)[i] = (int8_t)nearbyintf(val);
+    break;
+  case ZMI_DT_S32:
+    val = val < (float)INT32_MIN ? (float)INT32_MIN : (val > (float)INT32_MAX ? (float)INT32_MAX : val);
+    /* (float)INT32_MAX is 2^31; the reference's cast of it is out of range, so pin it */
+    ((int32_t *)dst)[i] = val >= 2147483648.0f ? INT32_MAX : (int32_t)nearbyintf(val);
+    break;
+  case ZMI_DT_BF16: ((uint16_t *)dst)[i] = zo_f32_to_bf16_ctor(val); break;
+  default: ((float *)dst)[i] = val; break;
+  }
+}
+
+/* matmul_direct for the int8 path.  Pipeline of lowoha_operators/matmul/
+ * lowoha_matmul.cpp:278-510: optional dynamic per-token quantization of a
+ * bf16/f32 source (matmul/quantization/reorder_quantization.cpp:43-280), then
+ * the int8 GEMM and the dequantization chain of
+ * operators/matmul/matmul_ref_kernel.cpp:1032-1053:
+ *   y = float(acc); y *= alpha (if != 1); y += beta * C (if beta);
+ *   y += float(zp_comp[n]); y *= src_scale[per-tensor | m]; y *= wei_scale[n % len];
+ *   y += bias[n]; post-ops in order; y = y * dst_scale + dst_zp (quantize_dst);
+ *   store with the dtype's rounding.
+ * Returns a ZMI_* status. */
+ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
+  const zmi_matmul_params_t *p = c->params;
+  const int64_t M = c->M, N = c->N, K = c->K;
+  if (p->dt_wei != ZMI_DT_S8) return ZMI_UNIMPLEMENTED;
+
+  const void *A = c->src;
+  int32_t a_dt = p->dt_src;
+  int64_t lda = c->lda;
+  int32_t transA = c->transA;
+  int8_t *qbuf = NULL;
+  float *sbuf = NULL;
+  const float *src_scale = NULL;
+  int64_t src_scale_n = p->src_scale.buff ? zo_nelems(&p->src_scale) : 0;
+  int32_t src_scale_dt = p->src_scale.dt;
+
+  const int dyn = p->dynamic_quant && (a_dt == ZMI_DT_BF16 || a_dt == ZMI_DT_F32) &&
+                  (p->dt_compute == ZMI_DT_S8 || p->dt_compute == ZMI_DT_U8);
+  if (dyn) {
+    if (transA) return ZMI_UNIMPLEMENTED;
+    qbuf = (int8_t *)malloc((size_t)M * K);
+    sbuf = (float *)malloc(sizeof(float) * (size_t)M);
+    int64_t dn = 1;
+    for (int i = 0; i < p->src_scale.ndims; ++i) dn *= p->src_scale.dims[i];
+    if (dn == M && M > 1) {
+      zo_quant_per_token(A, a_dt, M, K, lda, qbuf, K, sbuf);
+    } else {
+      /* per-tensor dynamic scale: same formula over the whole tensor,
+       * lowoha_operators/reorder/lowoha_reorder_utils.cpp:724-761 */
+      float absmax = 0.0f;
+      for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < K; ++k) {
+          float v = zo_read_f32(A, a_dt, m * lda + k);
+          if (isfinite(v) && fabsf(v) > absmax) absmax = fabsf(v);
+        }
+      if (absmax < 1e-10f) absmax = 1e-10f;
+      float s = absmax / 127.0f;
+      if (s < 1e-10f) s = 1e-10f;
+      for (int64_t m = 0; m < M; ++m) {
+        sbuf[m] = s;
+        for (int64_t k = 0; k < K; ++k) {
+          float v = zo_read_f32(A, a_dt, m * lda + k);
+          qbuf[m * K + k] = isfinite(v) ? (int8_t)(int32_t)nearbyintf(v / s) : 0;
+        }
+      }
+      dn = 1;
+    }
+    if (c->scale_out) memcpy(c->scale_out, sbuf, sizeof(float) * (size_t)(dn == 1 ? 1 : M));
+    A = qbuf; a_dt = ZMI_DT_S8; lda = K;
+    src_scale = sbuf; src_scale_n = dn == 1 ? 1 : M; src_scale_dt = ZMI_DT_F32;
+  } else if (a_dt != ZMI_DT_S8 && a_dt != ZMI_DT_U8) {
+    return ZMI_UNIMPLEMENTED;
+  } else {
+    src_scale = (const float *)p->src_scale.buff;
+  }
+
+  int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)M * N);
+  if (!transA && M * N * K > (1 << 22)) {
+    int8_t *Bt = (int8_t *)c->weight;
+    int64_t ldbt = c->ldb;
+    int8_t *tmp = NULL;
+    if (!c->transB) {
+      tmp = (int8_t *)malloc((size_t)N * K);
+      zo_transpose_s8((const int8_t *)c->weight, K, N, c->ldb, tmp);
+      Bt = tmp; ldbt = K;
+    }
+    zo_gemm_s32_bt(A, a_dt, lda, Bt, ldbt, M, N, K, acc, N);
+    free(tmp);
+  } else {
+    zo_gemm_s32(A, a_dt, transA, lda, (const int8_t *)c->weight, c->transB, c->ldb, M, N, K, acc, N);
+  }
+  if (c->acc_out) memcpy(c->acc_out, acc, sizeof(int32_t) * (size_t)M * N);
+
+  int32_t src_zp = p->src_zp.buff ? zo_read_s32(p->src_zp.buff, p->src_zp.dt, 0) : 0;
+  int32_t *comp = NULL;
+  if (src_zp) {
+    comp = (int32_t *)malloc(sizeof(int32_t) * (size_t)N);
+    zo_zp_comp((const int8_t *)c->weight, c->transB, c->ldb, K, N, src_zp, comp);
+  }
+  const int per_token = (src_scale_n == M && M > 1);
+  const int64_t wei_scale_n = p->wei_scale.buff ? zo_nelems(&p->wei_scale) : 0;
+  const float dst_scale = p->dst_scale.buff ? zo_read_f32(p->dst_scale.buff, p->dst_scale.dt, 0) : 1.0f;
+  const int has_dst_q = p->dst_scale.buff != NULL || p->dst_zp.buff != NULL;
+  const float dst_zp = p->dst_zp.buff ? zo_read_f32(p->dst_zp.buff, p->dst_zp.dt, 0) : 0.0f;
+
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      float y = (float)acc[m * N + n];
+      if (c->alpha != 1.0f) y *= c->alpha;
+      if (c->beta != 0.0f) y += zo_read_f32(c->dst, p->dt_dst, m * (int64_t)c->ldc + n) * c->beta;
+      if (comp) y += (float)comp[n];
+      if (src_scale_n) y *= zo_read_f32(src_scale, src_scale_dt, per_token ? m : 0);
+      if (wei_scale_n) y *= zo_read_f32(p->wei_scale.buff, p->wei_scale.dt, n % wei_scale_n);
+      if (c->bias) y += zo_read_f32(c->bias, p->dt_bias == ZMI_DT_NONE ? ZMI_DT_F32 : p->dt_bias, n);
+      for (int i = 0; i < p->n_postops; ++i) {
+        const zmi_post_op_t *po = &p->postops[i];
+        if (po->po_type == ZMI_PO_BINARY_ADD || po->po_type == ZMI_PO_BINARY_MUL) {
+          /* binary_add_fwd / binary_mul_fwd with scale 1,
+           * operators/matmul/matmul_ref_kernel.cpp:753-759; operand is
+           * {1,N} (row broadcast) or {M,N} with leading_dim */
+          int64_t ld = po->leading_dim > 0 ? po->leading_dim : N;
+          int rowb = (po->ndims == 2 && po->dims[0] == 1) || po->ndims == 1;
+          float t = zo_read_f32(po->buff, po->dtype, rowb ? n : m * ld + n);
+          y = po->po_type == ZMI_PO_BINARY_ADD ? y + t : y * t;
+        } else {
+          y = zo_eltwise(po->po_type, y, po->alpha, po->beta);
+        }
+      }
+      if (has_dst_q) y = y * dst_scale + dst_zp;
+      zo_store(c->dst, p->dt_dst, m * (int64_t)c->ldc + n, y);
+    }
+  }
+  free(acc); free(comp); free(qbuf); free(sbuf);
+  return ZMI_SUCCESS;
+}
+
+/* ---- gated activation ----------------------------------------------------- */
+
+/* silu_and_mul_row_scalar_{bf16,f32}, gelu_and_mul_*, swiglu_oai_mul_*,
+ * lowoha_operators/matmul/group_matmul/group_matmul_moe_act.cpp:88-154:
+ * split halves [gate | up], dst[:,0:dim] = act(gate) * up, f32 math,
+ * bf16 result through the bfloat16_t constructor. */
+static float zo_sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+ZO_EXPORT void zo_gated_act(int32_t act, void *buf, int32_t dt, int64_t M, int64_t N, int64_t ld) {
+  const int64_t dim = N / 2;
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < dim; ++n) {
+      float g, u, r;
+      if (act == ZMI_ACT_SWIGLU_OAI_MUL) {
+        g = zo_read_f32(buf, dt, m * ld + 2 * n);
+        u = zo_read_f32(buf, dt, m * ld + 2 * n + 1);
+        g = fmaxf(-7.0f, fminf(g, 7.0f));
+        u = fmaxf(-7.0f, fminf(u, 7.0f));
+        float sig = zo_sigmoid_f(g * 1.702f);
+        r = (1.0f + u) * g * sig;
+      } else {
+        g = zo_read_f32(buf, dt, m * ld + n);
+        u = zo_read_f32(buf, dt, m * ld + dim + n);
+        if (act == ZMI_ACT_SILU_AND_MUL) r = (g * zo_sigmoid_f(g)) * u;
+        else r = (g * 0.5f * (1.0f + erff(g * 0.7071067811865476f))) * u;
+      }
+      if (dt == ZMI_DT_BF16) ((uint16_t *)buf)[m * ld + n] = zo_f32_to_bf16_ctor(r);
+      else ((float *)buf)[m * ld + n] = r;
+    }
+  }
+}
+
+/* ---- MoE weighted reduce ---------------------------------------------------- */
+
+/* moe_weighted_reduce_avx512_{bf16,f32},
+ * lowoha_operators/matmul/group_matmul/group_matmul_moe_postop.cpp:191-286:
+ * acc = w0*x0 (one rounding), then acc = fma(wk, xk, acc) for k = 1..topk-1,
+ * bf16 store with the plain RNE bit trick.  (The scalar twin at :103-129 starts
+ * from 0 and uses mul+add; the two differ by at most one f32 rounding per term.) */
+ZO_EXPORT void zo_moe_reduce(const void *const *row_ptrs, const float *w, int32_t skip_weighted,
+                             int64_t T, int32_t topk, int64_t D, int32_t dt, void *out, int64_t ldo) {
+  #pragma omp parallel for schedule(static)
+  for (int64_t t = 0; t < T; ++t) {
+    for (int64_t d = 0; d < D; ++d) {
+      float acc = 0.0f;
+      for (int k = 0; k < topk; ++k) {
+        float wk = skip_weighted ? 1.0f : w[t * topk + k];
+        float x = zo_read_f32(row_ptrs[t * topk + k], dt, d);
+        acc = (k == 0) ? wk * x : fmaf(wk, x, acc);
+      }
+      if (dt == ZMI_DT_BF16) ((uint16_t *)out)[t * ldo + d] = zo_f32_to_bf16_rne(acc);
+      else ((float *)out)[t * ldo + d] = acc;
+    }
+  }
+}
+
+/* ---- timed CPU baseline helper ------------------------------------------------ */
+
+/* One decode-style call on already-quantized operands, the shape of work the
+ * reference's CPU path spends its time on (s8 x s8 -> s32 GEMM over
+ * pre-transposed weights, then scale * scale and SiLU, bf16 store).  Used only
+ * by bench.py's cpu_baseline leg. */
+ZO_EXPORT void zo_bench_s8_gemm(const int8_t *A, const int8_t *Bt, const float *sa, const float *sb,
+                                int64_t M, int64_t N, int64_t K, int32_t po, uint16_t *dst) {
+  #pragma omp parallel
+  {
+    int32_t *row = (int32_t *)malloc(sizeof(int32_t) * 256);
+    #pragma omp for schedule(static) collapse(2)
+    for (int64_t m = 0; m < M; ++m) {
+      for (int64_t n0 = 0; n0 < N; n0 += 256) {
+        int64_t nb = N - n0 < 256 ? N - n0 : 256;
+        zo_dot_rows_s8(A + m * K, Bt + n0 * K, K, nb, K, row);
+        for (int64_t j = 0; j < nb; ++j) {
+          float y = (float)row[j];
+          y *= sa[m];
+          y *= sb[n0 + j];
+          y = zo_eltwise(po, y, 0.0f, 0.0f);
+          dst[m * N + n0 + j] = zo_f32_to_bf16_ctor(y);
+        }
+      }
+    }
+    free(row);
+  }
+}

@@ -1,0 +1,332 @@
+"""Pins the CPU oracle against facts that do not come from the oracle itself:
+closed forms, integer identities, brute force in Python integers, libm in
+double precision, torch's bfloat16, and the deterministic recipes the
+reference's examples use.  A dropped term, a wrong sign or index, or a
+transposed operand fails at least one of these."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from zendnn_amd import capi
+
+
+# ---------------------------------------------------------------- bf16
+def test_bf16_ctor_matches_torch_on_normals(zo):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-20, 20, 200000).astype(np.float32)
+    ours = zo.f32_to_bf16(x, ctor=True)
+    ref = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(ours, ref)
+    assert np.array_equal(zo.f32_to_bf16(x, ctor=False), ref)
+
+
+def test_bf16_exhaustive_high_half_and_ties(zo):
+    hi = np.arange(65536, dtype=np.uint32) << 16
+    # exact, just-below-tie, tie, just-above-tie, all-ones low half
+    for lo in (0x0000, 0x7FFF, 0x8000, 0x8001, 0xFFFF):
+        bits = (hi | lo).astype(np.uint32)
+        x = bits.view(np.float32)
+        got = zo.f32_to_bf16(x, ctor=True).astype(np.uint32)
+        exp_field = (bits >> 23) & 0xFF
+        man = bits & 0x7FFFFF
+        normal = (exp_field != 0) & (exp_field != 0xFF)
+        up = (lo > 0x8000) | ((lo == 0x8000) & (((bits >> 16) & 1) == 1))
+        want_normal = ((bits >> 16) + up.astype(np.uint32)) & 0xFFFF
+        assert np.array_equal(got[normal], want_normal[normal])
+        sub = exp_field == 0                       # zero / subnormal -> signed zero
+        assert np.array_equal(got[sub], (bits[sub] >> 16) & 0x8000)
+        inf = (exp_field == 0xFF) & (man == 0)
+        assert np.array_equal(got[inf], bits[inf] >> 16)
+        nan = (exp_field == 0xFF) & (man != 0)
+        assert np.array_equal(got[nan], (bits[nan] >> 16) | 0x40)
+        # the plain bit trick has no special cases
+        got2 = zo.f32_to_bf16(x, ctor=False).astype(np.uint32)
+        want2 = ((bits.astype(np.uint64) + 0x7FFF + ((bits >> 16) & 1)) >> 16) & 0xFFFF
+        assert np.array_equal(got2, want2.astype(np.uint32))
+
+
+def test_bf16_round_trip(zo):
+    h = np.arange(65536, dtype=np.uint16)
+    f = zo.bf16_to_f32(h)
+    ok = ~np.isnan(f) & ((h & 0x7F80) != 0)
+    assert np.array_equal(zo.f32_to_bf16(f[ok]), h[ok])
+
+
+# ------------------------------------------------------- per-token quant
+def _bf16(x, zo):
+    return zo.f32_to_bf16(np.asarray(x, dtype=np.float32))
+
+
+def test_quant_constant_row_closed_form(zo):
+    for c in (0.5, -3.0, 127.0, 1e-3):
+        src = _bf16(np.full((1, 64), c), zo)
+        cb = float(zo.bf16_to_f32(src[0, :1])[0])
+        q, s = zo.quant_per_token(src, capi.DT_BF16)
+        assert s[0] == np.float32(abs(cb)) / np.float32(127.0)
+        assert np.all(q == (127 if c > 0 else -127))
+
+
+def test_quant_zero_row_and_nonfinite(zo):
+    src = np.zeros((3, 32), dtype=np.float32)
+    src[1, 3] = np.inf
+    src[1, 4] = np.nan
+    src[1, 5] = -np.inf
+    src[1, 6] = 2.0
+    src[2, :] = np.nan
+    q, s = zo.quant_per_token(src, capi.DT_F32)
+    assert s[0] == np.float32(1e-10)          # 1e-10/127 clamped back up to 1e-10
+    assert np.all(q[0] == 0)
+    assert s[1] == np.float32(2.0) / np.float32(127.0)   # non-finite excluded from absmax
+    assert q[1, 3] == 0 and q[1, 4] == 0 and q[1, 5] == 0 and q[1, 6] == 127
+    assert s[2] == np.float32(1e-10) and np.all(q[2] == 0)
+
+
+def test_quant_ties_round_to_even(zo):
+    # absmax 127 -> scale exactly 1 -> v/scale == v; halves must go to even
+    vals = np.array([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, 126.5, -126.5], dtype=np.float32)
+    q, s = zo.quant_per_token(vals[None, :], capi.DT_F32)
+    assert s[0] == 1.0
+    assert q[0].tolist() == [127, 0, 2, 2, 0, -2, -2, 4, 126, -126]
+
+
+def test_quant_invariants_random(zo):
+    rng = np.random.default_rng(7)
+    x = _bf16(rng.standard_normal((37, 515)), zo)
+    q, s = zo.quant_per_token(x, capi.DT_BF16)
+    xf = zo.bf16_to_f32(x)
+    assert np.all(np.abs(q.astype(np.int32)).max(axis=1) == 127)
+    assert np.array_equal(s, (np.abs(xf).max(axis=1) / np.float32(127.0)).astype(np.float32))
+    # independent evaluation of the rounding in float64 (v/s is far from a tie here or exactly on it)
+    want = np.rint((xf / s[:, None]).astype(np.float32)).astype(np.int8)
+    assert np.array_equal(q, want)
+
+
+# ------------------------------------------------------------ s32 GEMM
+def test_gemm_all_ones_closed_form(zo):
+    A = np.ones((5, 77), dtype=np.uint8)
+    B = np.ones((77, 9), dtype=np.int8)
+    acc, ov = zo.gemm_s32(A, B)
+    assert ov == 0 and np.all(acc == 77)
+
+
+def test_gemm_brute_force_python_ints_and_transposes(zo):
+    rng = np.random.default_rng(3)
+    M, K, N = 7, 19, 5
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    As = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    for a in (A, As):
+        want = [[sum(int(a[m, k]) * int(B[k, n]) for k in range(K)) for n in range(N)] for m in range(M)]
+        acc, ov = zo.gemm_s32(a, B)
+        assert ov == 0 and acc.tolist() == want
+        acc_t, _ = zo.gemm_s32(np.ascontiguousarray(a.T), np.ascontiguousarray(B.T), transA=True, transB=True)
+        assert acc_t.tolist() == want
+    # a non-symmetric case catches swapped operands: A @ B != (B.T @ A.T) elementwise unless transposed
+    assert acc.shape == (M, N)
+
+
+def test_gemm_reference_example_recipe(zo):
+    # deterministic recipe of the reference's int8 example
+    # (examples/lowoha_matmul_example.cpp:509-535): w = (i % 7) - 3, a = (i + 17*iter) % 256
+    M, K, N = 4, 64, 8
+    w = np.array([(i % 7) - 3 for i in range(K * N)], dtype=np.int8).reshape(K, N)
+    for it in range(3):
+        a = np.array([(i + 17 * it) % 256 for i in range(M * K)], dtype=np.uint8).reshape(M, K)
+        acc, ov = zo.gemm_s32(a, w)
+        want = a.astype(np.int64) @ w.astype(np.int64)
+        assert ov == 0 and np.array_equal(acc.astype(np.int64), want)
+
+
+def test_gemm_extremes_fit_int32(zo):
+    K = 14336
+    A = np.full((1, K), -128, dtype=np.int8)
+    B = np.full((K, 1), -127, dtype=np.int8)
+    acc, ov = zo.gemm_s32(A, B)
+    assert ov == 0 and acc[0, 0] == 128 * 127 * K
+
+
+def test_fast_and_general_gemm_agree(zo):
+    import ctypes as C
+    rng = np.random.default_rng(11)
+    M, K, N = 9, 300, 33
+    A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    Bt = np.empty((N, K), dtype=np.int8)
+    L = zo.lib()
+    L.zo_transpose_s8(B.ctypes.data, K, N, N, Bt.ctypes.data)
+    assert np.array_equal(Bt, B.T)
+    acc = np.empty((M, N), dtype=np.int32)
+    L.zo_gemm_s32_bt(A.ctypes.data, capi.DT_S8, K, Bt.ctypes.data, K, M, N, K, acc.ctypes.data, N)
+    assert np.array_equal(acc, A.astype(np.int32) @ B.astype(np.int32))
+
+
+# ------------------------------------------------- zero-point compensation
+def test_zp_identity(zo):
+    rng = np.random.default_rng(5)
+    M, K, N, zp = 6, 40, 11, 128
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    comp = np.empty(N, dtype=np.int32)
+    zo.lib().zo_zp_comp(B.ctypes.data, 0, N, K, N, zp, comp.ctypes.data)
+    acc, _ = zo.gemm_s32(A, B)
+    want = (A.astype(np.int64) - zp) @ B.astype(np.int64)
+    assert np.array_equal(acc.astype(np.int64) + comp[None, :], want)
+    comp0 = np.empty(N, dtype=np.int32)
+    zo.lib().zo_zp_comp(B.ctypes.data, 0, N, K, N, 0, comp0.ctypes.data)
+    assert np.all(comp0 == 0)
+
+
+# ------------------------------------------------------ dequant chain
+def _params(**kw):
+    p = capi.MatmulParamsT()
+    p.mem_format_a = b"n"
+    p.mem_format_b = b"n"
+    p.lowoha_algo = capi.ALGO_NONE
+    p.weight_cache_type = 2
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_chain_unit_scales_equals_accumulator(zo):
+    rng = np.random.default_rng(9)
+    M, K, N = 5, 48, 12
+    A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    one = np.ones(1, dtype=np.float32)
+    p = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32,
+                src_scale=capi.quant(one.ctypes.data, capi.DT_F32, (1,)),
+                wei_scale=capi.quant(one.ctypes.data, capi.DT_F32, (1,)))
+    st, dst, acc, _ = zo.matmul_int8(A, B, p, M, N, K, want_acc=True)
+    assert st == capi.SUCCESS
+    assert np.array_equal(dst[:, :N], acc.astype(np.float32))
+    # s32 destination without scales is the accumulator itself
+    p2 = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_S32)
+    st, dst2, _, _ = zo.matmul_int8(A, B, p2, M, N, K)
+    assert np.array_equal(dst2[:, :N], acc)
+
+
+def test_chain_per_channel_equal_is_per_tensor_and_order(zo):
+    rng = np.random.default_rng(10)
+    M, K, N = 4, 32, 10
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    ss = np.array([0.02], dtype=np.float32)
+    zp = np.array([128], dtype=np.int32)
+    ws1 = np.array([0.005], dtype=np.float32)
+    wsN = np.full(N, 0.005, dtype=np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    outs = []
+    for ws, dims in ((ws1, (1,)), (wsN, (1, N))):
+        p = _params(dt_src=capi.DT_U8, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32, dt_bias=capi.DT_F32,
+                    src_scale=capi.quant(ss.ctypes.data, capi.DT_F32, (1,)),
+                    src_zp=capi.quant(zp.ctypes.data, capi.DT_S32, (1,)),
+                    wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, dims))
+        st, dst, acc, _ = zo.matmul_int8(A, B, p, M, N, K, bias=bias, want_acc=True)
+        assert st == capi.SUCCESS
+        outs.append(dst.copy())
+    assert np.array_equal(outs[0], outs[1])
+    # independent statement of the chain, one float32 rounding per step
+    comp = (-128 * B.astype(np.int64).sum(axis=0)).astype(np.float32)
+    y = acc.astype(np.float32) + comp[None, :]
+    y = (y * np.float32(0.02)).astype(np.float32)
+    y = (y * wsN[None, :]).astype(np.float32)
+    y = (y + bias[None, :]).astype(np.float32)
+    assert np.array_equal(outs[0], y)
+    # and it is the dequantised product to float accuracy
+    exact = ((A.astype(np.float64) - 128) @ B.astype(np.float64)) * 0.02 * 0.005 + bias
+    assert np.allclose(outs[0], exact, rtol=1e-5, atol=1e-5)
+
+
+def test_chain_dynamic_quant_per_token(zo):
+    rng = np.random.default_rng(12)
+    M, K, N = 6, 64, 16
+    x = zo.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    p = _params(dt_src=capi.DT_BF16, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32, dt_compute=capi.DT_S8,
+                dynamic_quant=1,
+                src_scale=capi.quant(None, capi.DT_F32, (M, 1)),
+                wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, (1, N)))
+    st, dst, acc, scales = zo.matmul_int8(x, B, p, M, N, K, want_acc=True, want_scales=True)
+    assert st == capi.SUCCESS
+    q, s = zo.quant_per_token(x, capi.DT_BF16)
+    assert np.array_equal(s, scales)
+    assert np.array_equal(acc, q.astype(np.int32) @ B.astype(np.int32))
+    y = ((acc.astype(np.float32) * s[:, None]).astype(np.float32) * ws[None, :]).astype(np.float32)
+    assert np.array_equal(dst, y)
+    # close to the unquantised product (what the reference's dynamic-quant tests compare with)
+    full = zo.bf16_to_f32(x).astype(np.float64) @ (B.astype(np.float64) * ws[None, :])
+    assert np.abs(dst - full).max() < 0.02 * np.abs(full).max()
+
+
+# ------------------------------------------------------------- post-ops
+def test_eltwise_against_libm_double(zo):
+    xs = np.concatenate([np.linspace(-12, 12, 4001), [0.0, -0.0, 1e-6, -1e-6, 30.0, -30.0]]).astype(np.float32)
+    def ulp(a, b):
+        a = np.float32(a); b = np.float32(b)
+        sp = np.spacing(np.abs(b)) if b != 0 else np.float32(1e-45)
+        return abs(float(a) - float(b)) / float(sp)
+    silu = zo.eltwise(capi.PO_SWISH, xs)
+    gelu = zo.eltwise(capi.PO_GELU_TANH, xs)
+    gerf = zo.eltwise(capi.PO_GELU_ERF, xs)
+    sig = zo.eltwise(capi.PO_SIGMOID, xs)
+    for i, x in enumerate(xs.astype(np.float64)):
+        assert ulp(silu[i], x / (1 + math.exp(-x))) <= 2
+        assert ulp(sig[i], 1 / (1 + math.exp(-x))) <= 2
+        t = math.tanh(math.sqrt(2 / math.pi) * x * (1 + 0.044715 * x * x))
+        want = 0.5 * x * (1 + t)
+        # near the negative tail 1+tanh cancels; bound the absolute error there instead
+        assert ulp(gelu[i], want) <= 4 or abs(float(gelu[i]) - want) < 2e-7 * max(1.0, abs(x))
+        want_e = 0.5 * x * (1 + math.erf(x / math.sqrt(2)))
+        assert ulp(gerf[i], want_e) <= 4 or abs(float(gerf[i]) - want_e) < 2e-7 * max(1.0, abs(x))
+    assert np.array_equal(zo.eltwise(capi.PO_RELU, xs), np.maximum(xs, 0))
+    assert np.array_equal(zo.eltwise(capi.PO_CLIP, xs, -1.0, 2.0), np.clip(xs, -1.0, 2.0))
+    lr = zo.eltwise(capi.PO_LEAKY_RELU, xs)
+    assert np.array_equal(lr, np.where(xs > 0, xs, np.float32(0.01) * xs))
+
+
+# ---------------------------------------------------- gated act / reduce
+def test_gated_act_brute_force(zo):
+    rng = np.random.default_rng(13)
+    M, dim = 5, 24
+    buf = zo.f32_to_bf16(rng.standard_normal((M, 2 * dim)).astype(np.float32) * 3)
+    f = zo.bf16_to_f32(buf).astype(np.float64)
+    out = zo.gated_act(capi.ACT_SILU_AND_MUL, buf.copy(), capi.DT_BF16)
+    g, u = f[:, :dim], f[:, dim:]
+    want = zo.f32_to_bf16((g / (1 + np.exp(-g)) * u).astype(np.float32))
+    got = out[:, :dim]
+    d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 0.02       # double vs float evaluation: rare 1-ulp flips
+    assert np.array_equal(out[:, dim:], buf[:, dim:])    # the up half is left untouched
+    f32 = rng.standard_normal((M, 2 * dim)).astype(np.float32)
+    o32 = zo.gated_act(capi.ACT_SILU_AND_MUL, f32.copy(), capi.DT_F32)
+    w32 = f32[:, :dim].astype(np.float64)
+    assert np.allclose(o32[:, :dim], w32 / (1 + np.exp(-w32)) * f32[:, dim:], rtol=3e-7, atol=1e-7)
+
+
+def test_moe_reduce_closed_form_and_brute_force(zo):
+    # closed form of the reference example (examples/lowoha_group_matmul_example.cpp:320):
+    # all-ones src, expert e weight (e+1), K wide, routing weights 0.5/0.5
+    K, D = 64, 8
+    e0, e1 = 2, 5
+    rows = [np.full(D, K * (e0 + 1), dtype=np.float32), np.full(D, K * (e1 + 1), dtype=np.float32)]
+    out = zo.moe_reduce(rows, np.array([[0.5, 0.5]], dtype=np.float32), capi.DT_F32, D)
+    assert np.all(out == 0.5 * K * (e0 + 1) + 0.5 * K * (e1 + 1))
+    rng = np.random.default_rng(14)
+    T, topk, D = 6, 3, 20
+    rows = [zo.f32_to_bf16(rng.standard_normal(D).astype(np.float32)) for _ in range(T * topk)]
+    w = rng.uniform(0, 1, (T, topk)).astype(np.float32)
+    out = zo.moe_reduce(rows, w, capi.DT_BF16, D)
+    for t in range(T):
+        acc = np.zeros(D, dtype=np.float64)
+        for k in range(topk):
+            acc += float(w[t, k]) * zo.bf16_to_f32(rows[t * topk + k]).astype(np.float64)
+        want = zo.f32_to_bf16(acc.astype(np.float32), ctor=False)
+        d = np.abs(out[t].astype(np.int32) - want.astype(np.int32))
+        assert d.max() <= 1
+    ones = zo.moe_reduce(rows, w, capi.DT_BF16, D, skip_weighted=True)
+    t0 = sum(zo.bf16_to_f32(rows[k]).astype(np.float64) for k in range(topk))
+    assert np.abs(zo.bf16_to_f32(ones[0]) - t0).max() < 0.05
