@@ -34,6 +34,9 @@
 extern "C" {
 #endif
 
+/* Every entry point is exported; everything else in the library is hidden. */
+#define ZMI_API __attribute__((visibility("default")))
+
 /* ---- status_t (common/error_status.hpp:33-57) ------------------------- */
 #define ZMI_SUCCESS          1
 #define ZMI_FAILURE          0
@@ -125,13 +128,13 @@ typedef struct zmi_matmul_params_t {
 
 /* Sets every field of *p to the reference's constructor defaults
  * (matmul/lowoha_common.hpp:223-226). */
-void zmi_matmul_params_init(zmi_matmul_params_t *p);
-void zmi_batch_params_init(zmi_batch_params_t *p);
+ZMI_API void zmi_matmul_params_init(zmi_matmul_params_t *p);
+ZMI_API void zmi_batch_params_init(zmi_batch_params_t *p);
 
 /* matmul_direct (matmul/lowoha_matmul.hpp:104-108; body lowoha_matmul.cpp:278).
  * C = postops(alpha * A * B + beta * C + bias) for u8/s8 (or bf16/f32 with
  * dynamic_quant) activations x s8 weights, s32 accumulation. */
-int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB,
+ZMI_API int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB,
                           int32_t M, int32_t N, int32_t K, float alpha,
                           const void *src, int32_t lda,
                           const void *weight, int32_t ldb,
@@ -192,7 +195,7 @@ typedef struct zmi_group_args_t {
 /* group_matmul_direct (matmul/lowoha_matmul.hpp:204-223; body
  * matmul/group_matmul_direct.cpp:747).  gated_act is the value of
  * grp_matmul_gated_act_params::act, or ZMI_ACT_NONE for a null pointer. */
-int32_t zmi_group_matmul_direct(const zmi_group_args_t *args,
+ZMI_API int32_t zmi_group_matmul_direct(const zmi_group_args_t *args,
                                 const zmi_moe_postop_t *moe_postop,
                                 int32_t gated_act,
                                 const zmi_fused_moe_t *fused_moe);
@@ -225,18 +228,18 @@ typedef struct zmi_reorder_params_t {
   zmi_prepack_params_t prepack;
 } zmi_reorder_params_t;
 
-void zmi_reorder_params_init(zmi_reorder_params_t *p);
+ZMI_API void zmi_reorder_params_init(zmi_reorder_params_t *p);
 
 /* weight_prepack_size (reorder/prepack/lowoha_prepack.hpp:165; body
  * lowoha_prepack.cpp:285-313): bytes of the packed blob, a multiple of 64,
  * 0 on invalid parameters.  Also stores it in params->prepack.cached_size. */
-size_t zmi_weight_prepack_size(zmi_reorder_params_t *params);
+ZMI_API size_t zmi_weight_prepack_size(zmi_reorder_params_t *params);
 
 /* reorder_direct (reorder/lowoha_reorder.hpp:103; body lowoha_reorder.cpp:43):
  * is_prepack   -> pack [K,N] s8 weights into the MFMA-fragment blob at dst;
  * dynamic_quant-> per-token symmetric bf16/f32 -> s8 with scales written to
  *                 params->scale.buff (dst may be NULL: scales only). */
-int32_t zmi_reorder_direct(const void *src, void *dst,
+ZMI_API int32_t zmi_reorder_direct(const void *src, void *dst,
                            zmi_reorder_params_t *params);
 
 /* group_dynamic_quant_params_t (reorder/lowoha_reorder_common.hpp:357-368). */
@@ -249,7 +252,7 @@ typedef struct zmi_group_dq_params_t {
 /* group_dynamic_quant (reorder/lowoha_reorder.hpp:120-128; body
  * lowoha_reorder.cpp:279).  n matrices; strides are {row, col} pairs in
  * elements, row stride 0 meaning contiguous. */
-int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src,
+ZMI_API int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src,
                                 const int32_t *M, const int32_t *K,
                                 const int64_t *src_row_stride,
                                 void *const *dst,
@@ -261,22 +264,22 @@ int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src,
 
 /* Selects the GPU (hipSetDevice) and creates the per-device state.  Optional:
  * the first compute call does it for device 0. */
-int32_t zmi_init(int32_t device);
+ZMI_API int32_t zmi_init(int32_t device);
 /* hipStream_t used by the calling thread's later calls (NULL = null stream). */
-void zmi_set_stream(void *hip_stream);
-void *zmi_get_stream(void);
+ZMI_API void zmi_set_stream(void *hip_stream);
+ZMI_API void *zmi_get_stream(void);
 /* Text of the calling thread's most recent failure ("" if none). */
-const char *zmi_last_error(void);
+ZMI_API const char *zmi_last_error(void);
 /* Name of the kernel variant the calling thread's last compute call used. */
-const char *zmi_last_kernel(void);
+ZMI_API const char *zmi_last_kernel(void);
 /* Frees the packed-weight cache kept for mem_format_b == 'n' constant weights
  * (reference: clear_aocl_matmul_weight_caches, backends/aocl/aocl_kernel.cpp:294). */
-void zmi_clear_weight_cache(void);
+ZMI_API void zmi_clear_weight_cache(void);
 /* Frees the calling thread's scratch arena (reference: clear_fused_moe_scratch,
  * group_matmul/group_matmul_direct.hpp:683). */
-void zmi_clear_scratch(void);
+ZMI_API void zmi_clear_scratch(void);
 /* Library version string. */
-const char *zmi_version(void);
+ZMI_API const char *zmi_version(void);
 
 /* Device-side MoE routing glue.  In the reference the framework scatters
  * tokens to experts on the host (docs/operator/low_overhead_operator/
@@ -289,7 +292,7 @@ const char *zmi_version(void);
  *   slot_of[T*topk] position of (t,k) in the expert-sorted row order
  *                  (stable: within an expert rows keep (t,k) order).
  * All outputs are device s32 buffers. */
-int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk,
+ZMI_API int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk,
                       int32_t E, int32_t *counts, int32_t *offsets,
                       int32_t *slot_of);
 
@@ -304,14 +307,14 @@ typedef struct zmi_moe_device_t {
   const void *x;  int32_t ldx;              /* bf16 [T, ldx] */
   const int32_t *topk_ids;                  /* [T, topk] */
   const float *topk_weights;                /* [T, topk] */
-  const void *const *w13_blob;              /* host array [E] of gated prepack blobs [H, 2I] */
+  const void *const *w13_blob;              /* host array [E] of prepack blobs of [H, 2I] = [gate | up] */
   const void *const *w2_blob;               /* host array [E] of prepack blobs [I, H] */
   const float *const *w13_scale;            /* host array [E] of device f32 [2I] */
   const float *const *w2_scale;             /* host array [E] of device f32 [H] */
   int32_t gated_act;
   void *out; int32_t ldo;                   /* bf16 [T, ldo] */
 } zmi_moe_device_t;
-int32_t zmi_moe_fused_device(const zmi_moe_device_t *d);
+ZMI_API int32_t zmi_moe_fused_device(const zmi_moe_device_t *d);
 
 #ifdef __cplusplus
 }

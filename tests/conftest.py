@@ -18,3 +18,15 @@ def zo():
     from oracle import build, oracle
     build.build(force=False)
     return oracle
+
+
+@pytest.fixture(autouse=True)
+def _fresh_weight_cache(request):
+    """The packed-weight cache is keyed by weight address (as the reference's is)
+    and is_weights_const promises that address keeps its contents.  Tests free
+    and reallocate weights at recycled addresses, so each GPU test starts with
+    an empty cache."""
+    yield
+    if request.node.get_closest_marker("gpu") is not None:
+        from zendnn_amd import capi
+        capi.load().zmi_clear_weight_cache()

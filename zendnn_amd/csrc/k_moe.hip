@@ -1,0 +1,271 @@
+// MoE glue kernels for gfx950: stand-alone gated activation, weighted reduce
+// (combine), device-side routing (histogram / scan / stable slot assignment),
+// quantize-and-scatter, and the per-expert problem table.  All HBM-bound.
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+// ---------------------------------------------------------------------------
+// Gated activation in place: buf[m, 0:dim] = act(gate) * up, dim = N/2.
+// Reference: group_matmul_moe_act_execute / apply_gated_act_inplace
+// (zendnnl/src/lowoha_operators/matmul/group_matmul/group_matmul_moe_act.cpp:88-254).
+// One workgroup per row.  Results are staged in LDS and written after a
+// barrier because swiglu_oai's interleaved layout overlaps reads and writes.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void zmi_gated_act_kernel(ZmiActMat m0, const ZmiActMat *mats, int n_mat,
+                                                            int act, int dt) {
+  extern __shared__ float res[];
+  const int row = blockIdx.x;
+  ZmiActMat m = m0;
+  if (mats) {
+    int lo = 0, hi = n_mat - 1;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) / 2;
+      if (mats[mid].row_start <= row) lo = mid; else hi = mid - 1;
+    }
+    m = mats[lo];
+  }
+  const int r = row - m.row_start;
+  if (r >= m.M) return;
+  const int dim = m.N / 2;
+  const int64_t base = (int64_t)r * m.ld;
+  for (int n = threadIdx.x; n < dim; n += blockDim.x) {
+    float g, u;
+    if (act == ZMI_ACT_SWIGLU_OAI_MUL) {
+      g = zmi_ld_f32(m.buf, dt, base + 2 * n);
+      u = zmi_ld_f32(m.buf, dt, base + 2 * n + 1);
+    } else {
+      g = zmi_ld_f32(m.buf, dt, base + n);
+      u = zmi_ld_f32(m.buf, dt, base + dim + n);
+    }
+    res[n] = zmi_gated(act, g, u);
+  }
+  __syncthreads();
+  for (int n = threadIdx.x; n < dim; n += blockDim.x) {
+    if (dt == ZMI_DT_BF16) ((uint16_t *)m.buf)[base + n] = zmi_f32_to_bf16(res[n]);
+    else ((float *)m.buf)[base + n] = res[n];
+  }
+}
+
+hipError_t zmi_launch_gated_act(const ZmiActMat *mats_dev, const ZmiActMat *mat0, int n_mat,
+                                int64_t total_rows, int max_N, int32_t act, int32_t dt, hipStream_t stream) {
+  if (total_rows <= 0) return hipSuccess;
+  const size_t smem = (size_t)(max_N / 2) * sizeof(float);
+  if (smem > 160 * 1024) return hipErrorInvalidValue;
+  static size_t attr = 0;
+  if (smem > attr) {
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gated_act_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr = smem;
+  }
+  ZmiActMat m0 = {};
+  if (mat0) m0 = *mat0;
+  hipLaunchKernelGGL(zmi_gated_act_kernel, dim3((unsigned)total_rows), dim3(256), smem, stream, m0, mats_dev,
+                     n_mat, act, dt);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Weighted reduce: out[t, d] = sum_k w[t,k] * row(t,k)[d], f32 accumulation in
+// k order, first term a plain product, then fused multiply-adds; bf16 store
+// with the plain round-to-nearest-even bit trick.
+// Reference: moe_weighted_reduce_avx512_{bf16,f32}
+// (group_matmul/group_matmul_moe_postop.cpp:191-286).
+// Rows come either from a table of pointers (the reference's row_ptrs) or from
+// rows_base + slot_of[t*topk+k] * row_ld (device-side routing).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void zmi_moe_combine_kernel(const void *const *row_ptrs, const void *rows_base,
+                                                              int64_t row_ld, const int32_t *slot_of,
+                                                              const float *weights, int skip_weighted, int topk,
+                                                              int D, int dt, void *out, int64_t ldo) {
+  const int t = blockIdx.x;
+  const size_t es = dt == ZMI_DT_BF16 ? 2 : 4;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.0f;
+    for (int k = 0; k < topk; ++k) {
+      const int s = t * topk + k;
+      const void *row = row_ptrs ? row_ptrs[s]
+                                 : (const void *)((const char *)rows_base + (int64_t)slot_of[s] * row_ld * es);
+      const float w = skip_weighted ? 1.0f : weights[s];
+      const float x = zmi_ld_f32(row, dt, d);
+      acc = (k == 0) ? __fmul_rn(w, x) : __builtin_fmaf(w, x, acc);
+    }
+    if (dt == ZMI_DT_BF16) ((uint16_t *)out)[(int64_t)t * ldo + d] = zmi_f32_to_bf16_rne(acc);
+    else ((float *)out)[(int64_t)t * ldo + d] = acc;
+  }
+}
+
+hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *rows_base, int64_t row_ld,
+                                  const int32_t *slot_of, const float *weights, int skip_weighted, int T,
+                                  int topk, int D, int32_t dt, void *out, int64_t ldo, hipStream_t stream) {
+  if (T <= 0) return hipSuccess;
+  hipLaunchKernelGGL(zmi_moe_combine_kernel, dim3((unsigned)T), dim3(256), 0, stream, row_ptrs_dev, rows_base,
+                     row_ld, slot_of, weights, skip_weighted, topk, D, dt, out, ldo);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Routing.  One workgroup of 16 wavefronts; wavefront w owns the contiguous
+// segment w of the flat (t,k) index space.
+//   A: per-wavefront histograms hist[w][e] (LDS atomics);
+//   B: counts / exclusive offsets per expert, and cursor[w][e] = offsets[e] +
+//      sum of hist[w'][e] for w' < w;
+//   C: every wavefront walks its segment in order, 64 entries at a time; an
+//      entry's slot is cursor + (number of lower lanes with the same expert).
+// The order inside an expert is therefore the (t,k) order: deterministic.
+// ---------------------------------------------------------------------------
+#define RT_WAVES 16
+
+__global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int32_t *topk_ids, int n, int E,
+                                                                      int32_t *counts, int32_t *offsets,
+                                                                      int32_t *slot_of) {
+  extern __shared__ int32_t sh[];   // hist[RT_WAVES][E], then off[E+1]
+  int32_t *hist = sh;
+  int32_t *off = sh + RT_WAVES * E;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  for (int i = tid; i < RT_WAVES * E; i += blockDim.x) hist[i] = 0;
+  __syncthreads();
+  const int seg = (n + RT_WAVES - 1) / RT_WAVES;
+  const int s0 = wave * seg, s1 = (s0 + seg < n) ? s0 + seg : n;
+  for (int i = s0 + lane; i < s1; i += 64) {
+    const int e = topk_ids[i];
+    if (e >= 0 && e < E) atomicAdd(&hist[wave * E + e], 1);
+  }
+  __syncthreads();
+  // per-expert totals and the per-wavefront running starts (thread e handles expert e)
+  for (int e = tid; e < E; e += blockDim.x) {
+    int run = 0;
+    for (int w = 0; w < RT_WAVES; ++w) {
+      const int c = hist[w * E + e];
+      hist[w * E + e] = run;
+      run += c;
+    }
+    off[e] = run;
+    counts[e] = run;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) { const int c = off[e]; off[e] = run; offsets[e] = run; run += c; }
+    off[E] = run;
+    offsets[E] = run;
+  }
+  __syncthreads();
+  for (int i0 = s0; i0 < s1; i0 += 64) {
+    const int i = i0 + lane;
+    const bool live = i < s1;
+    int e = live ? topk_ids[i] : -1;
+    const bool ok = live && e >= 0 && e < E;
+    if (!ok) e = -1;
+    // lanes holding the same expert as this lane
+    unsigned long long same = __ballot(ok);
+    for (int bit = 0; bit < 11; ++bit) {
+      const unsigned long long b = __ballot((e >> bit) & 1);
+      same &= ((e >> bit) & 1) ? b : ~b;
+    }
+    if (ok) {
+      const int rank = __popcll(same & ((1ull << lane) - 1ull));
+      const int total = __popcll(same);
+      const int start = hist[wave * E + e];
+      slot_of[i] = off[e] + start + rank;
+      // the last lane of each expert group advances the cursor for the next 64 entries
+      if (rank == total - 1) hist[wave * E + e] = start + total;
+    } else if (live) {
+      slot_of[i] = -1;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int32_t *counts,
+                                int32_t *offsets, int32_t *slot_of, hipStream_t stream) {
+  if (E > 2047 || E <= 0) return hipErrorInvalidValue;
+  const size_t smem = ((size_t)RT_WAVES * E + E + 1) * sizeof(int32_t);
+  static size_t attr = 0;
+  if (smem > attr) {
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_moe_route_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr = smem;
+  }
+  hipLaunchKernelGGL(zmi_moe_route_kernel, dim3(1), dim3(RT_WAVES * 64), smem, stream, topk_ids, T * topk, E,
+                     counts, offsets, slot_of);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Quantize token t once (per-token symmetric s8, same arithmetic as
+// k_quant.hip) and write the row and its scale to each of its topk slots.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void zmi_moe_quant_scatter_kernel(const uint16_t *x, int64_t ldx, int H, int topk,
+                                                                    const int32_t *slot_of, int8_t *A1, float *s1) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const uint16_t *row = x + (int64_t)t * ldx;
+  float amax = 0.0f;
+  for (int k = threadIdx.x; k < H; k += blockDim.x) {
+    const float a = fabsf(zmi_bf16_to_f32(row[k]));
+    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+  }
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (threadIdx.x % 64 == 0) red[threadIdx.x / 64] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  for (int k = threadIdx.x; k < H; k += blockDim.x) {
+    const float v = zmi_bf16_to_f32(row[k]);
+    int8_t q = 0;
+    if ((__float_as_uint(v) & 0x7f800000u) != 0x7f800000u) q = (int8_t)(int32_t)rintf(__fdiv_rn(v, s));
+    for (int j = 0; j < topk; ++j) {
+      const int slot = slot_of[t * topk + j];
+      if (slot >= 0) A1[(int64_t)slot * H + k] = q;
+    }
+  }
+  if (threadIdx.x < topk) {
+    const int slot = slot_of[t * topk + threadIdx.x];
+    if (slot >= 0) s1[slot] = s;
+  }
+}
+
+hipError_t zmi_launch_moe_quant_scatter(const void *x, int64_t ldx, int T, int H, int topk,
+                                        const int32_t *slot_of, int8_t *A1, float *s1, hipStream_t stream) {
+  if (T <= 0) return hipSuccess;
+  hipLaunchKernelGGL(zmi_moe_quant_scatter_kernel, dim3((unsigned)T), dim3(256), 0, stream, (const uint16_t *)x,
+                     ldx, H, topk, slot_of, A1, s1);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Per-expert problem tables for Op1 (gate|up) and Op2 (down) from the device
+// side counts / offsets.
+// ---------------------------------------------------------------------------
+__global__ void zmi_moe_build_problems_kernel(ZmiMoeTables tb, int E, int H, int I, const int32_t *counts,
+                                              const int32_t *offsets, const int8_t *A1, const float *s1,
+                                              uint16_t *act, const int8_t *A2, const float *s2, uint16_t *Y,
+                                              ZmiProblem *op1, ZmiProblem *op2) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= E) return;
+  const int64_t o = offsets[e];
+  ZmiProblem a = {};
+  a.A = A1 + o * H; a.lda = H; a.blob = (const uint8_t *)tb.w13_blob[e];
+  a.dst = act + o * I; a.ldc = I; a.M = counts[e]; a.N = 2 * I; a.K = H; a.a_is_u8 = 0;
+  a.src_scale_ptr = s1 + o; a.wei_scale_ptr = tb.w13_scale[e];
+  op1[e] = a;
+  ZmiProblem b = {};
+  b.A = A2 + o * I; b.lda = I; b.blob = (const uint8_t *)tb.w2_blob[e];
+  b.dst = Y + o * H; b.ldc = H; b.M = counts[e]; b.N = H; b.K = I; b.a_is_u8 = 0;
+  b.src_scale_ptr = s2 + o; b.wei_scale_ptr = tb.w2_scale[e];
+  op2[e] = b;
+}
+
+hipError_t zmi_launch_moe_build_problems(ZmiMoeTables tb, int E, int H, int I, const int32_t *counts,
+                                         const int32_t *offsets, const int8_t *A1, const float *s1, void *act,
+                                         const int8_t *A2, const float *s2, void *Y, ZmiProblem *op1,
+                                         ZmiProblem *op2, hipStream_t stream) {
+  hipLaunchKernelGGL(zmi_moe_build_problems_kernel, dim3((E + 63) / 64), dim3(64), 0, stream, tb, E, H, I, counts,
+                     offsets, A1, s1, (uint16_t *)act, A2, s2, (uint16_t *)Y, op1, op2);
+  return hipGetLastError();
+}

@@ -1,0 +1,230 @@
+// Per-token symmetric dynamic quantization, bf16/f32 rows -> s8 rows + one f32
+// scale per row.  HBM-bound: M*K*2 bytes read, M*K + 4M written.
+//
+// Arithmetic of the reference's dynamic_per_token_quant_bf16_s8_native
+// (zendnnl/src/lowoha_operators/reorder/reorder_data_type/dynamic_quant_impl/
+// per_token_avx512_f32_fma_kernel.cpp:207-303; scalar twin
+// scalar_impl/dynamic_per_token_ref_kernel.cpp:70-96): absmax over the finite
+// values of the row, scale = max(absmax, 1e-10) / 127 clamped to >= 1e-10,
+// q = (int8) rint(v / scale) with a correctly rounded division, non-finite -> 0.
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+#define QT_THREADS 256
+#define QT_MAX_CHUNKS 8   // rows up to 256 * 8 * 8 = 16384 elements stay in registers
+
+__device__ __forceinline__ float zmi_block_max(float v, float *red) {
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  const int w = threadIdx.x / 64;
+  if (threadIdx.x % 64 == 0) red[w] = v;
+  __syncthreads();
+  float r = red[0];
+  #pragma unroll
+  for (int i = 1; i < QT_THREADS / 64; ++i) r = fmaxf(r, red[i]);
+  __syncthreads();
+  return r;
+}
+
+__device__ __forceinline__ int8_t zmi_quant_one(float v, float scale) {
+  // isfinite
+  if ((__float_as_uint(v) & 0x7f800000u) == 0x7f800000u) return 0;
+  return (int8_t)(int32_t)rintf(__fdiv_rn(v, scale));
+}
+
+template <bool BF16>
+__device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, void *scale, int scale_dt,
+                                              int K, float *red) {
+  const int t = threadIdx.x;
+  const bool vec_ok = (K % 8 == 0) && (((uintptr_t)srcv) % 16 == 0) &&
+                      (dst == nullptr || ((uintptr_t)dst) % 8 == 0);
+  if (vec_ok && K <= QT_THREADS * 8 * QT_MAX_CHUNKS) {
+    // 8 elements per thread per chunk, the row is held in registers between the passes
+    float v[QT_MAX_CHUNKS][8];
+    float amax = 0.0f;
+    #pragma unroll
+    for (int c = 0; c < QT_MAX_CHUNKS; ++c) {
+      const int k = (c * QT_THREADS + t) * 8;
+      if (k < K) {
+        if (BF16) {
+          v4i raw = *(const v4i *)((const uint16_t *)srcv + k);
+          #pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[c][2 * j] = __uint_as_float(((uint32_t)raw[j]) << 16);
+            v[c][2 * j + 1] = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+          }
+        } else {
+          const float4 *p = (const float4 *)((const float *)srcv + k);
+          float4 a = p[0], b = p[1];
+          v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
+          v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
+        }
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float a = fabsf(v[c][j]);
+          if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+        }
+      }
+    }
+    amax = zmi_block_max(amax, red);
+    if (amax < 1e-10f) amax = 1e-10f;
+    float s = __fdiv_rn(amax, 127.0f);
+    if (s < 1e-10f) s = 1e-10f;
+    if (t == 0) {
+      if (scale_dt == ZMI_DT_BF16) *(uint16_t *)scale = zmi_f32_to_bf16_rne(s);
+      else *(float *)scale = s;
+    }
+    if (!dst) return;
+    #pragma unroll
+    for (int c = 0; c < QT_MAX_CHUNKS; ++c) {
+      const int k = (c * QT_THREADS + t) * 8;
+      if (k < K) {
+        __attribute__((aligned(8))) int8_t q[8];
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = zmi_quant_one(v[c][j], s);
+        *(uint2 *)(dst + k) = *(const uint2 *)q;
+      }
+    }
+    return;
+  }
+  // generic path: any K, any alignment; the row is read twice
+  float amax = 0.0f;
+  for (int k = t; k < K; k += QT_THREADS) {
+    float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)srcv)[k]) : ((const float *)srcv)[k];
+    float a = fabsf(x);
+    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+  }
+  amax = zmi_block_max(amax, red);
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  if (t == 0) {
+    if (scale_dt == ZMI_DT_BF16) *(uint16_t *)scale = zmi_f32_to_bf16_rne(s);
+    else *(float *)scale = s;
+  }
+  if (!dst) return;
+  for (int k = t; k < K; k += QT_THREADS) {
+    float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)srcv)[k]) : ((const float *)srcv)[k];
+    dst[k] = zmi_quant_one(x, s);
+  }
+}
+
+// One workgroup per row.  mats has n_mat entries (device memory when n_mat > 1,
+// otherwise passed by value through mat0).
+template <bool BF16>
+__global__ __launch_bounds__(QT_THREADS) void zmi_quant_rows_kernel(ZmiQuantMat mat0,
+                                                                    const ZmiQuantMat *mats, int n_mat,
+                                                                    int scale_dt) {
+  __shared__ float red[QT_THREADS / 64];
+  const int row = blockIdx.x;
+  ZmiQuantMat m = mat0;
+  if (mats) {
+    // find the matrix that owns this global row (row_start is ascending)
+    int lo = 0, hi = n_mat - 1;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) / 2;
+      if (mats[mid].row_start <= row) lo = mid; else hi = mid - 1;
+    }
+    m = mats[lo];
+  }
+  const int r = row - m.row_start;
+  if (r >= m.M) return;
+  const size_t es = BF16 ? 2 : 4;
+  const void *src = (const char *)m.src + (size_t)r * m.ld_src * es;
+  int8_t *dst = m.dst ? m.dst + (size_t)r * m.ld_dst : nullptr;
+  void *sc = (char *)m.scale + (size_t)r * (scale_dt == ZMI_DT_BF16 ? 2 : 4);
+  zmi_quant_row<BF16>(src, dst, sc, scale_dt, m.K, red);
+}
+
+hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
+                                 int8_t *dst, int64_t ld_dst, void *scales, int32_t scale_dt,
+                                 hipStream_t stream) {
+  if (M <= 0) return hipSuccess;
+  ZmiQuantMat m;
+  m.src = src; m.dst = dst; m.scale = scales; m.ld_src = ld_src; m.ld_dst = ld_dst;
+  m.M = (int32_t)M; m.K = (int32_t)K; m.row_start = 0;
+  if (src_dt == ZMI_DT_BF16)
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, m,
+                       (const ZmiQuantMat *)nullptr, 1, scale_dt);
+  else
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, m,
+                       (const ZmiQuantMat *)nullptr, 1, scale_dt);
+  return hipGetLastError();
+}
+
+hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_t total_rows,
+                                  int32_t src_dt, int32_t scale_dt, hipStream_t stream) {
+  if (total_rows <= 0) return hipSuccess;
+  ZmiQuantMat m0 = {};
+  if (src_dt == ZMI_DT_BF16)
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)total_rows), dim3(QT_THREADS), 0,
+                       stream, m0, mats_dev, n_mat, scale_dt);
+  else
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<false>, dim3((unsigned)total_rows), dim3(QT_THREADS), 0,
+                       stream, m0, mats_dev, n_mat, scale_dt);
+  return hipGetLastError();
+}
+
+// Per-tensor dynamic scale (src_scale dims {1} / {1,1}): absmax over the whole
+// tensor, then every row is quantized with that one scale (reference:
+// zendnnl/src/lowoha_operators/reorder/lowoha_reorder_utils.cpp:724-761).  Two
+// small kernels: a grid-wide max through an ordered-int atomicMax, then the
+// element-wise quantization; scales[m] is filled for every row so the GEMM can
+// treat the result as per-token.
+template <bool BF16>
+__global__ __launch_bounds__(QT_THREADS) void zmi_absmax_kernel(const void *src, int64_t M, int64_t K,
+                                                                int64_t ld, unsigned int *amax_bits) {
+  __shared__ float red[QT_THREADS / 64];
+  const int64_t row = blockIdx.x;
+  float amax = 0.0f;
+  for (int64_t k = threadIdx.x; k < K; k += QT_THREADS) {
+    float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)src)[row * ld + k]) : ((const float *)src)[row * ld + k];
+    float a = fabsf(x);
+    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+  }
+  amax = zmi_block_max(amax, red);
+  // non-negative floats order like their bit patterns
+  if (threadIdx.x == 0) atomicMax(amax_bits, __float_as_uint(amax));
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(QT_THREADS) void zmi_quant_tensor_kernel(const void *src, int64_t M, int64_t K,
+                                                                      int64_t ld, int8_t *dst, int64_t ld_dst,
+                                                                      float *scales,
+                                                                      const unsigned int *amax_bits) {
+  const int64_t row = blockIdx.x;
+  float amax = __uint_as_float(*amax_bits);
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  if (threadIdx.x == 0) scales[row] = s;
+  if (!dst) return;
+  for (int64_t k = threadIdx.x; k < K; k += QT_THREADS) {
+    float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)src)[row * ld + k]) : ((const float *)src)[row * ld + k];
+    dst[row * ld_dst + k] = zmi_quant_one(x, s);
+  }
+}
+
+__global__ void zmi_zero_u32_kernel(unsigned int *p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
+                                   int8_t *dst, int64_t ld_dst, float *scales, unsigned int *amax_scratch,
+                                   hipStream_t stream) {
+  if (M <= 0) return hipSuccess;
+  hipLaunchKernelGGL(zmi_zero_u32_kernel, dim3(1), dim3(64), 0, stream, amax_scratch, 1);
+  if (src_dt == ZMI_DT_BF16) {
+    hipLaunchKernelGGL(zmi_absmax_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src, M, K,
+                       ld_src, amax_scratch);
+    hipLaunchKernelGGL(zmi_quant_tensor_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src,
+                       M, K, ld_src, dst, ld_dst, scales, amax_scratch);
+  } else {
+    hipLaunchKernelGGL(zmi_absmax_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src, M, K,
+                       ld_src, amax_scratch);
+    hipLaunchKernelGGL(zmi_quant_tensor_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src,
+                       M, K, ld_src, dst, ld_dst, scales, amax_scratch);
+  }
+  return hipGetLastError();
+}

@@ -1,0 +1,256 @@
+// Small-M (decode) int8 GEMM for gfx950 (HBM-bound weight streaming):
+// C[M<=128, N] = epilogue(A[M,K] x blob).
+//
+// Replaces, for decode shapes, the same aocl_gemm_s8s8s32o*_sym_quant call site
+// as the large-M kernel (zendnnl/src/lowoha_operators/matmul/backends/aocl/
+// aocl_kernel.cpp:1239-1257) and the reference's in-house decode microkernel
+// (matmul/group_matmul/custom_kernel/ukernel/int8_microkernel.cpp:196-606).
+//
+// The weights (K*N bytes) dominate the traffic and each byte is used once, so
+// the kernel is organised around streaming them at full HBM rate:
+//   * one workgroup per 32-column block of the blob (contiguous K_pad*32 bytes);
+//   * its W wavefronts split K: wavefront w streams one contiguous slice with
+//     16-byte-per-lane loads (all 64 lanes hit whole 256-byte segments) and keeps
+//     several loads in flight before the first MFMA;
+//   * the few activation rows come from L2 straight into the A operand
+//     registers; v_mfma_i32_16x16x64_i8 turns each 2 KiB of weights into two
+//     16x16 partial tiles per 16 rows;
+//   * the W partial tiles are summed through LDS (integer, so the order is
+//     immaterial and the result is bit-exact) and the epilogue runs once.
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+template <int MB, int UNROLL>
+__global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, const ZmiProblem *probs,
+                                                               int n_prob, int m_lo, int m_hi,
+                                                               ZmiEpilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) int32_t red[];   // [W][MB*2*4*64]
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int W = blockDim.x / 64;
+  const bool gated = epi.gated_act != 0;
+
+  // ---- which problem / column block ----
+  ZmiProblem p = p0;
+  int blk = blockIdx.x;
+  if (probs) {
+    int base = 0, e = 0;
+    for (; e < n_prob; ++e) {
+      const int M = probs[e].M;
+      if (!(M > m_lo && M <= m_hi)) continue;
+      const int cnt = gated ? probs[e].N / 2 / 16 : (int)(zmi_blob_npad(probs[e].N) / 32);
+      if (blk < base + cnt) break;
+      base += cnt;
+    }
+    if (e == n_prob) return;
+    p = probs[e];
+    blk -= base;
+  }
+  const int M = p.M, N = p.N, K = p.K;
+  const int64_t K_pad = zmi_blob_kpad(K);
+  const int64_t kblocks = K_pad / 32;
+  const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+
+  // the two 16-column groups h = 0, 1 this workgroup multiplies: weight column
+  // wcol[h], stored to output column ocol[h] (gated: h=0 gate, h=1 up, one output)
+  int wcol[2], ocol[2];
+  if (!gated) {
+    wcol[0] = blk * 32; wcol[1] = blk * 32 + 16;
+    ocol[0] = wcol[0]; ocol[1] = wcol[1];
+  } else {
+    wcol[0] = blk * 16; wcol[1] = blk * 16 + N / 2;
+    ocol[0] = blk * 16; ocol[1] = blk * 16;
+  }
+
+  // lane role inside a 16x16x64 operand: column / row c16, k group g (16 bytes each)
+  const int c16 = lane % 16, g = lane / 16;
+  const uint8_t *bsrc[2];
+  #pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t nb = wcol[h] / 32;
+    const int coff = wcol[h] % 32;
+    // fragment (nb, 2c + g/2), lane (g%2)*32 + coff + c16
+    bsrc[h] = tiles + (nb * kblocks + g / 2) * 1024 + ((g % 2) * 32 + coff + c16) * 16;
+  }
+  const int8_t *A = (const int8_t *)p.A;
+  const uint32_t xor_mask = p.a_is_u8 ? 0x80808080u : 0u;
+
+  v4i acc[MB][2];
+  #pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+    #pragma unroll
+    for (int h = 0; h < 2; ++h) acc[mb][h] = (v4i){0, 0, 0, 0};
+
+  const int nchunks = (int)(K_pad / 64);
+  const int c_begin = (int)((int64_t)wave * nchunks / W);
+  const int c_end = (int)((int64_t)(wave + 1) * nchunks / W);
+
+  for (int c = c_begin; c < c_end; c += UNROLL) {
+    v4i b[UNROLL][2], a[UNROLL][MB];
+    #pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int cc = c + u;
+      if (cc < c_end) {
+        b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)cc * 2048);
+        b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)cc * 2048);
+      } else {
+        b[u][0] = (v4i){0, 0, 0, 0};
+        b[u][1] = (v4i){0, 0, 0, 0};
+      }
+    }
+    #pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int cc = c + u;
+      const int k = cc * 64 + g * 16;
+      #pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int r = mb * 16 + c16;
+        v4i v = {0, 0, 0, 0};
+        if (cc < c_end && r < M && k < K) {
+          v = *(const v4i *)(A + (int64_t)r * p.lda + k);
+          if (xor_mask) { v[0] ^= xor_mask; v[1] ^= xor_mask; v[2] ^= xor_mask; v[3] ^= xor_mask; }
+        }
+        a[u][mb] = v;
+      }
+    }
+    #pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      #pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        acc[mb][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u][mb], b[u][0], acc[mb][0], 0, 0, 0);
+        acc[mb][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u][mb], b[u][1], acc[mb][1], 0, 0, 0);
+      }
+  }
+
+  // ---- cross-wavefront reduction through LDS ----
+  constexpr int PER_WAVE = MB * 2 * 4 * 64;
+  #pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+    #pragma unroll
+    for (int h = 0; h < 2; ++h)
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) red[wave * PER_WAVE + ((mb * 2 + h) * 4 + j) * 64 + lane] = acc[mb][h][j];
+  __syncthreads();
+
+  const void *bias = p.bias;
+  const int rows = M < MB * 16 ? M : MB * 16;
+
+  // acc[mb][h][j] of lane l is row mb*16 + (l/16)*4 + j, column h*16 + l%16
+  auto fetch = [&](int row, int h, int cidx) -> int32_t {
+    const int mb = row / 16, rr = row % 16;
+    const int off = ((mb * 2 + h) * 4 + rr % 4) * 64 + (rr / 4) * 16 + cidx;
+    int32_t s = 0;
+    for (int w = 0; w < W; ++w) s += red[w * PER_WAVE + off];
+    return s;
+  };
+
+  if (!gated) {
+    const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
+    for (int e = tid; e < rows * 32; e += blockDim.x) {
+      const int row = e / 32, col = e % 32;
+      const int h = col / 16, cidx = col % 16;
+      const int n = ocol[h] + cidx;
+      if (n >= N) continue;
+      const int32_t s = fetch(row, h, cidx);
+      ZmiColCtx cc = zmi_col_ctx(epi, p, colsum, n, N);
+      const int64_t o = (int64_t)row * p.ldc + n;
+      if (raw) {
+        ((int32_t *)p.dst)[o] = s + cc.comp;
+      } else {
+        const float rs = zmi_row_scale(epi, p, row);
+        zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, cc, rs, row, n, p.dst, p.ldc));
+      }
+    }
+  } else {
+    const int half = N / 2;
+    for (int e = tid; e < rows * 16; e += blockDim.x) {
+      const int row = e / 16, cidx = e % 16;
+      const int n = ocol[0] + cidx;
+      if (n >= half) continue;
+      const int32_t sg = fetch(row, 0, cidx), su = fetch(row, 1, cidx);
+      ZmiColCtx cg = zmi_col_ctx(epi, p, colsum, n, N);
+      ZmiColCtx cu = zmi_col_ctx(epi, p, colsum, n + half, N);
+      const float rs = zmi_row_scale(epi, p, row);
+      float gv = zmi_epilogue_value(epi, sg, cg, rs, row, n, p.dst, p.ldc);
+      float uv = zmi_epilogue_value(epi, su, cu, rs, row, n + half, p.dst, p.ldc);
+      if (epi.dst_dt == ZMI_DT_BF16) {
+        gv = zmi_bf16_to_f32(zmi_f32_to_bf16(gv));
+        uv = zmi_bf16_to_f32(zmi_f32_to_bf16(uv));
+      }
+      zmi_store(p.dst, epi.dst_dt, (int64_t)row * p.ldc + n, zmi_gated(epi.gated_act, gv, uv));
+    }
+  }
+}
+
+template <int MB, int UNROLL>
+static hipError_t launch_small(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int m_lo, int m_hi,
+                               int grid, int W, const ZmiEpilogue &epi, hipStream_t stream) {
+  const size_t smem = (size_t)W * MB * 2 * 4 * 64 * sizeof(int32_t);
+  static size_t attr_smem = 0;
+  if (smem > attr_smem) {
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_smallm_kernel<MB, UNROLL>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr_smem = smem;
+  }
+  hipLaunchKernelGGL((zmi_gemm_smallm_kernel<MB, UNROLL>), dim3(grid), dim3(W * 64), smem, stream, p0, probs,
+                     n_prob, m_lo, m_hi, epi);
+  return hipGetLastError();
+}
+
+// Picks the number of K-splitting wavefronts: enough workgroups*wavefronts to
+// keep about 8 wavefronts on every one of the 256 CUs, bounded by the chunks
+// available, by 16 wavefronts per workgroup and by the LDS the reduction needs.
+static int pick_waves(int grid, int MB, int64_t K_pad) {
+  const int nchunks = (int)(K_pad / 64);
+  int W = 4;
+  while (W < 16 && (int64_t)grid * W < 2048) W *= 2;
+  while (W > 1 && (size_t)W * MB * 2048 > 128 * 1024) W /= 2;
+  while (W > 1 && W > nchunks) W /= 2;
+  return W;
+}
+
+static hipError_t dispatch_small(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int m_lo,
+                                 int m_hi, int grid, int64_t K_pad, const ZmiEpilogue &epi,
+                                 hipStream_t stream) {
+  if (grid <= 0) return hipSuccess;
+  const int mb = (m_hi + 15) / 16;
+  if (mb <= 1) return launch_small<1, 4>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 1, K_pad), epi, stream);
+  if (mb <= 2) return launch_small<2, 4>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 2, K_pad), epi, stream);
+  if (mb <= 4) return launch_small<4, 2>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 4, K_pad), epi, stream);
+  return launch_small<8, 1>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 8, K_pad), epi, stream);
+}
+
+static int small_blocks(const ZmiProblem &p, bool gated) {
+  return gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
+}
+
+hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
+  if (p.M <= 0) return hipSuccess;
+  if (p.M > 128) return hipErrorInvalidValue;
+  return dispatch_small(p, nullptr, 1, 0, p.M, small_blocks(p, epi.gated_act != 0), zmi_blob_kpad(p.K), epi,
+                        stream);
+}
+
+// Runs every problem with m_lo < M <= m_hi (m_hi <= 128).  probs_host sizes
+// the grid; when it is null the grid is worst_grid (K_pad taken from kpad_hint)
+// and surplus workgroups exit at once.
+hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev,
+                                        int n_prob, int m_lo, int m_hi, int worst_grid, int64_t kpad_hint,
+                                        const ZmiEpilogue &epi, hipStream_t stream) {
+  int grid = worst_grid;
+  int64_t kpad_max = kpad_hint;
+  if (probs_host) {
+    grid = 0;
+    kpad_max = 0;
+    for (int e = 0; e < n_prob; ++e) {
+      if (probs_host[e].M > m_lo && probs_host[e].M <= m_hi) {
+        grid += small_blocks(probs_host[e], epi.gated_act != 0);
+        const int64_t kp = zmi_blob_kpad(probs_host[e].K);
+        if (kp > kpad_max) kpad_max = kp;
+      }
+    }
+  }
+  ZmiProblem dummy = {};
+  return dispatch_small(dummy, probs_dev, n_prob, m_lo, m_hi, grid, kpad_max, epi, stream);
+}

@@ -1,0 +1,13 @@
+// Internals shared by the C ABI translation units.
+#pragma once
+#include "zmi_host.h"
+
+namespace zmi {
+int32_t validate_matmul(const void *src, const void *weight, const void *dst, int M, int N, int K,
+                        int Batch_A, int Batch_B, const zmi_matmul_params_t &p, bool is_weights_const);
+bool is_dynamic_quant_config(const zmi_matmul_params_t &p);
+int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, float beta, const void *bias,
+                       ZmiEpilogue *out, ZmiProblem *prob);
+int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi);
+bool a_needs_repack(const void *A, int64_t lda, int K, bool transA);
+}  // namespace zmi

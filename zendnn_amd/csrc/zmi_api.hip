@@ -1,0 +1,531 @@
+// C ABI: matmul_direct, reorder_direct (prepack and dynamic per-token modes),
+// weight_prepack_size, group_dynamic_quant.
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#include "zmi_api.h"
+#include "zmi_host.h"
+
+namespace zmi {
+
+// Mirrors validate_matmul_direct_inputs of the reference
+// (zendnnl/src/lowoha_operators/matmul/lowoha_matmul_utils.cpp:180-411) for the
+// rules that concern the int8 path.  Every failure is status failure.
+int32_t validate_matmul(const void *src, const void *weight, const void *dst, int M, int N, int K,
+                        int Batch_A, int Batch_B, const zmi_matmul_params_t &p, bool is_weights_const) {
+  (void)is_weights_const;
+  if (!src || !weight || !dst) { set_error("null src / weight / dst"); return ZMI_FAILURE; }
+  if (M <= 0 || N <= 0 || K <= 0) { set_error("M, N, K must be positive"); return ZMI_FAILURE; }
+  if (Batch_A <= 0 || Batch_B <= 0) { set_error("batch sizes must be positive"); return ZMI_FAILURE; }
+  const bool is_int8 = p.dt_wei == ZMI_DT_S8;
+  if ((p.src_scale.buff || p.dst_scale.buff || p.src_zp.buff || p.dst_zp.buff) && !is_int8) {
+    set_error("source / destination quantization params need s8 weights");
+    return ZMI_FAILURE;
+  }
+  if (p.src_scale.buff) {
+    const int64_t n = nelems(p.src_scale);
+    if (n != 1) {
+      const bool src_ok = p.dt_src == ZMI_DT_S8 || p.dt_src == ZMI_DT_BF16 || p.dt_src == ZMI_DT_F32;
+      const bool sym = !p.src_zp.buff;
+      const bool dst_ok = p.dt_dst == ZMI_DT_F32 || p.dt_dst == ZMI_DT_BF16;
+      const bool per_token = n == M;
+      const bool per_group = n > M && n % M == 0 && K % (n / M) == 0;
+      if (!(src_ok && sym && dst_ok && (per_token || per_group))) {
+        set_error("per-token / per-group source scale needs s8/bf16/f32 src, no source zero-point and f32/bf16 dst");
+        return ZMI_FAILURE;
+      }
+      const int64_t wn = p.wei_scale.buff ? nelems(p.wei_scale) : 0;
+      if (per_token && wn != N) {
+        set_error("per-token source scale requires a per-channel weight scale of N elements");
+        return ZMI_FAILURE;
+      }
+      if (per_group && wn != (n / M) * N) {
+        set_error("per-group source scale requires a per-group weight scale");
+        return ZMI_FAILURE;
+      }
+    }
+  }
+  auto per_tensor = [](const zmi_quant_t &q, const char *name) {
+    if (q.buff && nelems(q) != 1) { set_error(std::string(name) + " supports only per-tensor"); return false; }
+    return true;
+  };
+  if (!per_tensor(p.src_zp, "source zero-point") || !per_tensor(p.dst_scale, "destination scale") ||
+      !per_tensor(p.dst_zp, "destination zero-point"))
+    return ZMI_FAILURE;
+  const int s = p.dt_src, d = p.dt_dst;
+  if (!(s == ZMI_DT_F32 || s == ZMI_DT_BF16 || s == ZMI_DT_U8 || s == ZMI_DT_S8 || s == ZMI_DT_F16)) {
+    set_error("unsupported source data type");
+    return ZMI_FAILURE;
+  }
+  if (!(d == ZMI_DT_F32 || d == ZMI_DT_BF16 || d == ZMI_DT_U8 || d == ZMI_DT_S8 || d == ZMI_DT_S32 ||
+        d == ZMI_DT_F16)) {
+    set_error("unsupported destination data type");
+    return ZMI_FAILURE;
+  }
+  if (s == ZMI_DT_F32 && (d == ZMI_DT_BF16 || d == ZMI_DT_F16)) {
+    set_error("f32 source with bf16 / f16 destination");
+    return ZMI_FAILURE;
+  }
+  if ((s == ZMI_DT_BF16 && d == ZMI_DT_F16) || (s == ZMI_DT_F16 && d == ZMI_DT_BF16)) {
+    set_error("mixed bf16 / f16 source and destination");
+    return ZMI_FAILURE;
+  }
+  const int bmax = Batch_A > Batch_B ? Batch_A : Batch_B, bmin = Batch_A < Batch_B ? Batch_A : Batch_B;
+  if (bmax % bmin != 0) { set_error("batch sizes do not broadcast"); return ZMI_FAILURE; }
+  for (int i = 0; i < p.n_postops; ++i) {
+    const zmi_post_op_t &po = p.postops[i];
+    if (po.po_type == ZMI_PO_CLIP && (!std::isfinite(po.alpha) || !std::isfinite(po.beta))) {
+      set_error("clip bounds must be finite");
+      return ZMI_FAILURE;
+    }
+    if (po.po_type == ZMI_PO_MISH) {
+      // rejected on the int8 sym-quant / dynamic-quant paths, which is every path here
+      set_error("mish is not supported on the int8 paths");
+      return ZMI_FAILURE;
+    }
+  }
+  return ZMI_SUCCESS;
+}
+
+bool is_dynamic_quant_config(const zmi_matmul_params_t &p) {
+  // reference: is_dynamic_quant_config, matmul/lowoha_matmul_utils.hpp:215-230
+  return p.dynamic_quant && p.dt_wei == ZMI_DT_S8 && (p.dt_src == ZMI_DT_BF16 || p.dt_src == ZMI_DT_F32) &&
+         (p.dt_compute == ZMI_DT_S8 || p.dt_compute == ZMI_DT_U8);
+}
+
+// Translates the quantization parameters and post-ops of one call into the
+// kernels' shared epilogue descriptor (*out) and the per-problem operands
+// (scale / zero-point / bias fields of *prob).  Returns a ZMI_* status.
+int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, float beta, const void *bias,
+                       ZmiEpilogue *out, ZmiProblem *prob) {
+  ZmiEpilogue e;
+  std::memset(&e, 0, sizeof(e));
+  e.alpha = alpha;
+  e.beta = beta;
+  e.dst_dt = p.dt_dst;
+  prob->bias = bias;
+  prob->src_scale_ptr = nullptr; prob->wei_scale_ptr = nullptr; prob->src_zp_ptr = nullptr;
+  prob->src_scale_val = 1.0f; prob->wei_scale_val = 1.0f; prob->src_zp_val = 0;
+  e.bias_dt = p.dt_bias == ZMI_DT_NONE ? ZMI_DT_F32 : p.dt_bias;
+  if (bias && !(e.bias_dt == ZMI_DT_F32 || e.bias_dt == ZMI_DT_BF16 || e.bias_dt == ZMI_DT_S32 ||
+                e.bias_dt == ZMI_DT_S8)) {
+    set_error("unsupported bias dtype");
+    return ZMI_UNIMPLEMENTED;
+  }
+  // source scale
+  e.src_scale_mode = ZMI_SS_NONE;
+  if (p.src_scale.buff) {
+    const int64_t n = nelems(p.src_scale);
+    e.src_scale_dt = p.src_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p.src_scale.dt;
+    if (e.src_scale_dt != ZMI_DT_F32 && e.src_scale_dt != ZMI_DT_BF16) {
+      set_error("source scale must be f32 or bf16");
+      return ZMI_UNIMPLEMENTED;
+    }
+    if (n == 1) {
+      const void *dp;
+      if (!scalar_param_f32(p.src_scale.buff, e.src_scale_dt, &prob->src_scale_val, &dp)) return ZMI_FAILURE;
+      prob->src_scale_ptr = dp;
+      e.src_scale_mode = dp ? ZMI_SS_TENSOR_PTR : ZMI_SS_VALUE;
+    } else if (n == M) {
+      prob->src_scale_ptr = p.src_scale.buff;
+      e.src_scale_mode = ZMI_SS_TOKEN_PTR;
+    } else {
+      set_error("per-group source scales are not implemented");
+      return ZMI_UNIMPLEMENTED;
+    }
+  }
+  // weight scale
+  if (p.wei_scale.buff) {
+    const int64_t n = nelems(p.wei_scale);
+    e.wei_scale_dt = p.wei_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p.wei_scale.dt;
+    if (e.wei_scale_dt != ZMI_DT_F32 && e.wei_scale_dt != ZMI_DT_BF16) {
+      set_error("weight scale must be f32 or bf16");
+      return ZMI_UNIMPLEMENTED;
+    }
+    if (n == 1) {
+      const void *dp;
+      if (!scalar_param_f32(p.wei_scale.buff, e.wei_scale_dt, &prob->wei_scale_val, &dp)) return ZMI_FAILURE;
+      prob->wei_scale_ptr = dp;
+      e.wei_scale_mode = 1;
+    } else if (n == N) {
+      prob->wei_scale_ptr = p.wei_scale.buff;
+      e.wei_scale_mode = 2;
+    } else {
+      set_error("per-group weight scales are not implemented");
+      return ZMI_UNIMPLEMENTED;
+    }
+  }
+  if (p.wei_zp.buff) {
+    set_error("weight zero-points are not implemented (symmetric s8 weights only)");
+    return ZMI_UNIMPLEMENTED;
+  }
+  if (p.src_zp.buff) {
+    if (!scalar_param_s32(p.src_zp.buff, p.src_zp.dt, &prob->src_zp_val, &prob->src_zp_ptr)) return ZMI_FAILURE;
+    e.has_zp = 1;
+  }
+  if (p.dst_scale.buff || p.dst_zp.buff) {
+    e.has_dst_q = 1;
+    e.dst_scale_val = 1.0f;
+    e.dst_zp_val = 0.0f;
+    e.dst_scale_dt = p.dst_scale.dt;
+    e.dst_zp_dt = p.dst_zp.dt;
+    if (p.dst_scale.buff && !scalar_param_f32(p.dst_scale.buff, p.dst_scale.dt, &e.dst_scale_val, &e.dst_scale_ptr))
+      return ZMI_FAILURE;
+    if (p.dst_zp.buff && !scalar_param_f32(p.dst_zp.buff, p.dst_zp.dt, &e.dst_zp_val, &e.dst_zp_ptr))
+      return ZMI_FAILURE;
+    if (!p.dst_zp.buff) e.dst_zp_val = 0.0f;
+  }
+  // post-ops (normalised like lowoha_matmul.cpp:335-356: leading_dim -1 -> N,
+  // reversed clip bounds swapped)
+  int n_po = 0;
+  for (int i = 0; i < p.n_postops; ++i) {
+    const zmi_post_op_t &po = p.postops[i];
+    if (po.po_type == ZMI_PO_NONE) continue;
+    if (n_po >= ZMI_MAX_PO) { set_error("too many post-ops"); return ZMI_UNIMPLEMENTED; }
+    ZmiPostOp &d = e.po[n_po];
+    d.type = po.po_type;
+    d.alpha = po.alpha;
+    d.beta = po.beta;
+    switch (po.po_type) {
+    case ZMI_PO_RELU: case ZMI_PO_LEAKY_RELU: case ZMI_PO_GELU_TANH: case ZMI_PO_GELU_ERF:
+    case ZMI_PO_SIGMOID: case ZMI_PO_SWISH: case ZMI_PO_TANH:
+      break;
+    case ZMI_PO_CLIP:
+      if (d.alpha > d.beta) { float t = d.alpha; d.alpha = d.beta; d.beta = t; }
+      break;
+    case ZMI_PO_BINARY_ADD: case ZMI_PO_BINARY_MUL: {
+      if (!po.buff) { set_error("binary post-op without operand"); return ZMI_FAILURE; }
+      d.buff = po.buff;
+      d.dtype = po.dtype == ZMI_DT_NONE ? ZMI_DT_F32 : po.dtype;
+      d.ld = po.leading_dim > 0 ? po.leading_dim : N;
+      const bool row = (po.ndims == 2 && po.dims[0] == 1 && po.dims[1] == N) || (po.ndims == 1 && po.dims[0] == N);
+      const bool full = po.ndims == 2 && po.dims[0] == M && po.dims[1] == N;
+      if (!row && !full) { set_error("binary post-op operand must be {1,N} or {M,N}"); return ZMI_UNIMPLEMENTED; }
+      d.rowb = row ? 1 : 0;
+      break;
+    }
+    default:
+      // the reference's AOCL wiring skips the remaining types silently
+      // (backends/aocl/aocl_postop.cpp:476-479); refusing is the safer reading
+      set_error("post-op type not implemented on the int8 path");
+      return ZMI_UNIMPLEMENTED;
+    }
+    ++n_po;
+  }
+  e.n_po = n_po;
+  *out = e;
+  return ZMI_SUCCESS;
+}
+
+static int pick_bm(int M, int N) {
+  if (const char *env = std::getenv("ZMI_GEMM_BM")) {
+    int v = std::atoi(env);
+    if (v == 64 || v == 128 || v == 256) return v;
+  }
+  auto tiles = [&](int bm) { return (int64_t)((M + bm - 1) / bm) * ((N + 255) / 256); };
+  if (tiles(256) >= 2 * 256 && M >= 256) return 256;
+  if (tiles(128) >= 256 || M > 64) return tiles(128) >= 128 ? 128 : 64;
+  return 64;
+}
+
+int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi) {
+  if (prob.M <= 128) {
+    set_kernel_name("smallm_splitk_mfma16x16x64");
+    if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
+  } else {
+    const int bm = pick_bm(prob.M, epi.gated_act ? prob.N / 2 : prob.N);
+    set_kernel_name(bm == 256 ? "mfma32x32x32_bm256" : (bm == 128 ? "mfma32x32x32_bm128" : "mfma32x32x32_bm64"));
+    if (!hip_ok(zmi_launch_gemm_mfma(prob, epi, bm, stream()), "MFMA GEMM launch")) return ZMI_FAILURE;
+  }
+  return ZMI_SUCCESS;
+}
+
+bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
+  return transA || (K % 16) != 0 || (lda % 16) != 0 || (((uintptr_t)A) % 16) != 0;
+}
+
+}  // namespace zmi
+
+using namespace zmi;
+
+extern "C" {
+
+void zmi_matmul_params_init(zmi_matmul_params_t *p) {
+  std::memset(p, 0, sizeof(*p));
+  p->mem_format_a = 'n';
+  p->mem_format_b = 'n';
+  p->lowoha_algo = ZMI_ALGO_NONE;
+  p->weight_cache_type = 2;
+}
+
+void zmi_batch_params_init(zmi_batch_params_t *p) {
+  p->Batch_A = 1;
+  p->Batch_B = 1;
+  p->batch_stride_src = p->batch_stride_wei = p->batch_stride_dst = (uint64_t)-1;
+}
+
+void zmi_reorder_params_init(zmi_reorder_params_t *p) {
+  std::memset(p, 0, sizeof(*p));
+  p->algo = 0;  // reorder_algo_t::DT
+  p->prepack.algo = ZMI_ALGO_NONE;
+}
+
+int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M, int32_t N, int32_t K,
+                          float alpha, const void *src, int32_t lda, const void *weight, int32_t ldb,
+                          const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
+                          const zmi_batch_params_t *batch_params, const zmi_matmul_params_t *params) {
+  clear_error();
+  if (!params) { set_error("null params"); return ZMI_FAILURE; }
+  const zmi_matmul_params_t &p = *params;
+  const int Batch_A = batch_params ? batch_params->Batch_A : 1;
+  const int Batch_B = batch_params ? batch_params->Batch_B : 1;
+  if (diagnostics_enabled()) {
+    int32_t st = validate_matmul(src, weight, dst, M, N, K, Batch_A, Batch_B, p, is_weights_const != 0);
+    if (st != ZMI_SUCCESS) return st;
+  } else if (!src || !weight || !dst || M <= 0 || N <= 0 || K <= 0) {
+    set_error("null pointer or non-positive dimension");
+    return ZMI_FAILURE;
+  }
+  // ---- what this library implements of matmul_direct: the int8 path ----
+  if (p.dt_wei != ZMI_DT_S8) { set_error("only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+  if (layout != 'r' && layout != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
+  if (Batch_A != 1 || Batch_B != 1) { set_error("batched matmul is not implemented"); return ZMI_UNIMPLEMENTED; }
+  if (p.pack_format_b != 0) { set_error("GGML-packed weights are not implemented"); return ZMI_UNIMPLEMENTED; }
+  if (p.mem_format_b == 'r' && p.lowoha_algo != ZMI_ALGO_AOCL_DLP_BLOCKED) {
+    // contract of the reference: prepacked weights require the blocked algo
+    set_error("mem_format_b == 'r' requires lowoha_algo == aocl_dlp_blocked");
+    return ZMI_FAILURE;
+  }
+  const bool dyn = is_dynamic_quant_config(p);
+  if (!dyn && p.dt_src != ZMI_DT_S8 && p.dt_src != ZMI_DT_U8) {
+    set_error("source must be u8 / s8, or bf16 / f32 with dynamic_quant and an s8 compute type");
+    return ZMI_UNIMPLEMENTED;
+  }
+  if (dyn && p.dt_compute == ZMI_DT_U8) { set_error("dynamic u8 (asymmetric) quantization is not implemented"); return ZMI_UNIMPLEMENTED; }
+  if (lda < (transA ? M : K) || ldc < N || ldb < (transB ? K : N)) {
+    if (p.mem_format_b != 'r' || lda < (transA ? M : K) || ldc < N) { set_error("leading dimension too small"); return ZMI_FAILURE; }
+  }
+  int64_t dyn_scale_n = 0;
+  if (dyn) {
+    dyn_scale_n = 1;
+    for (int i = 0; i < p.src_scale.ndims; ++i) dyn_scale_n *= p.src_scale.dims[i];
+    if (!(dyn_scale_n == 1 || dyn_scale_n == M)) { set_error("dynamic per-group source scales are not implemented"); return ZMI_UNIMPLEMENTED; }
+    if (p.src_zp.buff) { set_error("dynamic quantization is symmetric: no source zero-point"); return ZMI_FAILURE; }
+    if (transA) { set_error("dynamic quantization of a transposed source is not implemented"); return ZMI_UNIMPLEMENTED; }
+  }
+  if (!ensure_device()) return ZMI_FAILURE;
+
+  // ---- scratch plan ----
+  const bool use_cache = p.mem_format_b != 'r' && is_weights_const &&
+                         std::min(weight_cache_env(), p.weight_cache_type) > 0;
+  const bool pack_in_arena = p.mem_format_b != 'r' && !use_cache;
+  const int64_t K16 = zmi_round_up(K, 16);
+  const bool repack_a = !dyn && a_needs_repack(src, lda, K, transA != 0);
+  size_t need = 0;
+  if (pack_in_arena) need += Arena::padded((size_t)zmi_blob_bytes(K, N));
+  if (dyn) need += Arena::padded((size_t)M * K16) + Arena::padded(sizeof(float) * (size_t)M) + 256;
+  if (repack_a) need += Arena::padded((size_t)M * K16);
+  if (!arena().begin(need)) return ZMI_FAILURE;
+
+  // ---- weights ----
+  const uint8_t *blob;
+  if (p.mem_format_b == 'r') {
+    if (!blob_matches(weight, K, N)) return ZMI_FAILURE;
+    blob = (const uint8_t *)weight;
+  } else {
+    void *slot = pack_in_arena ? arena().alloc((size_t)zmi_blob_bytes(K, N)) : nullptr;
+    blob = packed_weights(weight, K, N, ldb, transB != 0, p.dt_src, use_cache, slot);
+    if (!blob) return ZMI_FAILURE;
+  }
+
+  // ---- source ----
+  zmi_matmul_params_t ep = p;   // working copy: the caller's struct is never modified
+  ZmiProblem prob;
+  std::memset(&prob, 0, sizeof(prob));
+  prob.blob = blob;
+  prob.dst = dst;
+  prob.ldc = ldc;
+  prob.M = M; prob.N = N; prob.K = K;
+  if (dyn) {
+    // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
+    int8_t *q = (int8_t *)arena().alloc((size_t)M * K16);
+    float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M);
+    unsigned int *amax = (unsigned int *)arena().alloc(256);
+    // bytes of q between K and K16 stay unwritten: the blob's rows beyond K are zero
+    int32_t sdt = p.src_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p.src_scale.dt;
+    if (dyn_scale_n == M && M > 1) {
+      void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
+      if (!p.src_scale.buff) sdt = ZMI_DT_F32;
+      if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, scale_out, sdt, stream()), "quant launch"))
+        return ZMI_FAILURE;
+      ep.src_scale.buff = scale_out;
+      ep.src_scale.dt = sdt;
+      ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = 1;
+    } else {
+      // one scale for the whole tensor; with M == 1 this is the per-token case too
+      if (!hip_ok(zmi_launch_quant_tensor(src, p.dt_src, M, K, lda, q, K16, sc, amax, stream()), "quant launch"))
+        return ZMI_FAILURE;
+      if (p.src_scale.buff) {
+        if (sdt != ZMI_DT_F32) { set_error("per-tensor dynamic scale output must be f32"); return ZMI_UNIMPLEMENTED; }
+        if (!hip_ok(hipMemcpyAsync((void *)p.src_scale.buff, sc, sizeof(float), hipMemcpyDeviceToDevice, stream()),
+                    "hipMemcpyAsync(scale)"))
+          return ZMI_FAILURE;
+      }
+      ep.src_scale.buff = sc;
+      ep.src_scale.dt = ZMI_DT_F32;
+      ep.src_scale.ndims = 1; ep.src_scale.dims[0] = 1;
+    }
+    prob.A = q; prob.lda = K16; prob.a_is_u8 = 0;
+    ep.dt_src = ZMI_DT_S8;
+  } else if (repack_a) {
+    int8_t *a2 = (int8_t *)arena().alloc((size_t)M * K16);
+    if (!hip_ok(zmi_launch_pad_rows(src, M, K, lda, transA != 0, a2, K16, stream()), "pad launch")) return ZMI_FAILURE;
+    prob.A = a2; prob.lda = K16; prob.a_is_u8 = p.dt_src == ZMI_DT_U8;
+  } else {
+    prob.A = src; prob.lda = lda; prob.a_is_u8 = p.dt_src == ZMI_DT_U8;
+  }
+
+  ZmiEpilogue epi;
+  int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
+  if (st != ZMI_SUCCESS) return st;
+  st = run_single_gemm(prob, epi);
+  upload_fence();
+  return st;
+}
+
+// ---- prepack ---------------------------------------------------------------------------------
+
+// reference: validate_prepack_params, reorder/prepack/lowoha_prepack.cpp:53-96
+static int32_t validate_prepack(const zmi_prepack_params_t &pp) {
+  if (pp.K <= 0 || pp.N <= 0) { set_error("prepack: K and N must be positive"); return ZMI_FAILURE; }
+  const int64_t min_ld = pp.transposed ? pp.K : pp.N;
+  if (pp.ldb < min_ld) { set_error("prepack: ldb too small"); return ZMI_FAILURE; }
+  if (pp.algo != ZMI_ALGO_AOCL_DLP_BLOCKED) { set_error("prepack: only aocl_dlp_blocked is supported"); return ZMI_UNIMPLEMENTED; }
+  if (pp.wei_dtype != ZMI_DT_S8) { set_error("prepack: only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+  return ZMI_SUCCESS;
+}
+
+size_t zmi_weight_prepack_size(zmi_reorder_params_t *params) {
+  clear_error();
+  if (!params) return 0;
+  params->prepack.cached_size = 0;
+  if (validate_prepack(params->prepack) != ZMI_SUCCESS) return 0;
+  const size_t sz = (size_t)zmi_round_up(zmi_blob_bytes(params->prepack.K, params->prepack.N), 64);
+  params->prepack.cached_size = sz;
+  return sz;
+}
+
+static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t &rp) {
+  // reference: validate_dynamic_quant_params + the fused per-token dispatch,
+  // reorder/lowoha_reorder.cpp:60-204
+  if (!src) { set_error("reorder: null src"); return ZMI_FAILURE; }
+  if (rp.n_src_shape != 2) { set_error("dynamic quantization: only 2-D [M,K] shapes are implemented"); return ZMI_UNIMPLEMENTED; }
+  if (rp.n_dst_shape != rp.n_src_shape || std::memcmp(rp.src_shape, rp.dst_shape, sizeof(int64_t) * rp.n_src_shape) != 0) {
+    set_error("reorder: src_shape and dst_shape differ");
+    return ZMI_FAILURE;
+  }
+  const int64_t M = rp.src_shape[0], K = rp.src_shape[1];
+  if (M <= 0 || K <= 0) { set_error("reorder: non-positive shape"); return ZMI_FAILURE; }
+  if (!(rp.src_dtype == ZMI_DT_BF16 || rp.src_dtype == ZMI_DT_F32) || rp.dst_dtype != ZMI_DT_S8) {
+    set_error("dynamic quantization: only bf16/f32 -> s8 is implemented");
+    return ZMI_UNIMPLEMENTED;
+  }
+  if (rp.zero_point.buff) { set_error("dynamic quantization: only symmetric (no zero-point buffer)"); return ZMI_UNIMPLEMENTED; }
+  if (!rp.scale.buff) { set_error("dynamic quantization: scale buffer is required"); return ZMI_FAILURE; }
+  const int32_t sdt = rp.scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : rp.scale.dt;
+  if (sdt != ZMI_DT_F32 && sdt != ZMI_DT_BF16) { set_error("dynamic quantization: scale must be f32 or bf16"); return ZMI_FAILURE; }
+  int64_t ld = K;
+  if (rp.n_src_strides == 2) {
+    if (rp.src_strides[1] != 1 || rp.src_strides[0] < K) { set_error("dynamic quantization: rows must be contiguous"); return ZMI_UNIMPLEMENTED; }
+    ld = rp.src_strides[0];
+  } else if (rp.n_src_strides != 0) {
+    set_error("reorder: strides do not match the shape");
+    return ZMI_FAILURE;
+  }
+  const int64_t sn = nelems(rp.scale);
+  if (!ensure_device()) return ZMI_FAILURE;
+  if (rp.scale.ndims == 2 && rp.scale.dims[0] == M && rp.scale.dims[1] == 1) {
+    if (!hip_ok(zmi_launch_quant_rows(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, (void *)rp.scale.buff, sdt, stream()),
+                "quant launch"))
+      return ZMI_FAILURE;
+    set_kernel_name("quant_rows_per_token");
+    return ZMI_SUCCESS;
+  }
+  if (sn == 1) {
+    if (sdt != ZMI_DT_F32) { set_error("per-tensor dynamic scale must be f32"); return ZMI_UNIMPLEMENTED; }
+    if (!arena().begin(Arena::padded(sizeof(float) * (size_t)M) + 256)) return ZMI_FAILURE;
+    float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M);
+    unsigned int *amax = (unsigned int *)arena().alloc(256);
+    if (!hip_ok(zmi_launch_quant_tensor(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, sc, amax, stream()), "quant launch"))
+      return ZMI_FAILURE;
+    if (!hip_ok(hipMemcpyAsync((void *)rp.scale.buff, sc, sizeof(float), hipMemcpyDeviceToDevice, stream()), "hipMemcpyAsync"))
+      return ZMI_FAILURE;
+    set_kernel_name("quant_tensor");
+    return ZMI_SUCCESS;
+  }
+  set_error("dynamic quantization: only per-token {M,1} and per-tensor scales are implemented");
+  return ZMI_UNIMPLEMENTED;
+}
+
+int32_t zmi_reorder_direct(const void *src, void *dst, zmi_reorder_params_t *params) {
+  clear_error();
+  if (!params) { set_error("null params"); return ZMI_FAILURE; }
+  if (params->is_prepack) {
+    // reference: weight_prepack_into, reorder/prepack/lowoha_prepack.cpp:315-373
+    int32_t st = validate_prepack(params->prepack);
+    if (st != ZMI_SUCCESS) return st;
+    if (!src || !dst) { set_error("prepack: null weights or destination"); return ZMI_FAILURE; }
+    if (!ensure_device()) return ZMI_FAILURE;
+    const zmi_prepack_params_t &pp = params->prepack;
+    if (!hip_ok(zmi_launch_prepack((const int8_t *)src, pp.K, pp.N, pp.ldb, pp.transposed, pp.src_dtype,
+                                   pp.sym_group_size, (uint8_t *)dst, stream()), "prepack launch"))
+      return ZMI_FAILURE;
+    set_kernel_name("prepack_mfma_fragments");
+    return ZMI_SUCCESS;
+  }
+  if (params->dynamic_quant) return reorder_dynamic(src, dst, *params);
+  set_error("static reorder / dtype conversion modes are not part of this path");
+  return ZMI_UNIMPLEMENTED;
+}
+
+int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src, const int32_t *M, const int32_t *K,
+                                const int64_t *src_row_stride, void *const *dst, const int64_t *dst_row_stride,
+                                void *const *scale, const zmi_group_dq_params_t *params) {
+  // reference: group_dynamic_quant, reorder/lowoha_reorder.cpp:279-404
+  clear_error();
+  if (!params || n <= 0 || !src || !M || !K || !dst || !scale) { set_error("group_dynamic_quant: bad arguments"); return ZMI_FAILURE; }
+  if (!(params->src_dtype == ZMI_DT_BF16 || params->src_dtype == ZMI_DT_F32) || params->dst_dtype != ZMI_DT_S8) {
+    set_error("group_dynamic_quant: only bf16/f32 -> s8");
+    return ZMI_FAILURE;
+  }
+  if (params->num_groups > 1) { set_error("group_dynamic_quant: per-group scales are not implemented"); return ZMI_UNIMPLEMENTED; }
+  const int32_t sdt = params->scale_dtype == ZMI_DT_NONE ? ZMI_DT_F32 : params->scale_dtype;
+  if (sdt != ZMI_DT_F32 && sdt != ZMI_DT_BF16) { set_error("group_dynamic_quant: scale must be f32 or bf16"); return ZMI_FAILURE; }
+  std::vector<ZmiQuantMat> mats;
+  int64_t rows = 0;
+  for (int i = 0; i < n; ++i) {
+    if (M[i] < 0 || K[i] <= 0) { set_error("group_dynamic_quant: bad shape"); return ZMI_FAILURE; }
+    if (M[i] == 0) continue;
+    if (!src[i] || !dst[i] || !scale[i]) { set_error("group_dynamic_quant: null buffer for an active matrix"); return ZMI_FAILURE; }
+    ZmiQuantMat m;
+    m.src = src[i]; m.dst = (int8_t *)dst[i]; m.scale = scale[i];
+    m.ld_src = src_row_stride && src_row_stride[i] ? src_row_stride[i] : K[i];
+    m.ld_dst = dst_row_stride && dst_row_stride[i] ? dst_row_stride[i] : K[i];
+    if (m.ld_src < K[i] || m.ld_dst < K[i]) { set_error("group_dynamic_quant: row stride smaller than K"); return ZMI_FAILURE; }
+    m.M = M[i]; m.K = K[i]; m.row_start = (int32_t)rows;
+    rows += M[i];
+    mats.push_back(m);
+  }
+  if (mats.empty()) return ZMI_SUCCESS;
+  if (!ensure_device()) return ZMI_FAILURE;
+  if (!arena().begin(0)) return ZMI_FAILURE;
+  const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
+  if (!dev) return ZMI_FAILURE;
+  bool ok = hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), rows, params->src_dtype, sdt, stream()), "quant launch");
+  upload_fence();
+  set_kernel_name("quant_rows_grouped");
+  return ok ? ZMI_SUCCESS : ZMI_FAILURE;
+}
+
+}  // extern "C"

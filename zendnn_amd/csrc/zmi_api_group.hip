@@ -1,0 +1,656 @@
+// C ABI: group_matmul_direct (independent expert GEMMs, gated activation,
+// fused MoE Op1 -> act -> Op2, weighted reduce) and the device-side MoE glue.
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "zmi_api.h"
+#include "zmi_host.h"
+
+using namespace zmi;
+
+namespace {
+
+struct SizeCheck {
+  size_t num_ops;
+  bool relaxed;
+  bool bad(size_t s) const { return relaxed ? s < num_ops : s != num_ops; }
+};
+
+// op2_k_for_act of the reference (group_matmul_parallel_common.hpp:202): a gated
+// activation halves the width of Op1's output.
+int op2_k_for_act(int N, int act) { return act != ZMI_ACT_NONE ? N / 2 : N; }
+
+bool all_null(void *const *v, int n, size_t num_ops) {
+  const size_t m = std::min((size_t)n, num_ops);
+  for (size_t i = 0; i < m; ++i)
+    if (v[i]) return false;
+  return true;
+}
+
+// Always-on guards and the diagnostics validator of the reference
+// (matmul/group_matmul_direct.cpp:185-699 and :768-1063), for the rules that do
+// not depend on the CPU scheduling.  Every failure is status failure.
+int32_t validate_group(const zmi_group_args_t &a, const zmi_moe_postop_t *postop, int gated_act,
+                       const zmi_fused_moe_t *fm, size_t *num_ops_out, bool *op1_internal_out,
+                       bool *op2_internal_out) {
+  if (a.n_M <= 0 || a.n_params <= 0 || a.n_src <= 0) { set_error("group_matmul_direct: required input vector is empty"); return ZMI_FAILURE; }
+  const bool opt_in = a.params[0].active_matmul > 0;
+  if (opt_in) {
+    const uint32_t am = a.params[0].active_matmul, tm = a.params[0].total_matmul;
+    if (am > (uint32_t)a.n_M) { set_error("active_matmul exceeds M.size()"); return ZMI_FAILURE; }
+    if (tm > 0 && tm < am) { set_error("total_matmul must be >= active_matmul"); return ZMI_FAILURE; }
+  }
+  const size_t num_ops = opt_in ? (size_t)a.params[0].active_matmul : (size_t)a.n_M;
+  *num_ops_out = num_ops;
+  const SizeCheck sc{num_ops, opt_in};
+
+  // library-managed outputs: with fused_moe, dst (Op1) and dst_down (Op2) may
+  // be empty / all null; a mix of null and non-null entries is an error
+  bool op1_internal = false, op2_internal = false;
+  if (fm) {
+    if (a.n_dst == 0 || all_null(a.dst, a.n_dst, num_ops)) op1_internal = true;
+    else {
+      for (size_t i = 0; i < std::min((size_t)a.n_dst, num_ops); ++i)
+        if (!a.dst[i] && i < (size_t)a.n_M && a.M[i] > 0) { set_error("fused_moe dst has a mixed null / non-null state"); return ZMI_FAILURE; }
+    }
+    if (fm->n_dst_down == 0 || all_null(fm->dst_down, fm->n_dst_down, num_ops)) op2_internal = true;
+    else {
+      for (size_t i = 0; i < std::min((size_t)fm->n_dst_down, num_ops); ++i)
+        if (!fm->dst_down[i] && i < (size_t)a.n_M && a.M[i] > 0) { set_error("fused_moe dst_down has a mixed null / non-null state"); return ZMI_FAILURE; }
+    }
+  }
+  *op1_internal_out = op1_internal;
+  *op2_internal_out = op2_internal;
+
+  if (sc.bad(a.n_N) || sc.bad(a.n_K) || sc.bad(a.n_weight) || sc.bad(a.n_lda) || sc.bad(a.n_ldb) ||
+      sc.bad(a.n_layout) || sc.bad(a.n_transA) || sc.bad(a.n_transB) || sc.bad(a.n_alpha) || sc.bad(a.n_beta) ||
+      sc.bad(a.n_bias) || sc.bad(a.n_is_weights_const) || sc.bad(a.n_params) ||
+      (!op1_internal && (sc.bad(a.n_dst) || sc.bad(a.n_ldc)))) {
+    set_error("group_matmul_direct: vector size mismatch");
+    return ZMI_FAILURE;
+  }
+  if (opt_in && a.params[0].total_matmul > a.params[0].active_matmul) {
+    const size_t tm = a.params[0].total_matmul;
+    if ((size_t)a.n_weight < tm || (size_t)a.n_K < tm || (size_t)a.n_N < tm || (size_t)a.n_ldb < tm ||
+        (size_t)a.n_transB < tm || (size_t)a.n_is_weights_const < tm) {
+      set_error("weight-side vectors must be sized to total_matmul");
+      return ZMI_FAILURE;
+    }
+  }
+  if (op1_internal) {
+    if (a.n_dst != 0 && sc.bad(a.n_dst)) { set_error("dst must be empty or sized to num_ops"); return ZMI_FAILURE; }
+    if (a.n_ldc != 0 && sc.bad(a.n_ldc)) { set_error("ldc must be empty or sized to num_ops"); return ZMI_FAILURE; }
+  }
+  if (op2_internal && fm->n_ldc_down != 0 && sc.bad(fm->n_ldc_down)) { set_error("ldc_down must be empty or sized to num_ops"); return ZMI_FAILURE; }
+  if (a.n_src != 1 && sc.bad(a.n_src)) { set_error("src.size() must be 1 or num_ops"); return ZMI_FAILURE; }
+  const bool run_act = gated_act != ZMI_ACT_NONE;
+  if (a.n_src == 1) {
+    if (postop) { set_error("moe_postop is only supported in parallel mode"); return ZMI_FAILURE; }
+    if (run_act) { set_error("gated_act is only supported in parallel mode"); return ZMI_FAILURE; }
+    if (fm) { set_error("fused_moe is only supported in parallel mode"); return ZMI_FAILURE; }
+  }
+  if (fm && fm->n_down_weight == 0) { set_error("fused_moe is non-null but down_weight is empty"); return ZMI_FAILURE; }
+  if (a.n_src == 1) {
+    // sequential chain
+    if (!a.src[0]) { set_error("group_matmul sequential: null src"); return ZMI_FAILURE; }
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (!a.weight[i] || !a.dst[i]) { set_error("group_matmul sequential: null pointer"); return ZMI_FAILURE; }
+      if (a.M[i] <= 0 || a.N[i] <= 0 || a.K[i] <= 0) { set_error("group_matmul sequential: invalid dimensions"); return ZMI_FAILURE; }
+    }
+    for (size_t i = 1; i < num_ops; ++i) {
+      if (a.M[i] != a.M[0]) { set_error("group_matmul sequential: M must be constant across layers"); return ZMI_FAILURE; }
+      if (a.K[i] != a.N[i - 1]) { set_error("group_matmul sequential: K[i] != N[i-1]"); return ZMI_FAILURE; }
+    }
+    return ZMI_SUCCESS;
+  }
+  for (size_t i = 0; i < num_ops; ++i) {
+    if (a.M[i] < 0 || a.N[i] <= 0 || a.K[i] <= 0) { set_error("group_matmul parallel: invalid dimensions"); return ZMI_FAILURE; }
+    if (a.M[i] > 0) {
+      if (!a.src[i] || !a.weight[i]) { set_error("group_matmul parallel: null src / weight at an active expert"); return ZMI_FAILURE; }
+      if (!op1_internal && !a.dst[i]) { set_error("group_matmul parallel: null dst at an active expert"); return ZMI_FAILURE; }
+    }
+  }
+  if (run_act) {
+    const int dt = a.params[0].dt_dst;
+    if (dt != ZMI_DT_F32 && dt != ZMI_DT_BF16 && dt != ZMI_DT_F16) { set_error("gated_act requires f32, bf16 or f16 dst"); return ZMI_FAILURE; }
+    for (size_t i = 1; i < num_ops; ++i)
+      if (a.params[i].dt_dst != dt) { set_error("gated_act requires uniform dst dtype"); return ZMI_FAILURE; }
+    for (size_t i = 0; i < num_ops; ++i)
+      if (a.N[i] % 2 != 0) { set_error("gated_act requires even N"); return ZMI_FAILURE; }
+    if (!op1_internal && !fm) {
+      bool tight = false, wide = false;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        if (a.ldc[i] < a.N[i]) tight = true; else wide = true;
+      }
+      if (tight && wide) { set_error("gated_act: mixed tight / wide dst layouts"); return ZMI_FAILURE; }
+    }
+  }
+  if (run_act || fm) {
+    for (size_t i = 0; i < num_ops; ++i)
+      if (a.layout[i] != 'r' && a.layout[i] != 'R') { set_error("gated_act / fused_moe require row-major layout"); return ZMI_FAILURE; }
+  }
+  if (fm) {
+    if (sc.bad(fm->n_down_weight) || sc.bad(fm->n_N_down) || sc.bad(fm->n_ldb_down) || sc.bad(fm->n_bias_down) ||
+        (!op2_internal && (sc.bad(fm->n_dst_down) || sc.bad(fm->n_ldc_down)))) {
+      set_error("fused_moe vector size mismatch");
+      return ZMI_FAILURE;
+    }
+    if (fm->n_down_scale != 0 && (size_t)fm->n_down_scale < num_ops) { set_error("fused_moe down_scale is shorter than num_ops"); return ZMI_FAILURE; }
+    if (fm->n_down_zp != 0 && (size_t)fm->n_down_zp < num_ops) { set_error("fused_moe down_zp is shorter than num_ops"); return ZMI_FAILURE; }
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (a.N[i] % 2 != 0) { set_error("fused_moe requires even N"); return ZMI_FAILURE; }
+      if (a.M[i] > 0) {
+        if (!fm->down_weight[i]) { set_error("fused_moe down_weight is null at an active expert"); return ZMI_FAILURE; }
+        if (!op2_internal && !fm->dst_down[i]) { set_error("fused_moe dst_down is null at an active expert"); return ZMI_FAILURE; }
+      }
+      if (fm->N_down[i] <= 0) { set_error("fused_moe N_down must be positive"); return ZMI_FAILURE; }
+      const int kd = op2_k_for_act(a.N[i], gated_act);
+      const int min_ldb = a.transB[i] ? kd : fm->N_down[i];
+      if (fm->ldb_down[i] < min_ldb) { set_error("fused_moe ldb_down too small"); return ZMI_FAILURE; }
+      if (!op2_internal) {
+        if (fm->ldc_down[i] < fm->N_down[i]) { set_error("fused_moe ldc_down < N_down"); return ZMI_FAILURE; }
+      } else {
+        if (a.M[i] > 0 && a.lda[i] < fm->N_down[i]) { set_error("fused_moe internal-alloc requires lda >= N_down"); return ZMI_FAILURE; }
+        if (a.M[i] > 0 && a.params[i].dt_src != a.params[i].dt_dst) { set_error("fused_moe internal-alloc requires matching src / dst dtypes"); return ZMI_FAILURE; }
+      }
+      if (fm->bias_down[i] && fm->bias_dt_down == ZMI_DT_NONE) { set_error("fused_moe bias_down is set but bias_dt_down is none"); return ZMI_FAILURE; }
+    }
+    if (postop)
+      for (size_t i = 1; i < num_ops; ++i)
+        if (fm->N_down[i] != fm->N_down[0]) { set_error("fused_moe + moe_postop requires uniform N_down"); return ZMI_FAILURE; }
+  }
+  if (postop) {
+    for (size_t i = 1; i < num_ops; ++i) {
+      if (a.N[i] != a.N[0]) { set_error("moe_postop requires identical N across experts"); return ZMI_FAILURE; }
+      if (a.params[i].dt_dst != a.params[0].dt_dst) { set_error("moe_postop requires identical dst dtype"); return ZMI_FAILURE; }
+    }
+    // validate_group_matmul_moe_postop (group_matmul/group_matmul_moe_postop.cpp)
+    const int D = fm ? fm->N_down[0] : a.N[0];
+    const int dt = a.params[0].dt_dst;
+    if (!postop->row_ptrs || !postop->output) { set_error("moe_postop: row_ptrs and output must be non-null"); return ZMI_FAILURE; }
+    if (postop->num_tokens <= 0 || postop->topk <= 0) { set_error("moe_postop: num_tokens and topk must be positive"); return ZMI_FAILURE; }
+    if (postop->ldc_output < D) { set_error("moe_postop: ldc_output < D"); return ZMI_FAILURE; }
+    if (dt != ZMI_DT_F32 && dt != ZMI_DT_BF16 && dt != ZMI_DT_F16) { set_error("moe_postop: dst dtype must be f32, bf16 or f16"); return ZMI_FAILURE; }
+    if (!postop->skip_weighted && !postop->topk_weights) { set_error("moe_postop: topk_weights required"); return ZMI_FAILURE; }
+  }
+  return ZMI_SUCCESS;
+}
+
+bool same_quant_shape(const zmi_quant_t &x, const zmi_quant_t &y, int Mx, int My, int Nx, int Ny) {
+  // same granularity class: absent / one element / per row / per column
+  auto cls = [](const zmi_quant_t &q, int M, int N, bool has) {
+    if (!has) return 0;
+    const int64_t n = nelems(q);
+    if (n == 1) return 1;
+    if (n == M) return 2;
+    if (n == N) return 3;
+    return 4;
+  };
+  return x.dt == y.dt && cls(x, Mx, Nx, x.buff != nullptr || x.ndims > 0) == cls(y, My, Ny, y.buff != nullptr || y.ndims > 0);
+}
+
+// One epilogue descriptor serves a grouped launch only if every expert asks for
+// the same arithmetic.
+bool params_uniform(const zmi_group_args_t &a, size_t num_ops) {
+  const zmi_matmul_params_t &p0 = a.params[0];
+  for (size_t i = 0; i < num_ops; ++i) {
+    const zmi_matmul_params_t &p = a.params[i];
+    if (p.dt_src != p0.dt_src || p.dt_wei != p0.dt_wei || p.dt_dst != p0.dt_dst || p.dt_bias != p0.dt_bias ||
+        p.dt_compute != p0.dt_compute || p.dynamic_quant != p0.dynamic_quant || p.mem_format_b != p0.mem_format_b ||
+        p.n_postops != p0.n_postops)
+      return false;
+    if (a.alpha[i] != a.alpha[0] || a.beta[i] != a.beta[0]) return false;
+    if ((a.bias[i] != nullptr) != (a.bias[0] != nullptr) && a.M[i] > 0 && a.M[0] > 0) return false;
+    for (int j = 0; j < p.n_postops; ++j) {
+      const zmi_post_op_t &x = p.postops[j], &y = p0.postops[j];
+      if (x.po_type != y.po_type || x.alpha != y.alpha || x.beta != y.beta) return false;
+      if (x.po_type == ZMI_PO_BINARY_ADD || x.po_type == ZMI_PO_BINARY_MUL) return false;
+    }
+    if ((p.src_zp.buff != nullptr) != (p0.src_zp.buff != nullptr)) return false;
+    if (p.dst_scale.buff || p.dst_zp.buff || p.wei_zp.buff) return false;
+    if ((p.wei_scale.buff != nullptr) != (p0.wei_scale.buff != nullptr)) return false;
+    if (p.wei_scale.buff && ((nelems(p.wei_scale) == 1) != (nelems(p0.wei_scale) == 1))) return false;
+    if (!p.dynamic_quant) {
+      if ((p.src_scale.buff != nullptr) != (p0.src_scale.buff != nullptr)) return false;
+      if (p.src_scale.buff && ((nelems(p.src_scale) == 1) != (nelems(p0.src_scale) == 1))) return false;
+    }
+  }
+  return true;
+}
+
+struct Stage {
+  std::vector<ZmiProblem> probs;
+  ZmiEpilogue epi;
+};
+
+int32_t launch_stage(const Stage &st, const char *what) {
+  if (st.probs.empty()) return ZMI_SUCCESS;
+  const ZmiProblem *dev = (const ZmiProblem *)upload(st.probs.data(), st.probs.size() * sizeof(ZmiProblem));
+  if (!dev) return ZMI_FAILURE;
+  const int n = (int)st.probs.size();
+  int bm = 128;
+  if (const char *env = std::getenv("ZMI_GROUP_BM")) { int v = std::atoi(env); if (v == 64 || v == 128 || v == 256) bm = v; }
+  // one small-M launch per row-count bucket so few-row experts do not pay for 128-row tiles
+  static const int kBuckets[5] = {0, 16, 32, 64, 128};
+  for (int b = 0; b < 4; ++b)
+    if (!hip_ok(zmi_launch_gemm_smallm_group(st.probs.data(), dev, n, kBuckets[b], kBuckets[b + 1], 0, 0, st.epi, stream()), what))
+      return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_mfma_group(st.probs.data(), dev, n, 128, 0, st.epi, bm, stream()), what)) return ZMI_FAILURE;
+  return ZMI_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_postop_t *moe_postop,
+                                int32_t gated_act, const zmi_fused_moe_t *fused_moe) {
+  clear_error();
+  if (!args) { set_error("null args"); return ZMI_FAILURE; }
+  const zmi_group_args_t &a = *args;
+  size_t num_ops = 0;
+  bool op1_internal = false, op2_internal = false;
+  int32_t st = validate_group(a, moe_postop, gated_act, fused_moe, &num_ops, &op1_internal, &op2_internal);
+  if (st != ZMI_SUCCESS) return st;
+  if (num_ops == 0) return ZMI_SUCCESS;
+
+  // ---- sequential chain: layer i consumes layer i-1's output (group_matmul_direct.cpp:1137-1164)
+  if (a.n_src == 1) {
+    const void *cur = a.src[0];
+    for (size_t i = 0; i < num_ops; ++i) {
+      zmi_batch_params_t bp;
+      zmi_batch_params_init(&bp);
+      zmi_matmul_params_t p = a.params[i];
+      st = zmi_matmul_direct(a.layout[i], a.transA[i], a.transB[i], a.M[i], a.N[i], a.K[i], a.alpha[i], cur, a.lda[i],
+                             a.weight[i], a.ldb[i], a.bias[i], a.beta[i], a.dst[i], a.ldc[i], a.is_weights_const[i], &bp, &p);
+      if (st != ZMI_SUCCESS) return st;
+      cur = a.dst[i];
+    }
+    return ZMI_SUCCESS;
+  }
+
+  // ---- per-expert validation through the single-matmul rules ----
+  for (size_t i = 0; i < num_ops; ++i) {
+    if (a.M[i] <= 0) continue;
+    const void *dsti = op1_internal ? (const void *)a.src[i] : (const void *)a.dst[i];
+    if (diagnostics_enabled()) {
+      st = validate_matmul(a.src[i], a.weight[i], dsti, a.M[i], a.N[i], a.K[i], 1, 1, a.params[i], a.is_weights_const[i] != 0);
+      if (st != ZMI_SUCCESS) return st;
+    }
+    if (a.params[i].dt_wei != ZMI_DT_S8) { set_error("only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+    if (a.layout[i] != 'r' && a.layout[i] != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
+    if (a.params[i].pack_format_b != 0) { set_error("GGML-packed weights are not implemented"); return ZMI_UNIMPLEMENTED; }
+  }
+  const bool run_act = gated_act != ZMI_ACT_NONE;
+
+  if (!params_uniform(a, num_ops)) {
+    // experts disagree on dtypes / post-ops: run them one by one
+    if (fused_moe || run_act) { set_error("fused_moe / gated_act need uniform per-expert params"); return ZMI_UNIMPLEMENTED; }
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (a.M[i] <= 0) continue;
+      zmi_batch_params_t bp;
+      zmi_batch_params_init(&bp);
+      st = zmi_matmul_direct(a.layout[i], a.transA[i], a.transB[i], a.M[i], a.N[i], a.K[i], a.alpha[i], a.src[i], a.lda[i],
+                             a.weight[i], a.ldb[i], a.bias[i], a.beta[i], a.dst[i], a.ldc[i], a.is_weights_const[i], &bp,
+                             &a.params[i]);
+      if (st != ZMI_SUCCESS) return st;
+    }
+    if (moe_postop) goto postop_only;
+    return ZMI_SUCCESS;
+  }
+
+  {
+    const zmi_matmul_params_t &p0 = a.params[0];
+    const bool dyn = is_dynamic_quant_config(p0);
+    if (!dyn && p0.dt_src != ZMI_DT_S8 && p0.dt_src != ZMI_DT_U8) {
+      set_error("source must be u8 / s8, or bf16 / f32 with dynamic_quant and an s8 compute type");
+      return ZMI_UNIMPLEMENTED;
+    }
+    if (dyn && p0.dt_compute == ZMI_DT_U8) { set_error("dynamic u8 quantization is not implemented"); return ZMI_UNIMPLEMENTED; }
+    const int dst_es = p0.dt_dst == ZMI_DT_BF16 ? 2 : (p0.dt_dst == ZMI_DT_F32 || p0.dt_dst == ZMI_DT_S32 ? 4 : 1);
+    if (fused_moe && !(p0.dt_dst == ZMI_DT_BF16 || p0.dt_dst == ZMI_DT_F32)) { set_error("fused_moe needs a bf16 or f32 dst"); return ZMI_UNIMPLEMENTED; }
+    if (fused_moe && !dyn) { set_error("fused_moe is implemented for dynamic_quant int8 only"); return ZMI_UNIMPLEMENTED; }
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (a.M[i] <= 0) continue;
+      if (a.transA[i]) { set_error("transposed sources are not implemented in group calls"); return ZMI_UNIMPLEMENTED; }
+      if (dyn) {
+        int64_t sn = 1;
+        for (int d = 0; d < a.params[i].src_scale.ndims; ++d) sn *= a.params[i].src_scale.dims[d];
+        if (!(sn == a.M[i] || sn == 1)) { set_error("dynamic per-group source scales are not implemented"); return ZMI_UNIMPLEMENTED; }
+        if (sn == 1 && a.M[i] > 1) { set_error("per-tensor dynamic scales are not implemented in group calls"); return ZMI_UNIMPLEMENTED; }
+        if (a.params[i].src_zp.buff) { set_error("dynamic quantization is symmetric"); return ZMI_FAILURE; }
+      }
+      if (run_act && a.beta[i] != 0.0f) { set_error("gated_act with beta != 0 is not implemented"); return ZMI_UNIMPLEMENTED; }
+    }
+    if (!ensure_device()) return ZMI_FAILURE;
+
+    // can the gated activation run inside the GEMM epilogue?
+    bool fuse_act = run_act && gated_act != ZMI_ACT_SWIGLU_OAI_MUL;
+    for (size_t i = 0; i < num_ops && fuse_act; ++i)
+      if (a.M[i] > 0 && (a.N[i] / 2) % 32 != 0) fuse_act = false;
+    // a caller-visible wide dst keeps the un-activated up half only in the unfused form
+    const bool tight_internal = op1_internal && run_act;
+
+    // ---- scratch plan ----
+    size_t need = 0;
+    int64_t rows = 0;
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (a.M[i] <= 0) continue;
+      rows += a.M[i];
+      const int64_t K16 = zmi_round_up(a.K[i], 16);
+      if (dyn) need += Arena::padded((size_t)a.M[i] * K16) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
+      else if (a_needs_repack(a.src[i], a.lda[i], a.K[i], false)) need += Arena::padded((size_t)a.M[i] * K16);
+      const bool cache = a.params[i].mem_format_b != 'r' && a.is_weights_const[i] &&
+                         std::min(weight_cache_env(), a.params[i].weight_cache_type) > 0;
+      if (a.params[i].mem_format_b != 'r' && !cache) need += Arena::padded((size_t)zmi_blob_bytes(a.K[i], a.N[i]));
+      if (op1_internal) {
+        const int w = tight_internal ? a.N[i] / 2 : a.N[i];
+        need += Arena::padded((size_t)a.M[i] * w * dst_es);
+      }
+      if (fused_moe) {
+        const int kd = op2_k_for_act(a.N[i], gated_act);
+        const int64_t kd16 = zmi_round_up(kd, 16);
+        need += Arena::padded((size_t)a.M[i] * kd16) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
+        const bool cache2 = a.is_weights_const[i] && std::min(weight_cache_env(), a.params[i].weight_cache_type) > 0;
+        if (!cache2) need += Arena::padded((size_t)zmi_blob_bytes(kd, fused_moe->N_down[i]));
+      }
+    }
+    if (moe_postop) {
+      const size_t tbl = sizeof(void *) * (size_t)moe_postop->num_tokens * moe_postop->topk;
+      need += Arena::padded(tbl);
+    }
+    need += 4096;
+    if (!arena().begin(need)) return ZMI_FAILURE;
+
+    // ---- stage 1: sources (dynamic per-token quantization of every expert in one launch)
+    std::vector<const void *> A1(num_ops, nullptr);
+    std::vector<int64_t> lda1(num_ops, 0);
+    std::vector<void *> s1(num_ops, nullptr);
+    int32_t s1_dt = ZMI_DT_F32;
+    if (dyn) {
+      // reference: group_reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:307-696
+      std::vector<ZmiQuantMat> mats;
+      int64_t r0 = 0;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        const int64_t K16 = zmi_round_up(a.K[i], 16);
+        ZmiQuantMat m;
+        m.src = a.src[i];
+        m.dst = (int8_t *)arena().alloc((size_t)a.M[i] * K16);
+        float *sc = (float *)arena().alloc(sizeof(float) * (size_t)a.M[i]);
+        m.scale = a.params[i].src_scale.buff ? (void *)a.params[i].src_scale.buff : (void *)sc;
+        m.ld_src = a.lda[i]; m.ld_dst = K16; m.M = a.M[i]; m.K = a.K[i]; m.row_start = (int32_t)r0;
+        r0 += a.M[i];
+        mats.push_back(m);
+        A1[i] = m.dst; lda1[i] = K16; s1[i] = m.scale;
+      }
+      s1_dt = (p0.src_scale.buff && p0.src_scale.dt != ZMI_DT_NONE) ? p0.src_scale.dt : ZMI_DT_F32;
+      if (s1_dt != ZMI_DT_F32 && s1_dt != ZMI_DT_BF16) { set_error("source scale must be f32 or bf16"); return ZMI_FAILURE; }
+      const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
+      if (!dev) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_src, s1_dt, stream()), "grouped quant launch")) return ZMI_FAILURE;
+    } else {
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        if (a_needs_repack(a.src[i], a.lda[i], a.K[i], false)) {
+          const int64_t K16 = zmi_round_up(a.K[i], 16);
+          int8_t *t = (int8_t *)arena().alloc((size_t)a.M[i] * K16);
+          if (!hip_ok(zmi_launch_pad_rows(a.src[i], a.M[i], a.K[i], a.lda[i], 0, t, K16, stream()), "pad launch")) return ZMI_FAILURE;
+          A1[i] = t; lda1[i] = K16;
+        } else {
+          A1[i] = a.src[i]; lda1[i] = a.lda[i];
+        }
+      }
+    }
+
+    // ---- stage 2: Op1 ----
+    Stage op1;
+    std::vector<void *> op1_dst(num_ops, nullptr);
+    std::vector<int64_t> op1_ld(num_ops, 0);
+    bool have_epi = false;
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (a.M[i] <= 0) continue;
+      const zmi_matmul_params_t &p = a.params[i];
+      ZmiProblem pr;
+      std::memset(&pr, 0, sizeof(pr));
+      if (p.mem_format_b == 'r') {
+        if (p.lowoha_algo != ZMI_ALGO_AOCL_DLP_BLOCKED) { set_error("mem_format_b == 'r' requires lowoha_algo == aocl_dlp_blocked"); return ZMI_FAILURE; }
+        if (!blob_matches(a.weight[i], a.K[i], a.N[i])) return ZMI_FAILURE;
+        pr.blob = (const uint8_t *)a.weight[i];
+      } else {
+        const bool cache = a.is_weights_const[i] && std::min(weight_cache_env(), p.weight_cache_type) > 0;
+        void *slot = cache ? nullptr : arena().alloc((size_t)zmi_blob_bytes(a.K[i], a.N[i]));
+        pr.blob = packed_weights(a.weight[i], a.K[i], a.N[i], a.ldb[i], a.transB[i] != 0, p.dt_src, cache, slot);
+        if (!pr.blob) return ZMI_FAILURE;
+      }
+      if (op1_internal) {
+        const int w = tight_internal ? a.N[i] / 2 : a.N[i];
+        op1_dst[i] = arena().alloc((size_t)a.M[i] * w * dst_es);
+        op1_ld[i] = w;
+      } else {
+        op1_dst[i] = a.dst[i];
+        op1_ld[i] = a.ldc[i];
+      }
+      pr.A = A1[i]; pr.lda = lda1[i]; pr.dst = op1_dst[i]; pr.ldc = op1_ld[i];
+      pr.M = a.M[i]; pr.N = a.N[i]; pr.K = a.K[i];
+      pr.a_is_u8 = (!dyn && p.dt_src == ZMI_DT_U8) ? 1 : 0;
+      zmi_matmul_params_t ep = p;
+      if (dyn) {
+        ep.dt_src = ZMI_DT_S8;
+        ep.src_scale.buff = s1[i]; ep.src_scale.dt = s1_dt; ep.src_scale.ndims = 2;
+        ep.src_scale.dims[0] = a.M[i]; ep.src_scale.dims[1] = 1;
+      }
+      ZmiEpilogue e;
+      st = build_epilogue(ep, a.M[i], a.N[i], a.alpha[i], a.beta[i], a.bias[i], &e, &pr);
+      if (st != ZMI_SUCCESS) return st;
+      // M == 1: a one-row per-token scale is the same thing as a per-tensor device scale
+      if (dyn && e.src_scale_mode == ZMI_SS_TENSOR_PTR) e.src_scale_mode = ZMI_SS_TOKEN_PTR;
+      if (!have_epi) { op1.epi = e; have_epi = true; }
+      else if (e.src_scale_mode != op1.epi.src_scale_mode || e.wei_scale_mode != op1.epi.wei_scale_mode) {
+        set_error("experts disagree on scale granularity or host/device placement of one-element scales");
+        return ZMI_UNIMPLEMENTED;
+      }
+      op1.probs.push_back(pr);
+    }
+    if (!have_epi) {
+      upload_fence();
+      if (moe_postop) goto postop_only;
+      return ZMI_SUCCESS;
+    }
+    op1.epi.gated_act = fuse_act ? gated_act : ZMI_ACT_NONE;
+    st = launch_stage(op1, "Op1 GEMM launch");
+    if (st != ZMI_SUCCESS) return st;
+    set_kernel_name(fuse_act ? "group: smallm + mfma32x32x32 (gated epilogue)" : "group: smallm + mfma32x32x32");
+
+    if (run_act && !fuse_act) {
+      // reference: group_matmul_moe_act_execute, group_matmul/group_matmul_moe_act.cpp
+      std::vector<ZmiActMat> mats;
+      int64_t r0 = 0;
+      int maxN = 0;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        ZmiActMat m;
+        m.buf = op1_dst[i]; m.ld = op1_ld[i]; m.M = a.M[i]; m.N = a.N[i]; m.row_start = (int32_t)r0;
+        r0 += a.M[i];
+        maxN = std::max(maxN, a.N[i]);
+        mats.push_back(m);
+      }
+      if (tight_internal) { set_error("internal: tight Op1 scratch needs the fused activation"); return ZMI_FAILURE; }
+      const ZmiActMat *dev = (const ZmiActMat *)upload(mats.data(), mats.size() * sizeof(ZmiActMat));
+      if (!dev) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_gated_act(dev, nullptr, (int)mats.size(), r0, maxN, gated_act, p0.dt_dst, stream()), "gated act launch")) return ZMI_FAILURE;
+    }
+
+    // ---- stage 3: Op2 (down projection), reference: run_fused_moe_legacy_two_pass,
+    // group_matmul/group_matmul_fused_moe.cpp:906-1078
+    if (fused_moe) {
+      const zmi_fused_moe_t &fm = *fused_moe;
+      std::vector<ZmiQuantMat> mats;
+      std::vector<int8_t *> A2(num_ops, nullptr);
+      std::vector<float *> s2(num_ops, nullptr);
+      std::vector<int64_t> lda2(num_ops, 0);
+      int64_t r0 = 0;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        const int kd = op2_k_for_act(a.N[i], gated_act);
+        const int64_t kd16 = zmi_round_up(kd, 16);
+        ZmiQuantMat m;
+        m.src = op1_dst[i];
+        m.dst = (int8_t *)arena().alloc((size_t)a.M[i] * kd16);
+        m.scale = arena().alloc(sizeof(float) * (size_t)a.M[i]);
+        m.ld_src = op1_ld[i]; m.ld_dst = kd16; m.M = a.M[i]; m.K = kd; m.row_start = (int32_t)r0;
+        r0 += a.M[i];
+        mats.push_back(m);
+        A2[i] = m.dst; s2[i] = (float *)m.scale; lda2[i] = kd16;
+      }
+      const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
+      if (!dev) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_dst, ZMI_DT_F32, stream()), "grouped quant launch (Op2)")) return ZMI_FAILURE;
+
+      Stage op2;
+      bool have2 = false;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        const int kd = op2_k_for_act(a.N[i], gated_act);
+        ZmiProblem pr;
+        std::memset(&pr, 0, sizeof(pr));
+        const bool cache = a.is_weights_const[i] && std::min(weight_cache_env(), a.params[i].weight_cache_type) > 0;
+        void *slot = cache ? nullptr : arena().alloc((size_t)zmi_blob_bytes(kd, fm.N_down[i]));
+        pr.blob = packed_weights(fm.down_weight[i], kd, fm.N_down[i], fm.ldb_down[i], a.transB[i] != 0, ZMI_DT_S8, cache, slot);
+        if (!pr.blob) return ZMI_FAILURE;
+        pr.A = A2[i]; pr.lda = lda2[i];
+        if (op2_internal) { pr.dst = const_cast<void *>(a.src[i]); pr.ldc = a.lda[i]; }
+        else { pr.dst = fm.dst_down[i]; pr.ldc = fm.ldc_down[i]; }
+        pr.M = a.M[i]; pr.N = fm.N_down[i]; pr.K = kd;
+        zmi_matmul_params_t ep;
+        zmi_matmul_params_init(&ep);
+        ep.dt_src = ZMI_DT_S8; ep.dt_wei = ZMI_DT_S8; ep.dt_dst = p0.dt_dst; ep.dt_bias = fm.bias_dt_down;
+        ep.src_scale.buff = s2[i]; ep.src_scale.dt = ZMI_DT_F32; ep.src_scale.ndims = 2;
+        ep.src_scale.dims[0] = a.M[i]; ep.src_scale.dims[1] = 1;
+        if (fm.n_down_scale) ep.wei_scale = fm.down_scale[i];
+        if (fm.n_down_zp && fm.down_zp[i].buff) { set_error("down_zp is not implemented (symmetric weights only)"); return ZMI_UNIMPLEMENTED; }
+        ZmiEpilogue e;
+        st = build_epilogue(ep, a.M[i], fm.N_down[i], 1.0f, 0.0f, fm.bias_down[i], &e, &pr);
+        if (st != ZMI_SUCCESS) return st;
+        if (e.src_scale_mode == ZMI_SS_TENSOR_PTR) e.src_scale_mode = ZMI_SS_TOKEN_PTR;
+        if (!have2) { op2.epi = e; have2 = true; }
+        else if (e.wei_scale_mode != op2.epi.wei_scale_mode) { set_error("experts disagree on down_scale granularity"); return ZMI_UNIMPLEMENTED; }
+        op2.probs.push_back(pr);
+      }
+      st = launch_stage(op2, "Op2 GEMM launch");
+      if (st != ZMI_SUCCESS) return st;
+    }
+  }
+
+postop_only:
+  if (moe_postop) {
+    // reference: group_matmul_moe_postop_execute, group_matmul/group_matmul_moe_postop.cpp:506
+    if (!ensure_device()) return ZMI_FAILURE;
+    const int D = fused_moe ? fused_moe->N_down[0] : a.N[0];
+    const int dt = a.params[0].dt_dst;
+    if (dt != ZMI_DT_BF16 && dt != ZMI_DT_F32) { set_error("moe_postop: f16 is not implemented"); return ZMI_UNIMPLEMENTED; }
+    const size_t tbl = sizeof(void *) * (size_t)moe_postop->num_tokens * moe_postop->topk;
+    const void *const *rp = (const void *const *)upload(moe_postop->row_ptrs, tbl);
+    if (!rp) return ZMI_FAILURE;
+    if (!hip_ok(zmi_launch_moe_combine(rp, nullptr, 0, nullptr, moe_postop->topk_weights, moe_postop->skip_weighted,
+                                       moe_postop->num_tokens, moe_postop->topk, D, dt, moe_postop->output,
+                                       moe_postop->ldc_output, stream()), "moe combine launch"))
+      return ZMI_FAILURE;
+  }
+  upload_fence();
+  return ZMI_SUCCESS;
+}
+
+int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk, int32_t E, int32_t *counts,
+                      int32_t *offsets, int32_t *slot_of) {
+  clear_error();
+  if (!topk_ids || !counts || !offsets || !slot_of || T <= 0 || topk <= 0 || E <= 0) { set_error("moe_route: bad arguments"); return ZMI_FAILURE; }
+  if (E > 2047) { set_error("moe_route: at most 2047 experts"); return ZMI_UNIMPLEMENTED; }
+  if (!ensure_device()) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, counts, offsets, slot_of, stream()), "moe route launch")) return ZMI_FAILURE;
+  set_kernel_name("moe_route");
+  return ZMI_SUCCESS;
+}
+
+int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
+  clear_error();
+  if (!d || !d->x || !d->topk_ids || !d->topk_weights || !d->w13_blob || !d->w2_blob || !d->w13_scale || !d->w2_scale || !d->out) {
+    set_error("moe_fused_device: null argument");
+    return ZMI_FAILURE;
+  }
+  const int T = d->T, H = d->H, I = d->I, E = d->E, topk = d->topk;
+  if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0 || d->ldx < H || d->ldo < H) { set_error("moe_fused_device: bad shape"); return ZMI_FAILURE; }
+  if (H % 16 != 0 || I % 32 != 0) { set_error("moe_fused_device: H must be a multiple of 16 and I of 32"); return ZMI_UNIMPLEMENTED; }
+  if (d->gated_act != ZMI_ACT_SILU_AND_MUL && d->gated_act != ZMI_ACT_GELU_AND_MUL) { set_error("moe_fused_device: silu_and_mul or gelu_and_mul"); return ZMI_UNIMPLEMENTED; }
+  if (E > 2047) { set_error("moe_fused_device: at most 2047 experts"); return ZMI_UNIMPLEMENTED; }
+  if (!ensure_device()) return ZMI_FAILURE;
+  const int64_t R = (int64_t)T * topk;
+  size_t need = 0;
+  need += Arena::padded(sizeof(int32_t) * E) + Arena::padded(sizeof(int32_t) * (E + 1)) + Arena::padded(sizeof(int32_t) * R);
+  need += Arena::padded((size_t)R * H) + Arena::padded(sizeof(float) * R);          // A1, s1
+  need += Arena::padded((size_t)R * I * 2);                                         // act bf16
+  need += Arena::padded((size_t)R * I) + Arena::padded(sizeof(float) * R);          // A2, s2
+  need += Arena::padded((size_t)R * H * 2);                                         // Y bf16
+  need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096;
+  if (!arena().begin(need)) return ZMI_FAILURE;
+  int32_t *counts = (int32_t *)arena().alloc(sizeof(int32_t) * E);
+  int32_t *offsets = (int32_t *)arena().alloc(sizeof(int32_t) * (E + 1));
+  int32_t *slot_of = (int32_t *)arena().alloc(sizeof(int32_t) * R);
+  int8_t *A1 = (int8_t *)arena().alloc((size_t)R * H);
+  float *s1 = (float *)arena().alloc(sizeof(float) * R);
+  void *act = arena().alloc((size_t)R * I * 2);
+  int8_t *A2 = (int8_t *)arena().alloc((size_t)R * I);
+  float *s2 = (float *)arena().alloc(sizeof(float) * R);
+  void *Y = arena().alloc((size_t)R * H * 2);
+  ZmiProblem *op1 = (ZmiProblem *)arena().alloc(sizeof(ZmiProblem) * E);
+  ZmiProblem *op2 = (ZmiProblem *)arena().alloc(sizeof(ZmiProblem) * E);
+
+  // the four per-expert pointer tables travel in one upload
+  std::vector<const void *> tbl(4 * (size_t)E);
+  for (int e = 0; e < E; ++e) {
+    tbl[e] = d->w13_blob[e]; tbl[E + e] = d->w2_blob[e]; tbl[2 * E + e] = d->w13_scale[e]; tbl[3 * E + e] = d->w2_scale[e];
+    if (!tbl[e] || !tbl[E + e] || !tbl[2 * E + e] || !tbl[3 * E + e]) { set_error("moe_fused_device: null expert table entry"); return ZMI_FAILURE; }
+  }
+  for (int e = 0; e < E; ++e) {
+    if (!blob_matches(d->w13_blob[e], H, 2 * I) || !blob_matches(d->w2_blob[e], I, H)) return ZMI_FAILURE;
+  }
+  const void *const *tdev = (const void *const *)upload(tbl.data(), tbl.size() * sizeof(void *));
+  if (!tdev) return ZMI_FAILURE;
+  ZmiMoeTables tb;
+  tb.w13_blob = tdev; tb.w2_blob = tdev + E;
+  tb.w13_scale = (const float *const *)(tdev + 2 * E); tb.w2_scale = (const float *const *)(tdev + 3 * E);
+
+  hipStream_t s = stream();
+  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, counts, offsets, slot_of, s), "moe route launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_quant_scatter(d->x, d->ldx, T, H, topk, slot_of, A1, s1, s), "quant scatter launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, s), "problem table launch")) return ZMI_FAILURE;
+
+  ZmiEpilogue e1;
+  std::memset(&e1, 0, sizeof(e1));
+  e1.src_scale_mode = ZMI_SS_TOKEN_PTR; e1.src_scale_dt = ZMI_DT_F32;
+  e1.wei_scale_mode = 2; e1.wei_scale_dt = ZMI_DT_F32;
+  e1.bias_dt = ZMI_DT_F32; e1.alpha = 1.0f; e1.beta = 0.0f; e1.dst_dt = ZMI_DT_BF16;
+  ZmiEpilogue e2 = e1;
+  e1.gated_act = d->gated_act;
+  // row counts live on the device: size the grids for the worst case
+  const int bm = 128;
+  const int small_grid1 = E * (I / 16), small_grid2 = E * (int)(zmi_blob_npad(H) / 32);
+  const int items1 = (int)((R / bm + E) * ((I + 127) / 128));
+  const int items2 = (int)((R / bm + E) * ((H + 255) / 256));
+  static const int kBuckets[5] = {0, 16, 32, 64, 128};
+  for (int b = 0; b < 4; ++b)
+    if (!hip_ok(zmi_launch_gemm_smallm_group(nullptr, op1, E, kBuckets[b], kBuckets[b + 1], small_grid1, zmi_blob_kpad(H), e1, s), "Op1 small-M launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_mfma_group(nullptr, op1, E, 128, items1, e1, bm, s), "Op1 MFMA launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, R, I, I, A2, I, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
+  for (int b = 0; b < 4; ++b)
+    if (!hip_ok(zmi_launch_gemm_smallm_group(nullptr, op2, E, kBuckets[b], kBuckets[b + 1], small_grid2, zmi_blob_kpad(I), e2, s), "Op2 small-M launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_mfma_group(nullptr, op2, E, 128, items2, e2, bm, s), "Op2 MFMA launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;
+  upload_fence();
+  set_kernel_name("moe_fused_device");
+  return ZMI_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,296 @@
+// Device-side types shared by the gfx950 kernels and the host dispatch code:
+// the packed-weight blob, the epilogue descriptor and the per-expert table.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/zmi_lowoha.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// ---------------------------------------------------------------------------
+// Packed weight blob ("mem_format_b == 'r'").
+//
+//   [ header 256 B ][ colsum int32[N_pad] ][ tiles ]
+//
+// tiles is an array [N_pad/32][K_pad/32] of 1 KiB fragments.  Fragment (nb,kb)
+// holds weight rows kb*32..+31 of columns nb*32..+31 exactly as one wavefront
+// feeds them to v_mfma_i32_32x32x32_i8 as the B operand: lane i owns bytes
+// [16i, 16i+16) = B[kb*32 + (i/32)*16 + b][nb*32 + i%32], b = 0..15.  A
+// wavefront therefore loads a fragment with one fully coalesced 16-byte-per-lane
+// load and needs no LDS staging or shuffles for B.  Fragments of one column
+// block are contiguous along K, so every wavefront streams contiguous memory.
+// Padding rows / columns are zero.  colsum[n] = sum_k B[k][n] feeds the source
+// zero-point compensation in the GEMM epilogue.
+// ---------------------------------------------------------------------------
+#define ZMI_BLOB_MAGIC 0x31424f4c42494d5aULL  // "ZMIBLOB1"
+#define ZMI_BLOB_HEADER_BYTES 256
+#define ZMI_KPAD 128
+#define ZMI_NPAD 64
+
+struct ZmiBlobHeader {
+  uint64_t magic;
+  uint32_t version;
+  uint32_t flags;
+  int64_t K, N, K_pad, N_pad;
+  int64_t colsum_off, tiles_off, total_bytes;
+  int32_t src_dtype, sym_group_size;
+};
+
+static inline __host__ __device__ int64_t zmi_round_up(int64_t x, int64_t m) {
+  return (x + m - 1) / m * m;
+}
+static inline __host__ __device__ int64_t zmi_blob_kpad(int64_t K) { return zmi_round_up(K, ZMI_KPAD); }
+static inline __host__ __device__ int64_t zmi_blob_npad(int64_t N) { return zmi_round_up(N, ZMI_NPAD); }
+static inline __host__ __device__ int64_t zmi_blob_colsum_off() { return ZMI_BLOB_HEADER_BYTES; }
+static inline __host__ __device__ int64_t zmi_blob_tiles_off(int64_t N) {
+  return zmi_round_up(ZMI_BLOB_HEADER_BYTES + zmi_blob_npad(N) * 4, 256);
+}
+static inline __host__ __device__ int64_t zmi_blob_bytes(int64_t K, int64_t N) {
+  return zmi_blob_tiles_off(N) + zmi_blob_kpad(K) * zmi_blob_npad(N);
+}
+
+// ---------------------------------------------------------------------------
+// Epilogue: everything between the s32 accumulator and the stored element.
+//   y = float(acc + comp[n])            comp[n] = -src_zp * colsum[n], in s32
+//   (alpha != 1 or beta != 0: y = float(acc)*alpha + beta*C + float(comp[n]))
+//   y *= src_scale (tensor or row m);  y *= wei_scale[n % len];  y += bias[n]
+//   post-ops in order;  y = y * dst_scale + dst_zp;  store as dst dtype.
+// ---------------------------------------------------------------------------
+#define ZMI_MAX_PO 4
+
+struct ZmiPostOp {
+  int32_t type;        // enum zmi_post_op_type
+  int32_t dtype;       // binary operand dtype
+  const void *buff;    // binary operand
+  int32_t ld;          // leading dimension of a {M,N} operand
+  int32_t rowb;        // 1: operand is {1,N} and broadcast over rows
+  float alpha, beta;   // clip bounds
+};
+
+enum { ZMI_SS_NONE = 0, ZMI_SS_VALUE = 1, ZMI_SS_TENSOR_PTR = 2, ZMI_SS_TOKEN_PTR = 3 };
+
+struct ZmiEpilogue {
+  int32_t src_scale_mode;  // ZMI_SS_*
+  int32_t src_scale_dt;
+  int32_t wei_scale_mode;  // 0: none; 1: per tensor; 2: per channel (indexed by n)
+  int32_t wei_scale_dt;
+  int32_t has_zp;
+  int32_t bias_dt;
+  float alpha, beta;
+  int32_t n_po;
+  ZmiPostOp po[ZMI_MAX_PO];
+  int32_t has_dst_q;
+  const void *dst_scale_ptr;
+  int32_t dst_scale_dt;
+  float dst_scale_val;
+  const void *dst_zp_ptr;
+  int32_t dst_zp_dt;
+  float dst_zp_val;
+  int32_t dst_dt;
+  int32_t gated_act;      // enum zmi_gated_act; != 0: columns are [gate | up] halves
+};
+
+// One GEMM problem: C[M,N] = epilogue(A[M,K] x blob), with the operands the
+// epilogue reads per problem.  The grouped kernels take an array of these in
+// device memory, one per expert; the epilogue descriptor is shared.
+struct ZmiProblem {
+  const void *A;          // u8 / s8, row-major, K contiguous
+  int64_t lda;
+  const uint8_t *blob;    // packed weights
+  void *dst;
+  int64_t ldc;
+  int32_t M, N, K;
+  int32_t a_is_u8;
+  const void *src_scale_ptr;   // ZMI_SS_TENSOR_PTR / ZMI_SS_TOKEN_PTR
+  const void *wei_scale_ptr;   // null with mode 1: wei_scale_val is used
+  const int32_t *src_zp_ptr;   // null: src_zp_val is used
+  const void *bias;
+  float src_scale_val;         // ZMI_SS_VALUE
+  float wei_scale_val;
+  int32_t src_zp_val;
+};
+
+#ifdef __HIPCC__
+// ------------------------------------------------------------------ device math
+__device__ __forceinline__ float zmi_bf16_to_f32(uint16_t h) {
+  return __uint_as_float(((uint32_t)h) << 16);
+}
+
+// Store rounding of the matmul output and the gated activation: normals round
+// to nearest even, zero and subnormal inputs give a signed zero, NaN keeps its
+// high half with the quiet bit set (reference: bfloat16_t(float),
+// zendnnl/src/common/bfloat16.cpp:27-51).
+__device__ __forceinline__ uint16_t zmi_f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t e = u & 0x7f800000u;
+  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  if (e == 0) r = (u >> 16) & 0x8000u;
+  if (e == 0x7f800000u) r = (u >> 16) | ((u & 0x007fffffu) ? 0x40u : 0u);
+  return (uint16_t)r;
+}
+
+// Plain round-to-nearest-even bit trick used by the MoE weighted reduce
+// (reference: bfloat16_t::f32_to_bf16_val, zendnnl/src/common/bfloat16.cpp:69-79).
+__device__ __forceinline__ uint16_t zmi_f32_to_bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__device__ __forceinline__ float zmi_ld_f32(const void *p, int dt, int64_t i) {
+  switch (dt) {
+  case ZMI_DT_BF16: return zmi_bf16_to_f32(((const uint16_t *)p)[i]);
+  case ZMI_DT_S32: return (float)((const int32_t *)p)[i];
+  case ZMI_DT_S8: return (float)((const int8_t *)p)[i];
+  case ZMI_DT_U8: return (float)((const uint8_t *)p)[i];
+  default: return ((const float *)p)[i];
+  }
+}
+
+// exp(x) from the hardware exp2 with a split product x*log2(e) so the argument
+// error does not grow with |x|; about 2 ulp over the range the activations use.
+__device__ __forceinline__ float zmi_expf(float x) {
+  const float l2e_hi = 1.44269502162933349609375f;
+  const float l2e_lo = 1.925963033500011e-08f;
+  float t = x * l2e_hi;
+  float r = __builtin_fmaf(x, l2e_hi, -t) + x * l2e_lo;   // rounding error of t plus the low part
+  float e = __builtin_amdgcn_exp2f(t);
+  // an overflowed e must stay +inf (inf * negative correction + inf would be NaN)
+  return e == __builtin_inff() ? e : __builtin_fmaf(e, r * 0.693147182464599609375f, e);
+}
+
+__device__ __forceinline__ float zmi_sigmoid(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + zmi_expf(-x));
+}
+
+// Element-wise post-ops (reference definitions:
+// zendnnl/src/operators/matmul/matmul_ref_kernel.cpp:694-761).
+__device__ __forceinline__ float zmi_eltwise(int type, float x, float alpha, float beta) {
+  switch (type) {
+  case ZMI_PO_RELU: return x > 0.0f ? x : 0.0f;
+  case ZMI_PO_LEAKY_RELU: return x > 0.0f ? x : 0.01f * x;
+  case ZMI_PO_GELU_TANH: {
+    // reference: v = tanhf(u); 0.5 * x * (1.0f + v), u = sqrt(2/pi) x (1 + 0.044715 x^2).
+    // 1 + tanh(u) == 2 sigmoid(2u) is evaluated accurately, then rounded through
+    // the float value of tanh (v) exactly as the reference's "1.0f + v" sees it,
+    // so the negative tail cancels onto the same 2^-24 grid.
+    float u = 0.79788458347320556640625f * x * (1.0f + 0.044715f * x * x);
+    float v = 2.0f * zmi_sigmoid(2.0f * u) - 1.0f;
+    return (0.5f * x) * (1.0f + v);
+  }
+  case ZMI_PO_GELU_ERF: return 0.5f * x * (1.0f + erff(x * 0.707106769084930419921875f));
+  case ZMI_PO_SIGMOID: return zmi_sigmoid(x);
+  case ZMI_PO_SWISH: return x * zmi_sigmoid(x);
+  case ZMI_PO_TANH: return tanhf(x);
+  case ZMI_PO_CLIP: { x = x > alpha ? x : alpha; return x > beta ? beta : x; }
+  default: return x;
+  }
+}
+
+// Gated activations (reference: group_matmul/group_matmul_moe_act.cpp:88-154).
+__device__ __forceinline__ float zmi_gated(int act, float g, float u) {
+  if (act == ZMI_ACT_SILU_AND_MUL) return (g * zmi_sigmoid(g)) * u;
+  if (act == ZMI_ACT_GELU_AND_MUL) return (g * 0.5f * (1.0f + erff(g * 0.7071067811865476f))) * u;
+  // swiglu_oai: clamp to [-7, 7], (1 + u) * g * sigmoid(1.702 g)
+  g = fmaxf(-7.0f, fminf(g, 7.0f));
+  u = fmaxf(-7.0f, fminf(u, 7.0f));
+  return (1.0f + u) * g * zmi_sigmoid(g * 1.702f);
+}
+
+// Per-column constants of the epilogue, loaded once per lane.
+struct ZmiColCtx {
+  float wscale;
+  float bias;
+  int32_t comp;
+};
+
+__device__ __forceinline__ ZmiColCtx zmi_col_ctx(const ZmiEpilogue &e, const ZmiProblem &p,
+                                                 const int32_t *colsum, int n, int N) {
+  ZmiColCtx c;
+  c.wscale = 1.0f;
+  c.bias = 0.0f;
+  c.comp = 0;
+  if (n < N) {
+    if (e.wei_scale_mode) {
+      c.wscale = p.wei_scale_ptr ? zmi_ld_f32(p.wei_scale_ptr, e.wei_scale_dt, e.wei_scale_mode == 1 ? 0 : n)
+                                 : p.wei_scale_val;
+    }
+    if (p.bias) c.bias = zmi_ld_f32(p.bias, e.bias_dt, n);
+    // u8 activations enter the MFMA as (a - 128): add 128 * colsum back, then
+    // subtract zp * colsum; both in s32
+    int32_t k = p.a_is_u8 ? 128 : 0;
+    if (e.has_zp) k -= p.src_zp_ptr ? *p.src_zp_ptr : p.src_zp_val;
+    if (k) c.comp = k * colsum[n];
+  }
+  return c;
+}
+
+__device__ __forceinline__ float zmi_row_scale(const ZmiEpilogue &e, const ZmiProblem &p, int m) {
+  switch (e.src_scale_mode) {
+  case ZMI_SS_VALUE: return p.src_scale_val;
+  case ZMI_SS_TENSOR_PTR: return zmi_ld_f32(p.src_scale_ptr, e.src_scale_dt, 0);
+  case ZMI_SS_TOKEN_PTR: return zmi_ld_f32(p.src_scale_ptr, e.src_scale_dt, m);
+  default: return 1.0f;
+  }
+}
+
+// acc -> f32 value before the store conversion (all steps separately rounded,
+// in the reference's order).
+__device__ __forceinline__ float zmi_epilogue_value(const ZmiEpilogue &e, int32_t acc, const ZmiColCtx &c,
+                                                    float rscale, int m, int n, const void *dst,
+                                                    int64_t ldc) {
+  float y;
+  if (e.alpha == 1.0f && e.beta == 0.0f) {
+    y = (float)(acc + c.comp);
+  } else {
+    // the reference scales and accumulates before it adds the compensation
+    y = (float)acc;
+    if (e.alpha != 1.0f) y = __fmul_rn(y, e.alpha);
+    if (e.beta != 0.0f) y = __fadd_rn(y, __fmul_rn(zmi_ld_f32(dst, e.dst_dt, (int64_t)m * ldc + n), e.beta));
+    y = __fadd_rn(y, (float)c.comp);
+  }
+  if (e.src_scale_mode) y = __fmul_rn(y, rscale);
+  if (e.wei_scale_mode) y = __fmul_rn(y, c.wscale);
+  y = __fadd_rn(y, c.bias);
+  for (int i = 0; i < e.n_po; ++i) {
+    const ZmiPostOp &po = e.po[i];
+    if (po.type == ZMI_PO_BINARY_ADD || po.type == ZMI_PO_BINARY_MUL) {
+      float t = zmi_ld_f32(po.buff, po.dtype, po.rowb ? (int64_t)n : (int64_t)m * po.ld + n);
+      y = po.type == ZMI_PO_BINARY_ADD ? __fadd_rn(y, t) : __fmul_rn(y, t);
+    } else {
+      y = zmi_eltwise(po.type, y, po.alpha, po.beta);
+    }
+  }
+  if (e.has_dst_q) {
+    float ds = e.dst_scale_ptr ? zmi_ld_f32(e.dst_scale_ptr, e.dst_scale_dt, 0) : e.dst_scale_val;
+    float dz = e.dst_zp_ptr ? zmi_ld_f32(e.dst_zp_ptr, e.dst_zp_dt, 0) : e.dst_zp_val;
+    y = __fadd_rn(__fmul_rn(y, ds), dz);
+  }
+  return y;
+}
+
+// Store conversions (reference: store_output,
+// zendnnl/src/operators/matmul/matmul_ref_kernel.cpp:154-254).
+__device__ __forceinline__ void zmi_store(void *dst, int dt, int64_t i, float y) {
+  switch (dt) {
+  case ZMI_DT_BF16: ((uint16_t *)dst)[i] = zmi_f32_to_bf16(y); break;
+  case ZMI_DT_S32: {
+    float v = fminf(fmaxf(y, -2147483648.0f), 2147483648.0f);
+    ((int32_t *)dst)[i] = v >= 2147483648.0f ? 2147483647 : (int32_t)rintf(v);
+    break;
+  }
+  case ZMI_DT_S8: ((int8_t *)dst)[i] = (int8_t)rintf(fminf(fmaxf(y, -128.0f), 127.0f)); break;
+  case ZMI_DT_U8: ((uint8_t *)dst)[i] = (uint8_t)rintf(fminf(fmaxf(y, 0.0f), 255.0f)); break;
+  default: ((float *)dst)[i] = y; break;
+  }
+}
+
+// True when the s32 accumulator (plus compensation) is the stored value: s32
+// destination, no scales, no bias, no post-ops.  The integer is then written
+// as is, which is exact where a float round trip would not be.
+__device__ __forceinline__ bool zmi_epilogue_is_raw_s32(const ZmiEpilogue &e, const void *bias) {
+  return e.dst_dt == ZMI_DT_S32 && !e.src_scale_mode && !e.wei_scale_mode && !bias && !e.n_po &&
+         !e.has_dst_q && e.alpha == 1.0f && e.beta == 0.0f;
+}
+#endif  // __HIPCC__

@@ -1,0 +1,75 @@
+// Host-side state shared by the C ABI entry points: error text, stream,
+// scratch arena, upload ring, packed-weight cache.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+namespace zmi {
+
+// ---- per-thread call context ------------------------------------------------
+void set_error(const std::string &msg);
+void clear_error();
+void set_kernel_name(const char *name);
+hipStream_t stream();
+
+// Returns false (and records the error) when a HIP call failed.
+bool hip_ok(hipError_t e, const char *what);
+
+// Makes sure a GPU is usable and the per-device state exists.
+bool ensure_device();
+
+// ---- scratch arena ------------------------------------------------------------
+// Grow-only device buffer owned by the calling thread.  begin() sizes it for
+// one API call (synchronising the stream only when it has to grow); alloc()
+// bump-allocates 256-byte aligned pieces until the next begin().
+class Arena {
+ public:
+  bool begin(size_t total_bytes);
+  void *alloc(size_t bytes);
+  void release();
+  static size_t padded(size_t bytes) { return (bytes + 255) / 256 * 256; }
+
+ private:
+  char *base_ = nullptr;
+  size_t cap_ = 0, used_ = 0;
+};
+Arena &arena();
+
+// ---- host -> device table upload ---------------------------------------------
+// Copies a small host table to device memory, ordered on the stream, without
+// synchronising: pinned staging slots recycled behind events.  Returns the
+// device address (valid until the slot is recycled, i.e. for this call).
+void *upload(const void *host, size_t bytes);
+// Ends a call's uploads: the slots it used stay reserved until the stream gets here.
+void upload_fence();
+
+// ---- one-element parameters ------------------------------------------------------
+// A scale / zero-point of one element may live in host or device memory.
+// Host: *value receives it and *dev_ptr is null.  Device: *dev_ptr receives
+// the pointer and the kernel reads it.
+bool scalar_param_f32(const void *buff, int32_t dt, float *value, const void **dev_ptr);
+bool scalar_param_s32(const void *buff, int32_t dt, int32_t *value, const int32_t **dev_ptr);
+
+// ---- packed weights ------------------------------------------------------------------
+// Returns the blob for plain [K,N] weights, packing on a miss.  With use_cache
+// the blob is kept for the life of the process keyed by (pointer, shape,
+// layout); otherwise it is packed into the arena (arena_slot must then have
+// been reserved by the caller with blob_bytes).
+const uint8_t *packed_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB,
+                              int32_t src_dtype, bool use_cache, void *arena_slot);
+void clear_weight_cache();
+
+// Checks (once per pointer) that a caller-supplied blob carries the header of a
+// blob packed for this K and N.
+bool blob_matches(const void *blob, int64_t K, int64_t N);
+
+int64_t nelems(const zmi_quant_t &q);
+bool diagnostics_enabled();
+int weight_cache_env();
+
+}  // namespace zmi

@@ -1,0 +1,338 @@
+// Host-side services behind the C ABI (see zmi_host.h).
+#include "zmi_host.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <list>
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <unordered_set>
+#include <vector>
+
+namespace zmi {
+
+namespace {
+struct ThreadCtx {
+  std::string error;
+  const char *kernel = "";
+  hipStream_t stream = nullptr;
+  Arena arena;
+  // upload ring
+  static constexpr int kSlots = 8;
+  static constexpr size_t kSlotBytes = 512 * 1024;
+  char *pinned = nullptr;
+  char *dev = nullptr;
+  hipEvent_t ev[kSlots] = {};
+  bool ev_live[kSlots] = {};   // an event is recorded and the slot is busy until it fires
+  bool used[kSlots] = {};      // written during the current call, not fenced yet
+  int next = 0;
+};
+thread_local ThreadCtx tctx;
+
+std::mutex g_mu;
+bool g_device_ready = false;
+
+struct CacheKey {
+  const void *ptr;
+  int64_t K, N, ldb;
+  bool transB;
+  bool operator<(const CacheKey &o) const {
+    return std::tie(ptr, K, N, ldb, transB) < std::tie(o.ptr, o.K, o.N, o.ldb, o.transB);
+  }
+};
+struct CacheVal {
+  uint8_t *blob;
+  std::list<CacheKey>::iterator lru;
+};
+std::map<CacheKey, CacheVal> g_cache;
+std::list<CacheKey> g_lru;
+std::unordered_set<const void *> g_checked_blobs;
+
+size_t cache_capacity() {
+  // same variable the reference reads for its weight caches
+  static const size_t cap = [] {
+    const char *e = std::getenv("ZENDNNL_LRU_CACHE_CAPACITY");
+    long v = e ? std::atol(e) : 0;
+    return v > 0 ? (size_t)v : (size_t)1 << 30;
+  }();
+  return cap;
+}
+}  // namespace
+
+void set_error(const std::string &msg) { tctx.error = msg; }
+void clear_error() { tctx.error.clear(); }
+void set_kernel_name(const char *name) { tctx.kernel = name; }
+hipStream_t stream() { return tctx.stream; }
+
+bool hip_ok(hipError_t e, const char *what) {
+  if (e == hipSuccess) return true;
+  set_error(std::string(what) + ": " + hipGetErrorString(e));
+  (void)hipGetLastError();
+  return false;
+}
+
+bool ensure_device() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_device_ready) return true;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n <= 0) {
+    set_error("no HIP device available (the library has no CPU fallback)");
+    (void)hipGetLastError();
+    return false;
+  }
+  g_device_ready = true;
+  return true;
+}
+
+// ---- arena ---------------------------------------------------------------------
+bool Arena::begin(size_t total) {
+  used_ = 0;
+  if (total <= cap_) return true;
+  // kernels of earlier calls may still read the old buffer
+  if (base_) {
+    if (!hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize")) return false;
+    if (!hip_ok(hipFree(base_), "hipFree(scratch)")) return false;
+    base_ = nullptr;
+    cap_ = 0;
+  }
+  size_t want = total + total / 4 + (1 << 20);
+  void *p = nullptr;
+  if (!hip_ok(hipMalloc(&p, want), "hipMalloc(scratch)")) return false;
+  base_ = (char *)p;
+  cap_ = want;
+  return true;
+}
+
+void *Arena::alloc(size_t bytes) {
+  size_t n = padded(bytes);
+  if (used_ + n > cap_) return nullptr;
+  void *p = base_ + used_;
+  used_ += n;
+  return p;
+}
+
+void Arena::release() {
+  if (base_) {
+    (void)hipStreamSynchronize(stream());
+    (void)hipFree(base_);
+  }
+  base_ = nullptr;
+  cap_ = used_ = 0;
+}
+
+Arena &arena() { return tctx.arena; }
+
+// ---- upload ring ------------------------------------------------------------------
+void *upload(const void *host, size_t bytes) {
+  ThreadCtx &c = tctx;
+  if (bytes == 0) return nullptr;
+  if (bytes > ThreadCtx::kSlotBytes) {
+    // too large for a ring slot: plain (synchronous for pageable memory) copy into the arena
+    void *d = c.arena.alloc(bytes);
+    if (!d) { set_error("upload: scratch arena too small"); return nullptr; }
+    if (!hip_ok(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, c.stream), "hipMemcpyAsync(upload)"))
+      return nullptr;
+    return d;
+  }
+  if (!c.pinned) {
+    void *p = nullptr, *d = nullptr;
+    if (!hip_ok(hipHostMalloc(&p, ThreadCtx::kSlots * ThreadCtx::kSlotBytes, hipHostMallocDefault),
+                "hipHostMalloc(upload ring)"))
+      return nullptr;
+    if (!hip_ok(hipMalloc(&d, ThreadCtx::kSlots * ThreadCtx::kSlotBytes), "hipMalloc(upload ring)")) return nullptr;
+    c.pinned = (char *)p;
+    c.dev = (char *)d;
+    for (int i = 0; i < ThreadCtx::kSlots; ++i)
+      if (!hip_ok(hipEventCreateWithFlags(&c.ev[i], hipEventDisableTiming), "hipEventCreate")) return nullptr;
+  }
+  const int s = c.next;
+  c.next = (c.next + 1) % ThreadCtx::kSlots;
+  if (c.used[s]) {
+    // the ring wrapped inside one call: fence the slot before it is rewritten
+    if (!hip_ok(hipEventRecord(c.ev[s], c.stream), "hipEventRecord(upload slot)")) return nullptr;
+    c.ev_live[s] = true;
+    c.used[s] = false;
+  }
+  if (c.ev_live[s]) {
+    if (!hip_ok(hipEventSynchronize(c.ev[s]), "hipEventSynchronize(upload slot)")) return nullptr;
+    c.ev_live[s] = false;
+  }
+  char *hp = c.pinned + (size_t)s * ThreadCtx::kSlotBytes;
+  char *dp = c.dev + (size_t)s * ThreadCtx::kSlotBytes;
+  std::memcpy(hp, host, bytes);
+  if (!hip_ok(hipMemcpyAsync(dp, hp, bytes, hipMemcpyHostToDevice, c.stream), "hipMemcpyAsync(upload)"))
+    return nullptr;
+  // the slot is free again once every kernel of this call that reads it has run;
+  // upload_fence() records that point
+  c.used[s] = true;
+  return dp;
+}
+
+// Marks every slot used since the last fence as busy until the stream reaches
+// this point.  Called at the end of each API entry point that uploaded tables.
+void upload_fence() {
+  ThreadCtx &c = tctx;
+  if (!c.pinned) return;
+  for (int i = 0; i < ThreadCtx::kSlots; ++i) {
+    if (c.used[i]) {
+      (void)hipEventRecord(c.ev[i], c.stream);
+      c.ev_live[i] = true;
+      c.used[i] = false;
+    }
+  }
+}
+
+// ---- one-element parameters ------------------------------------------------------
+static bool is_device_pointer(const void *p) {
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, p);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return false;   // ordinary host memory
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+bool scalar_param_f32(const void *buff, int32_t dt, float *value, const void **dev_ptr) {
+  *dev_ptr = nullptr;
+  *value = 1.0f;
+  if (!buff) return true;
+  if (is_device_pointer(buff)) {
+    *dev_ptr = buff;
+    return true;
+  }
+  switch (dt) {
+  case ZMI_DT_F32: *value = *(const float *)buff; return true;
+  case ZMI_DT_BF16: {
+    uint32_t u = ((uint32_t) * (const uint16_t *)buff) << 16;
+    std::memcpy(value, &u, 4);
+    return true;
+  }
+  case ZMI_DT_S32: *value = (float)*(const int32_t *)buff; return true;
+  case ZMI_DT_S8: *value = (float)*(const int8_t *)buff; return true;
+  case ZMI_DT_U8: *value = (float)*(const uint8_t *)buff; return true;
+  default: set_error("unsupported dtype for a one-element scale / zero-point"); return false;
+  }
+}
+
+bool scalar_param_s32(const void *buff, int32_t dt, int32_t *value, const int32_t **dev_ptr) {
+  *dev_ptr = nullptr;
+  *value = 0;
+  if (!buff) return true;
+  if (dt != ZMI_DT_S32) {
+    set_error("source zero-point must be s32");
+    return false;
+  }
+  if (is_device_pointer(buff)) {
+    *dev_ptr = (const int32_t *)buff;
+    return true;
+  }
+  *value = *(const int32_t *)buff;
+  return true;
+}
+
+// ---- packed weights ------------------------------------------------------------------
+const uint8_t *packed_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB,
+                              int32_t src_dtype, bool use_cache, void *arena_slot) {
+  if (!use_cache) {
+    if (!hip_ok(zmi_launch_prepack((const int8_t *)weight, K, N, ldb, transB, src_dtype, 0,
+                                   (uint8_t *)arena_slot, stream()), "prepack launch"))
+      return nullptr;
+    return (const uint8_t *)arena_slot;
+  }
+  std::lock_guard<std::mutex> lk(g_mu);
+  CacheKey key{weight, K, N, ldb, transB};
+  auto it = g_cache.find(key);
+  if (it != g_cache.end()) {
+    g_lru.splice(g_lru.begin(), g_lru, it->second.lru);
+    return it->second.blob;
+  }
+  void *blob = nullptr;
+  if (!hip_ok(hipMalloc(&blob, (size_t)zmi_blob_bytes(K, N)), "hipMalloc(packed weights)")) return nullptr;
+  if (!hip_ok(zmi_launch_prepack((const int8_t *)weight, K, N, ldb, transB, src_dtype, 0, (uint8_t *)blob,
+                                 stream()), "prepack launch")) {
+    (void)hipFree(blob);
+    return nullptr;
+  }
+  g_lru.push_front(key);
+  g_cache[key] = CacheVal{(uint8_t *)blob, g_lru.begin()};
+  while (g_cache.size() > cache_capacity()) {
+    // an evicted blob may still be read by enqueued kernels
+    (void)hipDeviceSynchronize();
+    CacheKey old = g_lru.back();
+    g_lru.pop_back();
+    (void)hipFree(g_cache[old].blob);
+    g_cache.erase(old);
+  }
+  return (const uint8_t *)blob;
+}
+
+void clear_weight_cache() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!g_cache.empty()) (void)hipDeviceSynchronize();
+  for (auto &kv : g_cache) (void)hipFree(kv.second.blob);
+  g_cache.clear();
+  g_lru.clear();
+  g_checked_blobs.clear();
+}
+
+bool blob_matches(const void *blob, int64_t K, int64_t N) {
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_checked_blobs.count(blob)) return true;
+  }
+  ZmiBlobHeader h;
+  if (!hip_ok(hipMemcpyAsync(&h, blob, sizeof(h), hipMemcpyDeviceToHost, stream()), "hipMemcpy(blob header)"))
+    return false;
+  if (!hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize")) return false;
+  if (h.magic != ZMI_BLOB_MAGIC || h.K != K || h.N != N) {
+    set_error("mem_format_b == 'r': the weight buffer is not a blob packed by reorder_direct for this K and N");
+    return false;
+  }
+  std::lock_guard<std::mutex> lk(g_mu);
+  g_checked_blobs.insert(blob);
+  return true;
+}
+
+int64_t nelems(const zmi_quant_t &q) {
+  int64_t n = 1;
+  for (int i = 0; i < q.ndims && i < ZMI_MAX_DIMS; ++i) n *= q.dims[i];
+  return n;
+}
+
+bool diagnostics_enabled() {
+  // validation gate of the reference (ZENDNNL_DIAGNOSTICS_ENABLE, on unless "0")
+  const char *e = std::getenv("ZENDNNL_DIAGNOSTICS_ENABLE");
+  return !(e && e[0] == '0' && e[1] == 0);
+}
+
+int weight_cache_env() {
+  const char *e = std::getenv("ZENDNNL_MATMUL_WEIGHT_CACHE");
+  if (!e) return 2;
+  int v = std::atoi(e);
+  return v < 0 ? 0 : (v > 2 ? 2 : v);
+}
+
+}  // namespace zmi
+
+// ---- C ABI: library services ---------------------------------------------------------
+extern "C" {
+
+int32_t zmi_init(int32_t device) {
+  zmi::clear_error();
+  if (!zmi::ensure_device()) return ZMI_FAILURE;
+  if (!zmi::hip_ok(hipSetDevice(device), "hipSetDevice")) return ZMI_FAILURE;
+  return ZMI_SUCCESS;
+}
+
+void zmi_set_stream(void *hip_stream) { zmi::tctx.stream = (hipStream_t)hip_stream; }
+void *zmi_get_stream(void) { return (void *)zmi::tctx.stream; }
+const char *zmi_last_error(void) { return zmi::tctx.error.c_str(); }
+const char *zmi_last_kernel(void) { return zmi::tctx.kernel; }
+void zmi_clear_weight_cache(void) { zmi::clear_weight_cache(); }
+void zmi_clear_scratch(void) { zmi::tctx.arena.release(); }
+const char *zmi_version(void) { return "zmi-lowoha 0.1.0 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,76 @@
+// Host-callable launchers of the gfx950 kernels (one per .hip file).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "zmi_device.h"
+
+// One matrix of a (possibly grouped) per-token quantization launch; row_start is
+// the index of its first row in the launch's global row numbering.
+struct ZmiQuantMat {
+  const void *src;
+  int8_t *dst;       // may be null: scales only
+  void *scale;
+  int64_t ld_src, ld_dst;
+  int32_t M, K;
+  int32_t row_start;
+};
+
+// k_prepack.hip
+hipError_t zmi_launch_prepack(const int8_t *B, int64_t K, int64_t N, int64_t ldb, int transposed,
+                              int32_t src_dtype, int32_t sym_group_size, uint8_t *blob,
+                              hipStream_t stream);
+
+// k_quant.hip
+hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
+                                 int8_t *dst, int64_t ld_dst, void *scales, int32_t scale_dt,
+                                 hipStream_t stream);
+hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_t total_rows,
+                                  int32_t src_dt, int32_t scale_dt, hipStream_t stream);
+hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
+                                   int8_t *dst, int64_t ld_dst, float *scales, unsigned int *amax_scratch,
+                                   hipStream_t stream);
+
+// k_gemm.hip
+hipError_t zmi_launch_gemm_mfma(const ZmiProblem &p, const ZmiEpilogue &epi, int BM, hipStream_t stream);
+hipError_t zmi_launch_gemm_mfma_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
+                                      int m_lo, int worst_items, const ZmiEpilogue &epi, int BM,
+                                      hipStream_t stream);
+
+// k_smallm.hip
+hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev,
+                                        int n_prob, int m_lo, int m_hi, int worst_grid, int64_t kpad_hint,
+                                        const ZmiEpilogue &epi, hipStream_t stream);
+
+// k_moe.hip
+struct ZmiActMat {
+  void *buf;
+  int64_t ld;
+  int32_t M, N;
+  int32_t row_start;
+};
+hipError_t zmi_launch_gated_act(const ZmiActMat *mats_dev, const ZmiActMat *mat0, int n_mat,
+                                int64_t total_rows, int max_N, int32_t act, int32_t dt, hipStream_t stream);
+hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *rows_base, int64_t row_ld,
+                                  const int32_t *slot_of, const float *weights, int skip_weighted,
+                                  int T, int topk, int D, int32_t dt, void *out, int64_t ldo,
+                                  hipStream_t stream);
+hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int32_t *counts,
+                                int32_t *offsets, int32_t *slot_of, hipStream_t stream);
+hipError_t zmi_launch_moe_quant_scatter(const void *x, int64_t ldx, int T, int H, int topk,
+                                        const int32_t *slot_of, int8_t *A1, float *s1, hipStream_t stream);
+struct ZmiMoeTables {   // device arrays of E entries each
+  const void *const *w13_blob;
+  const void *const *w2_blob;
+  const float *const *w13_scale;
+  const float *const *w2_scale;
+};
+hipError_t zmi_launch_moe_build_problems(ZmiMoeTables tb, int E, int H, int I, const int32_t *counts,
+                                         const int32_t *offsets, const int8_t *A1, const float *s1,
+                                         void *act, const int8_t *A2, const float *s2, void *Y,
+                                         ZmiProblem *op1, ZmiProblem *op2, hipStream_t stream);
+
+// k_util.hip
+hipError_t zmi_launch_pad_rows(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans,
+                               int8_t *dst, int64_t ld_dst, hipStream_t stream);
