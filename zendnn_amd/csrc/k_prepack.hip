@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void zmi_prepack_kernel(const int8_t *__restri
   #pragma unroll
   for (int b = 0; b < 16; ++b) out[b] = patch[krow + b][col];
   const int64_t nb = n0 / 32 + fnb, kb = k0 / 32 + fkb;
-  uint8_t *dst = tiles + (nb * kblocks + kb) * 1024 + lane * 16;
+  uint8_t *dst = tiles + nb * zmi_blob_nb_stride(K) + kb * 1024 + lane * 16;
   *(v4i *)dst = *(const v4i *)out;
 }
 
@@ -70,10 +70,11 @@ __global__ __launch_bounds__(256) void zmi_prepack_kernel(const int8_t *__restri
 // 32-column block; lane i adds its 16 bytes of every fragment, lanes i and
 // i+32 hold the two k halves of the same column.
 __global__ __launch_bounds__(64) void zmi_colsum_kernel(const uint8_t *__restrict__ tiles,
-                                                        int64_t kblocks, int32_t *__restrict__ colsum) {
+                                                        int64_t kblocks, int64_t nb_stride,
+                                                        int32_t *__restrict__ colsum) {
   const int lane = threadIdx.x;
   const int64_t nb = blockIdx.x;
-  const uint8_t *p = tiles + nb * kblocks * 1024 + lane * 16;
+  const uint8_t *p = tiles + nb * nb_stride + lane * 16;
   int32_t s = 0;
   for (int64_t kb = 0; kb < kblocks; ++kb) {
     v4i v = *(const v4i *)(p + kb * 1024);
@@ -118,7 +119,7 @@ hipError_t zmi_launch_prepack(const int8_t *B, int64_t K, int64_t N, int64_t ldb
   else
     hipLaunchKernelGGL(zmi_prepack_kernel<false>, grid, dim3(256), 0, stream, B, K, N, ldb, tiles, kblocks);
   hipLaunchKernelGGL(zmi_colsum_kernel, dim3((unsigned)(N_pad / 32)), dim3(64), 0, stream, tiles, kblocks,
-                     colsum);
+                     zmi_blob_nb_stride(K), colsum);
   hipLaunchKernelGGL(zmi_blob_header_kernel, dim3(1), dim3(64), 0, stream, (ZmiBlobHeader *)blob, K, N,
                      src_dtype, sym_group_size);
   return hipGetLastError();

@@ -47,7 +47,6 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
   }
   const int M = p.M, N = p.N, K = p.K;
   const int64_t K_pad = zmi_blob_kpad(K);
-  const int64_t kblocks = K_pad / 32;
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
 
@@ -70,7 +69,7 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
     const int64_t nb = wcol[h] / 32;
     const int coff = wcol[h] % 32;
     // fragment (nb, 2c + g/2), lane (g%2)*32 + coff + c16
-    bsrc[h] = tiles + (nb * kblocks + g / 2) * 1024 + ((g % 2) * 32 + coff + c16) * 16;
+    bsrc[h] = tiles + nb * zmi_blob_nb_stride(K) + (g / 2) * 1024 + ((g % 2) * 32 + coff + c16) * 16;
   }
   const int8_t *A = (const int8_t *)p.A;
   const uint32_t xor_mask = p.a_is_u8 ? 0x80808080u : 0u;

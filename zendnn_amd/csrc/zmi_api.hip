@@ -214,6 +214,13 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
     ++n_po;
   }
   e.n_po = n_po;
+  e.fast_kind = ZMI_EK_GENERIC;
+  if (alpha == 1.0f && beta == 0.0f && !e.has_dst_q && n_po <= 1 && (p.dt_dst == ZMI_DT_BF16 || p.dt_dst == ZMI_DT_F32)) {
+    if (n_po == 0) e.fast_kind = ZMI_EK_NONE;
+    else if (e.po[0].type == ZMI_PO_SWISH) e.fast_kind = ZMI_EK_SWISH;
+    else if (e.po[0].type == ZMI_PO_GELU_TANH) e.fast_kind = ZMI_EK_GELU_TANH;
+    else if (e.po[0].type == ZMI_PO_RELU) e.fast_kind = ZMI_EK_RELU;
+  }
   *out = e;
   return ZMI_SUCCESS;
 }
@@ -223,9 +230,11 @@ static int pick_bm(int M, int N) {
     int v = std::atoi(env);
     if (v == 64 || v == 128 || v == 256) return v;
   }
+  // Measured on MI355X (K = 4096): with 2 workgroups resident per CU the 64-row
+  // tile wins while there are fewer than about two 128-row tiles per CU, the
+  // 128-row tile after that.
   auto tiles = [&](int bm) { return (int64_t)((M + bm - 1) / bm) * ((N + 255) / 256); };
-  if (tiles(256) >= 2 * 256 && M >= 256) return 256;
-  if (tiles(128) >= 256 || M > 64) return tiles(128) >= 128 ? 128 : 64;
+  if (tiles(128) >= 2 * 256) return 128;
   return 64;
 }
 

@@ -631,7 +631,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   std::memset(&e1, 0, sizeof(e1));
   e1.src_scale_mode = ZMI_SS_TOKEN_PTR; e1.src_scale_dt = ZMI_DT_F32;
   e1.wei_scale_mode = 2; e1.wei_scale_dt = ZMI_DT_F32;
-  e1.bias_dt = ZMI_DT_F32; e1.alpha = 1.0f; e1.beta = 0.0f; e1.dst_dt = ZMI_DT_BF16;
+  e1.bias_dt = ZMI_DT_F32; e1.alpha = 1.0f; e1.beta = 0.0f; e1.dst_dt = ZMI_DT_BF16; e1.fast_kind = ZMI_EK_NONE;
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
   // row counts live on the device: size the grids for the worst case

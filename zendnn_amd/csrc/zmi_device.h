@@ -28,6 +28,12 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 #define ZMI_BLOB_HEADER_BYTES 256
 #define ZMI_KPAD 128
 #define ZMI_NPAD 64
+// Bytes skipped between consecutive column blocks.  Without it the streams of
+// all column blocks at the same K offset sit a power of two apart and land on
+// the same L2 / memory channel.
+#ifndef ZMI_NB_SKEW
+#define ZMI_NB_SKEW 0
+#endif
 
 struct ZmiBlobHeader {
   uint64_t magic;
@@ -47,8 +53,12 @@ static inline __host__ __device__ int64_t zmi_blob_colsum_off() { return ZMI_BLO
 static inline __host__ __device__ int64_t zmi_blob_tiles_off(int64_t N) {
   return zmi_round_up(ZMI_BLOB_HEADER_BYTES + zmi_blob_npad(N) * 4, 256);
 }
+// distance in bytes between the fragment streams of consecutive column blocks
+static inline __host__ __device__ int64_t zmi_blob_nb_stride(int64_t K) {
+  return zmi_blob_kpad(K) * 32 + ZMI_NB_SKEW;
+}
 static inline __host__ __device__ int64_t zmi_blob_bytes(int64_t K, int64_t N) {
-  return zmi_blob_tiles_off(N) + zmi_blob_kpad(K) * zmi_blob_npad(N);
+  return zmi_blob_tiles_off(N) + zmi_blob_nb_stride(K) * (zmi_blob_npad(N) / 32);
 }
 
 // ---------------------------------------------------------------------------
@@ -71,6 +81,11 @@ struct ZmiPostOp {
 
 enum { ZMI_SS_NONE = 0, ZMI_SS_VALUE = 1, ZMI_SS_TENSOR_PTR = 2, ZMI_SS_TOKEN_PTR = 3 };
 
+// Straight-line epilogue variants: alpha == 1, beta == 0, no destination
+// quantization, bf16 or f32 destination, at most one element-wise post-op of
+// the named type.  Everything else runs the generic interpreter.
+enum { ZMI_EK_GENERIC = 0, ZMI_EK_NONE = 1, ZMI_EK_SWISH = 2, ZMI_EK_GELU_TANH = 3, ZMI_EK_RELU = 4 };
+
 struct ZmiEpilogue {
   int32_t src_scale_mode;  // ZMI_SS_*
   int32_t src_scale_dt;
@@ -90,6 +105,7 @@ struct ZmiEpilogue {
   float dst_zp_val;
   int32_t dst_dt;
   int32_t gated_act;      // enum zmi_gated_act; != 0: columns are [gate | up] halves
+  int32_t fast_kind;      // ZMI_EK_*: straight-line epilogue variant, 0 = generic interpreter
 };
 
 // One GEMM problem: C[M,N] = epilogue(A[M,K] x blob), with the operands the
@@ -268,6 +284,27 @@ __device__ __forceinline__ float zmi_epilogue_value(const ZmiEpilogue &e, int32_
     y = __fadd_rn(__fmul_rn(y, ds), dz);
   }
   return y;
+}
+
+// Straight-line form of zmi_epilogue_value + zmi_store for the ZMI_EK_* variants:
+// same operations in the same order, no interpretation in the inner loop.
+template <int EK>
+__device__ __forceinline__ float zmi_fast_value(int32_t acc, const ZmiColCtx &c, float rscale, bool has_rs,
+                                                bool has_ws, bool has_bias) {
+  float y = (float)(acc + c.comp);
+  if (has_rs) y = __fmul_rn(y, rscale);
+  if (has_ws) y = __fmul_rn(y, c.wscale);
+  if (has_bias) y = __fadd_rn(y, c.bias);
+  if (EK == ZMI_EK_SWISH) y = zmi_eltwise(ZMI_PO_SWISH, y, 0.0f, 0.0f);
+  if (EK == ZMI_EK_GELU_TANH) y = zmi_eltwise(ZMI_PO_GELU_TANH, y, 0.0f, 0.0f);
+  if (EK == ZMI_EK_RELU) y = zmi_eltwise(ZMI_PO_RELU, y, 0.0f, 0.0f);
+  return y;
+}
+
+template <bool BF16>
+__device__ __forceinline__ void zmi_fast_store(void *dst, int64_t i, float y) {
+  if (BF16) ((uint16_t *)dst)[i] = zmi_f32_to_bf16(y);
+  else ((float *)dst)[i] = y;
 }
 
 // Store conversions (reference: store_output,
