@@ -1,0 +1,142 @@
+"""Synthetic MoE problems for the group_matmul_direct parity tests, the
+caller-side scatter the reference expects from the framework, and the oracle
+composition of the fused block."""
+import numpy as np
+import torch
+
+from zendnn_amd import capi, lowoha
+from tests import gpu_helpers as H
+
+
+class MoeCase:
+    pass
+
+
+def make_case(seed, T, Hd, I, E, topk, skew=False):
+    """Seeded problem on the host: tokens, routing, per-expert int8 weights and scales."""
+    rng = np.random.default_rng(seed)
+    c = MoeCase()
+    c.T, c.H, c.I, c.E, c.topk = T, Hd, I, E, topk
+    c.x = H.gen_bf16_normal(rng, (T, Hd))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if skew:
+        logits = logits + (rng.standard_normal(E) * 1.5).astype(np.float32)[None, :]
+    z = np.exp(logits - logits.max(axis=1, keepdims=True))
+    prob = (z / z.sum(axis=1, keepdims=True)).astype(np.float32)
+    c.ids = np.argsort(-prob, axis=1, kind="stable")[:, :topk].astype(np.int32)
+    # the two (or six) softmax probabilities themselves, not renormalised
+    c.w = np.take_along_axis(prob, c.ids, axis=1).astype(np.float32)
+    c.w13 = [H.gen_weights(rng, Hd, 2 * I) for _ in range(E)]
+    c.w2 = [H.gen_weights(rng, I, Hd) for _ in range(E)]
+    c.s13 = [rng.uniform(0.001, 0.01, 2 * I).astype(np.float32) for _ in range(E)]
+    c.s2 = [rng.uniform(0.001, 0.01, Hd).astype(np.float32) for _ in range(E)]
+    # caller-side scatter: rows of expert e in (t, k) order
+    c.rows_of = [[] for _ in range(E)]
+    c.slot = np.zeros((T, topk, 2), dtype=np.int64)      # (expert, row index inside the expert)
+    for t in range(T):
+        for k in range(topk):
+            e = int(c.ids[t, k])
+            c.slot[t, k] = (e, len(c.rows_of[e]))
+            c.rows_of[e].append(t)
+    c.M = [len(r) for r in c.rows_of]
+    return c
+
+
+def dyn_params(M, N, ws_buf, dst_dt=capi.DT_BF16, packed=False):
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=dst_dt, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_buf, capi.DT_F32, (1, N))
+    if packed:
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+    return p
+
+
+def oracle_expert(zo, c, e, x_rows, act=capi.ACT_SILU_AND_MUL):
+    """Reference composition for the rows of one expert: dynamic-quant Op1 -> bf16 ->
+    gated activation -> bf16 -> dynamic-quant Op2 -> bf16
+    (group_matmul_fused_moe.cpp:906-1078, the two-pass form)."""
+    M = x_rows.shape[0]
+    keep = []
+    p1 = dyn_params(M, 2 * c.I, c.s13[e].ctypes.data).flat(keep)
+    st, y1, _, _ = zo.matmul_int8(x_rows, c.w13[e], p1, M, 2 * c.I, c.H)
+    assert st == capi.SUCCESS
+    zo.gated_act(act, y1, capi.DT_BF16)
+    a = np.ascontiguousarray(y1[:, :c.I])
+    p2 = dyn_params(M, c.H, c.s2[e].ctypes.data).flat(keep)
+    st, y2, _, _ = zo.matmul_int8(a, c.w2[e], p2, M, c.H, c.I)
+    assert st == capi.SUCCESS
+    return a, y2
+
+
+def oracle_moe(zo, c, tokens):
+    """Final output rows for the given token indices."""
+    need = {}
+    for t in tokens:
+        for k in range(c.topk):
+            e, j = c.slot[t, k]
+            need.setdefault(int(e), []).append((int(t), k))
+    y2_of = {}
+    for e, lst in need.items():
+        xr = np.ascontiguousarray(c.x[[t for t, _ in lst]])
+        _, y2 = oracle_expert(zo, c, e, xr)
+        for i, (t, k) in enumerate(lst):
+            y2_of[(t, k)] = y2[i]
+    rows = [np.ascontiguousarray(y2_of[(int(t), k)]) for t in tokens for k in range(c.topk)]
+    wsel = np.ascontiguousarray(c.w[list(tokens)])
+    return zo.moe_reduce(rows, wsel, capi.DT_BF16, c.H)
+
+
+class DeviceMoe:
+    """Device buffers of a case plus the per-expert scattered sources."""
+
+    def __init__(self, c, packed=False):
+        self.c = c
+        x_d = H.to_dev(c.x)
+        self.x = x_d
+        self.src, self.dst_down = [], []
+        for e in range(c.E):
+            if c.M[e]:
+                idx = torch.tensor(c.rows_of[e], dtype=torch.long, device=H.DEV)
+                self.src.append(x_d.index_select(0, idx).contiguous())
+                self.dst_down.append(torch.zeros((c.M[e], c.H), dtype=torch.bfloat16, device=H.DEV))
+            else:
+                self.src.append(None)
+                self.dst_down.append(None)
+        self.w13 = [H.to_dev(w) for w in c.w13]
+        self.w2 = [H.to_dev(w) for w in c.w2]
+        self.s13 = [H.to_dev(s) for s in c.s13]
+        self.s2 = [H.to_dev(s) for s in c.s2]
+        self.topk_w = H.to_dev(c.w)
+        self.out = torch.zeros((c.T, c.H), dtype=torch.bfloat16, device=H.DEV)
+        self.w13_arg = self.w13
+        if packed:
+            self.w13_arg = [H.prepack(w, c.H, 2 * c.I) for w in self.w13]
+        self.packed = packed
+
+    def row_ptrs(self):
+        c = self.c
+        out = []
+        for t in range(c.T):
+            for k in range(c.topk):
+                e, j = c.slot[t, k]
+                out.append(self.dst_down[e].data_ptr() + int(j) * c.H * 2)
+        return out
+
+    def call_fused(self, with_postop=True, act=capi.ACT_SILU_AND_MUL):
+        c = self.c
+        E = c.E
+        params = [dyn_params(max(c.M[e], 0), 2 * c.I, self.s13[e], packed=self.packed) for e in range(E)]
+        fm = lowoha.FusedMoe(
+            down_weight=self.w2, N_down=[c.H] * E, ldb_down=[c.H] * E,
+            down_scale=[lowoha.QuantParam(self.s2[e], capi.DT_F32, (1, c.H)) for e in range(E)],
+            dst_down=self.dst_down, ldc_down=[c.H] * E)
+        pp = None
+        if with_postop:
+            pp = lowoha.MoePostop(c.T, c.topk, self.out, c.H, self.topk_w, self.row_ptrs())
+        return lowoha.group_matmul_direct(
+            ["r"] * E, [False] * E, [False] * E, c.M, [2 * c.I] * E, [c.H] * E, [1.0] * E,
+            self.src, [c.H] * E, self.w13_arg, [2 * c.I] * E, [None] * E, [0.0] * E,
+            [None] * E, [2 * c.I] * E, [True] * E, params,
+            moe_postop=pp, gated_act=act, fused_moe=fm)
