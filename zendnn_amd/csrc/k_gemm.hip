@@ -177,8 +177,10 @@ __global__ __launch_bounds__(G_THREADS, (BM > 128 ? 1 : 2)) void zmi_gemm_mfma_k
   // valid chunk of the row instead (the blob's rows beyond K are zero, so the
   // values do not matter, only that the address is valid).
   auto load_a = [&](int kt, v4i (&r)[A_CHUNKS]) {
+    // rows are readable up to K rounded up to 16 (the host repacks A otherwise)
+    const int k_last = ((K + 15) & ~15) - 16;
     int k = kt * G_BK + a_kc * 16;
-    if (k > K - 16) k = K - 16;
+    if (k > k_last) k = k_last;
     #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) r[i] = *(const v4i *)(a_src[i] + k);
   };

@@ -218,7 +218,8 @@ __device__ __forceinline__ float zmi_gated(int act, float g, float u) {
 struct ZmiColCtx {
   float wscale;
   float bias;
-  int32_t comp;
+  int32_t comp;    // everything added to the MFMA accumulator: u8 shift and zero-point compensation
+  int32_t shift;   // the u8 part alone (128 * colsum): accumulator + shift is the true sum of a*w
 };
 
 __device__ __forceinline__ ZmiColCtx zmi_col_ctx(const ZmiEpilogue &e, const ZmiProblem &p,
@@ -227,6 +228,7 @@ __device__ __forceinline__ ZmiColCtx zmi_col_ctx(const ZmiEpilogue &e, const Zmi
   c.wscale = 1.0f;
   c.bias = 0.0f;
   c.comp = 0;
+  c.shift = 0;
   if (n < N) {
     if (e.wei_scale_mode) {
       c.wscale = p.wei_scale_ptr ? zmi_ld_f32(p.wei_scale_ptr, e.wei_scale_dt, e.wei_scale_mode == 1 ? 0 : n)
@@ -238,6 +240,7 @@ __device__ __forceinline__ ZmiColCtx zmi_col_ctx(const ZmiEpilogue &e, const Zmi
     int32_t k = p.a_is_u8 ? 128 : 0;
     if (e.has_zp) k -= p.src_zp_ptr ? *p.src_zp_ptr : p.src_zp_val;
     if (k) c.comp = k * colsum[n];
+    if (p.a_is_u8) c.shift = 128 * colsum[n];
   }
   return c;
 }
@@ -261,10 +264,10 @@ __device__ __forceinline__ float zmi_epilogue_value(const ZmiEpilogue &e, int32_
     y = (float)(acc + c.comp);
   } else {
     // the reference scales and accumulates before it adds the compensation
-    y = (float)acc;
+    y = (float)(acc + c.shift);
     if (e.alpha != 1.0f) y = __fmul_rn(y, e.alpha);
     if (e.beta != 0.0f) y = __fadd_rn(y, __fmul_rn(zmi_ld_f32(dst, e.dst_dt, (int64_t)m * ldc + n), e.beta));
-    y = __fadd_rn(y, (float)c.comp);
+    if (e.has_zp) y = __fadd_rn(y, (float)(c.comp - c.shift));
   }
   if (e.src_scale_mode) y = __fmul_rn(y, rscale);
   if (e.wei_scale_mode) y = __fmul_rn(y, c.wscale);
