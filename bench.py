@@ -1,0 +1,308 @@
+#!/usr/bin/env python3
+"""Benchmark of the LowOHA int8 matmul path on one MI355X.
+
+Headline workload (BASELINE.json configs[1], the decode shape): one
+matmul_direct call per step, M=16, K=4096, N=14336, bf16 activations quantized
+per token to s8 inside the call, prepacked s8 weights with per-channel scales,
+fused SiLU, bf16 output.  The metric is the algorithmic bytes of one call
+(weights K*N + activations M*K*2 + scales N*4 + output M*N*2) divided by the
+time of one call, in GB/s; the roofline that bounds it is HBM (8 TB/s).
+
+Weights rotate through enough prepacked copies to exceed the 256 MB on-die
+cache, so every step streams its weights from HBM (the reference's "warm"
+benchmark mode, benchdnn/doc/matmul.md:171-181).  Inputs are resident in HBM
+before the timed region.
+
+Prints ONE JSON line.  The other BASELINE.json configs are timed briefly and
+reported under "other_configs" in the same line.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+INT8_PEAK_TOPS = 5000.0
+K_DEC, N_DEC = 4096, 14336
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; the path has no multi-GPU part (--gpus must be 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from zendnn_amd import capi, lowoha
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = capi.load()      # raises if the HIP library is not built: there is no fallback
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    lib.zmi_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    g = torch.Generator(device=dev)
+    g.manual_seed(0x5EED0002)
+
+    def prepack(w, K, N, src_dt=capi.DT_S8):
+        rp = lowoha.ReorderParams()
+        rp.is_prepack = True
+        rp.prepack_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        rp.prepack_wei_dtype = capi.DT_S8
+        rp.prepack_src_dtype = src_dt
+        rp.prepack_K, rp.prepack_N, rp.prepack_ldb = K, N, N
+        size = lowoha.weight_prepack_size(rp)
+        blob = torch.empty(size, dtype=torch.uint8, device=dev)
+        assert lowoha.reorder_direct(w, blob, rp) == capi.SUCCESS, lowoha.last_error()
+        return blob
+
+    def rand_w(K, N):
+        return torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+
+    def ev_time(fn, steps, warmup):
+        """Average milliseconds per call: warmup untimed calls, then `steps` calls between two
+        events on the library's stream, synchronised on both sides."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    # ------------------------------------------------------------ decode (headline)
+    def decode_setup(M, n_sets):
+        blobs = [prepack(rand_w(K_DEC, N_DEC), K_DEC, N_DEC) for _ in range(n_sets)]
+        ws = torch.rand(N_DEC, device=dev, generator=g) * 0.009 + 0.001
+        x = torch.randn((M, K_DEC), device=dev, generator=g).to(torch.bfloat16)
+        dst = torch.zeros((M, N_DEC), dtype=torch.bfloat16, device=dev)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (M, 1))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N_DEC))
+        p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        state = {"i": 0}
+
+        def step():
+            blob = blobs[state["i"] % n_sets]
+            state["i"] += 1
+            st = lowoha.matmul_direct("r", False, False, M, N_DEC, K_DEC, 1.0, x, K_DEC, blob, N_DEC, None, 0.0,
+                                      dst, N_DEC, True, p)
+            if st != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+
+        # the GEMM kernel alone: the same call on rows that are already s8 with given scales
+        xq = torch.randint(-127, 128, (M, K_DEC), dtype=torch.int8, device=dev, generator=g)
+        xs = torch.rand(M, device=dev, generator=g) * 0.02 + 0.01
+        pk = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16)
+        pk.src_scale = lowoha.QuantParam(xs, capi.DT_F32, (M, 1) if M > 1 else (1,))
+        pk.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N_DEC))
+        pk.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+        pk.mem_format_b = "r"
+        pk.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+
+        def kernel_only():
+            blob = blobs[state["i"] % n_sets]
+            state["i"] += 1
+            st = lowoha.matmul_direct("r", False, False, M, N_DEC, K_DEC, 1.0, xq, K_DEC, blob, N_DEC, None, 0.0,
+                                      dst, N_DEC, True, pk)
+            if st != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+
+        keep = (blobs, ws, x, dst, xq, xs)
+        return step, kernel_only, keep
+
+    def decode_bytes(M):
+        return K_DEC * N_DEC + M * K_DEC * 2 + N_DEC * 4 + M * N_DEC * 2
+
+    M = 16
+    n_sets = 8
+    step, kernel_only, keep = decode_setup(M, n_sets)
+    ms = ev_time(step, args.steps, args.warmup)
+    value = decode_bytes(M) / (ms * 1e-3) / 1e9
+    ms_k = ev_time(kernel_only, args.steps, args.warmup)
+    kernel_name = lowoha.last_kernel()
+    # algorithmic bytes of the kernel launch: s8 rows instead of bf16 rows, plus the row scales
+    kbytes = K_DEC * N_DEC + M * K_DEC + M * 4 + N_DEC * 4 + M * N_DEC * 2
+    achieved = kbytes / (ms_k * 1e-3) / 1e9
+
+    result = {
+        "metric": "decode_int8_gemm_weight_streaming",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "s8 x s8 -> s32 (f32 epilogue, bf16 store)",
+        "data": "synthetic",
+        "config": {"workload": "matmul_direct decode: M=16 K=4096 N=14336, bf16 -> per-token s8, "
+                               "prepacked s8 weights, per-channel scales, SiLU, bf16 out",
+                   "weight_sets_rotated": n_sets, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1)},
+        "roofline": {"bound": "hbm", "kernel": "zmi_gemm_smallm_kernel<1,4> (" + kernel_name + ")",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": kbytes,
+                     "avg_launch_us": round(ms_k * 1e3, 2),
+                     "note": "launches timed back to back between two events on the kernel's stream, "
+                             "so the figure includes the dispatch gap between launches"},
+    }
+
+    if not args.no_extras:
+        other = {}
+        del keep
+        torch.cuda.empty_cache()
+        # decode at M = 1 and 4
+        for m in (1, 4):
+            s, k, kp = decode_setup(m, n_sets)
+            t = ev_time(s, 100, 10)
+            tk = ev_time(k, 100, 10)
+            other[f"decode_M{m}"] = {"GBps": round(decode_bytes(m) / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2),
+                                     "kernel_GBps": round((K_DEC * N_DEC + m * K_DEC + m * 4 + N_DEC * 4 + m * N_DEC * 2) / (tk * 1e-3) / 1e9, 1)}
+            del s, k, kp
+            torch.cuda.empty_cache()
+        # prefill (config 3): whole call (quantization + GEMM) and the GEMM kernel alone
+        for N in (4096, 14336):
+            Mp, K = 2048, 4096
+            blob = prepack(rand_w(K, N), K, N)
+            ws = torch.rand(N, device=dev, generator=g) * 0.009 + 0.001
+            bias = torch.randn(N, device=dev, generator=g) * 0.1
+            x = torch.randn((Mp, K), device=dev, generator=g).to(torch.bfloat16)
+            dst = torch.zeros((Mp, N), dtype=torch.bfloat16, device=dev)
+            p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32, compute=capi.DT_S8)
+            p.dynamic_quant = True
+            p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (Mp, 1))
+            p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+            p.postop_ = [lowoha.PostOp(capi.PO_GELU_TANH)]
+            p.mem_format_b = "r"
+            p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+            t = ev_time(lambda: lowoha.matmul_direct("r", False, False, Mp, N, K, 1.0, x, K, blob, N, bias, 0.0, dst, N, True, p), 30, 5)
+            xq = torch.randint(-127, 128, (Mp, K), dtype=torch.int8, device=dev, generator=g)
+            xs = torch.rand(Mp, device=dev, generator=g) * 0.02 + 0.01
+            pk = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32)
+            pk.src_scale = lowoha.QuantParam(xs, capi.DT_F32, (Mp, 1))
+            pk.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+            pk.postop_ = [lowoha.PostOp(capi.PO_GELU_TANH)]
+            pk.mem_format_b = "r"
+            pk.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+            tk = ev_time(lambda: lowoha.matmul_direct("r", False, False, Mp, N, K, 1.0, xq, K, blob, N, bias, 0.0, dst, N, True, pk), 30, 5)
+            ops = 2.0 * Mp * N * K
+            other[f"prefill_N{N}"] = {"TOPS_whole_call": round(ops / (t * 1e-3) / 1e12, 1),
+                                      "TOPS_gemm_kernel": round(ops / (tk * 1e-3) / 1e12, 1),
+                                      "pct_of_int8_mfma_peak": round(100 * ops / (tk * 1e-3) / 1e12 / INT8_PEAK_TOPS, 1),
+                                      "us_gemm_kernel": round(tk * 1e3, 1), "kernel": lowoha.last_kernel()}
+            del blob, x, dst, xq
+            torch.cuda.empty_cache()
+        # config 1
+        Mc, K, N = 128, 4096, 4096
+        blobs = [prepack(rand_w(K, N), K, N, capi.DT_U8) for _ in range(20)]
+        a = torch.randint(0, 256, (Mc, K), dtype=torch.uint8, device=dev, generator=g)
+        ws = torch.rand(N, device=dev, generator=g) * 0.009 + 0.001
+        bias = torch.randn(N, device=dev, generator=g)
+        dst = torch.zeros((Mc, N), dtype=torch.float32, device=dev)
+        ss = np.array([0.02], dtype=np.float32)
+        zp = np.array([128], dtype=np.int32)
+        p = lowoha.MatmulParams(src=capi.DT_U8, wei=capi.DT_S8, dst=capi.DT_F32, bias=capi.DT_F32)
+        p.src_scale = lowoha.QuantParam(ss.ctypes.data, capi.DT_F32, (1,))
+        p.src_zp = lowoha.QuantParam(zp.ctypes.data, capi.DT_S32, (1,))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        st = {"i": 0}
+
+        def c1():
+            b = blobs[st["i"] % len(blobs)]
+            st["i"] += 1
+            lowoha.matmul_direct("r", False, False, Mc, N, K, 1.0, a, K, b, N, bias, 0.0, dst, N, True, p)
+        t = ev_time(c1, 100, 10)
+        other["config1_u8s8_M128"] = {"us_per_call": round(t * 1e3, 2), "GBps": round(19431424 / (t * 1e-3) / 1e9, 1),
+                                      "TOPS": round(2.0 * Mc * N * K / (t * 1e-3) / 1e12, 1)}
+        del blobs
+        torch.cuda.empty_cache()
+        # MoE configs 4 and 5: tokens/s through the device-routed fused block
+        for name, T, Hd, I, E, topk, skew in (("moe_config4", 512, 4096, 14336, 8, 2, False),
+                                              ("moe_config5", 4096, 2048, 1408, 64, 6, True)):
+            w13 = [prepack(rand_w(Hd, 2 * I), Hd, 2 * I) for _ in range(E)]
+            w2 = [prepack(rand_w(I, Hd), I, Hd) for _ in range(E)]
+            s13 = [torch.rand(2 * I, device=dev, generator=g) * 0.009 + 0.001 for _ in range(E)]
+            s2 = [torch.rand(Hd, device=dev, generator=g) * 0.009 + 0.001 for _ in range(E)]
+            x = torch.randn((T, Hd), device=dev, generator=g).to(torch.bfloat16)
+            logits = torch.randn((T, E), device=dev, generator=g)
+            if skew:
+                logits = logits + torch.randn(E, device=dev, generator=g) * 1.5
+            prob = torch.softmax(logits, dim=1)
+            tw, ids = torch.topk(prob, topk, dim=1)
+            ids = ids.to(torch.int32).contiguous()
+            tw = tw.contiguous()
+            out = torch.zeros((T, Hd), dtype=torch.bfloat16, device=dev)
+
+            def moe():
+                r = lowoha.moe_fused_device(x, ids, tw, w13, w2, s13, s2, I, capi.ACT_SILU_AND_MUL, out)
+                if r != capi.SUCCESS:
+                    raise RuntimeError(lowoha.last_error())
+            t = ev_time(moe, 10, 3)
+            cnt = torch.bincount(ids.flatten().long(), minlength=E)
+            ops = 2.0 * T * topk * 3 * Hd * I
+            other[name] = {"tokens_per_s": round(T / (t * 1e-3), 0), "ms_per_call": round(t, 4),
+                           "TOPS": round(ops / (t * 1e-3) / 1e12, 1),
+                           "weight_GBps": round(E * 3 * Hd * I / (t * 1e-3) / 1e9, 1),
+                           "expert_rows_min_max": [int(cnt.min()), int(cnt.max())]}
+            del w13, w2, x, out
+            torch.cuda.empty_cache()
+        result["other_configs"] = other
+
+        # ------------------------------------------------------ CPU baseline (oracle port)
+        from oracle import build as obuild, oracle as zo
+        obuild.build(force=False)
+        rng = np.random.default_rng(1)
+        Mb = 16
+        A = rng.integers(-127, 128, (Mb, K_DEC), dtype=np.int8)
+        Bt = rng.integers(-127, 128, (N_DEC, K_DEC), dtype=np.int8)   # pre-transposed: the packed form of the CPU path
+        sa = rng.uniform(0.01, 0.03, Mb).astype(np.float32)
+        sb = rng.uniform(0.001, 0.01, N_DEC).astype(np.float32)
+        out = np.zeros((Mb, N_DEC), dtype=np.uint16)
+        L = zo.lib()
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+
+        def cpu_call():
+            L.zo_bench_s8_gemm(A.ctypes.data, Bt.ctypes.data, sa.ctypes.data, sb.ctypes.data, Mb, N_DEC, K_DEC,
+                               capi.PO_SWISH, out.ctypes.data)
+        cpu_call()
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < 10.0:
+            cpu_call()
+            n += 1
+        dt = (time.perf_counter() - t0) / n
+        cb = K_DEC * N_DEC + Mb * K_DEC + Mb * 4 + N_DEC * 4 + Mb * N_DEC * 2
+        result["cpu_baseline"] = {"value": round(cb / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                                  "sample": f"{n} calls of the same M=16 K=4096 N=14336 s8 x s8 GEMM + scales + SiLU + bf16 "
+                                            f"store through the oracle's OpenMP port (about 10 s); not AOCL-DLP",
+                                  "ms_per_call": round(dt * 1e3, 3)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
