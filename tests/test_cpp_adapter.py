@@ -1,0 +1,26 @@
+"""The C++ front end (reference signatures over the C ABI), driven by a small
+C++ program: validation outcomes on the CPU, the reference example's
+deterministic int8 recipe on the GPU."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "zendnn_amd", "lib", "adapter_example")
+
+
+def _run(args):
+    assert os.path.exists(EXE), "run __graft_entry__.build() first"
+    r = subprocess.run([EXE] + args, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "adapter example: ok" in r.stdout
+
+
+def test_cpp_adapter_validation_paths():
+    _run(["--validate-only"])
+
+
+@pytest.mark.gpu
+def test_cpp_adapter_reference_example_recipe():
+    _run([])

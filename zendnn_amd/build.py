@@ -50,8 +50,9 @@ def build(verbose=False, force=True):
         if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(path), hdr):
             continue
         jobs.append(["hipcc"] + HIPCC_FLAGS + ["-c", path, "-o", obj])
-    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
-        list(ex.map(_run, jobs))
+    if jobs:
+        with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
+            list(ex.map(_run, jobs))
     lib = os.path.join(LIBDIR, "libzmi_lowoha.so")
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs)
     # C++ adapter: plain g++, sees only the C ABI header
@@ -60,6 +61,12 @@ def build(verbose=False, force=True):
     if os.path.exists(host_src):
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(HERE, "..", "include"),
               "-I", HOST, host_src, "-o", host_lib, "-L", LIBDIR, "-lzmi_lowoha", "-Wl,-rpath,$ORIGIN"])
+        # C++ usage example / adapter test (host code only; hipcc for the HIP runtime headers)
+        ex_src = os.path.join(HERE, "..", "tests", "cpp", "adapter_example.cpp")
+        if os.path.exists(ex_src):
+            _run(["hipcc", "-O1", "-std=c++17", "-w", "-I", HOST, "-I", os.path.join(HERE, "..", "include"), ex_src,
+                  "-o", os.path.join(LIBDIR, "adapter_example"), "-L", LIBDIR, "-lzendnnl_mi355x", "-lzmi_lowoha",
+                  "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", lib)
     return lib
