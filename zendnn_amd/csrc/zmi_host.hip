@@ -27,6 +27,8 @@ struct ThreadCtx {
   bool ev_live[kSlots] = {};   // an event is recorded and the slot is busy until it fires
   bool used[kSlots] = {};      // written during the current call, not fenced yet
   int next = 0;
+  unsigned int *fq_counter = nullptr;
+  unsigned int fq_total = 0;
 };
 thread_local ThreadCtx tctx;
 
@@ -182,6 +184,23 @@ void upload_fence() {
       c.used[i] = false;
     }
   }
+}
+
+unsigned int *fused_counter() {
+  ThreadCtx &c = tctx;
+  if (!c.fq_counter) {
+    void *p = nullptr;
+    if (!hip_ok(hipMalloc(&p, 256), "hipMalloc(counter)")) return nullptr;
+    if (!hip_ok(hipMemset(p, 0, 256), "hipMemset(counter)")) return nullptr;
+    c.fq_counter = (unsigned int *)p;
+    c.fq_total = 0;
+  }
+  return c.fq_counter;
+}
+
+unsigned int fused_next_target(int rows) {
+  tctx.fq_total += (unsigned int)rows;
+  return tctx.fq_total;
 }
 
 // ---- one-element parameters ------------------------------------------------------

@@ -38,6 +38,22 @@ hipError_t zmi_launch_gemm_mfma_group(const ZmiProblem *probs_host, const ZmiPro
                                       hipStream_t stream);
 
 // k_smallm.hip
+struct ZmiFusedQuant {
+  const void *x;          // bf16 / f32 rows, null: no fused quantization
+  int64_t ldx;
+  int32_t x_dt;
+  int8_t *q;              // s8 rows out (== ZmiProblem::A)
+  int64_t ldq;
+  float *scales;          // f32 scale per row out (== ZmiProblem::src_scale_ptr)
+  void *user_scales;      // optional copy in user_dt
+  int32_t user_dt;
+  unsigned int *counter;  // device counter, monotonically increasing across launches
+  unsigned int target;    // value the counter reaches when all M rows of this launch are published
+};
+
+int zmi_smallm_grid(const ZmiProblem &p, bool gated);
+hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
+                                        hipStream_t stream);
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
 hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev,
                                         int n_prob, int m_lo, int m_hi, int worst_grid, int64_t kpad_hint,

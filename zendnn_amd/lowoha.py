@@ -123,6 +123,31 @@ def matmul_direct(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb,
                                  C.byref(b), C.byref(p))
 
 
+def prepared_matmul(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc,
+                    is_weights_const, params):
+    """Flattens the arguments once and returns (call, rebind): call() issues the same
+    matmul_direct with no per-call Python work beyond the foreign call; rebind(weight=...)
+    swaps the weight pointer.  For timing loops and serving loops."""
+    lib = capi.load()
+    keep = []
+    p = params.flat(keep)
+    b = capi.BatchParamsT()
+    lib.zmi_batch_params_init(C.byref(b))
+    state = {"w": C.c_void_p(_ptr(weight)), "keep": (keep, params, src, bias, dst, weight)}
+    fixed_a = (layout.encode(), int(transA), int(transB), M, N, K, alpha, C.c_void_p(_ptr(src)), lda)
+    fixed_b = (ldb, C.c_void_p(_ptr(bias)), beta, C.c_void_p(_ptr(dst)), ldc, int(is_weights_const),
+               C.byref(b), C.byref(p))
+    fn = lib.zmi_matmul_direct
+
+    def call():
+        return fn(*fixed_a, state["w"], *fixed_b)
+
+    def rebind(weight):
+        state["w"] = C.c_void_p(_ptr(weight))
+
+    return call, rebind
+
+
 class ReorderParams:
     """reorder_params_t (prepack and dynamic per-token fields)."""
 
