@@ -157,9 +157,9 @@ def main():
     gemm_kernel = lowoha.last_kernel()
     # algorithmic bytes of the GEMM-only launch: s8 rows instead of bf16 rows, plus the row scales
     kbytes = K_DEC * N_DEC + M * K_DEC + M * 4 + N_DEC * 4 + M * N_DEC * 2
-    # One step is one launch of zmi_gemm_smallm_kernel<1,8> (quantization fused in), so the step
-    # time between the two events is that kernel's average launch duration.
-    achieved = value
+    # One step is the per-token quantization launch plus the GEMM launch; the GEMM kernel
+    # dominates, and the second timed loop runs that kernel alone, back to back.
+    achieved = kbytes / (ms_k * 1e-3) / 1e9
 
     result = {
         "metric": "decode_int8_gemm_weight_streaming",
@@ -177,17 +177,16 @@ def main():
         "config": {"workload": "matmul_direct decode: M=16 K=4096 N=14336, bf16 -> per-token s8, "
                                "prepacked s8 weights, per-channel scales, SiLU, bf16 out",
                    "weight_sets_rotated": n_sets, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1)},
-        "roofline": {"bound": "hbm", "kernel": "zmi_gemm_smallm_kernel<1,8>: " + step_kernel,
+        "roofline": {"bound": "hbm", "kernel": "zmi_gemm_decode_kernel: " + gemm_kernel,
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "algorithmic_bytes_per_launch": decode_bytes(M),
-                     "avg_launch_us": round(ms * 1e3, 2),
-                     "gemm_only": {"kernel": gemm_kernel, "avg_launch_us": round(ms_k * 1e3, 2),
-                                   "algorithmic_bytes_per_launch": kbytes,
-                                   "GBps": round(kbytes / (ms_k * 1e-3) / 1e9, 1),
-                                   "what": "the same launch on rows that are already s8 (no fused quantization)"},
-                     "note": "launches timed back to back between two events on the kernel's stream, "
-                             "so the figure includes the dispatch gap between launches"},
+                     "algorithmic_bytes_per_launch": kbytes,
+                     "avg_launch_us": round(ms_k * 1e3, 2),
+                     "whole_call": {"kernels": "zmi_quant_rows_kernel + " + step_kernel, "us": round(ms * 1e3, 2),
+                                    "algorithmic_bytes": decode_bytes(M)},
+                     "note": "the GEMM kernel launched back to back on s8 rows, timed between two events on "
+                             "its stream (includes the dispatch gap); value above is the whole call "
+                             "(quantization launch + this kernel)"},
     }
 
     if not args.no_extras:

@@ -89,7 +89,7 @@ def test_decode_dynamic_quant_bf16_silu(zo, M, K, N):
     dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
     st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, blob, N, None, 0.0, dst, N, True, p)
     assert st == capi.SUCCESS, lowoha.last_error()
-    assert "smallm" in lowoha.last_kernel()
+    assert "decode" in lowoha.last_kernel() or "smallm" in lowoha.last_kernel()
     ph = H.host_params(p, src_scale=None, wei_scale=ws)
     ph.mem_format_b = "n"
     want, _, scales = _oracle(zo, ph, x, w, M, N, K, want_scales=True)

@@ -1,0 +1,216 @@
+// Decode int8 GEMM for gfx950: C[M<=16, N] = epilogue(A[M,K] x blob), K_pad <= 4096.
+//
+// Same call sites as k_smallm.hip (the aocl_gemm_s8s8s32o*_sym_quant call,
+// zendnnl/src/lowoha_operators/matmul/backends/aocl/aocl_kernel.cpp:1239-1257, and the
+// in-house decode microkernel, matmul/group_matmul/custom_kernel/ukernel/
+// int8_microkernel.cpp:196-606), specialised for the one-to-sixteen-token case, where
+// the weights are streamed once from HBM and everything else has to stay out of
+// the way of that stream:
+//   * one workgroup (8 wavefronts) per 32 weight columns; wavefront w streams the
+//     w-th eighth of K with 16-byte-per-lane loads, all issued up front;
+//   * the activation rows are read from L2 with row-contiguous loads (consecutive
+//     lanes, consecutive bytes) BEFORE the weight loads, so they return first,
+//     and are laid out in LDS in MFMA operand order (bank-swizzled); the MFMA A
+//     operands then come from LDS.  Loading the operands straight from global
+//     memory instead touches 16 different rows per load and costs ~2 us of the
+//     ~13 us launch;
+//   * the per-column / per-row epilogue constants are fetched before anything
+//     else, so the tail after the last weight byte is LDS-only.
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+#define DEC_WAVES 8
+#define DEC_THREADS (DEC_WAVES * 64)
+#define DEC_RED_BYTES (DEC_WAVES * 2 * 4 * 64 * 4)   // 16 KiB of partial tiles
+
+// Byte offset in LDS of the 16-byte operand granule of chunk cc (64 k), k group g
+// (16 k), row r.  Chunk-major so that one ds_read_b128 per lane fetches a whole
+// 16x64 operand; the row index is XOR-swizzled with (g, cc) so that the
+// row-contiguous writes (one row, 16 consecutive granules per 16 lanes) spread
+// over all banks as well.
+__device__ __forceinline__ int dec_lds_off(int cc, int g, int r) {
+  return cc * 1024 + ((g * 16 + (r ^ ((g * 4 + (cc & 3)) & 15))) << 4);
+}
+
+__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProblem p, ZmiEpilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);   // scalar: slice bounds and addresses stay in SGPRs
+  const int M = p.M, N = p.N, K = p.K;
+  const int K_pad = (int)zmi_blob_kpad(K);
+  const int nchunks = K_pad / 64;
+  const bool gated = epi.gated_act != 0;
+  const int blk = blockIdx.x;
+  const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+
+  // the two 16-column groups h = 0, 1: weight column wcol[h], output column ocol[h]
+  // (gated: h = 0 gate, h = 1 up, one output column)
+  int wcol[2], ocol[2];
+  if (!gated) {
+    wcol[0] = blk * 32; wcol[1] = blk * 32 + 16;
+    ocol[0] = wcol[0]; ocol[1] = wcol[1];
+  } else {
+    wcol[0] = blk * 16; wcol[1] = blk * 16 + N / 2;
+    ocol[0] = blk * 16; ocol[1] = blk * 16;
+  }
+
+  // ---- epilogue constants of this thread's output element, fetched first ----
+  // plain: element (row tid/32, column tid%32); gated: threads < 256, (row tid/16, column tid%16)
+  const int e_row = gated ? tid / 16 : tid / 32;
+  const int e_h = gated ? 0 : (tid % 32) / 16;
+  const int e_c = tid % 16;
+  const int e_n = ocol[e_h] + e_c;
+  const bool e_live = e_row < M && e_row < 16 && (gated ? e_n < N / 2 : e_n < N);
+  ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_live ? e_n : N, N);
+  ZmiColCtx cc1 = cc0;
+  if (gated) cc1 = zmi_col_ctx(epi, p, colsum, e_live ? e_n + N / 2 : N, N);
+  const float rs = zmi_row_scale(epi, p, e_live ? e_row : 0);
+
+  // ---- activation loads (row-contiguous), before the weight stream ----
+  // 64 items (row, 1 KiB segment); wavefront w takes rows w and w + 8.
+  const int c16 = lane % 16, g = lane / 16;
+  v4i araw[2][4];
+  {
+    const int8_t *A = (const int8_t *)p.A;
+    const int G = ((K + 15) & ~15) / 16;   // readable 16-byte granules per row
+    #pragma unroll
+    for (int i = 0; i < 2; ++i)
+      #pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int row = wave + 8 * i, gran = s * 64 + lane;
+        v4i v = {0, 0, 0, 0};
+        if (row < M && gran < G) v = *(const v4i *)(A + (int64_t)row * p.lda + gran * 16);
+        araw[i][s] = v;
+      }
+  }
+
+  // ---- weight stream: this wavefront's slice of K, at most 8 chunks of 64 ----
+  const int c_begin = wave * nchunks / DEC_WAVES;
+  const int c_end = (wave + 1) * nchunks / DEC_WAVES;
+  const uint8_t *bsrc[2];
+  #pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t nb = wcol[h] / 32;
+    const int coff = wcol[h] % 32;
+    bsrc[h] = tiles + nb * zmi_blob_nb_stride(K) + (g / 2) * 1024 + ((g % 2) * 32 + coff + c16) * 16;
+  }
+  v4i b[8][2];
+  auto load_b = [&](int u) {
+    // past the end of the slice: re-read the slice's first chunk (valid memory), result unused
+    const int c = c_begin + u < c_end ? c_begin + u : c_begin;
+    b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)c * 2048);
+    b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)c * 2048);
+  };
+  #pragma unroll
+  for (int u = 0; u < 8; ++u) load_b(u);
+
+  // ---- rows -> LDS in operand order ----
+  {
+    const uint32_t xm = p.a_is_u8 ? 0x80808080u : 0u;
+    #pragma unroll
+    for (int i = 0; i < 2; ++i)
+      #pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int row = wave + 8 * i, gran = s * 64 + lane;
+        v4i v = araw[i][s];
+        v[0] ^= xm; v[1] ^= xm; v[2] ^= xm; v[3] ^= xm;
+        if (row >= M) v = (v4i){0, 0, 0, 0};
+        // granule s*64 + lane: chunk s*16 + lane/4, k group lane%4 (the swizzle does not depend on s)
+        if (gran * 16 < K_pad) *(v4i *)(lds + dec_lds_off(lane / 4, lane % 4, row) + s * 16384) = v;
+      }
+  }
+  __syncthreads();
+
+  // ---- MFMA: one 16x16x64 per chunk and column group ----
+  v4i acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  #pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const bool live = c_begin + u < c_end;
+    const int c = live ? c_begin + u : c_begin;
+    v4i a = *(const v4i *)(lds + dec_lds_off(c, g, c16));
+    if (!live) a = (v4i){0, 0, 0, 0};   // whatever b holds then adds nothing
+    acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[1], 0, 0, 0);
+  }
+
+  // ---- cross-wavefront reduction through LDS (reuses the operand area) ----
+  __syncthreads();
+  int32_t *red = (int32_t *)lds;
+  #pragma unroll
+  for (int h = 0; h < 2; ++h)
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) red[wave * 512 + (h * 4 + j) * 64 + lane] = acc[h][j];
+  __syncthreads();
+  if (!e_live) return;
+
+  // acc[h][j] of lane l is row (l/16)*4 + j, column h*16 + l%16
+  auto fetch = [&](int h) -> int32_t {
+    const int off = (h * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_c;
+    int32_t s = 0;
+    #pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) s += red[w * 512 + off];
+    return s;
+  };
+
+  if (!gated) {
+    const int32_t s = fetch(e_h);
+    const void *bias = p.bias;
+    const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+    const bool has_bias = bias != nullptr;
+    const int64_t o = (int64_t)e_row * p.ldc + e_n;
+    const bool bf = epi.dst_dt == ZMI_DT_BF16;
+    switch (epi.fast_kind) {
+    case ZMI_EK_NONE: {
+      const float y = zmi_fast_value<ZMI_EK_NONE>(s, cc0, rs, has_rs, has_ws, has_bias);
+      if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+      break;
+    }
+    case ZMI_EK_SWISH: {
+      const float y = zmi_fast_value<ZMI_EK_SWISH>(s, cc0, rs, has_rs, has_ws, has_bias);
+      if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+      break;
+    }
+    case ZMI_EK_GELU_TANH: {
+      const float y = zmi_fast_value<ZMI_EK_GELU_TANH>(s, cc0, rs, has_rs, has_ws, has_bias);
+      if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+      break;
+    }
+    default:
+      if (zmi_epilogue_is_raw_s32(epi, bias)) ((int32_t *)p.dst)[o] = s + cc0.comp;
+      else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, cc0, rs, e_row, e_n, p.dst, p.ldc));
+    }
+  } else {
+    const int half = N / 2;
+    const int32_t sg = fetch(0), su = fetch(1);
+    float gv = zmi_epilogue_value(epi, sg, cc0, rs, e_row, e_n, p.dst, p.ldc);
+    float uv = zmi_epilogue_value(epi, su, cc1, rs, e_row, e_n + half, p.dst, p.ldc);
+    if (epi.dst_dt == ZMI_DT_BF16) {
+      gv = zmi_bf16_to_f32(zmi_f32_to_bf16(gv));
+      uv = zmi_bf16_to_f32(zmi_f32_to_bf16(uv));
+    }
+    zmi_store(p.dst, epi.dst_dt, (int64_t)e_row * p.ldc + e_n, zmi_gated(epi.gated_act, gv, uv));
+  }
+}
+
+bool zmi_decode_kernel_fits(const ZmiProblem &p) {
+  return p.M > 0 && p.M <= 16 && zmi_blob_kpad(p.K) <= 4096;
+}
+
+hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
+  if (!zmi_decode_kernel_fits(p)) return hipErrorInvalidValue;
+  const bool gated = epi.gated_act != 0;
+  const int grid = gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
+  if (grid <= 0) return hipSuccess;
+  const size_t a_bytes = (size_t)zmi_blob_kpad(p.K) * 16;
+  const size_t smem = a_bytes > DEC_RED_BYTES ? a_bytes : (size_t)DEC_RED_BYTES;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_decode_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * 16);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(zmi_gemm_decode_kernel, dim3(grid), dim3(DEC_THREADS), smem, stream, p, epi);
+  return hipGetLastError();
+}

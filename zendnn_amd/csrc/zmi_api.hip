@@ -239,7 +239,10 @@ static int pick_bm(int M, int N) {
 }
 
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi) {
-  if (prob.M <= 128) {
+  if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
+    set_kernel_name("decode_lds_rows_mfma16x16x64");
+    if (!hip_ok(zmi_launch_gemm_decode(prob, epi, stream()), "decode GEMM launch")) return ZMI_FAILURE;
+  } else if (prob.M <= 128) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
   } else {
@@ -370,7 +373,9 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     prob.A = q; prob.lda = K16;
     const bool per_token = (dyn_scale_n == M && M > 1) || M == 1;
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
-    if (per_token && M <= 128 && K % 4 == 0 && zmi_smallm_grid(prob, false) <= 512 && !std::getenv("ZMI_NO_FUSED_QUANT")) {
+    const bool decode_kernel = M <= 16 && zmi_blob_kpad(K) <= 4096 && !std::getenv("ZMI_NO_DECODE_KERNEL");
+    if (per_token && !decode_kernel && M <= 128 && K % 4 == 0 && zmi_smallm_grid(prob, false) <= 512 &&
+        !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
       if (!ctr) return ZMI_FAILURE;
       fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;

@@ -59,6 +59,10 @@ hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiP
                                         int n_prob, int m_lo, int m_hi, int worst_grid, int64_t kpad_hint,
                                         const ZmiEpilogue &epi, hipStream_t stream);
 
+// k_decode.hip: single problem, M <= 16, K_pad <= 4096
+bool zmi_decode_kernel_fits(const ZmiProblem &p);
+hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+
 // k_moe.hip
 struct ZmiActMat {
   void *buf;
