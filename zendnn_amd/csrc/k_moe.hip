@@ -80,14 +80,40 @@ __global__ __launch_bounds__(256) void zmi_moe_combine_kernel(const void *const 
                                                               int D, int dt, void *out, int64_t ldo) {
   const int t = blockIdx.x;
   const size_t es = dt == ZMI_DT_BF16 ? 2 : 4;
+  auto row_of = [&](int k) -> const void * {
+    const int s = t * topk + k;
+    return row_ptrs ? row_ptrs[s] : (const void *)((const char *)rows_base + (int64_t)slot_of[s] * row_ld * es);
+  };
+  // bf16 rows, 8 columns (16 bytes) per thread and step, when everything is 16-byte aligned
+  bool vec = dt == ZMI_DT_BF16 && D % 8 == 0 && ldo % 8 == 0 && ((uintptr_t)out) % 16 == 0;
+  for (int k = 0; k < topk && vec; ++k) vec = ((uintptr_t)row_of(k)) % 16 == 0;
+  if (vec) {
+    for (int d = threadIdx.x * 8; d < D; d += blockDim.x * 8) {
+      float acc[8];
+      for (int k = 0; k < topk; ++k) {
+        const v4i raw = *(const v4i *)((const uint16_t *)row_of(k) + d);
+        const float w = skip_weighted ? 1.0f : weights[t * topk + k];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float x0 = __uint_as_float(((uint32_t)raw[j]) << 16);
+          const float x1 = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+          acc[2 * j] = (k == 0) ? __fmul_rn(w, x0) : __builtin_fmaf(w, x0, acc[2 * j]);
+          acc[2 * j + 1] = (k == 0) ? __fmul_rn(w, x1) : __builtin_fmaf(w, x1, acc[2 * j + 1]);
+        }
+      }
+      v4i o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        o[j] = (int)((uint32_t)zmi_f32_to_bf16_rne(acc[2 * j]) | ((uint32_t)zmi_f32_to_bf16_rne(acc[2 * j + 1]) << 16));
+      *(v4i *)((uint16_t *)out + (int64_t)t * ldo + d) = o;
+    }
+    return;
+  }
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float acc = 0.0f;
     for (int k = 0; k < topk; ++k) {
-      const int s = t * topk + k;
-      const void *row = row_ptrs ? row_ptrs[s]
-                                 : (const void *)((const char *)rows_base + (int64_t)slot_of[s] * row_ld * es);
-      const float w = skip_weighted ? 1.0f : weights[s];
-      const float x = zmi_ld_f32(row, dt, d);
+      const float w = skip_weighted ? 1.0f : weights[t * topk + k];
+      const float x = zmi_ld_f32(row_of(k), dt, d);
       acc = (k == 0) ? __fmul_rn(w, x) : __builtin_fmaf(w, x, acc);
     }
     if (dt == ZMI_DT_BF16) ((uint16_t *)out)[(int64_t)t * ldo + d] = zmi_f32_to_bf16_rne(acc);
@@ -117,8 +143,8 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
 #define RT_WAVES 16
 
 __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int32_t *topk_ids, int n, int E,
-                                                                      int32_t *counts, int32_t *offsets,
-                                                                      int32_t *slot_of) {
+                                                                      int align, int32_t *counts,
+                                                                      int32_t *offsets, int32_t *slot_of) {
   extern __shared__ int32_t sh[];   // hist[RT_WAVES][E], then off[E+1]
   int32_t *hist = sh;
   int32_t *off = sh + RT_WAVES * E;
@@ -146,7 +172,7 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
   __syncthreads();
   if (tid == 0) {
     int run = 0;
-    for (int e = 0; e < E; ++e) { const int c = off[e]; off[e] = run; offsets[e] = run; run += c; }
+    for (int e = 0; e < E; ++e) { const int c = off[e]; off[e] = run; offsets[e] = run; run += (c + align - 1) / align * align; }
     off[E] = run;
     offsets[E] = run;
   }
@@ -177,7 +203,7 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
   }
 }
 
-hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int32_t *counts,
+hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
                                 int32_t *offsets, int32_t *slot_of, hipStream_t stream) {
   if (E > 2047 || E <= 0) return hipErrorInvalidValue;
   const size_t smem = ((size_t)RT_WAVES * E + E + 1) * sizeof(int32_t);
@@ -189,23 +215,45 @@ hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E,
     attr = smem;
   }
   hipLaunchKernelGGL(zmi_moe_route_kernel, dim3(1), dim3(RT_WAVES * 64), smem, stream, topk_ids, T * topk, E,
-                     counts, offsets, slot_of);
+                     align < 1 ? 1 : align, counts, offsets, slot_of);
   return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
 // Quantize token t once (per-token symmetric s8, same arithmetic as
-// k_quant.hip) and write the row and its scale to each of its topk slots.
+// k_quant.hip) and write the row (fragment-major over the slot numbering) and
+// its scale to each of its topk slots.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void zmi_moe_quant_scatter_kernel(const uint16_t *x, int64_t ldx, int H, int topk,
                                                                     const int32_t *slot_of, int8_t *A1, float *s1) {
+  const int64_t k_pad = zmi_blob_kpad(H);
   __shared__ float red[4];
   const int t = blockIdx.x;
   const uint16_t *row = x + (int64_t)t * ldx;
+  // 8 consecutive elements per thread and step (H is a multiple of 16); 16-byte loads when the row allows
+  const bool vec = ((uintptr_t)row) % 16 == 0;
+  auto load8 = [&](int k, float (&v)[8]) {
+    if (vec) {
+      const v4i raw = *(const v4i *)(row + k);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float(((uint32_t)raw[j]) << 16);
+        v[2 * j + 1] = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = zmi_bf16_to_f32(row[k + j]);
+    }
+  };
   float amax = 0.0f;
-  for (int k = threadIdx.x; k < H; k += blockDim.x) {
-    const float a = fabsf(zmi_bf16_to_f32(row[k]));
-    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+  for (int k = threadIdx.x * 8; k < H; k += blockDim.x * 8) {
+    float v[8];
+    load8(k, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = fabsf(v[j]);
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
   }
   #pragma unroll
   for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
@@ -215,13 +263,19 @@ __global__ __launch_bounds__(256) void zmi_moe_quant_scatter_kernel(const uint16
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
-  for (int k = threadIdx.x; k < H; k += blockDim.x) {
-    const float v = zmi_bf16_to_f32(row[k]);
-    int8_t q = 0;
-    if ((__float_as_uint(v) & 0x7f800000u) != 0x7f800000u) q = (int8_t)(int32_t)rintf(__fdiv_rn(v, s));
+  for (int k = threadIdx.x * 8; k < H; k += blockDim.x * 8) {
+    float v[8];
+    load8(k, v);
+    __attribute__((aligned(8))) int8_t q[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      q[j] = 0;
+      if ((__float_as_uint(v[j]) & 0x7f800000u) != 0x7f800000u) q[j] = (int8_t)(int32_t)rintf(__fdiv_rn(v[j], s));
+    }
     for (int j = 0; j < topk; ++j) {
       const int slot = slot_of[t * topk + j];
-      if (slot >= 0) A1[(int64_t)slot * H + k] = q;
+      // 8 consecutive k starting at a multiple of 8 are contiguous in fragment order
+      if (slot >= 0) *(uint2 *)(A1 + zmi_afrag_off(slot, k, k_pad)) = *(const uint2 *)q;
     }
   }
   if (threadIdx.x < topk) {
@@ -248,14 +302,14 @@ __global__ void zmi_moe_build_problems_kernel(ZmiMoeTables tb, int E, int H, int
                                               ZmiProblem *op1, ZmiProblem *op2) {
   const int e = blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= E) return;
-  const int64_t o = offsets[e];
+  const int64_t o = offsets[e];   // a multiple of 32: every expert starts on a fragment row
   ZmiProblem a = {};
-  a.A = A1 + o * H; a.lda = H; a.blob = (const uint8_t *)tb.w13_blob[e];
+  a.A = A1 + o * zmi_blob_kpad(H); a.lda = H; a.blob = (const uint8_t *)tb.w13_blob[e];
   a.dst = act + o * I; a.ldc = I; a.M = counts[e]; a.N = 2 * I; a.K = H; a.a_is_u8 = 0;
   a.src_scale_ptr = s1 + o; a.wei_scale_ptr = tb.w13_scale[e];
   op1[e] = a;
   ZmiProblem b = {};
-  b.A = A2 + o * I; b.lda = I; b.blob = (const uint8_t *)tb.w2_blob[e];
+  b.A = A2 + o * zmi_blob_kpad(I); b.lda = I; b.blob = (const uint8_t *)tb.w2_blob[e];
   b.dst = Y + o * H; b.ldc = H; b.M = counts[e]; b.N = H; b.K = I; b.a_is_u8 = 0;
   b.src_scale_ptr = s2 + o; b.wei_scale_ptr = tb.w2_scale[e];
   op2[e] = b;

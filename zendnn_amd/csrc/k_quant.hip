@@ -32,10 +32,14 @@ __device__ __forceinline__ int8_t zmi_quant_one(float v, float scale) {
   return (int8_t)(int32_t)rintf(__fdiv_rn(v, scale));
 }
 
+// dst + dst_off(k) is where element k of this row goes: k itself for K-contiguous
+// rows, the fragment-major position otherwise (8 consecutive k starting at a
+// multiple of 8 stay contiguous in both).
 template <bool BF16>
-__device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, void *scale, int scale_dt,
-                                              int K, float *red) {
+__device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, int r_frag, int64_t frag_kpad,
+                                              void *scale, int scale_dt, int K, float *red) {
   const int t = threadIdx.x;
+  auto dst_off = [&](int k) -> int64_t { return frag_kpad ? zmi_afrag_off(r_frag, k, frag_kpad) : (int64_t)k; };
   const bool vec_ok = (K % 8 == 0) && (((uintptr_t)srcv) % 16 == 0) &&
                       (dst == nullptr || ((uintptr_t)dst) % 8 == 0);
   if (vec_ok && K <= QT_THREADS * 8 * QT_MAX_CHUNKS) {
@@ -82,7 +86,7 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, voi
         __attribute__((aligned(8))) int8_t q[8];
         #pragma unroll
         for (int j = 0; j < 8; ++j) q[j] = zmi_quant_one(v[c][j], s);
-        *(uint2 *)(dst + k) = *(const uint2 *)q;
+        *(uint2 *)(dst + dst_off(k)) = *(const uint2 *)q;
       }
     }
     return;
@@ -105,7 +109,7 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, voi
   if (!dst) return;
   for (int k = t; k < K; k += QT_THREADS) {
     float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)srcv)[k]) : ((const float *)srcv)[k];
-    dst[k] = zmi_quant_one(x, s);
+    dst[dst_off(k)] = zmi_quant_one(x, s);
   }
 }
 
@@ -131,18 +135,18 @@ __global__ __launch_bounds__(QT_THREADS) void zmi_quant_rows_kernel(ZmiQuantMat 
   if (r >= m.M) return;
   const size_t es = BF16 ? 2 : 4;
   const void *src = (const char *)m.src + (size_t)r * m.ld_src * es;
-  int8_t *dst = m.dst ? m.dst + (size_t)r * m.ld_dst : nullptr;
+  int8_t *dst = m.dst ? (m.frag_kpad ? m.dst : m.dst + (size_t)r * m.ld_dst) : nullptr;
   void *sc = (char *)m.scale + (size_t)r * (scale_dt == ZMI_DT_BF16 ? 2 : 4);
-  zmi_quant_row<BF16>(src, dst, sc, scale_dt, m.K, red);
+  zmi_quant_row<BF16>(src, dst, r, m.frag_kpad, sc, scale_dt, m.K, red);
 }
 
 hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
-                                 int8_t *dst, int64_t ld_dst, void *scales, int32_t scale_dt,
+                                 int8_t *dst, int64_t ld_dst, int64_t frag_kpad, void *scales, int32_t scale_dt,
                                  hipStream_t stream) {
   if (M <= 0) return hipSuccess;
   ZmiQuantMat m;
   m.src = src; m.dst = dst; m.scale = scales; m.ld_src = ld_src; m.ld_dst = ld_dst;
-  m.M = (int32_t)M; m.K = (int32_t)K; m.row_start = 0;
+  m.M = (int32_t)M; m.K = (int32_t)K; m.row_start = 0; m.frag_kpad = (int32_t)frag_kpad;
   if (src_dt == ZMI_DT_BF16)
     hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, m,
                        (const ZmiQuantMat *)nullptr, 1, scale_dt);
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(QT_THREADS) void zmi_absmax_kernel(const void *src,
 template <bool BF16>
 __global__ __launch_bounds__(QT_THREADS) void zmi_quant_tensor_kernel(const void *src, int64_t M, int64_t K,
                                                                       int64_t ld, int8_t *dst, int64_t ld_dst,
-                                                                      float *scales,
+                                                                      int64_t frag_kpad, float *scales,
                                                                       const unsigned int *amax_bits) {
   const int64_t row = blockIdx.x;
   float amax = __uint_as_float(*amax_bits);
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(QT_THREADS) void zmi_quant_tensor_kernel(const void
   if (!dst) return;
   for (int64_t k = threadIdx.x; k < K; k += QT_THREADS) {
     float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)src)[row * ld + k]) : ((const float *)src)[row * ld + k];
-    dst[row * ld_dst + k] = zmi_quant_one(x, s);
+    dst[frag_kpad ? zmi_afrag_off(row, k, frag_kpad) : row * ld_dst + k] = zmi_quant_one(x, s);
   }
 }
 
@@ -211,20 +215,20 @@ __global__ void zmi_zero_u32_kernel(unsigned int *p, int n) {
 }
 
 hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
-                                   int8_t *dst, int64_t ld_dst, float *scales, unsigned int *amax_scratch,
-                                   hipStream_t stream) {
+                                   int8_t *dst, int64_t ld_dst, int64_t frag_kpad, float *scales,
+                                   unsigned int *amax_scratch, hipStream_t stream) {
   if (M <= 0) return hipSuccess;
   hipLaunchKernelGGL(zmi_zero_u32_kernel, dim3(1), dim3(64), 0, stream, amax_scratch, 1);
   if (src_dt == ZMI_DT_BF16) {
     hipLaunchKernelGGL(zmi_absmax_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src, M, K,
                        ld_src, amax_scratch);
     hipLaunchKernelGGL(zmi_quant_tensor_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src,
-                       M, K, ld_src, dst, ld_dst, scales, amax_scratch);
+                       M, K, ld_src, dst, ld_dst, frag_kpad, scales, amax_scratch);
   } else {
     hipLaunchKernelGGL(zmi_absmax_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src, M, K,
                        ld_src, amax_scratch);
     hipLaunchKernelGGL(zmi_quant_tensor_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src,
-                       M, K, ld_src, dst, ld_dst, scales, amax_scratch);
+                       M, K, ld_src, dst, ld_dst, frag_kpad, scales, amax_scratch);
   }
   return hipGetLastError();
 }

@@ -1,0 +1,626 @@
+// Large-M int8 GEMM for gfx950 (MFMA-bound), single and grouped:
+//   C = epilogue(A[M,K] x blob), s32 accumulation on v_mfma_i32_32x32x32_i8.
+//
+// Replaces the reference's aocl_gemm_u8s8s32o* / aocl_gemm_s8s8s32o*[_sym_quant]
+// call sites (zendnnl/src/lowoha_operators/matmul/backends/aocl/
+// aocl_kernel.cpp:1190-1295) and, in grouped form, the per-expert GEMMs of
+// group_matmul_run_parallel_dispatch (matmul/group_matmul/
+// group_matmul_dispatch.cpp:1096).
+//
+// Both operands arrive in MFMA fragment order (1 KiB fragments of 32 rows x 32 k,
+// see zmi_device.h): the weights from the prepack, the activations from the
+// quantization / repack pass that precedes the GEMM.  A workgroup of 4 wavefronts
+// (2 x 2) owns a BM x 256 tile (gated: BM x 128 outputs from 2 x 128 weight
+// columns) and walks K in stages of 64:
+//   * every stage is BM/32 + 8 contiguous 2 KiB fragment pairs; each wavefront
+//     moves its share with global_load_lds_dwordx4 (global memory -> LDS without
+//     passing through registers) into a ring of NS stages, NS-1 stages ahead;
+//   * a wavefront computes (BM/2) x 128: per 32-wide k block it reads BM/64 + 4
+//     fragments from LDS (linear 16 bytes per lane, conflict free) for
+//     (BM/64) x 4 MFMAs; the reads of the next k block are interleaved with the
+//     MFMAs of the current one, two register sets;
+//   * one workgroup barrier per stage, placed between the two k blocks, where it
+//     orders "stage s+1 has landed" and "stage s-1 is free" at once.
+// The MFMA takes the weight fragment as its first operand, so a lane's 16
+// accumulators of a 32 x 32 block are 4 runs of 4 consecutive output columns of
+// one output row.  The epilogue moves each 32 x 128 strip through LDS and reads
+// it back with 16 lanes per row, so the arithmetic runs in a rolled loop with
+// the per-column constants of a lane fixed in registers, and a row is stored as
+// 128-byte (bf16) or 256-byte (f32) runs.
+#include <type_traits>
+
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+#define R_THREADS 256
+#define R_BN 256
+#define R_EPI_LD 132                       // words per staged row (128 + 4: rows 4 banks apart)
+#define R_EPI_WAVE_WORDS (32 * R_EPI_LD)
+
+extern __shared__ __attribute__((aligned(16))) char zmi_ring_smem[];
+
+__device__ __forceinline__ void zmi_dma_pair(const void *base, uint32_t voff, uint32_t lds) {
+  // two consecutive 1 KiB fragments: LDS address = m0 + offset + lane * 16
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024"
+               ::"s"(lds), "v"(voff), "s"(base)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void zmi_wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void zmi_wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+template <int BM>
+struct RingCfg {
+  static constexpr int AF = BM / 32;                 // activation fragment rows per tile
+  static constexpr int P = AF + 8;                   // 2 KiB pairs per stage
+  static constexpr int STAGE = P * 2048;
+  static constexpr int NS = BM == 256 ? 4 : 3;
+  static constexpr int OCC = BM == 256 ? 1 : 2;
+  static constexpr int NPAIR_MAX = (P + 3) / 4;
+  static constexpr int RING = STAGE * NS;
+  static constexpr int EPI = 4 * R_EPI_WAVE_WORDS * 4 + BM * 4;
+  static constexpr int SMEM = RING > EPI ? RING : EPI;
+};
+
+// Row blocks of one problem for a launch whose largest tile has `top` rows:
+// floor(M / top) full blocks (handled by the BM == top kernel) and one remainder
+// block handled by the smallest of {64, 128, 256} that holds it.
+template <int BM>
+__device__ __host__ __forceinline__ void zmi_ring_rows(int M, int top, int &full, bool &has_rem) {
+  full = BM == top ? M / top : 0;
+  const int r = M % top;
+  has_rem = r > 0 && r <= BM && (BM == 64 || r > BM / 2);
+}
+
+template <int BM>
+__host__ __device__ __forceinline__ int zmi_ring_items(int M, int N, int top, bool gated) {
+  int full; bool rem;
+  zmi_ring_rows<BM>(M, top, full, rem);
+  const int ncols = gated ? N / 2 : N;
+  const int per = gated ? 128 : 256;
+  return (full + (rem ? 1 : 0)) * ((ncols + per - 1) / per);
+}
+
+template <int BM>
+__global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_kernel(ZmiProblem p0,
+                                                                                   const ZmiProblem *probs,
+                                                                                   int n_prob, int n_items,
+                                                                                   const int *n_items_dev, int top,
+                                                                                   ZmiEpilogue epi) {
+  using Cfg = RingCfg<BM>;
+  constexpr int MI = BM / 64, NI = 4;
+  constexpr int AF = Cfg::AF, STAGE = Cfg::STAGE, NS = Cfg::NS, NPM = Cfg::NPAIR_MAX;
+  char *smem = zmi_ring_smem;
+
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int wm = wave / 2, wn = wave % 2;
+  const bool gated = epi.gated_act != 0;
+
+  // ---- which tile -------------------------------------------------------------------
+  // Workgroup ids go round robin over the 8 XCDs; renumber so that every XCD gets
+  // a contiguous range of tiles, and order tiles so that neighbours share weight
+  // columns (and, for one problem, a band of activation rows).
+  // (with row counts known only on the device the grid is a bound and the real tile count is read here)
+  if (n_items_dev) n_items = *n_items_dev;
+  const int b = blockIdx.x;
+  const int per_xcd = (n_items + 7) / 8;
+  const int id = (b % 8) * per_xcd + b / 8;
+  if (b / 8 >= per_xcd || id >= n_items) return;
+  ZmiProblem p;
+  int tm, tn, m0;
+  {
+    const int per = gated ? 128 : 256;
+    if (!probs) {
+      p = p0;
+      int full; bool rem;
+      zmi_ring_rows<BM>(p.M, top, full, rem);
+      const int tiles_m = full + (rem ? 1 : 0);
+      const int ncols = gated ? p.N / 2 : p.N;
+      const int tiles_n = (ncols + per - 1) / per;
+      const int GM = tiles_m < 8 ? tiles_m : 8;
+      const int per_group = GM * tiles_n;
+      const int group = id / per_group;
+      const int first_m = group * GM;
+      const int gm = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+      const int r = id % per_group;
+      tm = first_m + r % gm;
+      tn = r / gm;
+      m0 = tm < full ? tm * top : (p.M / top) * top;
+    } else {
+      int base = 0, e = 0;
+      tm = tn = m0 = 0;
+      bool found = false;
+      for (; e < n_prob; ++e) {
+        const int M = probs[e].M;
+        if (M <= 0) continue;
+        int full; bool rem;
+        zmi_ring_rows<BM>(M, top, full, rem);
+        const int tiles_m = full + (rem ? 1 : 0);
+        if (!tiles_m) continue;
+        const int ncols = gated ? probs[e].N / 2 : probs[e].N;
+        const int tiles_n = (ncols + per - 1) / per;
+        const int cnt = tiles_m * tiles_n;
+        if (id < base + cnt) {
+          const int r = id - base;
+          tm = r % tiles_m;
+          tn = r / tiles_m;
+          m0 = tm < full ? tm * top : (M / top) * top;
+          found = true;
+          break;
+        }
+        base += cnt;
+      }
+      if (!found) return;
+      p = probs[e];
+    }
+  }
+
+  const int M = p.M, N = p.N, K = p.K;
+  const int K_pad = (int)zmi_blob_kpad(K);
+  const int nk = K_pad / 64;
+  const int64_t frow_bytes = (int64_t)K_pad * 32;
+  const uint8_t *Afr = (const uint8_t *)p.A;
+  const uint8_t *Bfr = p.blob + zmi_blob_tiles_off(N);
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+  const int a_last = (M + 31) / 32 - 1;
+  const int b_last = (int)(zmi_blob_npad(N) / 32) - 1;
+  const int half = N / 2;
+
+  // ---- this wavefront's share of a stage: pairs wave, wave+4, ... ---------------------
+  const uint8_t *gbase[NPM];
+  uint32_t lds_dst[NPM];
+#pragma unroll
+  for (int j = 0; j < NPM; ++j) {
+    int r = wave + 4 * j;
+    if (r >= Cfg::P) r = Cfg::P - 1;       // surplus slot of a short wavefront: never issued
+    int64_t frow;
+    const uint8_t *base;
+    if (r < AF) {
+      int fr = m0 / 32 + r;
+      frow = fr < a_last ? fr : a_last;
+      base = Afr;
+    } else {
+      const int q = r - AF;
+      int fc;
+      if (!gated) {
+        fc = tn * 8 + q;
+      } else {
+        // LDS order per wavefront column half: [gate 2w, gate 2w+1, up 2w, up 2w+1]
+        const int w = q / 4, qq = q % 4;
+        fc = tn * 4 + w * 2 + (qq & 1);
+        const int lim = half / 32 - 1;
+        if (fc > lim) fc = lim;
+        if (qq >= 2) fc += half / 32;
+      }
+      frow = fc < b_last ? fc : b_last;
+      base = Bfr;
+    }
+    gbase[j] = base + frow * frow_bytes;
+    lds_dst[j] = r * 2048;
+  }
+  const int n_my = (Cfg::P - wave + 3) / 4;      // pairs this wavefront really loads
+  const bool short_wave = n_my < NPM;
+
+  uint32_t voff = lane * 16;
+  const uint32_t voff_max = lane * 16 + (nk - 1) * 2048;
+  auto issue_all = [&](int slot) {
+#pragma unroll
+    for (int j = 0; j < NPM; ++j)
+      if (j < NPM - 1 || !short_wave) zmi_dma_pair(gbase[j], voff, lds_dst[j] + slot * STAGE);
+    voff = voff + 2048 < voff_max ? voff + 2048 : voff_max;
+  };
+
+  v16i acc[NI][MI];
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[ni][mi][j] = 0;
+
+  v4i fa[2][MI], fb[2][NI];
+  const char *lbase = smem + lane * 16;
+
+  // One phase = MI*NI MFMAs on the fragments of set `cur`; the first MI+NI of them
+  // are each followed by one LDS fragment read into the other set.  In the second
+  // phase of a stage the global->LDS pairs of the stage NS-1 ahead are spread over
+  // the phase so that no wavefront sits in a queue of loads while its MFMAs wait.
+  auto phase = [&](int cur, int rd_slot, int rd_kb, bool do_issue, int is_slot) {
+    const char *pr = lbase + rd_slot * STAGE + rd_kb * 1024;
+    constexpr int NM = MI * NI;
+    constexpr int ISTEP = NM / NPM > 0 ? NM / NPM : 1;
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      const int ni = i / MI, mi = i % MI;
+      acc[ni][mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[cur][ni], fa[cur][mi], acc[ni][mi], 0, 0, 0);
+      if (i < NI) fb[cur ^ 1][i] = *(const v4i *)(pr + (AF + wn * NI + i) * 2048);
+      else if (i < NI + MI) fa[cur ^ 1][i - NI] = *(const v4i *)(pr + (wm * MI + (i - NI)) * 2048);
+      if (do_issue && i % ISTEP == 0 && i / ISTEP < NPM) {
+        const int j = i / ISTEP;
+        if (j < NPM - 1 || !short_wave) zmi_dma_pair(gbase[j], voff, lds_dst[j] + is_slot * STAGE);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (NM < NI + MI) {
+      // fewer MFMAs than fragments (BM == 64): the remaining reads follow
+#pragma unroll
+      for (int i = NM; i < NI + MI; ++i) {
+        if (i < NI) fb[cur ^ 1][i] = *(const v4i *)(pr + (AF + wn * NI + i) * 2048);
+        else fa[cur ^ 1][i - NI] = *(const v4i *)(pr + (wm * MI + (i - NI)) * 2048);
+      }
+    }
+    if (do_issue && NM / ISTEP < NPM) {
+#pragma unroll
+      for (int j = NM / ISTEP; j < NPM; ++j)
+        if (j < NPM - 1 || !short_wave) zmi_dma_pair(gbase[j], voff, lds_dst[j] + is_slot * STAGE);
+    }
+  };
+
+#ifdef ZMI_RING_PRIO
+  // Two workgroups share a CU (BM < 256): the one with the even workgroup slot issues its
+  // MFMAs first, so the pair drifts half a tile apart and one's epilogue runs under the
+  // other's main loop.
+  if (Cfg::OCC > 1) {
+    const int tg = __builtin_amdgcn_s_getreg(4 | (16 << 6) | (3 << 11));   // HW_ID.TG_ID
+    if (tg & 1) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(3);
+#ifdef ZMI_RING_DELAY
+    if (tg & 1) { const long long t0 = wall_clock64(); while (wall_clock64() - t0 < ZMI_RING_DELAY) __builtin_amdgcn_s_sleep(16); }
+#endif
+  }
+#endif
+  // ---- prologue: NS-1 stages in flight, the first one landed --------------------------
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s) issue_all(s);
+  if (short_wave) zmi_wait_vm<(NS - 2) * (NPM - 1) * 2>();
+  else zmi_wait_vm<(NS - 2) * NPM * 2>();
+  zmi_wg_barrier();
+  {
+    const char *pr = lbase;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) fb[0][i] = *(const v4i *)(pr + (AF + wn * NI + i) * 2048);
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[0][i] = *(const v4i *)(pr + (wm * MI + i) * 2048);
+  }
+
+  int slot = 0;
+  for (int s = 0; s < nk; ++s) {
+    const int slot_next = slot + 1 == NS ? 0 : slot + 1;
+    const int slot_prev = slot == 0 ? NS - 1 : slot - 1;
+    phase(0, slot, 1, false, 0);
+    // stage s+1 has landed (loads are issued every stage, clamped at the end, so the count is uniform)
+    if (short_wave) zmi_wait_vm<(NS - 3) * (NPM - 1) * 2>();
+    else zmi_wait_vm<(NS - 3) * NPM * 2>();
+    zmi_wg_barrier();
+    phase(1, slot_next, 0, true, slot_prev);
+    voff = voff + 2048 < voff_max ? voff + 2048 : voff_max;
+    slot = slot_next;
+  }
+  zmi_wait_vm<0>();
+  zmi_wg_barrier();
+
+  // ------------------------------------------------------------------------ epilogue
+#ifdef ZMI_RING_PRIO
+  __builtin_amdgcn_s_setprio(0);
+#endif
+#ifdef ZMI_RING_NO_EPI
+  if (acc[0][0][0] != 0x12345678) return;
+#endif
+  int32_t *stage = reinterpret_cast<int32_t *>(smem) + wave * R_EPI_WAVE_WORDS;
+  float *row_scale = reinterpret_cast<float *>(smem) + 4 * R_EPI_WAVE_WORDS;
+  for (int r = tid; r < BM; r += R_THREADS) {
+    const int m = m0 + r;
+    row_scale[r] = m < M ? zmi_row_scale(epi, p, m) : 1.0f;
+  }
+  __syncthreads();
+
+  const int hi = lane / 32, cl = lane % 32;
+  const int c16 = lane % 16, r4 = lane / 16;
+  const void *bias = p.bias;
+  const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+  const bool has_bias = bias != nullptr;
+  const int dst_dt = epi.dst_dt;
+
+  // output columns of this lane: two runs of 4
+  int n_run[2];
+  ZmiColCtx cc[2][4];
+  if (!gated) {
+    n_run[0] = tn * 256 + wn * 128 + c16 * 4;
+    n_run[1] = n_run[0] + 64;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cc[h][j] = zmi_col_ctx(epi, p, colsum, n_run[h] + j, N);
+  } else {
+    // run 0: gate columns n, run 1: the matching up columns n + N/2; output column n
+    n_run[0] = tn * 128 + wn * 64 + c16 * 4;
+    n_run[1] = n_run[0] + half;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      cc[0][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j, half);
+      cc[1][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j < half ? n_run[1] + j : N, N);
+    }
+  }
+  // the bf16 fast forms multiply / add unconditionally: absent scales are 1, an absent bias is -0
+  if (dst_dt == ZMI_DT_BF16 && epi.fast_kind != ZMI_EK_GENERIC) {
+    zmi_set_f32_flush();
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (!has_bias) cc[h][j].bias = -0.0f;
+  }
+  const int n_lim = gated ? half : N;
+  // vector stores need every row start aligned
+  const int es = dst_dt == ZMI_DT_BF16 ? 2 : (dst_dt == ZMI_DT_S8 || dst_dt == ZMI_DT_U8 ? 1 : 4);
+  const bool vec_ok = (((uintptr_t)p.dst) % 16 == 0) && ((p.ldc * es) % 16 == 0);
+  const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
+
+  // The strips are visited by a static loop (the accumulators are registers: a
+  // dynamic index would make the compiler select among all of them); the
+  // arithmetic inside a strip is a rolled loop.
+  auto do_strip = [&](auto mic) {
+    constexpr int mi = decltype(mic)::value;
+    // this wavefront's 32 x 128 strip -> LDS (row = lane % 32, 4 consecutive columns per store)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        v4i o = {acc[ni][mi][g * 4], acc[ni][mi][g * 4 + 1], acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]};
+        *(v4i *)&stage[cl * R_EPI_LD + ni * 32 + g * 8 + hi * 4] = o;
+      }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+
+    const int mbase = m0 + wm * (BM / 2) + mi * 32;
+    const float *rsc = row_scale + wm * (BM / 2) + mi * 32;
+
+    auto run = [&](auto ek, auto dtc) {
+      constexpr int EK = decltype(ek)::value;
+      constexpr int DT = decltype(dtc)::value;    // 0: f32, 1: bf16
+#pragma unroll 2
+      for (int it = 0; it < 8; ++it) {
+        const int r = it * 4 + r4;
+        const int m = mbase + r;
+        const v4i a0 = *(const v4i *)&stage[r * R_EPI_LD + c16 * 4];
+        const v4i a1 = *(const v4i *)&stage[r * R_EPI_LD + 64 + c16 * 4];
+        const float rs = rsc[r];
+        if (m >= M) continue;
+#ifdef ZMI_RING_NO_STORE
+        if (rs != 12345.0f) continue;
+#endif
+        float y0[4], y1[4];
+        if (DT == 1) {
+          // bf16 store: scale chain with one fused multiply-add (absent scales are 1, absent bias -0)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            y0[j] = __builtin_fmaf((float)(a0[j] + cc[0][j].comp) * rs, cc[0][j].wscale, cc[0][j].bias);
+            y1[j] = __builtin_fmaf((float)(a1[j] + cc[1][j].comp) * rs, cc[1][j].wscale, cc[1][j].bias);
+            if (!gated) { y0[j] = zmi_act_bf16<EK>(y0[j]); y1[j] = zmi_act_bf16<EK>(y1[j]); }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            y0[j] = zmi_fast_value<EK>(a0[j], cc[0][j], rs, has_rs, has_ws, has_bias);
+            y1[j] = zmi_fast_value<EK>(a1[j], cc[1][j], rs, has_rs, has_ws, has_bias);
+          }
+        }
+        if (!gated) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const float *y = h ? y1 : y0;
+            const int n = n_run[h];
+            if (n >= N) continue;
+            const int64_t o = (int64_t)m * p.ldc + n;
+            if (vec_ok && n + 3 < N) {
+              if (DT == 1) {
+                const v2u v = {zmi_pack_bf16(y[0], y[1]), zmi_pack_bf16(y[2], y[3])};
+                *zmi_global<v2u>((uint16_t *)p.dst + o) = v;
+              } else {
+                *zmi_global<v4f>((float *)p.dst + o) = (v4f){y[0], y[1], y[2], y[3]};
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if (n + j < N) {
+                  if (DT == 1) zmi_global<uint16_t>(p.dst)[o + j] = (uint16_t)zmi_pack_bf16(y[j], 0.0f);
+                  else zmi_global<float>(p.dst)[o + j] = y[j];
+                }
+            }
+          }
+        } else {
+          const int n = n_run[0];
+          if (n >= half) continue;
+          float z[4];
+          if (DT == 1) {
+            // the unfused path stores the GEMM result as bf16 before the activation reads it
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const uint32_t gu = zmi_pack_bf16(y0[j], y1[j]);
+              const float g = __uint_as_float(gu << 16), u = __uint_as_float(gu & 0xffff0000u);
+              z[j] = epi.gated_act == ZMI_ACT_SILU_AND_MUL ? zmi_act_bf16<ZMI_EK_SWISH>(g) * u
+                                                           : zmi_gated(epi.gated_act, g, u);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) z[j] = zmi_gated(epi.gated_act, y0[j], y1[j]);
+          }
+          const int64_t o = (int64_t)m * p.ldc + n;
+          if (vec_ok && n + 3 < half) {
+            if (DT == 1) {
+              const v2u v = {zmi_pack_bf16(z[0], z[1]), zmi_pack_bf16(z[2], z[3])};
+              *zmi_global<v2u>((uint16_t *)p.dst + o) = v;
+            } else {
+              *zmi_global<v4f>((float *)p.dst + o) = (v4f){z[0], z[1], z[2], z[3]};
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (n + j < half) {
+                if (DT == 1) zmi_global<uint16_t>(p.dst)[o + j] = (uint16_t)zmi_pack_bf16(z[j], 0.0f);
+                else zmi_global<float>(p.dst)[o + j] = z[j];
+              }
+          }
+        }
+      }
+    };
+    using std::integral_constant;
+    const bool bf16 = dst_dt == ZMI_DT_BF16;
+    const bool fast_ok = epi.fast_kind != ZMI_EK_GENERIC && (bf16 || dst_dt == ZMI_DT_F32);
+    // the gated form applies no element-wise post-op of its own before the activation
+    const int kind = fast_ok ? (gated && epi.fast_kind != ZMI_EK_NONE ? -1 : epi.fast_kind * 2 + (bf16 ? 1 : 0)) : -1;
+    switch (kind) {
+    case ZMI_EK_NONE * 2: run(integral_constant<int, ZMI_EK_NONE>{}, integral_constant<int, 0>{}); break;
+    case ZMI_EK_NONE * 2 + 1: run(integral_constant<int, ZMI_EK_NONE>{}, integral_constant<int, 1>{}); break;
+    case ZMI_EK_SWISH * 2: run(integral_constant<int, ZMI_EK_SWISH>{}, integral_constant<int, 0>{}); break;
+    case ZMI_EK_SWISH * 2 + 1: run(integral_constant<int, ZMI_EK_SWISH>{}, integral_constant<int, 1>{}); break;
+    case ZMI_EK_GELU_TANH * 2: run(integral_constant<int, ZMI_EK_GELU_TANH>{}, integral_constant<int, 0>{}); break;
+    case ZMI_EK_GELU_TANH * 2 + 1: run(integral_constant<int, ZMI_EK_GELU_TANH>{}, integral_constant<int, 1>{}); break;
+    case ZMI_EK_RELU * 2: run(integral_constant<int, ZMI_EK_RELU>{}, integral_constant<int, 0>{}); break;
+    case ZMI_EK_RELU * 2 + 1: run(integral_constant<int, ZMI_EK_RELU>{}, integral_constant<int, 1>{}); break;
+    default:
+      // generic interpreter: any post-op chain, alpha / beta, destination quantization, raw s32
+#pragma unroll 1
+      for (int it = 0; it < 8; ++it) {
+        const int r = it * 4 + r4;
+        const int m = mbase + r;
+        if (m >= M) continue;
+        const float rs = rsc[r];
+#pragma unroll 1
+        for (int j = 0; j < 4; ++j) {
+          const int32_t a0 = stage[r * R_EPI_LD + c16 * 4 + j];
+          const int32_t a1 = stage[r * R_EPI_LD + 64 + c16 * 4 + j];
+          if (!gated) {
+#pragma unroll 1
+            for (int h = 0; h < 2; ++h) {
+              const int n = n_run[h] + j;
+              if (n >= N) continue;
+              const int64_t o = (int64_t)m * p.ldc + n;
+              const ZmiColCtx c = zmi_col_ctx(epi, p, colsum, n, N);
+              const int32_t a = h ? a1 : a0;
+              if (raw) ((int32_t *)p.dst)[o] = a + c.comp;
+              else zmi_store(p.dst, dst_dt, o, zmi_epilogue_value(epi, a, c, rs, m, n, p.dst, p.ldc));
+            }
+          } else {
+            const int n = n_run[0] + j;
+            if (n >= half) continue;
+            const ZmiColCtx cg = zmi_col_ctx(epi, p, colsum, n, half);
+            const ZmiColCtx cu = zmi_col_ctx(epi, p, colsum, n + half, N);
+            float g = zmi_epilogue_value(epi, a0, cg, rs, m, n, p.dst, p.ldc);
+            float u = zmi_epilogue_value(epi, a1, cu, rs, m, n + half, p.dst, p.ldc);
+            if (dst_dt == ZMI_DT_BF16) {
+              g = zmi_bf16_to_f32(zmi_f32_to_bf16(g));
+              u = zmi_bf16_to_f32(zmi_f32_to_bf16(u));
+            }
+            zmi_store(p.dst, dst_dt, (int64_t)m * p.ldc + n, zmi_gated(epi.gated_act, g, u));
+          }
+        }
+      }
+    }
+    (void)n_lim;
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+  };
+  do_strip(std::integral_constant<int, 0>{});
+  if constexpr (MI > 1) do_strip(std::integral_constant<int, 1>{});
+  if constexpr (MI > 2) {
+    do_strip(std::integral_constant<int, 2>{});
+    do_strip(std::integral_constant<int, 3>{});
+  }
+}
+
+// Tile counts of a problem table for the three tile heights, computed where the row counts live.
+__global__ void zmi_ring_count_kernel(const ZmiProblem *probs, int n_prob, int top, int gated, int *out) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int c256 = 0, c128 = 0, c64 = 0;
+  for (int e = 0; e < n_prob; ++e) {
+    const int M = probs[e].M, N = probs[e].N;
+    if (M <= 0) continue;
+    if (top == 256) c256 += zmi_ring_items<256>(M, N, top, gated != 0);
+    c128 += zmi_ring_items<128>(M, N, top, gated != 0);
+    c64 += zmi_ring_items<64>(M, N, top, gated != 0);
+  }
+  out[0] = c256; out[1] = c128; out[2] = c64;
+}
+
+template <int BM>
+static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items,
+                              const int *n_items_dev, int top, const ZmiEpilogue &epi, hipStream_t stream) {
+  if (n_items <= 0) return hipSuccess;
+  const size_t smem = RingCfg<BM>::SMEM;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_ring_kernel<BM>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  const int grid = (n_items + 7) / 8 * 8;   // a multiple of 8 so the XCD renumbering applies
+  hipLaunchKernelGGL(zmi_gemm_ring_kernel<BM>, dim3(grid), dim3(R_THREADS), smem, stream, p0, probs, n_prob,
+                     n_items, n_items_dev, top, epi);
+  return hipGetLastError();
+}
+
+// Largest tile height for a problem set: 256-row tiles once they fill the chip,
+// 128-row tiles for smaller problems (more tiles, two workgroups per CU).
+int zmi_ring_pick_top(int64_t rows, int64_t out_cols) {
+  const int64_t t256 = ((rows + 255) / 256) * ((out_cols + 255) / 256);
+  return t256 >= 192 ? 256 : 128;
+}
+
+// One problem, M rows in fragment-major order at p.A.
+hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream) {
+  if (p.M <= 0) return hipSuccess;
+  const bool gated = epi.gated_act != 0;
+  hipError_t e = hipSuccess;
+  if (top == 256) {
+    e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), nullptr, top, epi, stream);
+    if (e != hipSuccess) return e;
+  }
+  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), nullptr, top, epi, stream);
+  if (e != hipSuccess) return e;
+  return ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), nullptr, top, epi, stream);
+}
+
+// Every problem of the table.  probs_host mirrors probs_dev and sizes the grids;
+// when it is null (row counts known only on the device) worst_rows / worst_cols
+// bound them, the real tile counts are computed on the device into counts_dev
+// (3 ints of scratch) and surplus workgroups exit at once.
+hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
+                                      int top, int64_t worst_rows, int worst_cols, int *counts_dev,
+                                      const ZmiEpilogue &epi, hipStream_t stream) {
+  const bool gated = epi.gated_act != 0;
+  int items[3] = {0, 0, 0};   // 256, 128, 64
+  if (probs_host) {
+    for (int e = 0; e < n_prob; ++e) {
+      const ZmiProblem &q = probs_host[e];
+      if (q.M <= 0) continue;
+      items[0] += top == 256 ? zmi_ring_items<256>(q.M, q.N, top, gated) : 0;
+      items[1] += zmi_ring_items<128>(q.M, q.N, top, gated);
+      items[2] += zmi_ring_items<64>(q.M, q.N, top, gated);
+    }
+  } else {
+    const int per = gated ? 128 : 256;
+    const int ncols = gated ? worst_cols / 2 : worst_cols;
+    const int tiles_n = (ncols + per - 1) / per;
+    // at most rows/top full blocks in total and one remainder block per problem
+    items[top == 256 ? 0 : 1] = (int)(worst_rows / top + n_prob) * tiles_n;
+    if (top == 256) items[1] = n_prob * tiles_n;
+    items[2] = n_prob * tiles_n;
+    if (!counts_dev) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0,
+                       counts_dev);
+  }
+  const int *cd = probs_host ? nullptr : counts_dev;
+  ZmiProblem dummy = {};
+  hipError_t e = hipSuccess;
+  if (top == 256) {
+    e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], cd, top, epi, stream);
+    if (e != hipSuccess) return e;
+  }
+  e = ring_launch<128>(dummy, probs_dev, n_prob, items[1], cd ? cd + 1 : nullptr, top, epi, stream);
+  if (e != hipSuccess) return e;
+  return ring_launch<64>(dummy, probs_dev, n_prob, items[2], cd ? cd + 2 : nullptr, top, epi, stream);
+}

@@ -225,32 +225,38 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
   return ZMI_SUCCESS;
 }
 
-static int pick_bm(int M, int N) {
-  if (const char *env = std::getenv("ZMI_GEMM_BM")) {
+static int pick_top(int M, int N) {
+  if (const char *env = std::getenv("ZMI_GEMM_TOP")) {
     int v = std::atoi(env);
-    if (v == 64 || v == 128 || v == 256) return v;
+    if (v == 128 || v == 256) return v;
   }
-  // Measured on MI355X (K = 4096): with 2 workgroups resident per CU the 64-row
-  // tile wins while there are fewer than about two 128-row tiles per CU, the
-  // 128-row tile after that.
-  auto tiles = [&](int bm) { return (int64_t)((M + bm - 1) / bm) * ((N + 255) / 256); };
-  if (tiles(128) >= 2 * 256) return 128;
-  return 64;
+  return zmi_ring_pick_top(M, N);
 }
 
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi) {
   if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
     set_kernel_name("decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, stream()), "decode GEMM launch")) return ZMI_FAILURE;
-  } else if (prob.M <= 128) {
+  } else if (!use_ring_kernel(prob.M)) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
   } else {
-    const int bm = pick_bm(prob.M, epi.gated_act ? prob.N / 2 : prob.N);
-    set_kernel_name(bm == 256 ? "mfma32x32x32_bm256" : (bm == 128 ? "mfma32x32x32_bm128" : "mfma32x32x32_bm64"));
-    if (!hip_ok(zmi_launch_gemm_mfma(prob, epi, bm, stream()), "MFMA GEMM launch")) return ZMI_FAILURE;
+    // prob.A is fragment-major here (see use_ring_kernel)
+    const int top = pick_top(prob.M, epi.gated_act ? prob.N / 2 : prob.N);
+    set_kernel_name(top == 256 ? "ring_mfma32x32x32_top256" : "ring_mfma32x32x32_top128");
+    if (!hip_ok(zmi_launch_gemm_ring(prob, epi, top, stream()), "MFMA GEMM launch")) return ZMI_FAILURE;
   }
   return ZMI_SUCCESS;
+}
+
+// Problems with more rows than the small-M kernels take run on the MFMA-bound
+// kernel, which reads the activations in fragment-major order.
+bool use_ring_kernel(int M) {
+  static const int min_m = [] {
+    const char *env = std::getenv("ZMI_RING_MIN_M");
+    return env ? std::atoi(env) : 129;
+  }();
+  return M >= min_m;
 }
 
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
@@ -333,11 +339,14 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                          std::min(weight_cache_env(), p.weight_cache_type) > 0;
   const bool pack_in_arena = p.mem_format_b != 'r' && !use_cache;
   const int64_t K16 = zmi_round_up(K, 16);
-  const bool repack_a = !dyn && a_needs_repack(src, lda, K, transA != 0);
+  const bool ring = use_ring_kernel(M);
+  const int64_t frag_kpad = ring ? zmi_blob_kpad(K) : 0;
+  const size_t a_bytes = ring ? (size_t)zmi_afrag_bytes(M, K) : (size_t)M * K16;
+  const bool repack_a = !dyn && (ring || a_needs_repack(src, lda, K, transA != 0));
   size_t need = 0;
   if (pack_in_arena) need += Arena::padded((size_t)zmi_blob_bytes(K, N));
-  if (dyn) need += Arena::padded((size_t)M * K16) + Arena::padded(sizeof(float) * (size_t)M) + 256;
-  if (repack_a) need += Arena::padded((size_t)M * K16);
+  if (dyn) need += Arena::padded(a_bytes) + Arena::padded(sizeof(float) * (size_t)M) + 256;
+  if (repack_a) need += Arena::padded(a_bytes);
   if (!arena().begin(need)) return ZMI_FAILURE;
 
   // ---- weights ----
@@ -364,7 +373,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   bool use_fused = false;
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
-    int8_t *q = (int8_t *)arena().alloc((size_t)M * K16);
+    int8_t *q = (int8_t *)arena().alloc(a_bytes);
     float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M);
     unsigned int *amax = (unsigned int *)arena().alloc(256);
     // bytes of q between K and K16 stay unwritten: the blob's rows beyond K are zero
@@ -374,7 +383,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     const bool per_token = (dyn_scale_n == M && M > 1) || M == 1;
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
     const bool decode_kernel = M <= 16 && zmi_blob_kpad(K) <= 4096 && !std::getenv("ZMI_NO_DECODE_KERNEL");
-    if (per_token && !decode_kernel && M <= 128 && K % 4 == 0 && zmi_smallm_grid(prob, false) <= 512 &&
+    if (per_token && !decode_kernel && !ring && M <= 128 && K % 4 == 0 && zmi_smallm_grid(prob, false) <= 512 &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
       if (!ctr) return ZMI_FAILURE;
@@ -389,14 +398,14 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     } else if (dyn_scale_n == M && M > 1) {
       void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
       if (!p.src_scale.buff) sdt = ZMI_DT_F32;
-      if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, scale_out, sdt, stream()), "quant launch"))
+      if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, frag_kpad, scale_out, sdt, stream()), "quant launch"))
         return ZMI_FAILURE;
       ep.src_scale.buff = scale_out;
       ep.src_scale.dt = sdt;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = 1;
     } else {
       // one scale for the whole tensor; with M == 1 this is the per-token case too
-      if (!hip_ok(zmi_launch_quant_tensor(src, p.dt_src, M, K, lda, q, K16, sc, amax, stream()), "quant launch"))
+      if (!hip_ok(zmi_launch_quant_tensor(src, p.dt_src, M, K, lda, q, K16, frag_kpad, sc, amax, stream()), "quant launch"))
         return ZMI_FAILURE;
       if (p.src_scale.buff) {
         if (sdt != ZMI_DT_F32) { set_error("per-tensor dynamic scale output must be f32"); return ZMI_UNIMPLEMENTED; }
@@ -411,8 +420,12 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     prob.A = q; prob.lda = K16; prob.a_is_u8 = 0;
     ep.dt_src = ZMI_DT_S8;
   } else if (repack_a) {
-    int8_t *a2 = (int8_t *)arena().alloc((size_t)M * K16);
-    if (!hip_ok(zmi_launch_pad_rows(src, M, K, lda, transA != 0, a2, K16, stream()), "pad launch")) return ZMI_FAILURE;
+    int8_t *a2 = (int8_t *)arena().alloc(a_bytes);
+    if (ring) {
+      if (!hip_ok(zmi_launch_repack_frag(src, M, K, lda, transA != 0, p.dt_src == ZMI_DT_U8, a2, stream()), "repack launch")) return ZMI_FAILURE;
+    } else {
+      if (!hip_ok(zmi_launch_pad_rows(src, M, K, lda, transA != 0, a2, K16, stream()), "pad launch")) return ZMI_FAILURE;
+    }
     prob.A = a2; prob.lda = K16; prob.a_is_u8 = p.dt_src == ZMI_DT_U8;
   } else {
     prob.A = src; prob.lda = lda; prob.a_is_u8 = p.dt_src == ZMI_DT_U8;
@@ -485,7 +498,7 @@ static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t 
   const int64_t sn = nelems(rp.scale);
   if (!ensure_device()) return ZMI_FAILURE;
   if (rp.scale.ndims == 2 && rp.scale.dims[0] == M && rp.scale.dims[1] == 1) {
-    if (!hip_ok(zmi_launch_quant_rows(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, (void *)rp.scale.buff, sdt, stream()),
+    if (!hip_ok(zmi_launch_quant_rows(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, 0, (void *)rp.scale.buff, sdt, stream()),
                 "quant launch"))
       return ZMI_FAILURE;
     set_kernel_name("quant_rows_per_token");
@@ -496,7 +509,7 @@ static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t 
     if (!arena().begin(Arena::padded(sizeof(float) * (size_t)M) + 256)) return ZMI_FAILURE;
     float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M);
     unsigned int *amax = (unsigned int *)arena().alloc(256);
-    if (!hip_ok(zmi_launch_quant_tensor(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, sc, amax, stream()), "quant launch"))
+    if (!hip_ok(zmi_launch_quant_tensor(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, 0, sc, amax, stream()), "quant launch"))
       return ZMI_FAILURE;
     if (!hip_ok(hipMemcpyAsync((void *)rp.scale.buff, sc, sizeof(float), hipMemcpyDeviceToDevice, stream()), "hipMemcpyAsync"))
       return ZMI_FAILURE;
@@ -547,7 +560,7 @@ int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src, const int32_t
     if (M[i] < 0 || K[i] <= 0) { set_error("group_dynamic_quant: bad shape"); return ZMI_FAILURE; }
     if (M[i] == 0) continue;
     if (!src[i] || !dst[i] || !scale[i]) { set_error("group_dynamic_quant: null buffer for an active matrix"); return ZMI_FAILURE; }
-    ZmiQuantMat m;
+    ZmiQuantMat m = {};
     m.src = src[i]; m.dst = (int8_t *)dst[i]; m.scale = scale[i];
     m.ld_src = src_row_stride && src_row_stride[i] ? src_row_stride[i] : K[i];
     m.ld_dst = dst_row_stride && dst_row_stride[i] ? dst_row_stride[i] : K[i];

@@ -225,19 +225,22 @@ struct Stage {
   ZmiEpilogue epi;
 };
 
+int group_top(int64_t rows, int64_t out_cols) {
+  if (const char *env = std::getenv("ZMI_GROUP_TOP")) { int v = std::atoi(env); if (v == 128 || v == 256) return v; }
+  return zmi_ring_pick_top(rows, out_cols);
+}
+
+// Every expert's activations are fragment-major; one launch per tile height.
 int32_t launch_stage(const Stage &st, const char *what) {
   if (st.probs.empty()) return ZMI_SUCCESS;
   const ZmiProblem *dev = (const ZmiProblem *)upload(st.probs.data(), st.probs.size() * sizeof(ZmiProblem));
   if (!dev) return ZMI_FAILURE;
   const int n = (int)st.probs.size();
-  int bm = 128;
-  if (const char *env = std::getenv("ZMI_GROUP_BM")) { int v = std::atoi(env); if (v == 64 || v == 128 || v == 256) bm = v; }
-  // one small-M launch per row-count bucket so few-row experts do not pay for 128-row tiles
-  static const int kBuckets[5] = {0, 16, 32, 64, 128};
-  for (int b = 0; b < 4; ++b)
-    if (!hip_ok(zmi_launch_gemm_smallm_group(st.probs.data(), dev, n, kBuckets[b], kBuckets[b + 1], 0, 0, st.epi, stream()), what))
-      return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_gemm_mfma_group(st.probs.data(), dev, n, 128, 0, st.epi, bm, stream()), what)) return ZMI_FAILURE;
+  int64_t rows = 0;
+  int cols = 0;
+  for (const ZmiProblem &q : st.probs) { rows += q.M; cols = std::max(cols, (int)q.N); }
+  const int top = group_top(rows, st.epi.gated_act ? cols / 2 : cols);
+  if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, nullptr, st.epi, stream()), what)) return ZMI_FAILURE;
   return ZMI_SUCCESS;
 }
 
@@ -339,9 +342,8 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     for (size_t i = 0; i < num_ops; ++i) {
       if (a.M[i] <= 0) continue;
       rows += a.M[i];
-      const int64_t K16 = zmi_round_up(a.K[i], 16);
-      if (dyn) need += Arena::padded((size_t)a.M[i] * K16) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
-      else if (a_needs_repack(a.src[i], a.lda[i], a.K[i], false)) need += Arena::padded((size_t)a.M[i] * K16);
+      if (dyn) need += Arena::padded((size_t)zmi_afrag_bytes(a.M[i], a.K[i])) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
+      else need += Arena::padded((size_t)zmi_afrag_bytes(a.M[i], a.K[i]));
       const bool cache = a.params[i].mem_format_b != 'r' && a.is_weights_const[i] &&
                          std::min(weight_cache_env(), a.params[i].weight_cache_type) > 0;
       if (a.params[i].mem_format_b != 'r' && !cache) need += Arena::padded((size_t)zmi_blob_bytes(a.K[i], a.N[i]));
@@ -351,8 +353,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       }
       if (fused_moe) {
         const int kd = op2_k_for_act(a.N[i], gated_act);
-        const int64_t kd16 = zmi_round_up(kd, 16);
-        need += Arena::padded((size_t)a.M[i] * kd16) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
+        need += Arena::padded((size_t)zmi_afrag_bytes(a.M[i], kd)) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
         const bool cache2 = a.is_weights_const[i] && std::min(weight_cache_env(), a.params[i].weight_cache_type) > 0;
         if (!cache2) need += Arena::padded((size_t)zmi_blob_bytes(kd, fused_moe->N_down[i]));
       }
@@ -375,16 +376,17 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       int64_t r0 = 0;
       for (size_t i = 0; i < num_ops; ++i) {
         if (a.M[i] <= 0) continue;
-        const int64_t K16 = zmi_round_up(a.K[i], 16);
-        ZmiQuantMat m;
+        const int64_t kp = zmi_blob_kpad(a.K[i]);
+        ZmiQuantMat m = {};
         m.src = a.src[i];
-        m.dst = (int8_t *)arena().alloc((size_t)a.M[i] * K16);
+        m.dst = (int8_t *)arena().alloc((size_t)zmi_afrag_bytes(a.M[i], a.K[i]));
         float *sc = (float *)arena().alloc(sizeof(float) * (size_t)a.M[i]);
         m.scale = a.params[i].src_scale.buff ? (void *)a.params[i].src_scale.buff : (void *)sc;
-        m.ld_src = a.lda[i]; m.ld_dst = K16; m.M = a.M[i]; m.K = a.K[i]; m.row_start = (int32_t)r0;
+        m.ld_src = a.lda[i]; m.ld_dst = kp; m.M = a.M[i]; m.K = a.K[i]; m.row_start = (int32_t)r0;
+        m.frag_kpad = (int32_t)kp;
         r0 += a.M[i];
         mats.push_back(m);
-        A1[i] = m.dst; lda1[i] = K16; s1[i] = m.scale;
+        A1[i] = m.dst; lda1[i] = kp; s1[i] = m.scale;
       }
       s1_dt = (p0.src_scale.buff && p0.src_scale.dt != ZMI_DT_NONE) ? p0.src_scale.dt : ZMI_DT_F32;
       if (s1_dt != ZMI_DT_F32 && s1_dt != ZMI_DT_BF16) { set_error("source scale must be f32 or bf16"); return ZMI_FAILURE; }
@@ -394,14 +396,9 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     } else {
       for (size_t i = 0; i < num_ops; ++i) {
         if (a.M[i] <= 0) continue;
-        if (a_needs_repack(a.src[i], a.lda[i], a.K[i], false)) {
-          const int64_t K16 = zmi_round_up(a.K[i], 16);
-          int8_t *t = (int8_t *)arena().alloc((size_t)a.M[i] * K16);
-          if (!hip_ok(zmi_launch_pad_rows(a.src[i], a.M[i], a.K[i], a.lda[i], 0, t, K16, stream()), "pad launch")) return ZMI_FAILURE;
-          A1[i] = t; lda1[i] = K16;
-        } else {
-          A1[i] = a.src[i]; lda1[i] = a.lda[i];
-        }
+        int8_t *t = (int8_t *)arena().alloc((size_t)zmi_afrag_bytes(a.M[i], a.K[i]));
+        if (!hip_ok(zmi_launch_repack_frag(a.src[i], a.M[i], a.K[i], a.lda[i], 0, a.params[i].dt_src == ZMI_DT_U8, t, stream()), "repack launch")) return ZMI_FAILURE;
+        A1[i] = t; lda1[i] = zmi_blob_kpad(a.K[i]);
       }
     }
 
@@ -462,7 +459,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     op1.epi.gated_act = fuse_act ? gated_act : ZMI_ACT_NONE;
     st = launch_stage(op1, "Op1 GEMM launch");
     if (st != ZMI_SUCCESS) return st;
-    set_kernel_name(fuse_act ? "group: smallm + mfma32x32x32 (gated epilogue)" : "group: smallm + mfma32x32x32");
+    set_kernel_name(fuse_act ? "group: ring_mfma32x32x32 (gated epilogue)" : "group: ring_mfma32x32x32");
 
     if (run_act && !fuse_act) {
       // reference: group_matmul_moe_act_execute, group_matmul/group_matmul_moe_act.cpp
@@ -495,15 +492,16 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       for (size_t i = 0; i < num_ops; ++i) {
         if (a.M[i] <= 0) continue;
         const int kd = op2_k_for_act(a.N[i], gated_act);
-        const int64_t kd16 = zmi_round_up(kd, 16);
-        ZmiQuantMat m;
+        const int64_t kp = zmi_blob_kpad(kd);
+        ZmiQuantMat m = {};
         m.src = op1_dst[i];
-        m.dst = (int8_t *)arena().alloc((size_t)a.M[i] * kd16);
+        m.dst = (int8_t *)arena().alloc((size_t)zmi_afrag_bytes(a.M[i], kd));
         m.scale = arena().alloc(sizeof(float) * (size_t)a.M[i]);
-        m.ld_src = op1_ld[i]; m.ld_dst = kd16; m.M = a.M[i]; m.K = kd; m.row_start = (int32_t)r0;
+        m.ld_src = op1_ld[i]; m.ld_dst = kp; m.M = a.M[i]; m.K = kd; m.row_start = (int32_t)r0;
+        m.frag_kpad = (int32_t)kp;
         r0 += a.M[i];
         mats.push_back(m);
-        A2[i] = m.dst; s2[i] = (float *)m.scale; lda2[i] = kd16;
+        A2[i] = m.dst; s2[i] = (float *)m.scale; lda2[i] = kp;
       }
       const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
       if (!dev) return ZMI_FAILURE;
@@ -569,7 +567,7 @@ int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk, int32_t 
   if (!topk_ids || !counts || !offsets || !slot_of || T <= 0 || topk <= 0 || E <= 0) { set_error("moe_route: bad arguments"); return ZMI_FAILURE; }
   if (E > 2047) { set_error("moe_route: at most 2047 experts"); return ZMI_UNIMPLEMENTED; }
   if (!ensure_device()) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, counts, offsets, slot_of, stream()), "moe route launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, 1, counts, offsets, slot_of, stream()), "moe route launch")) return ZMI_FAILURE;
   set_kernel_name("moe_route");
   return ZMI_SUCCESS;
 }
@@ -587,23 +585,27 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   if (E > 2047) { set_error("moe_fused_device: at most 2047 experts"); return ZMI_UNIMPLEMENTED; }
   if (!ensure_device()) return ZMI_FAILURE;
   const int64_t R = (int64_t)T * topk;
+  // every expert's rows start on a fragment row (multiple of 32 slots): at most 31 idle slots per expert
+  const int64_t Rp = zmi_round_up(R + 31 * (int64_t)E, 32);
+  const int64_t kpH = zmi_blob_kpad(H), kpI = zmi_blob_kpad(I);
   size_t need = 0;
   need += Arena::padded(sizeof(int32_t) * E) + Arena::padded(sizeof(int32_t) * (E + 1)) + Arena::padded(sizeof(int32_t) * R);
-  need += Arena::padded((size_t)R * H) + Arena::padded(sizeof(float) * R);          // A1, s1
-  need += Arena::padded((size_t)R * I * 2);                                         // act bf16
-  need += Arena::padded((size_t)R * I) + Arena::padded(sizeof(float) * R);          // A2, s2
-  need += Arena::padded((size_t)R * H * 2);                                         // Y bf16
-  need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096;
+  need += Arena::padded((size_t)Rp * kpH) + Arena::padded(sizeof(float) * Rp);       // A1, s1
+  need += Arena::padded((size_t)Rp * I * 2);                                         // act bf16
+  need += Arena::padded((size_t)Rp * kpI) + Arena::padded(sizeof(float) * Rp);       // A2, s2
+  need += Arena::padded((size_t)Rp * H * 2);                                         // Y bf16
+  need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096 + 256;
   if (!arena().begin(need)) return ZMI_FAILURE;
   int32_t *counts = (int32_t *)arena().alloc(sizeof(int32_t) * E);
   int32_t *offsets = (int32_t *)arena().alloc(sizeof(int32_t) * (E + 1));
   int32_t *slot_of = (int32_t *)arena().alloc(sizeof(int32_t) * R);
-  int8_t *A1 = (int8_t *)arena().alloc((size_t)R * H);
-  float *s1 = (float *)arena().alloc(sizeof(float) * R);
-  void *act = arena().alloc((size_t)R * I * 2);
-  int8_t *A2 = (int8_t *)arena().alloc((size_t)R * I);
-  float *s2 = (float *)arena().alloc(sizeof(float) * R);
-  void *Y = arena().alloc((size_t)R * H * 2);
+  int8_t *A1 = (int8_t *)arena().alloc((size_t)Rp * kpH);
+  float *s1 = (float *)arena().alloc(sizeof(float) * Rp);
+  void *act = arena().alloc((size_t)Rp * I * 2);
+  int8_t *A2 = (int8_t *)arena().alloc((size_t)Rp * kpI);
+  float *s2 = (float *)arena().alloc(sizeof(float) * Rp);
+  void *Y = arena().alloc((size_t)Rp * H * 2);
+  int *tile_counts = (int *)arena().alloc(256);
   ZmiProblem *op1 = (ZmiProblem *)arena().alloc(sizeof(ZmiProblem) * E);
   ZmiProblem *op2 = (ZmiProblem *)arena().alloc(sizeof(ZmiProblem) * E);
 
@@ -623,7 +625,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   tb.w13_scale = (const float *const *)(tdev + 2 * E); tb.w2_scale = (const float *const *)(tdev + 3 * E);
 
   hipStream_t s = stream();
-  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, counts, offsets, slot_of, s), "moe route launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, 32, counts, offsets, slot_of, s), "moe route launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_quant_scatter(d->x, d->ldx, T, H, topk, slot_of, A1, s1, s), "quant scatter launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, s), "problem table launch")) return ZMI_FAILURE;
 
@@ -634,19 +636,12 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   e1.bias_dt = ZMI_DT_F32; e1.alpha = 1.0f; e1.beta = 0.0f; e1.dst_dt = ZMI_DT_BF16; e1.fast_kind = ZMI_EK_NONE;
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
-  // row counts live on the device: size the grids for the worst case
-  const int bm = 128;
-  const int small_grid1 = E * (I / 16), small_grid2 = E * (int)(zmi_blob_npad(H) / 32);
-  const int items1 = (int)((R / bm + E) * ((I + 127) / 128));
-  const int items2 = (int)((R / bm + E) * ((H + 255) / 256));
-  static const int kBuckets[5] = {0, 16, 32, 64, 128};
-  for (int b = 0; b < 4; ++b)
-    if (!hip_ok(zmi_launch_gemm_smallm_group(nullptr, op1, E, kBuckets[b], kBuckets[b + 1], small_grid1, zmi_blob_kpad(H), e1, s), "Op1 small-M launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_gemm_mfma_group(nullptr, op1, E, 128, items1, e1, bm, s), "Op1 MFMA launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, R, I, I, A2, I, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
-  for (int b = 0; b < 4; ++b)
-    if (!hip_ok(zmi_launch_gemm_smallm_group(nullptr, op2, E, kBuckets[b], kBuckets[b + 1], small_grid2, zmi_blob_kpad(I), e2, s), "Op2 small-M launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_gemm_mfma_group(nullptr, op2, E, 128, items2, e2, bm, s), "Op2 MFMA launch")) return ZMI_FAILURE;
+  // row counts live on the device: the grids are sized for the worst case
+  const int top1 = group_top(R, I), top2 = group_top(R, H);
+  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_counts, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+  // idle slots between experts are quantized too (their values are never read back)
+  if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_counts + 4, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;
   upload_fence();
   set_kernel_name("moe_fused_device");

@@ -8,6 +8,8 @@
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------------------
 // Packed weight blob ("mem_format_b == 'r'").
@@ -59,6 +61,16 @@ static inline __host__ __device__ int64_t zmi_blob_nb_stride(int64_t K) {
 }
 static inline __host__ __device__ int64_t zmi_blob_bytes(int64_t K, int64_t N) {
   return zmi_blob_tiles_off(N) + zmi_blob_nb_stride(K) * (zmi_blob_npad(N) / 32);
+}
+
+// Activations for the large-M kernel use the same fragment order: an array
+// [ceil(M/32)][K_pad/32] of 1 KiB fragments, fragment (mb, kb) lane i bytes
+// [16i, 16i+16) = A[mb*32 + i%32][kb*32 + (i/32)*16 + b].  Byte offset of A[r][k]:
+static inline __host__ __device__ int64_t zmi_afrag_off(int64_t r, int64_t k, int64_t k_pad) {
+  return ((r >> 5) * (k_pad >> 5) + (k >> 5)) * 1024 + ((((k >> 4) & 1) << 5) + (r & 31)) * 16 + (k & 15);
+}
+static inline __host__ __device__ int64_t zmi_afrag_bytes(int64_t M, int64_t K) {
+  return zmi_round_up(M, 32) * zmi_blob_kpad(K);
 }
 
 // ---------------------------------------------------------------------------
@@ -129,6 +141,16 @@ struct ZmiProblem {
 };
 
 #ifdef __HIPCC__
+// A pointer that is known to address global memory.  Pointers that reach a kernel
+// inside a problem table are generic to the compiler, and accesses through them
+// become flat instructions, which share a counter with LDS reads: a wait for an
+// LDS read then also waits for every store in flight.
+#define ZMI_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ ZMI_GLOBAL T *zmi_global(const void *p) {
+  return (ZMI_GLOBAL T *)(uintptr_t)p;
+}
+
 // ------------------------------------------------------------------ device math
 __device__ __forceinline__ float zmi_bf16_to_f32(uint16_t h) {
   return __uint_as_float(((uint32_t)h) << 16);
@@ -308,6 +330,44 @@ template <bool BF16>
 __device__ __forceinline__ void zmi_fast_store(void *dst, int64_t i, float y) {
   if (BF16) ((uint16_t *)dst)[i] = zmi_f32_to_bf16(y);
   else ((float *)dst)[i] = y;
+}
+
+// ---- bf16-destination forms used by the large-M kernel ---------------------------
+// Two f32 values -> packed bf16 with the hardware conversion.  With the
+// wavefront's f32 denormal mode set to flush (zmi_set_f32_flush) it is
+// bit-identical to zmi_f32_to_bf16 on every input: round to nearest even,
+// zero / subnormal -> signed zero, NaN quieted with its payload kept.
+typedef __bf16 zmi_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float zmi_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t zmi_pack_bf16(float lo, float hi) {
+  zmi_f32x2 v = {lo, hi};
+  zmi_bf16x2 r = __builtin_convertvector(v, zmi_bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+// MODE register, bits [5:4]: single-precision denormal mode, 0 = flush inputs and results
+__device__ __forceinline__ void zmi_set_f32_flush() { __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0); }
+
+// Activations evaluated for a bf16 store: plain hardware exp2 / reciprocal, fused
+// multiply-adds.  The result differs from the separately rounded f32 form by
+// about 1e-6 relative, 1/2000 of half a bf16 unit in the last place.
+template <int EK>
+__device__ __forceinline__ float zmi_act_bf16(float x) {
+  if (EK == ZMI_EK_RELU) return x > 0.0f ? x : 0.0f;
+  if (EK == ZMI_EK_SWISH) {
+    const float e = __builtin_amdgcn_exp2f(x * -1.44269502162933349609375f);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+  }
+  if (EK == ZMI_EK_GELU_TANH) {
+    // exp(-2u) = exp2(x * (c0 + c1 x^2)), u = sqrt(2/pi) x (1 + 0.044715 x^2); then the
+    // reference's "0.5 x (1.0f + tanhf(u))" with tanh(u) = 2 sigmoid(2u) - 1 rounded to float
+    const float c0 = -2.0f * 1.44269502162933349609375f * 0.79788458347320556640625f;
+    const float c1 = c0 * 0.044715f;
+    const float a = x * __builtin_fmaf(c1, x * x, c0);
+    const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a));
+    const float v = __builtin_fmaf(2.0f, s, -1.0f);
+    return (0.5f * x) * (1.0f + v);
+  }
+  return x;
 }
 
 // Store conversions (reference: store_output,

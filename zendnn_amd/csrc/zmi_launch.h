@@ -14,6 +14,7 @@ struct ZmiQuantMat {
   int64_t ld_src, ld_dst;
   int32_t M, K;
   int32_t row_start;
+  int32_t frag_kpad;   // 0: dst rows are K-contiguous with stride ld_dst; > 0: dst is fragment-major with this K_pad
 };
 
 // k_prepack.hip
@@ -23,19 +24,26 @@ hipError_t zmi_launch_prepack(const int8_t *B, int64_t K, int64_t N, int64_t ldb
 
 // k_quant.hip
 hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
-                                 int8_t *dst, int64_t ld_dst, void *scales, int32_t scale_dt,
+                                 int8_t *dst, int64_t ld_dst, int64_t frag_kpad, void *scales, int32_t scale_dt,
                                  hipStream_t stream);
 hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_t total_rows,
                                   int32_t src_dt, int32_t scale_dt, hipStream_t stream);
 hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
-                                   int8_t *dst, int64_t ld_dst, float *scales, unsigned int *amax_scratch,
-                                   hipStream_t stream);
+                                   int8_t *dst, int64_t ld_dst, int64_t frag_kpad, float *scales,
+                                   unsigned int *amax_scratch, hipStream_t stream);
 
 // k_gemm.hip
 hipError_t zmi_launch_gemm_mfma(const ZmiProblem &p, const ZmiEpilogue &epi, int BM, hipStream_t stream);
 hipError_t zmi_launch_gemm_mfma_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int m_lo, int worst_items, const ZmiEpilogue &epi, int BM,
                                       hipStream_t stream);
+
+// k_ring.hip: A in fragment-major order; `top` is the largest tile height (128 or 256)
+int zmi_ring_pick_top(int64_t rows, int64_t out_cols);
+hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream);
+hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
+                                      int top, int64_t worst_rows, int worst_cols, int *counts_dev,
+                                      const ZmiEpilogue &epi, hipStream_t stream);
 
 // k_smallm.hip
 struct ZmiFusedQuant {
@@ -76,8 +84,10 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
                                   const int32_t *slot_of, const float *weights, int skip_weighted,
                                   int T, int topk, int D, int32_t dt, void *out, int64_t ldo,
                                   hipStream_t stream);
-hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int32_t *counts,
+// align: every expert's first slot is rounded up to a multiple of it (1: dense numbering)
+hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
                                 int32_t *offsets, int32_t *slot_of, hipStream_t stream);
+// A1 is fragment-major over the slot numbering, K_pad = zmi_blob_kpad(H)
 hipError_t zmi_launch_moe_quant_scatter(const void *x, int64_t ldx, int T, int H, int topk,
                                         const int32_t *slot_of, int8_t *A1, float *s1, hipStream_t stream);
 struct ZmiMoeTables {   // device arrays of E entries each
@@ -94,3 +104,6 @@ hipError_t zmi_launch_moe_build_problems(ZmiMoeTables tb, int E, int H, int I, c
 // k_util.hip
 hipError_t zmi_launch_pad_rows(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans,
                                int8_t *dst, int64_t ld_dst, hipStream_t stream);
+// u8 / s8 rows (or their transpose) -> fragment-major s8; u8 values are shifted by -128
+hipError_t zmi_launch_repack_frag(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans, int is_u8,
+                                  int8_t *dst, hipStream_t stream);
