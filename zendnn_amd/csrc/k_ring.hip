@@ -60,8 +60,9 @@ struct RingCfg {
   static constexpr int OCC = BM == 256 ? 1 : 2;
   static constexpr int NPAIR_MAX = (P + 3) / 4;
   static constexpr int RING = STAGE * NS;
-  static constexpr int EPI = 4 * R_EPI_WAVE_WORDS * 4 + BM * 4;
-  static constexpr int SMEM = RING > EPI ? RING : EPI;
+  static constexpr int EPI = 4 * R_EPI_WAVE_WORDS * 4;     // epilogue staging, reuses the ring
+  static constexpr int ROWS_OFF = RING > EPI ? RING : EPI;  // BM row scales, live during the main loop
+  static constexpr int SMEM = ROWS_OFF + BM * 4;
 };
 
 // Row blocks of one problem for a launch whose largest tile has `top` rows:
@@ -81,6 +82,52 @@ __host__ __device__ __forceinline__ int zmi_ring_items(int M, int N, int top, bo
   const int ncols = gated ? N / 2 : N;
   const int per = gated ? 128 : 256;
   return (full + (rem ? 1 : 0)) * ((ncols + per - 1) / per);
+}
+
+// Interior strips with a bf16 destination: every row and column of the strip is
+// valid and 8-byte stores are aligned, so the loop body is straight-line code.
+// GATED pairs run 0 (gate) with run 1 (up) through silu(g) * u.
+template <int EK, bool GATED>
+__device__ __forceinline__ void zmi_ring_strip_bf16(const int32_t *stage, const float *rsc, const ZmiColCtx (&cc)[2][4],
+                                                    int r4, int c16, uint16_t *dst0, int64_t ldc, int run1_off) {
+  // dst0: element (first row of the strip + r4, first column of run 0)
+  ZMI_GLOBAL uint16_t *o = zmi_global<uint16_t>(dst0);
+  const int32_t *sp = stage + r4 * R_EPI_LD + c16 * 4;
+  const float *rp = rsc + r4;
+#pragma unroll 2
+  for (int it = 0; it < 8; ++it) {
+    const v4i a0 = *(const v4i *)sp;
+    const v4i a1 = *(const v4i *)(sp + 64);
+    const float rs = *rp;
+    float y0[4], y1[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      y0[j] = __builtin_fmaf((float)(a0[j] + cc[0][j].comp) * rs, cc[0][j].wscale, cc[0][j].bias);
+      y1[j] = __builtin_fmaf((float)(a1[j] + cc[1][j].comp) * rs, cc[1][j].wscale, cc[1][j].bias);
+    }
+    if (!GATED) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { y0[j] = zmi_act_bf16<EK>(y0[j]); y1[j] = zmi_act_bf16<EK>(y1[j]); }
+      const v2u v0 = {zmi_pack_bf16(y0[0], y0[1]), zmi_pack_bf16(y0[2], y0[3])};
+      const v2u v1 = {zmi_pack_bf16(y1[0], y1[1]), zmi_pack_bf16(y1[2], y1[3])};
+      *(ZMI_GLOBAL v2u *)o = v0;
+      *(ZMI_GLOBAL v2u *)(o + run1_off) = v1;
+    } else {
+      float z[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // gate and up are rounded to bf16 first, as when the activation reads a stored GEMM result
+        const uint32_t gu = zmi_pack_bf16(y0[j], y1[j]);
+        const float g = __uint_as_float(gu << 16), u = __uint_as_float(gu & 0xffff0000u);
+        z[j] = zmi_act_bf16<ZMI_EK_SWISH>(g) * u;
+      }
+      const v2u v = {zmi_pack_bf16(z[0], z[1]), zmi_pack_bf16(z[2], z[3])};
+      *(ZMI_GLOBAL v2u *)o = v;
+    }
+    sp += 4 * R_EPI_LD;
+    rp += 4;
+    o += 4 * ldc;
+  }
 }
 
 template <int BM>
@@ -271,9 +318,53 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
 #endif
   }
 #endif
+#ifdef ZMI_RING_TRACE
+  const long long tr_t0 = wall_clock64();
+#endif
   // ---- prologue: NS-1 stages in flight, the first one landed --------------------------
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) issue_all(s);
+
+  // ---- epilogue constants, requested behind the first stages so their latency hides under the main loop:
+  // the row scales of the tile (LDS) and this lane's eight column contexts (registers)
+  float *row_scale = reinterpret_cast<float *>(smem + Cfg::ROWS_OFF);
+  for (int r = tid; r < BM; r += R_THREADS) {
+    const int m = m0 + r;
+    row_scale[r] = m < M ? zmi_row_scale(epi, p, m) : 1.0f;
+  }
+  const int hi = lane / 32, cl = lane % 32;
+  const int c16 = lane % 16, r4 = lane / 16;
+  const void *bias = p.bias;
+  const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+  const bool has_bias = bias != nullptr;
+  const int dst_dt = epi.dst_dt;
+
+  // output columns of this lane: two runs of 4
+  int n_run[2];
+  ZmiColCtx cc[2][4];
+  if (!gated) {
+    n_run[0] = tn * 256 + wn * 128 + c16 * 4;
+    n_run[1] = n_run[0] + 64;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cc[h][j] = zmi_col_ctx(epi, p, colsum, n_run[h] + j, N);
+  } else {
+    // run 0: gate columns n, run 1: the matching up columns n + N/2; output column n
+    n_run[0] = tn * 128 + wn * 64 + c16 * 4;
+    n_run[1] = n_run[0] + half;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      cc[0][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j, half);
+      cc[1][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j < half ? n_run[1] + j : N, N);
+    }
+  }
+  const int n_lim = gated ? half : N;
+  // vector stores need every row start aligned
+  const int es = dst_dt == ZMI_DT_BF16 ? 2 : (dst_dt == ZMI_DT_S8 || dst_dt == ZMI_DT_U8 ? 1 : 4);
+  const bool vec_ok = (((uintptr_t)p.dst) % 16 == 0) && ((p.ldc * es) % 16 == 0);
+  const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
+
   if (short_wave) zmi_wait_vm<(NS - 2) * (NPM - 1) * 2>();
   else zmi_wait_vm<(NS - 2) * NPM * 2>();
   zmi_wg_barrier();
@@ -302,6 +393,9 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
   zmi_wg_barrier();
 
   // ------------------------------------------------------------------------ epilogue
+#ifdef ZMI_RING_TRACE
+  const long long tr_t1 = wall_clock64();
+#endif
 #ifdef ZMI_RING_PRIO
   __builtin_amdgcn_s_setprio(0);
 #endif
@@ -309,40 +403,6 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
   if (acc[0][0][0] != 0x12345678) return;
 #endif
   int32_t *stage = reinterpret_cast<int32_t *>(smem) + wave * R_EPI_WAVE_WORDS;
-  float *row_scale = reinterpret_cast<float *>(smem) + 4 * R_EPI_WAVE_WORDS;
-  for (int r = tid; r < BM; r += R_THREADS) {
-    const int m = m0 + r;
-    row_scale[r] = m < M ? zmi_row_scale(epi, p, m) : 1.0f;
-  }
-  __syncthreads();
-
-  const int hi = lane / 32, cl = lane % 32;
-  const int c16 = lane % 16, r4 = lane / 16;
-  const void *bias = p.bias;
-  const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
-  const bool has_bias = bias != nullptr;
-  const int dst_dt = epi.dst_dt;
-
-  // output columns of this lane: two runs of 4
-  int n_run[2];
-  ZmiColCtx cc[2][4];
-  if (!gated) {
-    n_run[0] = tn * 256 + wn * 128 + c16 * 4;
-    n_run[1] = n_run[0] + 64;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) cc[h][j] = zmi_col_ctx(epi, p, colsum, n_run[h] + j, N);
-  } else {
-    // run 0: gate columns n, run 1: the matching up columns n + N/2; output column n
-    n_run[0] = tn * 128 + wn * 64 + c16 * 4;
-    n_run[1] = n_run[0] + half;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      cc[0][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j, half);
-      cc[1][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j < half ? n_run[1] + j : N, N);
-    }
-  }
   // the bf16 fast forms multiply / add unconditionally: absent scales are 1, an absent bias is -0
   if (dst_dt == ZMI_DT_BF16 && epi.fast_kind != ZMI_EK_GENERIC) {
     zmi_set_f32_flush();
@@ -352,12 +412,6 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
       for (int j = 0; j < 4; ++j)
         if (!has_bias) cc[h][j].bias = -0.0f;
   }
-  const int n_lim = gated ? half : N;
-  // vector stores need every row start aligned
-  const int es = dst_dt == ZMI_DT_BF16 ? 2 : (dst_dt == ZMI_DT_S8 || dst_dt == ZMI_DT_U8 ? 1 : 4);
-  const bool vec_ok = (((uintptr_t)p.dst) % 16 == 0) && ((p.ldc * es) % 16 == 0);
-  const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
-
   // The strips are visited by a static loop (the accumulators are registers: a
   // dynamic index would make the compiler select among all of them); the
   // arithmetic inside a strip is a rolled loop.
@@ -468,6 +522,23 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
     };
     using std::integral_constant;
     const bool bf16 = dst_dt == ZMI_DT_BF16;
+    // interior strip: all 32 rows and all columns of the tile valid, aligned rows
+    const bool interior = bf16 && vec_ok && epi.fast_kind != ZMI_EK_GENERIC && mbase + 32 <= M &&
+                          (gated ? (tn + 1) * 128 <= half && epi.gated_act == ZMI_ACT_SILU_AND_MUL && epi.fast_kind == ZMI_EK_NONE
+                                 : (tn + 1) * 256 <= N);
+    if (interior) {
+      uint16_t *d0 = (uint16_t *)p.dst + (int64_t)(mbase + r4) * p.ldc + n_run[0];
+      if (gated) zmi_ring_strip_bf16<ZMI_EK_NONE, true>(stage, rsc, cc, r4, c16, d0, p.ldc, 0);
+      else switch (epi.fast_kind) {
+        case ZMI_EK_SWISH: zmi_ring_strip_bf16<ZMI_EK_SWISH, false>(stage, rsc, cc, r4, c16, d0, p.ldc, 64); break;
+        case ZMI_EK_GELU_TANH: zmi_ring_strip_bf16<ZMI_EK_GELU_TANH, false>(stage, rsc, cc, r4, c16, d0, p.ldc, 64); break;
+        case ZMI_EK_RELU: zmi_ring_strip_bf16<ZMI_EK_RELU, false>(stage, rsc, cc, r4, c16, d0, p.ldc, 64); break;
+        default: zmi_ring_strip_bf16<ZMI_EK_NONE, false>(stage, rsc, cc, r4, c16, d0, p.ldc, 64); break;
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      return;
+    }
     const bool fast_ok = epi.fast_kind != ZMI_EK_GENERIC && (bf16 || dst_dt == ZMI_DT_F32);
     // the gated form applies no element-wise post-op of its own before the activation
     const int kind = fast_ok ? (gated && epi.fast_kind != ZMI_EK_NONE ? -1 : epi.fast_kind * 2 + (bf16 ? 1 : 0)) : -1;
@@ -529,6 +600,14 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
     do_strip(std::integral_constant<int, 2>{});
     do_strip(std::integral_constant<int, 3>{});
   }
+#ifdef ZMI_RING_TRACE
+  if (tid == 0) {
+    extern __device__ long long zmi_ring_trace[];
+    long long *t = zmi_ring_trace + (size_t)blockIdx.x * 4;
+    t[0] = ((long long)__builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11)) & 0xffffffffll) | ((long long)__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) << 32);
+    t[1] = tr_t0; t[2] = tr_t1; t[3] = wall_clock64();
+  }
+#endif
 }
 
 // Tile counts of a problem table for the three tile heights, computed where the row counts live.
