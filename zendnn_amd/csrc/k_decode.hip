@@ -15,12 +15,21 @@
 //     memory instead touches 16 different rows per load and costs ~2 us of the
 //     ~13 us launch;
 //   * the per-column / per-row epilogue constants are fetched before anything
-//     else, so the tail after the last weight byte is LDS-only.
+//     else, so the tail after the last weight byte is LDS-only;
+//   * optionally the per-token quantization of the M source rows is part of the
+//     launch: M extra workgroups at the head of the grid quantize one row each and publish it, every
+//     workgroup puts the first half of its weight stream in flight, waits for the
+//     rows (the wait is bounded, producers wait for nothing and are dispatched
+//     first), then requests the rows and the second half of the stream.
 #include "zmi_device.h"
+#include "zmi_fused_quant.h"
 #include "zmi_launch.h"
 
 #define DEC_WAVES 8
 #define DEC_THREADS (DEC_WAVES * 64)
+#ifndef DEC_FQ_FIRST
+#define DEC_FQ_FIRST 6   // chunks of the slice requested before the wait for the quantized rows (measured best of 2, 4, 6, 8)
+#endif
 #define DEC_RED_BYTES (DEC_WAVES * 2 * 4 * 64 * 4)   // 16 KiB of partial tiles
 
 // Byte offset in LDS of the 16-byte operand granule of chunk cc (64 k), k group g
@@ -32,7 +41,8 @@ __device__ __forceinline__ int dec_lds_off(int cc, int g, int r) {
   return cc * 1024 + ((g * 16 + (r ^ ((g * 4 + (cc & 3)) & 15))) << 4);
 }
 
-__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProblem p, ZmiEpilogue epi) {
+__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProblem p, ZmiEpilogue epi,
+                                                                        ZmiFusedQuant fq) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);   // scalar: slice bounds and addresses stay in SGPRs
@@ -40,7 +50,16 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
   const int K_pad = (int)zmi_blob_kpad(K);
   const int nchunks = K_pad / 64;
   const bool gated = epi.gated_act != 0;
-  const int blk = blockIdx.x;
+  // With fused quantization the first M workgroups only quantize one source row each,
+  // publish it and leave; the streaming workgroups follow them in dispatch order.
+  if (fq.x && (int)blockIdx.x < M) {
+    zmi_fused_quant_row(fq, blockIdx.x, K, reinterpret_cast<float *>(lds));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
+    __syncthreads();
+    if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
+    return;
+  }
+  const int blk = fq.x ? (int)blockIdx.x - M : (int)blockIdx.x;
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
 
@@ -65,13 +84,13 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
   ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_live ? e_n : N, N);
   ZmiColCtx cc1 = cc0;
   if (gated) cc1 = zmi_col_ctx(epi, p, colsum, e_live ? e_n + N / 2 : N, N);
-  const float rs = zmi_row_scale(epi, p, e_live ? e_row : 0);
+  // (with fused quantization the row scales exist only after the wait below)
+  float rs = fq.x ? 1.0f : zmi_row_scale(epi, p, e_live ? e_row : 0);
 
-  // ---- activation loads (row-contiguous), before the weight stream ----
-  // 64 items (row, 1 KiB segment); wavefront w takes rows w and w + 8.
+  // ---- activation loads (row-contiguous): 64 items (row, 1 KiB segment); wavefront w takes rows w and w + 8 ----
   const int c16 = lane % 16, g = lane / 16;
   v4i araw[2][4];
-  {
+  auto load_rows = [&]() {
     const int8_t *A = (const int8_t *)p.A;
     const int G = ((K + 15) & ~15) / 16;   // readable 16-byte granules per row
     #pragma unroll
@@ -83,7 +102,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
         if (row < M && gran < G) v = *(const v4i *)(A + (int64_t)row * p.lda + gran * 16);
         araw[i][s] = v;
       }
-  }
+  };
 
   // ---- weight stream: this wavefront's slice of K, at most 8 chunks of 64 ----
   const int c_begin = wave * nchunks / DEC_WAVES;
@@ -102,8 +121,29 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
     b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)c * 2048);
     b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)c * 2048);
   };
-  #pragma unroll
-  for (int u = 0; u < 8; ++u) load_b(u);
+
+  if (!fq.x) {
+    // rows first, so they return first; then the whole slice
+    load_rows();
+    #pragma unroll
+    for (int u = 0; u < 8; ++u) load_b(u);
+  } else {
+    #pragma unroll
+    for (int u = 0; u < DEC_FQ_FIRST; ++u) load_b(u);
+    if (tid == 0) {
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        const unsigned int v = __hip_atomic_load(fq.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((int)(v - fq.target) >= 0) break;
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    __syncthreads();
+    asm volatile("" ::: "memory");   // the loads below stay below the wait
+    rs = zmi_row_scale(epi, p, e_live ? e_row : 0);
+    load_rows();
+    #pragma unroll
+    for (int u = DEC_FQ_FIRST; u < 8; ++u) load_b(u);
+  }
 
   // ---- rows -> LDS in operand order ----
   {
@@ -193,11 +233,16 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
   }
 }
 
+int zmi_decode_grid(const ZmiProblem &p, bool gated) {
+  return gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
+}
+
 bool zmi_decode_kernel_fits(const ZmiProblem &p) {
   return p.M > 0 && p.M <= 16 && zmi_blob_kpad(p.K) <= 4096;
 }
 
-hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
+hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
+                                  hipStream_t stream) {
   if (!zmi_decode_kernel_fits(p)) return hipErrorInvalidValue;
   const bool gated = epi.gated_act != 0;
   const int grid = gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
@@ -211,6 +256,8 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, h
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  hipLaunchKernelGGL(zmi_gemm_decode_kernel, dim3(grid), dim3(DEC_THREADS), smem, stream, p, epi);
+  ZmiFusedQuant none = {};
+  hipLaunchKernelGGL(zmi_gemm_decode_kernel, dim3(grid + (fq ? p.M : 0)), dim3(DEC_THREADS), smem, stream, p, epi,
+                     fq ? *fq : none);
   return hipGetLastError();
 }

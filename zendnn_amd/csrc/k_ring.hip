@@ -67,12 +67,18 @@ struct RingCfg {
 
 // Row blocks of one problem for a launch whose largest tile has `top` rows:
 // floor(M / top) full blocks (handled by the BM == top kernel) and one remainder
-// block handled by the smallest of {64, 128, 256} that holds it.
+// block handled by the smallest of {64, 128, 256} that holds it.  `top` may carry
+// ZMI_RING_PAD: the remainder then stays with the BM == top kernel as a partly
+// filled block, so that the weights of a problem are streamed by one launch only
+// (the choice when the launch is bound by weight traffic, not by MFMA work).
+#define ZMI_RING_PAD 0x10000
 template <int BM>
-__device__ __host__ __forceinline__ void zmi_ring_rows(int M, int top, int &full, bool &has_rem) {
+__device__ __host__ __forceinline__ void zmi_ring_rows(int M, int top_flags, int &full, bool &has_rem) {
+  const int top = top_flags & 0xffff;
   full = BM == top ? M / top : 0;
   const int r = M % top;
-  has_rem = r > 0 && r <= BM && (BM == 64 || r > BM / 2);
+  if (top_flags & ZMI_RING_PAD) has_rem = BM == top && r > 0;
+  else has_rem = r > 0 && r <= BM && (BM == 64 || r > BM / 2);
 }
 
 template <int BM>
@@ -134,13 +140,14 @@ template <int BM>
 __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_kernel(ZmiProblem p0,
                                                                                    const ZmiProblem *probs,
                                                                                    int n_prob, int n_items,
-                                                                                   const int *n_items_dev, int top,
+                                                                                   const int *n_items_dev, int top_flags,
                                                                                    ZmiEpilogue epi) {
   using Cfg = RingCfg<BM>;
   constexpr int MI = BM / 64, NI = 4;
   constexpr int AF = Cfg::AF, STAGE = Cfg::STAGE, NS = Cfg::NS, NPM = Cfg::NPAIR_MAX;
   char *smem = zmi_ring_smem;
 
+  const int top = top_flags & 0xffff;
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int wm = wave / 2, wn = wave % 2;
@@ -163,7 +170,7 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
     if (!probs) {
       p = p0;
       int full; bool rem;
-      zmi_ring_rows<BM>(p.M, top, full, rem);
+      zmi_ring_rows<BM>(p.M, top_flags, full, rem);
       const int tiles_m = full + (rem ? 1 : 0);
       const int ncols = gated ? p.N / 2 : p.N;
       const int tiles_n = (ncols + per - 1) / per;
@@ -184,7 +191,7 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
         const int M = probs[e].M;
         if (M <= 0) continue;
         int full; bool rem;
-        zmi_ring_rows<BM>(M, top, full, rem);
+        zmi_ring_rows<BM>(M, top_flags, full, rem);
         const int tiles_m = full + (rem ? 1 : 0);
         if (!tiles_m) continue;
         const int ncols = gated ? probs[e].N / 2 : probs[e].N;
@@ -611,17 +618,23 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
 }
 
 // Tile counts of a problem table for the three tile heights, computed where the row counts live.
-__global__ void zmi_ring_count_kernel(const ZmiProblem *probs, int n_prob, int top, int gated, int *out) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+__global__ __launch_bounds__(64) void zmi_ring_count_kernel(const ZmiProblem *probs, int n_prob, int top, int gated,
+                                                             int *out) {
   int c256 = 0, c128 = 0, c64 = 0;
-  for (int e = 0; e < n_prob; ++e) {
+  for (int e = threadIdx.x; e < n_prob; e += 64) {
     const int M = probs[e].M, N = probs[e].N;
     if (M <= 0) continue;
-    if (top == 256) c256 += zmi_ring_items<256>(M, N, top, gated != 0);
+    if ((top & 0xffff) == 256) c256 += zmi_ring_items<256>(M, N, top, gated != 0);
     c128 += zmi_ring_items<128>(M, N, top, gated != 0);
     c64 += zmi_ring_items<64>(M, N, top, gated != 0);
   }
-  out[0] = c256; out[1] = c128; out[2] = c64;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    c256 += __shfl_xor(c256, o);
+    c128 += __shfl_xor(c128, o);
+    c64 += __shfl_xor(c64, o);
+  }
+  if (threadIdx.x == 0) { out[0] = c256; out[1] = c128; out[2] = c64; }
 }
 
 template <int BM>
@@ -649,12 +662,25 @@ int zmi_ring_pick_top(int64_t rows, int64_t out_cols) {
   return t256 >= 192 ? 256 : 128;
 }
 
+// Grouped launches (n_prob problems, rows / n_prob rows each on average): every
+// problem is covered by one launch whose tile height fits the typical problem
+// (ZMI_RING_PAD), so its weights are streamed once and the launch count stays at
+// one.  Measured on MI355X on 8 x ~128-row and 64 x 0..3900-row expert sets, the
+// 128-row tile (two workgroups per CU, one's epilogue under the other's main
+// loop) beats both the 256-row tile and full tiles plus right-sized remainders.
+int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated) {
+  (void)K; (void)N; (void)gated;
+  if (n_prob <= 0 || rows <= 0) return 128 | ZMI_RING_PAD;
+  const int64_t avg = (rows + n_prob - 1) / n_prob;
+  return (avg <= 64 ? 64 : 128) | ZMI_RING_PAD;
+}
+
 // One problem, M rows in fragment-major order at p.A.
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream) {
   if (p.M <= 0) return hipSuccess;
   const bool gated = epi.gated_act != 0;
   hipError_t e = hipSuccess;
-  if (top == 256) {
+  if ((top & 0xffff) == 256) {
     e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), nullptr, top, epi, stream);
     if (e != hipSuccess) return e;
   }
@@ -676,7 +702,7 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
     for (int e = 0; e < n_prob; ++e) {
       const ZmiProblem &q = probs_host[e];
       if (q.M <= 0) continue;
-      items[0] += top == 256 ? zmi_ring_items<256>(q.M, q.N, top, gated) : 0;
+      items[0] += (top & 0xffff) == 256 ? zmi_ring_items<256>(q.M, q.N, top, gated) : 0;
       items[1] += zmi_ring_items<128>(q.M, q.N, top, gated);
       items[2] += zmi_ring_items<64>(q.M, q.N, top, gated);
     }
@@ -685,9 +711,12 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
     const int ncols = gated ? worst_cols / 2 : worst_cols;
     const int tiles_n = (ncols + per - 1) / per;
     // at most rows/top full blocks in total and one remainder block per problem
-    items[top == 256 ? 0 : 1] = (int)(worst_rows / top + n_prob) * tiles_n;
-    if (top == 256) items[1] = n_prob * tiles_n;
-    items[2] = n_prob * tiles_n;
+    const int th = top & 0xffff;
+    items[th == 256 ? 0 : (th == 128 ? 1 : 2)] = (int)(worst_rows / th + n_prob) * tiles_n;
+    if (!(top & ZMI_RING_PAD)) {
+      if (th == 256) items[1] = n_prob * tiles_n;
+      if (th >= 128) items[2] = n_prob * tiles_n;
+    }
     if (!counts_dev) return hipErrorInvalidValue;
     hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0,
                        counts_dev);
@@ -695,7 +724,7 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
   const int *cd = probs_host ? nullptr : counts_dev;
   ZmiProblem dummy = {};
   hipError_t e = hipSuccess;
-  if (top == 256) {
+  if ((top & 0xffff) == 256) {
     e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], cd, top, epi, stream);
     if (e != hipSuccess) return e;
   }

@@ -236,7 +236,7 @@ static int pick_top(int M, int N) {
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi) {
   if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
     set_kernel_name("decode_lds_rows_mfma16x16x64");
-    if (!hip_ok(zmi_launch_gemm_decode(prob, epi, stream()), "decode GEMM launch")) return ZMI_FAILURE;
+    if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
   } else if (!use_ring_kernel(prob.M)) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
@@ -383,7 +383,8 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     const bool per_token = (dyn_scale_n == M && M > 1) || M == 1;
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
     const bool decode_kernel = M <= 16 && zmi_blob_kpad(K) <= 4096 && !std::getenv("ZMI_NO_DECODE_KERNEL");
-    if (per_token && !decode_kernel && !ring && M <= 128 && K % 4 == 0 && zmi_smallm_grid(prob, false) <= 512 &&
+    // (the decode kernel's producers are its first workgroups and wait for nothing, so its grid need not be resident)
+    if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob, false) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
       if (!ctr) return ZMI_FAILURE;
@@ -437,8 +438,13 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (use_fused) {
     // a one-row scale in device memory reads like a per-token scale
     if (epi.src_scale_mode == ZMI_SS_TENSOR_PTR) epi.src_scale_mode = ZMI_SS_TOKEN_PTR;
-    set_kernel_name("smallm_splitk_mfma16x16x64 (fused per-token quant)");
-    st = hip_ok(zmi_launch_gemm_smallm_fused(prob, epi, fused, stream()), "fused small-M GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+    if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
+      set_kernel_name("decode_lds_rows_mfma16x16x64 (fused per-token quant)");
+      st = hip_ok(zmi_launch_gemm_decode(prob, epi, &fused, stream()), "fused decode GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+    } else {
+      set_kernel_name("smallm_splitk_mfma16x16x64 (fused per-token quant)");
+      st = hip_ok(zmi_launch_gemm_smallm_fused(prob, epi, fused, stream()), "fused small-M GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+    }
   } else {
     st = run_single_gemm(prob, epi);
   }

@@ -225,9 +225,9 @@ struct Stage {
   ZmiEpilogue epi;
 };
 
-int group_top(int64_t rows, int64_t out_cols) {
-  if (const char *env = std::getenv("ZMI_GROUP_TOP")) { int v = std::atoi(env); if (v == 128 || v == 256) return v; }
-  return zmi_ring_pick_top(rows, out_cols);
+int group_top(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated) {
+  if (const char *env = std::getenv("ZMI_GROUP_TOP")) { int v = std::atoi(env); if (v > 0) return v; }
+  return zmi_ring_pick_top_group(rows, n_prob, K, N, gated);
 }
 
 // Every expert's activations are fragment-major; one launch per tile height.
@@ -237,9 +237,9 @@ int32_t launch_stage(const Stage &st, const char *what) {
   if (!dev) return ZMI_FAILURE;
   const int n = (int)st.probs.size();
   int64_t rows = 0;
-  int cols = 0;
-  for (const ZmiProblem &q : st.probs) { rows += q.M; cols = std::max(cols, (int)q.N); }
-  const int top = group_top(rows, st.epi.gated_act ? cols / 2 : cols);
+  int cols = 0, kmax = 0;
+  for (const ZmiProblem &q : st.probs) { rows += q.M; cols = std::max(cols, (int)q.N); kmax = std::max(kmax, (int)q.K); }
+  const int top = group_top(rows, n, kmax, cols, st.epi.gated_act != 0);
   if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, nullptr, st.epi, stream()), what)) return ZMI_FAILURE;
   return ZMI_SUCCESS;
 }
@@ -637,7 +637,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
   // row counts live on the device: the grids are sized for the worst case
-  const int top1 = group_top(R, I), top2 = group_top(R, H);
+  const int top1 = group_top(R, E, H, 2 * I, true), top2 = group_top(R, E, I, H, false);
   if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_counts, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;

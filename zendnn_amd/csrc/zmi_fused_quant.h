@@ -1,0 +1,158 @@
+// Per-token quantization of one source row by a whole workgroup, used by the
+// small-M kernels that fuse the quantization into the GEMM launch: the
+// workgroups with the lowest indices quantize one row each, publish it with a
+// device-scope counter, and every workgroup waits for the counter before it
+// reads the s8 rows (same arithmetic as k_quant.hip).
+#pragma once
+#include "zmi_device.h"
+#include "zmi_launch.h"
+
+__device__ __forceinline__ int8_t zmi_sq_quant(float v, float scale) {
+  if ((__float_as_uint(v) & 0x7f800000u) == 0x7f800000u) return 0;
+  return (int8_t)(int32_t)rintf(__fdiv_rn(v, scale));
+}
+
+// Quantizes one source row with the whole workgroup.  The s8 row and its scale
+// are written with device-scope (write-through) stores: the eight XCDs have
+// private, mutually non-coherent L2s, and a full release / acquire fence pair
+// would write back and invalidate whole caches in the middle of the weight
+// stream.  Readers on other XCDs miss in their own L2 (invalidated when the
+// kernel started) and fetch the fresh bytes.
+static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int K, float *red) {
+  const int t = threadIdx.x, nt = blockDim.x;
+  const bool bf16 = fq.x_dt == ZMI_DT_BF16;
+  const char *src = (const char *)fq.x + (size_t)row * fq.ldx * (bf16 ? 2 : 4);
+  auto ld = [&](int k) { return bf16 ? zmi_bf16_to_f32(((const uint16_t *)src)[k]) : ((const float *)src)[k]; };
+  // one 16-byte chunk (8 bf16) per thread held in registers when the row fits
+  const bool vec = bf16 && K % 8 == 0 && K <= nt * 8 && ((uintptr_t)src % 16) == 0;
+  float v8[8];
+  float amax = 0.0f;
+  if (vec) {
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) v8[j] = 0.0f;
+    if (t * 8 < K) {
+      const v4i raw = *(const v4i *)((const uint16_t *)src + t * 8);
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v8[2 * j] = __uint_as_float(((uint32_t)raw[j]) << 16);
+        v8[2 * j + 1] = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+      }
+    }
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = fabsf(v8[j]);
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+  } else {
+    for (int k = t; k < K; k += nt) {
+      const float a = fabsf(ld(k));
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+  }
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (t % 64 == 0) red[t / 64] = amax;
+  __syncthreads();
+  amax = red[0];
+  for (int i = 1; i < nt / 64; ++i) amax = fmaxf(amax, red[i]);
+  __syncthreads();
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  if (t == 0) {
+    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (fq.user_scales) {
+      if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[row] = zmi_f32_to_bf16_rne(s);
+      else ((float *)fq.user_scales)[row] = s;
+    }
+  }
+  unsigned int *dst = (unsigned int *)(fq.q + (size_t)row * fq.ldq);
+  if (vec) {
+    if (t * 8 < K) {
+      #pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        unsigned int w = 0;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(v8[h * 4 + j], s)) << (8 * j);
+        __hip_atomic_store(&dst[t * 2 + h], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    return;
+  }
+  for (int k4 = t; k4 < K / 4; k4 += nt) {
+    unsigned int w = 0;
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(ld(k4 * 4 + j), s)) << (8 * j);
+    __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+
+// The same by a single wavefront (no workgroup barrier), for kernels whose other
+// wavefronts must not wait for the quantization: two passes over the row, the
+// second one re-reads it from L2.  K must be a multiple of 4.
+static __device__ void zmi_fused_quant_row_wave(const ZmiFusedQuant &fq, int row, int K) {
+  const int lane = threadIdx.x % 64;
+  const bool bf16 = fq.x_dt == ZMI_DT_BF16;
+  const char *src = (const char *)fq.x + (size_t)row * fq.ldx * (bf16 ? 2 : 4);
+  const bool vec = bf16 && K % 8 == 0 && ((uintptr_t)src % 16) == 0;
+  auto ld = [&](int k) { return bf16 ? zmi_bf16_to_f32(((const uint16_t *)src)[k]) : ((const float *)src)[k]; };
+  auto ld8 = [&](int k, float (&v)[8]) {
+    const v4i raw = *(const v4i *)((const uint16_t *)src + k);
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[2 * j] = __uint_as_float(((uint32_t)raw[j]) << 16);
+      v[2 * j + 1] = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+    }
+  };
+  float amax = 0.0f;
+  if (vec) {
+    for (int k = lane * 8; k < K; k += 512) {
+      float v[8];
+      ld8(k, v);
+      #pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float a = fabsf(v[j]);
+        if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+      }
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) {
+      const float a = fabsf(ld(k));
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+  }
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  if (lane == 0) {
+    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (fq.user_scales) {
+      if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[row] = zmi_f32_to_bf16_rne(s);
+      else ((float *)fq.user_scales)[row] = s;
+    }
+  }
+  unsigned int *dst = (unsigned int *)(fq.q + (size_t)row * fq.ldq);
+  if (vec) {
+    for (int k = lane * 8; k < K; k += 512) {
+      float v[8];
+      ld8(k, v);
+      #pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        unsigned int w = 0;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(v[h * 4 + j], s)) << (8 * j);
+        __hip_atomic_store(&dst[k / 4 + h], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    return;
+  }
+  for (int k4 = lane; k4 < K / 4; k4 += 64) {
+    unsigned int w = 0;
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(ld(k4 * 4 + j), s)) << (8 * j);
+    __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}

@@ -40,6 +40,7 @@ hipError_t zmi_launch_gemm_mfma_group(const ZmiProblem *probs_host, const ZmiPro
 
 // k_ring.hip: A in fragment-major order; `top` is the largest tile height (128 or 256)
 int zmi_ring_pick_top(int64_t rows, int64_t out_cols);
+int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated);
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *counts_dev,
@@ -69,7 +70,10 @@ hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiP
 
 // k_decode.hip: single problem, M <= 16, K_pad <= 4096
 bool zmi_decode_kernel_fits(const ZmiProblem &p);
-hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+// fq != null: the launch also quantizes the M source rows (its grid must be resident at once)
+hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
+                                  hipStream_t stream);
+int zmi_decode_grid(const ZmiProblem &p, bool gated);
 
 // k_moe.hip
 struct ZmiActMat {
