@@ -32,6 +32,9 @@
 #include "zmi_device.h"
 #include "zmi_launch.h"
 
+#ifndef ZMI_RING_EPI_UNROLL
+#define ZMI_RING_EPI_UNROLL 2
+#endif
 #define R_THREADS 256
 #define R_BN 256
 #define R_EPI_LD 132                       // words per staged row (128 + 4: rows 4 banks apart)
@@ -100,7 +103,7 @@ __device__ __forceinline__ void zmi_ring_strip_bf16(const int32_t *stage, const 
   ZMI_GLOBAL uint16_t *o = zmi_global<uint16_t>(dst0);
   const int32_t *sp = stage + r4 * R_EPI_LD + c16 * 4;
   const float *rp = rsc + r4;
-#pragma unroll 2
+#pragma unroll ZMI_RING_EPI_UNROLL
   for (int it = 0; it < 8; ++it) {
     const v4i a0 = *(const v4i *)sp;
     const v4i a1 = *(const v4i *)(sp + 64);

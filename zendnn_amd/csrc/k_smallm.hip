@@ -305,27 +305,3 @@ hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &
   return dispatch_small(p, nullptr, 1, 0, p.M, small_blocks(p, epi.gated_act != 0), zmi_blob_kpad(p.K), epi,
                         fq, stream);
 }
-
-// Runs every problem with m_lo < M <= m_hi (m_hi <= 128).  probs_host sizes
-// the grid; when it is null the grid is worst_grid (K_pad taken from kpad_hint)
-// and surplus workgroups exit at once.
-hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev,
-                                        int n_prob, int m_lo, int m_hi, int worst_grid, int64_t kpad_hint,
-                                        const ZmiEpilogue &epi, hipStream_t stream) {
-  int grid = worst_grid;
-  int64_t kpad_max = kpad_hint;
-  if (probs_host) {
-    grid = 0;
-    kpad_max = 0;
-    for (int e = 0; e < n_prob; ++e) {
-      if (probs_host[e].M > m_lo && probs_host[e].M <= m_hi) {
-        grid += small_blocks(probs_host[e], epi.gated_act != 0);
-        const int64_t kp = zmi_blob_kpad(probs_host[e].K);
-        if (kp > kpad_max) kpad_max = kp;
-      }
-    }
-  }
-  ZmiProblem dummy = {};
-  ZmiFusedQuant none = {};
-  return dispatch_small(dummy, probs_dev, n_prob, m_lo, m_hi, grid, kpad_max, epi, none, stream);
-}

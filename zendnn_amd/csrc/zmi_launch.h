@@ -32,12 +32,6 @@ hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, i
                                    int8_t *dst, int64_t ld_dst, int64_t frag_kpad, float *scales,
                                    unsigned int *amax_scratch, hipStream_t stream);
 
-// k_gemm.hip
-hipError_t zmi_launch_gemm_mfma(const ZmiProblem &p, const ZmiEpilogue &epi, int BM, hipStream_t stream);
-hipError_t zmi_launch_gemm_mfma_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
-                                      int m_lo, int worst_items, const ZmiEpilogue &epi, int BM,
-                                      hipStream_t stream);
-
 // k_ring.hip: A in fragment-major order; `top` is the largest tile height (128 or 256)
 int zmi_ring_pick_top(int64_t rows, int64_t out_cols);
 int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated);
@@ -64,9 +58,6 @@ int zmi_smallm_grid(const ZmiProblem &p, bool gated);
 hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
                                         hipStream_t stream);
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
-hipError_t zmi_launch_gemm_smallm_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev,
-                                        int n_prob, int m_lo, int m_hi, int worst_grid, int64_t kpad_hint,
-                                        const ZmiEpilogue &epi, hipStream_t stream);
 
 // k_decode.hip: single problem, M <= 16, K_pad <= 4096
 bool zmi_decode_kernel_fits(const ZmiProblem &p);
