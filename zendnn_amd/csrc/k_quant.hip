@@ -140,6 +140,160 @@ __global__ __launch_bounds__(QT_THREADS) void zmi_quant_rows_kernel(ZmiQuantMat 
   zmi_quant_row<BF16>(src, dst, r, m.frag_kpad, sc, scale_dt, m.K, red);
 }
 
+#define FR_THREADS 512
+// Fragment-major destination, K a multiple of 16, 16-byte aligned rows: one
+// workgroup per 8 rows.  Thread (r = t % 8, q = t / 8) owns the 16 consecutive k
+// starting at 16 q + 1024 step, i.e. exactly one 16-byte chunk of the fragment
+// layout, and the 8 threads of one q write 8 consecutive chunks (128 bytes).
+// The rows are read twice (absmax, then quantize); the second read hits L2.
+template <bool BF16>
+__global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat mat0, const ZmiQuantMat *mats, int n_mat,
+                                                              int scale_dt) {
+  __shared__ float red[FR_THREADS / 64][8];
+  const int t = threadIdx.x, r8 = t % 8, q = t / 8;
+  const int grp = blockIdx.x;                 // group of 8 rows in the launch's numbering
+  ZmiQuantMat m = mat0;
+  if (mats) {
+    int lo = 0, hi = n_mat - 1;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) / 2;
+      if (mats[mid].row_start <= grp * 8) lo = mid; else hi = mid - 1;
+    }
+    m = mats[lo];
+  }
+  // row_start of every matrix is a multiple of 8 in this launch form
+  const int r = grp * 8 - m.row_start + r8;
+  const bool live = r < m.M;
+  const int K = m.K;
+  const size_t es = BF16 ? 2 : 4;
+  const char *src = (const char *)m.src + (size_t)(live ? r : 0) * m.ld_src * es;
+  // raw 32-byte (bf16) / 64-byte (f32) pieces -> 16 floats
+  auto load_raw = [&](int k, v4i (&w)[4]) {
+    if (BF16) {
+      w[0] = *(const v4i *)(src + (size_t)k * 2);
+      w[1] = *(const v4i *)(src + (size_t)k * 2 + 16);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = *(const v4i *)(src + (size_t)k * 4 + j * 16);
+    }
+  };
+  auto unpack = [&](const v4i (&w)[4], float (&v)[16]) {
+    if (BF16) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[8 * h + 2 * j] = __uint_as_float(((uint32_t)w[h][j]) << 16);
+          v[8 * h + 2 * j + 1] = __uint_as_float(((uint32_t)w[h][j]) & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) v[4 * j + b] = __int_as_float(w[j][b]);
+    }
+  };
+  auto absmax16 = [&](const float (&v)[16], float amax) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float a = fabsf(v[j]);
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+    return amax;
+  };
+  auto quant_store = [&](const float (&v)[16], float s, int k) {
+    v4i o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t w = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) w |= ((uint32_t)(uint8_t)zmi_quant_one(v[4 * j + b], s)) << (8 * b);
+      o[j] = (int)w;
+    }
+    *(v4i *)(m.dst + zmi_afrag_off(r, k, m.frag_kpad)) = o;
+  };
+  // rows of up to FR_STEPS * FR_THREADS * 2 elements stay in registers between the two passes
+  // (bf16 only: 8 registers per step); longer rows are read twice, the second time from L2
+  constexpr int FR_STEPS = 8;
+  const bool in_regs = BF16 && K <= FR_STEPS * FR_THREADS * 2;
+  v4i keep[FR_STEPS][2];
+  float amax = 0.0f;
+  if (live) {
+    if (in_regs) {
+#pragma unroll
+      for (int st = 0; st < FR_STEPS; ++st) {
+        const int k = q * 16 + st * (FR_THREADS * 2);
+        if (k < K) {
+          keep[st][0] = *(const v4i *)(src + (size_t)k * 2);
+          keep[st][1] = *(const v4i *)(src + (size_t)k * 2 + 16);
+        }
+      }
+#pragma unroll
+      for (int st = 0; st < FR_STEPS; ++st) {
+        const int k = q * 16 + st * (FR_THREADS * 2);
+        if (k < K) {
+          v4i w[4] = {keep[st][0], keep[st][1], keep[st][0], keep[st][1]};
+          float v[16];
+          unpack(w, v);
+          amax = absmax16(v, amax);
+        }
+      }
+    } else {
+      for (int k = q * 16; k < K; k += FR_THREADS * 2) {
+        v4i w[4];
+        float v[16];
+        load_raw(k, w);
+        unpack(w, v);
+        amax = absmax16(v, amax);
+      }
+    }
+  }
+  // the threads of one row inside a wavefront are 8 lanes apart
+  amax = fmaxf(amax, __shfl_xor(amax, 8));
+  amax = fmaxf(amax, __shfl_xor(amax, 16));
+  amax = fmaxf(amax, __shfl_xor(amax, 32));
+  if (t % 64 < 8) red[t / 64][r8] = amax;
+  __syncthreads();
+  amax = red[0][r8];
+#pragma unroll
+  for (int w = 1; w < FR_THREADS / 64; ++w) amax = fmaxf(amax, red[w][r8]);
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  if (!live) return;
+  if (q == 0) {
+    void *sc = (char *)m.scale + (size_t)r * (scale_dt == ZMI_DT_BF16 ? 2 : 4);
+    if (scale_dt == ZMI_DT_BF16) *(uint16_t *)sc = zmi_f32_to_bf16_rne(s);
+    else *(float *)sc = s;
+  }
+  if (!m.dst) return;
+  if (in_regs) {
+#pragma unroll
+    for (int st = 0; st < FR_STEPS; ++st) {
+      const int k = q * 16 + st * (FR_THREADS * 2);
+      if (k < K) {
+        v4i w[4] = {keep[st][0], keep[st][1], keep[st][0], keep[st][1]};
+        float v[16];
+        unpack(w, v);
+        quant_store(v, s, k);
+      }
+    }
+  } else {
+    for (int k = q * 16; k < K; k += FR_THREADS * 2) {
+      v4i w[4];
+      float v[16];
+      load_raw(k, w);
+      unpack(w, v);
+      quant_store(v, s, k);
+    }
+  }
+}
+
+static bool zmi_quant_frag8_ok(const void *src, int64_t K, int64_t ld_src, int32_t src_dt) {
+  const int64_t es = src_dt == ZMI_DT_BF16 ? 2 : 4;
+  return K % 16 == 0 && ((uintptr_t)src) % 16 == 0 && (ld_src * es) % 16 == 0;
+}
+
 hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
                                  int8_t *dst, int64_t ld_dst, int64_t frag_kpad, void *scales, int32_t scale_dt,
                                  hipStream_t stream) {
@@ -147,6 +301,14 @@ hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int
   ZmiQuantMat m;
   m.src = src; m.dst = dst; m.scale = scales; m.ld_src = ld_src; m.ld_dst = ld_dst;
   m.M = (int32_t)M; m.K = (int32_t)K; m.row_start = 0; m.frag_kpad = (int32_t)frag_kpad;
+  if (frag_kpad && zmi_quant_frag8_ok(src, K, ld_src, src_dt)) {
+    const unsigned grid = (unsigned)((M + 7) / 8);
+    if (src_dt == ZMI_DT_BF16)
+      hipLaunchKernelGGL(zmi_quant_frag8_kernel<true>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, scale_dt);
+    else
+      hipLaunchKernelGGL(zmi_quant_frag8_kernel<false>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, scale_dt);
+    return hipGetLastError();
+  }
   if (src_dt == ZMI_DT_BF16)
     hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, m,
                        (const ZmiQuantMat *)nullptr, 1, scale_dt);
@@ -156,10 +318,23 @@ hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int
   return hipGetLastError();
 }
 
+bool zmi_quant_mat_frag8_ok(const ZmiQuantMat &m, int32_t src_dt) {
+  return m.frag_kpad > 0 && zmi_quant_frag8_ok(m.src, m.K, m.ld_src, src_dt);
+}
+
 hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_t total_rows,
-                                  int32_t src_dt, int32_t scale_dt, hipStream_t stream) {
+                                  int32_t src_dt, int32_t scale_dt, int rows8, hipStream_t stream) {
   if (total_rows <= 0) return hipSuccess;
   ZmiQuantMat m0 = {};
+  if (rows8) {
+    // every matrix is fragment-major, eligible for the 8-row kernel, and starts at a multiple of 8 rows
+    const unsigned grid = (unsigned)((total_rows + 7) / 8);
+    if (src_dt == ZMI_DT_BF16)
+      hipLaunchKernelGGL(zmi_quant_frag8_kernel<true>, dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats_dev, n_mat, scale_dt);
+    else
+      hipLaunchKernelGGL(zmi_quant_frag8_kernel<false>, dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats_dev, n_mat, scale_dt);
+    return hipGetLastError();
+  }
   if (src_dt == ZMI_DT_BF16)
     hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)total_rows), dim3(QT_THREADS), 0,
                        stream, m0, mats_dev, n_mat, scale_dt);

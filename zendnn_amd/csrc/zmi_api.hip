@@ -580,7 +580,7 @@ int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src, const int32_t
   if (!arena().begin(0)) return ZMI_FAILURE;
   const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
   if (!dev) return ZMI_FAILURE;
-  bool ok = hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), rows, params->src_dtype, sdt, stream()), "quant launch");
+  bool ok = hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), rows, params->src_dtype, sdt, 0, stream()), "quant launch");
   upload_fence();
   set_kernel_name("quant_rows_grouped");
   return ok ? ZMI_SUCCESS : ZMI_FAILURE;

@@ -220,6 +220,18 @@ bool params_uniform(const zmi_group_args_t &a, size_t num_ops) {
   return true;
 }
 
+// When every matrix of a grouped quantization qualifies for the 8-rows-per-workgroup
+// kernel, its rows are renumbered so that each matrix starts at a multiple of 8.
+int64_t renumber_rows8(std::vector<ZmiQuantMat> &mats, int32_t src_dt, int64_t total_rows, int *rows8) {
+  *rows8 = 0;
+  for (const ZmiQuantMat &m : mats)
+    if (!zmi_quant_mat_frag8_ok(m, src_dt)) return total_rows;
+  int64_t r = 0;
+  for (ZmiQuantMat &m : mats) { m.row_start = (int32_t)r; r += zmi_round_up(m.M, 8); }
+  *rows8 = 1;
+  return r;
+}
+
 struct Stage {
   std::vector<ZmiProblem> probs;
   ZmiEpilogue epi;
@@ -374,6 +386,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       // reference: group_reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:307-696
       std::vector<ZmiQuantMat> mats;
       int64_t r0 = 0;
+      int rows8 = 0;
       for (size_t i = 0; i < num_ops; ++i) {
         if (a.M[i] <= 0) continue;
         const int64_t kp = zmi_blob_kpad(a.K[i]);
@@ -390,9 +403,10 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       }
       s1_dt = (p0.src_scale.buff && p0.src_scale.dt != ZMI_DT_NONE) ? p0.src_scale.dt : ZMI_DT_F32;
       if (s1_dt != ZMI_DT_F32 && s1_dt != ZMI_DT_BF16) { set_error("source scale must be f32 or bf16"); return ZMI_FAILURE; }
+      r0 = renumber_rows8(mats, p0.dt_src, r0, &rows8);
       const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
       if (!dev) return ZMI_FAILURE;
-      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_src, s1_dt, stream()), "grouped quant launch")) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_src, s1_dt, rows8, stream()), "grouped quant launch")) return ZMI_FAILURE;
     } else {
       for (size_t i = 0; i < num_ops; ++i) {
         if (a.M[i] <= 0) continue;
@@ -503,9 +517,11 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
         mats.push_back(m);
         A2[i] = m.dst; s2[i] = (float *)m.scale; lda2[i] = kp;
       }
+      int rows8 = 0;
+      r0 = renumber_rows8(mats, p0.dt_dst, r0, &rows8);
       const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
       if (!dev) return ZMI_FAILURE;
-      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_dst, ZMI_DT_F32, stream()), "grouped quant launch (Op2)")) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_dst, ZMI_DT_F32, rows8, stream()), "grouped quant launch (Op2)")) return ZMI_FAILURE;
 
       Stage op2;
       bool have2 = false;

@@ -26,8 +26,10 @@ hipError_t zmi_launch_prepack(const int8_t *B, int64_t K, int64_t N, int64_t ldb
 hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
                                  int8_t *dst, int64_t ld_dst, int64_t frag_kpad, void *scales, int32_t scale_dt,
                                  hipStream_t stream);
+// rows8 != 0: row_start of every matrix is a multiple of 8 and zmi_quant_mat_frag8_ok holds for all of them
 hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_t total_rows,
-                                  int32_t src_dt, int32_t scale_dt, hipStream_t stream);
+                                  int32_t src_dt, int32_t scale_dt, int rows8, hipStream_t stream);
+bool zmi_quant_mat_frag8_ok(const ZmiQuantMat &m, int32_t src_dt);
 hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
                                    int8_t *dst, int64_t ld_dst, int64_t frag_kpad, float *scales,
                                    unsigned int *amax_scratch, hipStream_t stream);
