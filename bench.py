@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0
 K_DEC, N_DEC = 4096, 14336
+# HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
+# size), measured with the commands recorded in profiles/zmi_gemm_decode_kernel_decode_M16_K4096_N14336.md
+DECODE_TRAFFIC_BYTES = 60274942
 
 
 def main():
@@ -37,6 +40,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
+    ap.add_argument("--only", default=None,
+                    choices=["decode_M1", "decode_M4", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
+                             "moe_config4", "moe_config5"],
+                    help="run one of the other configs alone and print its entry (for profiler runs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run")
@@ -149,92 +156,87 @@ def main():
 
     M = 16
     n_sets = 8
-    step, kernel_only, keep = decode_setup(M, n_sets)
-    ms = ev_time(step, args.steps, args.warmup)
-    step_kernel = lowoha.last_kernel()
-    value = decode_bytes(M) / (ms * 1e-3) / 1e9
-    ms_k = ev_time(kernel_only, args.steps, args.warmup)
-    gemm_kernel = lowoha.last_kernel()
-    # algorithmic bytes of the GEMM-only launch: s8 rows instead of bf16 rows, plus the row scales
-    kbytes = K_DEC * N_DEC + M * K_DEC + M * 4 + N_DEC * 4 + M * N_DEC * 2
-    # One step is the per-token quantization launch plus the GEMM launch; the GEMM kernel
-    # dominates, and the second timed loop runs that kernel alone, back to back.
-    achieved = kbytes / (ms_k * 1e-3) / 1e9
+    keep = None
+    result = None
+    if not args.only:
+        step, kernel_only, keep = decode_setup(M, n_sets)
+        ms = ev_time(step, args.steps, args.warmup)
+        step_kernel = lowoha.last_kernel()
+        value = decode_bytes(M) / (ms * 1e-3) / 1e9
+        ms_k = ev_time(kernel_only, args.steps, args.warmup)
+        gemm_kernel = lowoha.last_kernel()
+        # One step is ONE launch: the decode kernel with the per-token quantization fused in (its
+        # first M workgroups quantize, the rest stream the weights).  The timed region above is
+        # therefore already "that kernel launched back to back between two events on its stream".
+        fused = "fused" in step_kernel
+        achieved = value if fused else None
+        # the same kernel on rows that are already s8 (no quantization part), for comparison
+        kbytes = K_DEC * N_DEC + M * K_DEC + M * 4 + N_DEC * 4 + M * N_DEC * 2
+        gemm_only = kbytes / (ms_k * 1e-3) / 1e9
+        if achieved is None:
+            achieved = gemm_only
 
-    result = {
-        "metric": "decode_int8_gemm_weight_streaming",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "s8 x s8 -> s32 (f32 epilogue, bf16 store)",
-        "data": "synthetic",
-        "config": {"workload": "matmul_direct decode: M=16 K=4096 N=14336, bf16 -> per-token s8, "
-                               "prepacked s8 weights, per-channel scales, SiLU, bf16 out",
-                   "weight_sets_rotated": n_sets, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1)},
-        "roofline": {"bound": "hbm", "kernel": "zmi_gemm_decode_kernel: " + gemm_kernel,
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "algorithmic_bytes_per_launch": kbytes,
-                     "avg_launch_us": round(ms_k * 1e3, 2),
-                     "whole_call": {"kernels": "zmi_quant_rows_kernel + " + step_kernel, "us": round(ms * 1e3, 2),
-                                    "algorithmic_bytes": decode_bytes(M)},
-                     "note": "the GEMM kernel launched back to back on s8 rows, timed between two events on "
-                             "its stream (includes the dispatch gap); value above is the whole call "
-                             "(quantization launch + this kernel)"},
-    }
+        result = {
+            "metric": "decode_int8_gemm_weight_streaming",
+            "value": round(value, 1),
+            "unit": "GB/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(ms, 5),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "s8 x s8 -> s32 (f32 epilogue, bf16 store)",
+            "data": "synthetic",
+            "config": {"workload": "matmul_direct decode: M=16 K=4096 N=14336, bf16 -> per-token s8, "
+                                   "prepacked s8 weights, per-channel scales, SiLU, bf16 out",
+                       "weight_sets_rotated": n_sets, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1)},
+            "roofline": {"bound": "hbm", "kernel": "zmi_gemm_decode_kernel: " + (step_kernel if fused else gemm_kernel),
+                         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": DECODE_TRAFFIC_BYTES,
+                         "algorithmic_bytes_per_launch": decode_bytes(M) if fused else kbytes,
+                         "avg_launch_us": round((ms if fused else ms_k) * 1e3, 2),
+                         "gemm_only": {"kernel": gemm_kernel, "us": round(ms_k * 1e3, 2), "GBps": round(gemm_only, 1),
+                                       "algorithmic_bytes": kbytes},
+                         "note": "launches timed back to back between two events on the kernel's stream, so the "
+                                 "figure includes the dispatch gap; traffic is FETCH_SIZE + WRITE_SIZE per launch "
+                                 "from the rocprofv3 --pmc runs summarised under profiles/ (null if not measured "
+                                 "for this build)"},
+        }
 
-    if not args.no_extras:
-        other = {}
-        del keep
-        torch.cuda.empty_cache()
-        # decode at M = 1 and 4
-        for m in (1, 4):
-            s, k, kp = decode_setup(m, n_sets)
-            t = ev_time(s, 100, 10)
-            tk = ev_time(k, 100, 10)
-            other[f"decode_M{m}"] = {"GBps": round(decode_bytes(m) / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2),
-                                     "kernel_GBps": round((K_DEC * N_DEC + m * K_DEC + m * 4 + N_DEC * 4 + m * N_DEC * 2) / (tk * 1e-3) / 1e9, 1)}
-            del s, k, kp
-            torch.cuda.empty_cache()
-        # prefill (config 3): whole call (quantization + GEMM) and the GEMM kernel alone
-        for N in (4096, 14336):
-            Mp, K = 2048, 4096
-            blob = prepack(rand_w(K, N), K, N)
-            ws = torch.rand(N, device=dev, generator=g) * 0.009 + 0.001
-            bias = torch.randn(N, device=dev, generator=g) * 0.1
-            x = torch.randn((Mp, K), device=dev, generator=g).to(torch.bfloat16)
-            dst = torch.zeros((Mp, N), dtype=torch.bfloat16, device=dev)
-            p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32, compute=capi.DT_S8)
-            p.dynamic_quant = True
-            p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (Mp, 1))
-            p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
-            p.postop_ = [lowoha.PostOp(capi.PO_GELU_TANH)]
-            p.mem_format_b = "r"
-            p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
-            t = ev_time(lambda: lowoha.matmul_direct("r", False, False, Mp, N, K, 1.0, x, K, blob, N, bias, 0.0, dst, N, True, p), 30, 5)
-            xq = torch.randint(-127, 128, (Mp, K), dtype=torch.int8, device=dev, generator=g)
-            xs = torch.rand(Mp, device=dev, generator=g) * 0.02 + 0.01
-            pk = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32)
-            pk.src_scale = lowoha.QuantParam(xs, capi.DT_F32, (Mp, 1))
-            pk.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
-            pk.postop_ = [lowoha.PostOp(capi.PO_GELU_TANH)]
-            pk.mem_format_b = "r"
-            pk.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
-            tk = ev_time(lambda: lowoha.matmul_direct("r", False, False, Mp, N, K, 1.0, xq, K, blob, N, bias, 0.0, dst, N, True, pk), 30, 5)
-            ops = 2.0 * Mp * N * K
-            other[f"prefill_N{N}"] = {"TOPS_whole_call": round(ops / (t * 1e-3) / 1e12, 1),
-                                      "TOPS_gemm_kernel": round(ops / (tk * 1e-3) / 1e12, 1),
-                                      "pct_of_int8_mfma_peak": round(100 * ops / (tk * 1e-3) / 1e12 / INT8_PEAK_TOPS, 1),
-                                      "us_gemm_kernel": round(tk * 1e3, 1), "kernel": lowoha.last_kernel()}
-            del blob, x, dst, xq
-            torch.cuda.empty_cache()
-        # config 1
+    # ---------------------------------------------------------------- other configs
+    def run_decode_m(m):
+        s_, k_, kp_ = decode_setup(m, n_sets)
+        t = ev_time(s_, 100, 10)
+        tk = ev_time(k_, 100, 10)
+        return {"GBps": round(decode_bytes(m) / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2),
+                "gemm_only_GBps": round((K_DEC * N_DEC + m * K_DEC + m * 4 + N_DEC * 4 + m * N_DEC * 2) / (tk * 1e-3) / 1e9, 1),
+                "kernel": lowoha.last_kernel()}
+
+    def run_prefill(N):
+        # config 3: whole call = per-token quantization launch (rows written in MFMA fragment order) + GEMM launch;
+        # the per-kernel split is in the rocprofv3 summaries under profiles/
+        Mp, K = 2048, 4096
+        blob = prepack(rand_w(K, N), K, N)
+        ws = torch.rand(N, device=dev, generator=g) * 0.009 + 0.001
+        bias = torch.randn(N, device=dev, generator=g) * 0.1
+        x = torch.randn((Mp, K), device=dev, generator=g).to(torch.bfloat16)
+        dst = torch.zeros((Mp, N), dtype=torch.bfloat16, device=dev)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (Mp, 1))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+        p.postop_ = [lowoha.PostOp(capi.PO_GELU_TANH)]
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        t = ev_time(lambda: lowoha.matmul_direct("r", False, False, Mp, N, K, 1.0, x, K, blob, N, bias, 0.0, dst, N, True, p), 30, 5)
+        ops = 2.0 * Mp * N * K
+        return {"TOPS_whole_call": round(ops / (t * 1e-3) / 1e12, 1),
+                "pct_of_int8_mfma_peak": round(100 * ops / (t * 1e-3) / 1e12 / INT8_PEAK_TOPS, 1),
+                "us_whole_call": round(t * 1e3, 1), "kernel": lowoha.last_kernel()}
+
+    def run_config1():
         Mc, K, N = 128, 4096, 4096
         blobs = [prepack(rand_w(K, N), K, N, capi.DT_U8) for _ in range(20)]
         a = torch.randint(0, 256, (Mc, K), dtype=torch.uint8, device=dev, generator=g)
@@ -256,39 +258,59 @@ def main():
             st["i"] += 1
             lowoha.matmul_direct("r", False, False, Mc, N, K, 1.0, a, K, b, N, bias, 0.0, dst, N, True, p)
         t = ev_time(c1, 100, 10)
-        other["config1_u8s8_M128"] = {"us_per_call": round(t * 1e3, 2), "GBps": round(19431424 / (t * 1e-3) / 1e9, 1),
-                                      "TOPS": round(2.0 * Mc * N * K / (t * 1e-3) / 1e12, 1)}
-        del blobs
-        torch.cuda.empty_cache()
-        # MoE configs 4 and 5: tokens/s through the device-routed fused block
-        for name, T, Hd, I, E, topk, skew in (("moe_config4", 512, 4096, 14336, 8, 2, False),
-                                              ("moe_config5", 4096, 2048, 1408, 64, 6, True)):
-            w13 = [prepack(rand_w(Hd, 2 * I), Hd, 2 * I) for _ in range(E)]
-            w2 = [prepack(rand_w(I, Hd), I, Hd) for _ in range(E)]
-            s13 = [torch.rand(2 * I, device=dev, generator=g) * 0.009 + 0.001 for _ in range(E)]
-            s2 = [torch.rand(Hd, device=dev, generator=g) * 0.009 + 0.001 for _ in range(E)]
-            x = torch.randn((T, Hd), device=dev, generator=g).to(torch.bfloat16)
-            logits = torch.randn((T, E), device=dev, generator=g)
-            if skew:
-                logits = logits + torch.randn(E, device=dev, generator=g) * 1.5
-            prob = torch.softmax(logits, dim=1)
-            tw, ids = torch.topk(prob, topk, dim=1)
-            ids = ids.to(torch.int32).contiguous()
-            tw = tw.contiguous()
-            out = torch.zeros((T, Hd), dtype=torch.bfloat16, device=dev)
+        return {"us_per_call": round(t * 1e3, 2), "GBps": round(19431424 / (t * 1e-3) / 1e9, 1),
+                "TOPS": round(2.0 * Mc * N * K / (t * 1e-3) / 1e12, 1), "kernel": lowoha.last_kernel()}
 
-            def moe():
-                r = lowoha.moe_fused_device(x, ids, tw, w13, w2, s13, s2, I, capi.ACT_SILU_AND_MUL, out)
-                if r != capi.SUCCESS:
-                    raise RuntimeError(lowoha.last_error())
-            t = ev_time(moe, 10, 3)
-            cnt = torch.bincount(ids.flatten().long(), minlength=E)
-            ops = 2.0 * T * topk * 3 * Hd * I
-            other[name] = {"tokens_per_s": round(T / (t * 1e-3), 0), "ms_per_call": round(t, 4),
-                           "TOPS": round(ops / (t * 1e-3) / 1e12, 1),
-                           "weight_GBps": round(E * 3 * Hd * I / (t * 1e-3) / 1e9, 1),
-                           "expert_rows_min_max": [int(cnt.min()), int(cnt.max())]}
-            del w13, w2, x, out
+    def run_moe(T, Hd, I, E, topk, skew):
+        # configs 4 and 5: tokens/s through the device-routed fused block
+        w13 = [prepack(rand_w(Hd, 2 * I), Hd, 2 * I) for _ in range(E)]
+        w2 = [prepack(rand_w(I, Hd), I, Hd) for _ in range(E)]
+        s13 = [torch.rand(2 * I, device=dev, generator=g) * 0.009 + 0.001 for _ in range(E)]
+        s2 = [torch.rand(Hd, device=dev, generator=g) * 0.009 + 0.001 for _ in range(E)]
+        x = torch.randn((T, Hd), device=dev, generator=g).to(torch.bfloat16)
+        logits = torch.randn((T, E), device=dev, generator=g)
+        if skew:
+            logits = logits + torch.randn(E, device=dev, generator=g) * 1.5
+        prob = torch.softmax(logits, dim=1)
+        tw, ids = torch.topk(prob, topk, dim=1)
+        ids = ids.to(torch.int32).contiguous()
+        tw = tw.contiguous()
+        out = torch.zeros((T, Hd), dtype=torch.bfloat16, device=dev)
+
+        def moe():
+            r = lowoha.moe_fused_device(x, ids, tw, w13, w2, s13, s2, I, capi.ACT_SILU_AND_MUL, out)
+            if r != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+        t = ev_time(moe, 10, 3)
+        cnt = torch.bincount(ids.flatten().long(), minlength=E)
+        ops = 2.0 * T * topk * 3 * Hd * I
+        touched = int((cnt > 0).sum())
+        return {"tokens_per_s": round(T / (t * 1e-3), 0), "ms_per_call": round(t, 4),
+                "TOPS": round(ops / (t * 1e-3) / 1e12, 1),
+                "weight_GBps": round(touched * 3 * Hd * I / (t * 1e-3) / 1e9, 1),
+                "expert_rows_min_max": [int(cnt.min()), int(cnt.max())],
+                "experts_under_8_rows": int((cnt < 8).sum()), "experts_over_1000_rows": int((cnt > 1000).sum())}
+
+    extras = {
+        "decode_M1": lambda: run_decode_m(1),
+        "decode_M4": lambda: run_decode_m(4),
+        "prefill_N4096": lambda: run_prefill(4096),
+        "prefill_N14336": lambda: run_prefill(14336),
+        "config1_u8s8_M128": run_config1,
+        "moe_config4": lambda: run_moe(512, 4096, 14336, 8, 2, False),
+        "moe_config5": lambda: run_moe(4096, 2048, 1408, 64, 6, True),
+    }
+    if args.only:
+        # one of the other configs alone (the form the profiler runs use); prints its entry only
+        print(json.dumps({args.only: extras[args.only]()}))
+        return
+
+    if not args.no_extras:
+        other = {}
+        del keep
+        torch.cuda.empty_cache()
+        for name, fn in extras.items():
+            other[name] = fn()
             torch.cuda.empty_cache()
         result["other_configs"] = other
 
