@@ -54,13 +54,15 @@ __device__ __forceinline__ void zmi_wait_vm() {
 }
 __device__ __forceinline__ void zmi_wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
-template <int BM>
+// DEEP: the launch has at most one workgroup per CU, so the ring takes the whole LDS
+// (more stages in flight) instead of leaving room for a second workgroup.
+template <int BM, bool DEEP = false>
 struct RingCfg {
   static constexpr int AF = BM / 32;                 // activation fragment rows per tile
   static constexpr int P = AF + 8;                   // 2 KiB pairs per stage
   static constexpr int STAGE = P * 2048;
-  static constexpr int NS = BM == 256 ? 4 : 3;
-  static constexpr int OCC = BM == 256 ? 1 : 2;
+  static constexpr int NS = BM == 256 ? 4 : (DEEP ? (BM == 128 ? 6 : 7) : 3);
+  static constexpr int OCC = (BM == 256 || DEEP) ? 1 : 2;
   static constexpr int NPAIR_MAX = (P + 3) / 4;
   static constexpr int RING = STAGE * NS;
   static constexpr int EPI = 4 * R_EPI_WAVE_WORDS * 4;     // epilogue staging, reuses the ring
@@ -139,13 +141,13 @@ __device__ __forceinline__ void zmi_ring_strip_bf16(const int32_t *stage, const 
   }
 }
 
-template <int BM>
-__global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_kernel(ZmiProblem p0,
+template <int BM, bool DEEP>
+__global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_ring_kernel(ZmiProblem p0,
                                                                                    const ZmiProblem *probs,
                                                                                    int n_prob, int n_items,
-                                                                                   const int *n_items_dev, int top_flags,
+                                                                                   const int *tile_tab, int bm_idx, int top_flags,
                                                                                    ZmiEpilogue epi) {
-  using Cfg = RingCfg<BM>;
+  using Cfg = RingCfg<BM, DEEP>;
   constexpr int MI = BM / 64, NI = 4;
   constexpr int AF = Cfg::AF, STAGE = Cfg::STAGE, NS = Cfg::NS, NPM = Cfg::NPAIR_MAX;
   char *smem = zmi_ring_smem;
@@ -160,8 +162,10 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
   // Workgroup ids go round robin over the 8 XCDs; renumber so that every XCD gets
   // a contiguous range of tiles, and order tiles so that neighbours share weight
   // columns (and, for one problem, a band of activation rows).
-  // (with row counts known only on the device the grid is a bound and the real tile count is read here)
-  if (n_items_dev) n_items = *n_items_dev;
+  // Grouped launches read the tile table made by zmi_ring_count_kernel: the real tile count
+  // (the grid is only a bound when the row counts live on the device) and, per problem,
+  // the index of its first tile.
+  if (tile_tab) n_items = tile_tab[bm_idx];
   const int b = blockIdx.x;
   const int per_xcd = (n_items + 7) / 8;
   const int id = (b % 8) * per_xcd + b / 8;
@@ -187,28 +191,31 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
       tn = r / gm;
       m0 = tm < full ? tm * top : (p.M / top) * top;
     } else {
-      int base = 0, e = 0;
+      // the problem that owns tile `id`: the last one whose first tile is <= id (64 candidates per step)
+      const int *starts = tile_tab + 4 + bm_idx * n_prob;
+      int e = -1;
+      for (int e0 = 0; e0 < n_prob; e0 += 64) {
+        const int ee = e0 + lane;
+        const int st = ee < n_prob ? starts[ee] : 0x7fffffff;
+        const int c = __popcll(__ballot(st <= id));
+        if (c > 0) e = e0 + c - 1;
+        if (c < 64) break;
+      }
+      e = __builtin_amdgcn_readfirstlane(e);
+      bool found = e >= 0;
       tm = tn = m0 = 0;
-      bool found = false;
-      for (; e < n_prob; ++e) {
+      if (found) {
         const int M = probs[e].M;
-        if (M <= 0) continue;
         int full; bool rem;
         zmi_ring_rows<BM>(M, top_flags, full, rem);
         const int tiles_m = full + (rem ? 1 : 0);
-        if (!tiles_m) continue;
-        const int ncols = gated ? probs[e].N / 2 : probs[e].N;
-        const int tiles_n = (ncols + per - 1) / per;
-        const int cnt = tiles_m * tiles_n;
-        if (id < base + cnt) {
-          const int r = id - base;
+        const int r = id - starts[e];
+        found = tiles_m > 0;
+        if (found) {
           tm = r % tiles_m;
           tn = r / tiles_m;
           m0 = tm < full ? tm * top : (M / top) * top;
-          found = true;
-          break;
         }
-        base += cnt;
       }
       if (!found) return;
       p = probs[e];
@@ -392,9 +399,13 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
     const int slot_prev = slot == 0 ? NS - 1 : slot - 1;
     phase(0, slot, 1, false, 0);
     // stage s+1 has landed (loads are issued every stage, clamped at the end, so the count is uniform)
+#ifndef ZMI_RING_TEST_NOWAIT
     if (short_wave) zmi_wait_vm<(NS - 3) * (NPM - 1) * 2>();
     else zmi_wait_vm<(NS - 3) * NPM * 2>();
+#endif
+#ifndef ZMI_RING_TEST_NOBAR
     zmi_wg_barrier();
+#endif
     phase(1, slot_next, 0, true, slot_prev);
     voff = voff + 2048 < voff_max ? voff + 2048 : voff_max;
     slot = slot_next;
@@ -620,42 +631,70 @@ __global__ __launch_bounds__(R_THREADS, RingCfg<BM>::OCC) void zmi_gemm_ring_ker
 #endif
 }
 
-// Tile counts of a problem table for the three tile heights, computed where the row counts live.
+// Tile table of a problem set, computed where the row counts live: tab[0..2] = number of
+// tiles of the 256 / 128 / 64 row kernels, tab[4 + b * n_prob + e] = index of the first
+// tile of problem e in kernel b.  One wavefront, 64 problems per step.
 __global__ __launch_bounds__(64) void zmi_ring_count_kernel(const ZmiProblem *probs, int n_prob, int top, int gated,
-                                                             int *out) {
-  int c256 = 0, c128 = 0, c64 = 0;
-  for (int e = threadIdx.x; e < n_prob; e += 64) {
-    const int M = probs[e].M, N = probs[e].N;
-    if (M <= 0) continue;
-    if ((top & 0xffff) == 256) c256 += zmi_ring_items<256>(M, N, top, gated != 0);
-    c128 += zmi_ring_items<128>(M, N, top, gated != 0);
-    c64 += zmi_ring_items<64>(M, N, top, gated != 0);
-  }
+                                                             int *tab) {
+  const int lane = threadIdx.x;
+  int run[3] = {0, 0, 0};
+  for (int e0 = 0; e0 < n_prob; e0 += 64) {
+    const int e = e0 + lane;
+    int c[3] = {0, 0, 0};
+    if (e < n_prob) {
+      const int M = probs[e].M, N = probs[e].N;
+      if (M > 0) {
+        if ((top & 0xffff) == 256) c[0] = zmi_ring_items<256>(M, N, top, gated != 0);
+        c[1] = zmi_ring_items<128>(M, N, top, gated != 0);
+        c[2] = zmi_ring_items<64>(M, N, top, gated != 0);
+      }
+    }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    c256 += __shfl_xor(c256, o);
-    c128 += __shfl_xor(c128, o);
-    c64 += __shfl_xor(c64, o);
+    for (int b = 0; b < 3; ++b) {
+      // inclusive prefix over the wavefront
+      int x = c[b];
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int y = __shfl_up(x, o);
+        if (lane >= o) x += y;
+      }
+      if (e < n_prob) tab[4 + b * n_prob + e] = run[b] + x - c[b];
+      run[b] += __shfl(x, 63);
+    }
   }
-  if (threadIdx.x == 0) { out[0] = c256; out[1] = c128; out[2] = c64; }
+  if (lane == 0) { tab[0] = run[0]; tab[1] = run[1]; tab[2] = run[2]; }
 }
 
-template <int BM>
-static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items,
-                              const int *n_items_dev, int top, const ZmiEpilogue &epi, hipStream_t stream) {
-  if (n_items <= 0) return hipSuccess;
-  const size_t smem = RingCfg<BM>::SMEM;
+template <int BM, bool DEEP>
+static hipError_t ring_launch_cfg(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items,
+                                  const int *tile_tab, int top, const ZmiEpilogue &epi, hipStream_t stream) {
+  const size_t smem = RingCfg<BM, DEEP>::SMEM;
   static bool attr_done = false;
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_ring_kernel<BM>,
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_ring_kernel<BM, DEEP>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
   const int grid = (n_items + 7) / 8 * 8;   // a multiple of 8 so the XCD renumbering applies
-  hipLaunchKernelGGL(zmi_gemm_ring_kernel<BM>, dim3(grid), dim3(R_THREADS), smem, stream, p0, probs, n_prob,
-                     n_items, n_items_dev, top, epi);
+  hipLaunchKernelGGL((zmi_gemm_ring_kernel<BM, DEEP>), dim3(grid), dim3(R_THREADS), smem, stream, p0, probs, n_prob,
+                     n_items, tile_tab, BM == 256 ? 0 : (BM == 128 ? 1 : 2), top, epi);
   return hipGetLastError();
+}
+
+template <int BM>
+static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items, bool exact,
+                              const int *tile_tab, int top, const ZmiEpilogue &epi, hipStream_t stream) {
+  if (n_items <= 0) return hipSuccess;
+  // at most one workgroup per CU anyway: let it have the whole LDS for its ring
+  static const int n_cu = [] {
+    int dev = 0, n = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    return n;
+  }();
+  if (BM != 256 && n_items <= n_cu && exact)
+    return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, epi, stream);
+  return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, epi, stream);
 }
 
 // Largest tile height for a problem set: 256-row tiles once they fill the chip,
@@ -684,22 +723,22 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
   const bool gated = epi.gated_act != 0;
   hipError_t e = hipSuccess;
   if ((top & 0xffff) == 256) {
-    e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), nullptr, top, epi, stream);
+    e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), true, nullptr, top, epi, stream);
     if (e != hipSuccess) return e;
   }
-  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), nullptr, top, epi, stream);
+  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, epi, stream);
   if (e != hipSuccess) return e;
-  return ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), nullptr, top, epi, stream);
+  return ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, epi, stream);
 }
 
-// Every problem of the table.  probs_host mirrors probs_dev and sizes the grids;
-// when it is null (row counts known only on the device) worst_rows / worst_cols
-// bound them, the real tile counts are computed on the device into counts_dev
-// (3 ints of scratch) and surplus workgroups exit at once.
+// Every problem of the table.  probs_host mirrors probs_dev and sizes the grids; when it is
+// null (row counts known only on the device) worst_rows / worst_cols bound them and surplus
+// workgroups exit at once.  tab_dev is 4 + 3 * n_prob ints of scratch for the tile table.
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
-                                      int top, int64_t worst_rows, int worst_cols, int *counts_dev,
+                                      int top, int64_t worst_rows, int worst_cols, int *tab_dev,
                                       const ZmiEpilogue &epi, hipStream_t stream) {
   const bool gated = epi.gated_act != 0;
+  if (!tab_dev) return hipErrorInvalidValue;
   int items[3] = {0, 0, 0};   // 256, 128, 64
   if (probs_host) {
     for (int e = 0; e < n_prob; ++e) {
@@ -720,18 +759,17 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
       if (th == 256) items[1] = n_prob * tiles_n;
       if (th >= 128) items[2] = n_prob * tiles_n;
     }
-    if (!counts_dev) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0,
-                       counts_dev);
   }
-  const int *cd = probs_host ? nullptr : counts_dev;
+  if (items[0] + items[1] + items[2] <= 0) return hipSuccess;
+  hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0, tab_dev);
+  const bool exact = probs_host != nullptr;
   ZmiProblem dummy = {};
   hipError_t e = hipSuccess;
   if ((top & 0xffff) == 256) {
-    e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], cd, top, epi, stream);
+    e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], exact, tab_dev, top, epi, stream);
     if (e != hipSuccess) return e;
   }
-  e = ring_launch<128>(dummy, probs_dev, n_prob, items[1], cd ? cd + 1 : nullptr, top, epi, stream);
+  e = ring_launch<128>(dummy, probs_dev, n_prob, items[1], exact, tab_dev, top, epi, stream);
   if (e != hipSuccess) return e;
-  return ring_launch<64>(dummy, probs_dev, n_prob, items[2], cd ? cd + 2 : nullptr, top, epi, stream);
+  return ring_launch<64>(dummy, probs_dev, n_prob, items[2], exact, tab_dev, top, epi, stream);
 }

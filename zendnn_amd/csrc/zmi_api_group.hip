@@ -252,7 +252,9 @@ int32_t launch_stage(const Stage &st, const char *what) {
   int cols = 0, kmax = 0;
   for (const ZmiProblem &q : st.probs) { rows += q.M; cols = std::max(cols, (int)q.N); kmax = std::max(kmax, (int)q.K); }
   const int top = group_top(rows, n, kmax, cols, st.epi.gated_act != 0);
-  if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, nullptr, st.epi, stream()), what)) return ZMI_FAILURE;
+  int *tab = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)n));
+  if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
+  if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, st.epi, stream()), what)) return ZMI_FAILURE;
   return ZMI_SUCCESS;
 }
 
@@ -374,7 +376,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       const size_t tbl = sizeof(void *) * (size_t)moe_postop->num_tokens * moe_postop->topk;
       need += Arena::padded(tbl);
     }
-    need += 4096;
+    need += 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * num_ops));
     if (!arena().begin(need)) return ZMI_FAILURE;
 
     // ---- stage 1: sources (dynamic per-token quantization of every expert in one launch)
@@ -610,7 +612,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   need += Arena::padded((size_t)Rp * I * 2);                                         // act bf16
   need += Arena::padded((size_t)Rp * kpI) + Arena::padded(sizeof(float) * Rp);       // A2, s2
   need += Arena::padded((size_t)Rp * H * 2);                                         // Y bf16
-  need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096 + 256;
+  need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * (size_t)E));
   if (!arena().begin(need)) return ZMI_FAILURE;
   int32_t *counts = (int32_t *)arena().alloc(sizeof(int32_t) * E);
   int32_t *offsets = (int32_t *)arena().alloc(sizeof(int32_t) * (E + 1));
@@ -621,7 +623,8 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   int8_t *A2 = (int8_t *)arena().alloc((size_t)Rp * kpI);
   float *s2 = (float *)arena().alloc(sizeof(float) * Rp);
   void *Y = arena().alloc((size_t)Rp * H * 2);
-  int *tile_counts = (int *)arena().alloc(256);
+  int *tile_tab1 = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)E));
+  int *tile_tab2 = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)E));
   ZmiProblem *op1 = (ZmiProblem *)arena().alloc(sizeof(ZmiProblem) * E);
   ZmiProblem *op2 = (ZmiProblem *)arena().alloc(sizeof(ZmiProblem) * E);
 
@@ -654,10 +657,10 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   e1.gated_act = d->gated_act;
   // row counts live on the device: the grids are sized for the worst case
   const int top1 = group_top(R, E, H, 2 * I, true), top2 = group_top(R, E, I, H, false);
-  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_counts, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_counts + 4, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;
   upload_fence();
   set_kernel_name("moe_fused_device");

@@ -39,7 +39,7 @@ int zmi_ring_pick_top(int64_t rows, int64_t out_cols);
 int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated);
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
-                                      int top, int64_t worst_rows, int worst_cols, int *counts_dev,
+                                      int top, int64_t worst_rows, int worst_cols, int *tab_dev,
                                       const ZmiEpilogue &epi, hipStream_t stream);
 
 // k_smallm.hip
