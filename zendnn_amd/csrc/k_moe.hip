@@ -144,11 +144,14 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
 
 __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int32_t *topk_ids, int n, int E,
                                                                       int align, int32_t *counts,
-                                                                      int32_t *offsets, int32_t *slot_of) {
+                                                                      int32_t *offsets, int32_t *slot_of,
+                                                                      int32_t *src_of, int n_slots) {
   extern __shared__ int32_t sh[];   // hist[RT_WAVES][E], then off[E+1]
   int32_t *hist = sh;
   int32_t *off = sh + RT_WAVES * E;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  if (src_of)
+    for (int i = tid; i < n_slots; i += blockDim.x) src_of[i] = -1;
   for (int i = tid; i < RT_WAVES * E; i += blockDim.x) hist[i] = 0;
   __syncthreads();
   const int seg = (n + RT_WAVES - 1) / RT_WAVES;
@@ -177,6 +180,8 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
     offsets[E] = run;
   }
   __syncthreads();
+  int ebits = 1;
+  while ((1 << ebits) < E) ++ebits;          // expert ids fit in ebits bits
   for (int i0 = s0; i0 < s1; i0 += 64) {
     const int i = i0 + lane;
     const bool live = i < s1;
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
     if (!ok) e = -1;
     // lanes holding the same expert as this lane
     unsigned long long same = __ballot(ok);
-    for (int bit = 0; bit < 11; ++bit) {
+    for (int bit = 0; bit < ebits; ++bit) {
       const unsigned long long b = __ballot((e >> bit) & 1);
       same &= ((e >> bit) & 1) ? b : ~b;
     }
@@ -194,6 +199,7 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
       const int total = __popcll(same);
       const int start = hist[wave * E + e];
       slot_of[i] = off[e] + start + rank;
+      if (src_of) src_of[off[e] + start + rank] = i;
       // the last lane of each expert group advances the cursor for the next 64 entries
       if (rank == total - 1) hist[wave * E + e] = start + total;
     } else if (live) {
@@ -204,7 +210,8 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
 }
 
 hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
-                                int32_t *offsets, int32_t *slot_of, hipStream_t stream) {
+                                int32_t *offsets, int32_t *slot_of, int32_t *src_of, int n_slots,
+                                hipStream_t stream) {
   if (E > 2047 || E <= 0) return hipErrorInvalidValue;
   const size_t smem = ((size_t)RT_WAVES * E + E + 1) * sizeof(int32_t);
   static size_t attr = 0;
@@ -215,7 +222,7 @@ hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E,
     attr = smem;
   }
   hipLaunchKernelGGL(zmi_moe_route_kernel, dim3(1), dim3(RT_WAVES * 64), smem, stream, topk_ids, T * topk, E,
-                     align < 1 ? 1 : align, counts, offsets, slot_of);
+                     align < 1 ? 1 : align, counts, offsets, slot_of, src_of, n_slots);
   return hipGetLastError();
 }
 

@@ -163,10 +163,16 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
   }
   // row_start of every matrix is a multiple of 8 in this launch form
   const int r = grp * 8 - m.row_start + r8;
-  const bool live = r < m.M;
+  bool live = r < m.M;
   const int K = m.K;
   const size_t es = BF16 ? 2 : 4;
-  const char *src = (const char *)m.src + (size_t)(live ? r : 0) * m.ld_src * es;
+  int64_t src_row = live ? r : 0;
+  if (m.gather && live) {
+    const int g = m.gather[r];
+    live = g >= 0;
+    src_row = live ? g / m.gather_div : 0;
+  }
+  const char *src = (const char *)m.src + (size_t)src_row * m.ld_src * es;
   // raw 32-byte (bf16) / 64-byte (f32) pieces -> 16 floats
   auto load_raw = [&](int k, v4i (&w)[4]) {
     if (BF16) {
@@ -301,6 +307,7 @@ hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int
   ZmiQuantMat m;
   m.src = src; m.dst = dst; m.scale = scales; m.ld_src = ld_src; m.ld_dst = ld_dst;
   m.M = (int32_t)M; m.K = (int32_t)K; m.row_start = 0; m.frag_kpad = (int32_t)frag_kpad;
+  m.gather = nullptr; m.gather_div = 1;
   if (frag_kpad && zmi_quant_frag8_ok(src, K, ld_src, src_dt)) {
     const unsigned grid = (unsigned)((M + 7) / 8);
     if (src_dt == ZMI_DT_BF16)
@@ -405,5 +412,24 @@ hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, i
     hipLaunchKernelGGL(zmi_quant_tensor_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, src,
                        M, K, ld_src, dst, ld_dst, frag_kpad, scales, amax_scratch);
   }
+  return hipGetLastError();
+}
+
+// Fragment-major per-token quantization with a row gather: destination row r (of n_rows) takes
+// source row gather[r] / gather_div of x; rows with gather[r] < 0 are left alone.
+hipError_t zmi_launch_quant_gather(const void *x, int32_t x_dt, int64_t ldx, int64_t K, const int32_t *gather,
+                                   int32_t gather_div, int64_t n_rows, int8_t *dst, int64_t frag_kpad, float *scales,
+                                   hipStream_t stream) {
+  if (n_rows <= 0) return hipSuccess;
+  if (!zmi_quant_frag8_ok(x, K, ldx, x_dt) || !frag_kpad) return hipErrorInvalidValue;
+  ZmiQuantMat m = {};
+  m.src = x; m.dst = dst; m.scale = scales; m.ld_src = ldx; m.ld_dst = frag_kpad;
+  m.M = (int32_t)n_rows; m.K = (int32_t)K; m.row_start = 0; m.frag_kpad = (int32_t)frag_kpad;
+  m.gather = gather; m.gather_div = gather_div;
+  const unsigned grid = (unsigned)((n_rows + 7) / 8);
+  if (x_dt == ZMI_DT_BF16)
+    hipLaunchKernelGGL(zmi_quant_frag8_kernel<true>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, ZMI_DT_F32);
+  else
+    hipLaunchKernelGGL(zmi_quant_frag8_kernel<false>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, ZMI_DT_F32);
   return hipGetLastError();
 }

@@ -692,7 +692,8 @@ static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
     return n;
   }();
-  if (BM != 256 && n_items <= n_cu && exact)
+  (void)exact;   // a bound that fits one workgroup per CU is as good as the exact count
+  if (BM != 256 && n_items <= n_cu)
     return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, epi, stream);
   return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, epi, stream);
 }

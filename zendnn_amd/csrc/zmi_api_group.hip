@@ -585,7 +585,7 @@ int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk, int32_t 
   if (!topk_ids || !counts || !offsets || !slot_of || T <= 0 || topk <= 0 || E <= 0) { set_error("moe_route: bad arguments"); return ZMI_FAILURE; }
   if (E > 2047) { set_error("moe_route: at most 2047 experts"); return ZMI_UNIMPLEMENTED; }
   if (!ensure_device()) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, 1, counts, offsets, slot_of, stream()), "moe route launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, 1, counts, offsets, slot_of, nullptr, 0, stream()), "moe route launch")) return ZMI_FAILURE;
   set_kernel_name("moe_route");
   return ZMI_SUCCESS;
 }
@@ -608,6 +608,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   const int64_t kpH = zmi_blob_kpad(H), kpI = zmi_blob_kpad(I);
   size_t need = 0;
   need += Arena::padded(sizeof(int32_t) * E) + Arena::padded(sizeof(int32_t) * (E + 1)) + Arena::padded(sizeof(int32_t) * R);
+  need += Arena::padded(sizeof(int32_t) * Rp);
   need += Arena::padded((size_t)Rp * kpH) + Arena::padded(sizeof(float) * Rp);       // A1, s1
   need += Arena::padded((size_t)Rp * I * 2);                                         // act bf16
   need += Arena::padded((size_t)Rp * kpI) + Arena::padded(sizeof(float) * Rp);       // A2, s2
@@ -617,6 +618,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   int32_t *counts = (int32_t *)arena().alloc(sizeof(int32_t) * E);
   int32_t *offsets = (int32_t *)arena().alloc(sizeof(int32_t) * (E + 1));
   int32_t *slot_of = (int32_t *)arena().alloc(sizeof(int32_t) * R);
+  int32_t *src_of = (int32_t *)arena().alloc(sizeof(int32_t) * Rp);
   int8_t *A1 = (int8_t *)arena().alloc((size_t)Rp * kpH);
   float *s1 = (float *)arena().alloc(sizeof(float) * Rp);
   void *act = arena().alloc((size_t)Rp * I * 2);
@@ -644,8 +646,13 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   tb.w13_scale = (const float *const *)(tdev + 2 * E); tb.w2_scale = (const float *const *)(tdev + 3 * E);
 
   hipStream_t s = stream();
-  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, 32, counts, offsets, slot_of, s), "moe route launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_moe_quant_scatter(d->x, d->ldx, T, H, topk, slot_of, A1, s1, s), "quant scatter launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, 32, counts, offsets, slot_of, src_of, (int)Rp, s), "moe route launch")) return ZMI_FAILURE;
+  // every slot quantizes its token's row itself (8 slots per workgroup, whole 128-byte lines of the
+  // fragment layout); rows that do not allow 16-byte loads take the per-token scatter form
+  if (hipSuccess != zmi_launch_quant_gather(d->x, ZMI_DT_BF16, d->ldx, H, src_of, topk, Rp, A1, kpH, s1, s)) {
+    (void)hipGetLastError();
+    if (!hip_ok(zmi_launch_moe_quant_scatter(d->x, d->ldx, T, H, topk, slot_of, A1, s1, s), "quant scatter launch")) return ZMI_FAILURE;
+  }
   if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, s), "problem table launch")) return ZMI_FAILURE;
 
   ZmiEpilogue e1;

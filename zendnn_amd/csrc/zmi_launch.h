@@ -15,6 +15,10 @@ struct ZmiQuantMat {
   int32_t M, K;
   int32_t row_start;
   int32_t frag_kpad;   // 0: dst rows are K-contiguous with stride ld_dst; > 0: dst is fragment-major with this K_pad
+  // optional row gather (8-rows-per-workgroup kernel only): destination row r is quantized from
+  // source row gather[r] / gather_div, rows with gather[r] < 0 are skipped
+  const int32_t *gather;
+  int32_t gather_div;
 };
 
 // k_prepack.hip
@@ -30,6 +34,9 @@ hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int
 hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_t total_rows,
                                   int32_t src_dt, int32_t scale_dt, int rows8, hipStream_t stream);
 bool zmi_quant_mat_frag8_ok(const ZmiQuantMat &m, int32_t src_dt);
+hipError_t zmi_launch_quant_gather(const void *x, int32_t x_dt, int64_t ldx, int64_t K, const int32_t *gather,
+                                   int32_t gather_div, int64_t n_rows, int8_t *dst, int64_t frag_kpad, float *scales,
+                                   hipStream_t stream);
 hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t ld_src,
                                    int8_t *dst, int64_t ld_dst, int64_t frag_kpad, float *scales,
                                    unsigned int *amax_scratch, hipStream_t stream);
@@ -81,9 +88,11 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
                                   const int32_t *slot_of, const float *weights, int skip_weighted,
                                   int T, int topk, int D, int32_t dt, void *out, int64_t ldo,
                                   hipStream_t stream);
-// align: every expert's first slot is rounded up to a multiple of it (1: dense numbering)
+// align: every expert's first slot is rounded up to a multiple of it (1: dense numbering).
+// src_of (optional, n_slots entries): the flat (token, k) index that fills each slot, -1 for idle slots.
 hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
-                                int32_t *offsets, int32_t *slot_of, hipStream_t stream);
+                                int32_t *offsets, int32_t *slot_of, int32_t *src_of, int n_slots,
+                                hipStream_t stream);
 // A1 is fragment-major over the slot numbering, K_pad = zmi_blob_kpad(H)
 hipError_t zmi_launch_moe_quant_scatter(const void *x, int64_t ldx, int T, int H, int topk,
                                         const int32_t *slot_of, int8_t *A1, float *s1, hipStream_t stream);
