@@ -323,21 +323,6 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
     }
   };
 
-#ifdef ZMI_RING_PRIO
-  // Two workgroups share a CU (BM < 256): the one with the even workgroup slot issues its
-  // MFMAs first, so the pair drifts half a tile apart and one's epilogue runs under the
-  // other's main loop.
-  if (Cfg::OCC > 1) {
-    const int tg = __builtin_amdgcn_s_getreg(4 | (16 << 6) | (3 << 11));   // HW_ID.TG_ID
-    if (tg & 1) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(3);
-#ifdef ZMI_RING_DELAY
-    if (tg & 1) { const long long t0 = wall_clock64(); while (wall_clock64() - t0 < ZMI_RING_DELAY) __builtin_amdgcn_s_sleep(16); }
-#endif
-  }
-#endif
-#ifdef ZMI_RING_TRACE
-  const long long tr_t0 = wall_clock64();
-#endif
   // ---- prologue: NS-1 stages in flight, the first one landed --------------------------
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) issue_all(s);
@@ -399,13 +384,9 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
     const int slot_prev = slot == 0 ? NS - 1 : slot - 1;
     phase(0, slot, 1, false, 0);
     // stage s+1 has landed (loads are issued every stage, clamped at the end, so the count is uniform)
-#ifndef ZMI_RING_TEST_NOWAIT
     if (short_wave) zmi_wait_vm<(NS - 3) * (NPM - 1) * 2>();
     else zmi_wait_vm<(NS - 3) * NPM * 2>();
-#endif
-#ifndef ZMI_RING_TEST_NOBAR
     zmi_wg_barrier();
-#endif
     phase(1, slot_next, 0, true, slot_prev);
     voff = voff + 2048 < voff_max ? voff + 2048 : voff_max;
     slot = slot_next;
@@ -414,15 +395,6 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   zmi_wg_barrier();
 
   // ------------------------------------------------------------------------ epilogue
-#ifdef ZMI_RING_TRACE
-  const long long tr_t1 = wall_clock64();
-#endif
-#ifdef ZMI_RING_PRIO
-  __builtin_amdgcn_s_setprio(0);
-#endif
-#ifdef ZMI_RING_NO_EPI
-  if (acc[0][0][0] != 0x12345678) return;
-#endif
   int32_t *stage = reinterpret_cast<int32_t *>(smem) + wave * R_EPI_WAVE_WORDS;
   // the bf16 fast forms multiply / add unconditionally: absent scales are 1, an absent bias is -0
   if (dst_dt == ZMI_DT_BF16 && epi.fast_kind != ZMI_EK_GENERIC) {
@@ -463,9 +435,6 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
         const v4i a1 = *(const v4i *)&stage[r * R_EPI_LD + 64 + c16 * 4];
         const float rs = rsc[r];
         if (m >= M) continue;
-#ifdef ZMI_RING_NO_STORE
-        if (rs != 12345.0f) continue;
-#endif
         float y0[4], y1[4];
         if (DT == 1) {
           // bf16 store: scale chain with one fused multiply-add (absent scales are 1, absent bias -0)
@@ -621,14 +590,6 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
     do_strip(std::integral_constant<int, 2>{});
     do_strip(std::integral_constant<int, 3>{});
   }
-#ifdef ZMI_RING_TRACE
-  if (tid == 0) {
-    extern __device__ long long zmi_ring_trace[];
-    long long *t = zmi_ring_trace + (size_t)blockIdx.x * 4;
-    t[0] = ((long long)__builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11)) & 0xffffffffll) | ((long long)__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) << 32);
-    t[1] = tr_t0; t[2] = tr_t1; t[3] = wall_clock64();
-  }
-#endif
 }
 
 // Tile table of a problem set, computed where the row counts live: tab[0..2] = number of
