@@ -1,7 +1,8 @@
 """GPU parity of the large-M (fragment-major, MFMA-bound) kernel through matmul_direct:
 tile-edge shapes for every tile height, the straight-line bf16 epilogues next to
-their edge forms, unaligned destinations, u8 sources, and the destination dtypes
-that go through its generic epilogue."""
+their edge forms, unaligned destinations, u8 sources, the destination dtypes
+that go through its generic epilogue, and the K-sliced launch (partial tiles + reduction
+kernel) for both of its tile heights."""
 import os
 
 import numpy as np
@@ -104,3 +105,123 @@ def test_transposed_source_and_weights(zo, top):
     p.weight_cache_type = 0
     got, want = _run_both(zo, p, a, w, M, N, K, lda=M + 2, ldb=K + 6, transA=True, transB=True)
     assert np.array_equal(got, want)
+
+
+@pytest.fixture
+def env():
+    """Sets environment switches for one test and restores them afterwards."""
+    saved = {}
+
+    def set_(**kv):
+        for k, v in kv.items():
+            saved.setdefault(k, os.environ.get(k))
+            os.environ[k] = str(v)
+
+    yield set_
+    for k, v in saved.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
+
+
+# 64-row tiles (M <= 64) and 128-row tiles; K not a multiple of the slice count, fewer
+# 64-k stages than slices asked for (K = 100: two stages), several row and column tiles
+@pytest.mark.parametrize("slices", [2, 3, 8])
+@pytest.mark.parametrize("M,K,N", [(20, 256, 256), (64, 1000, 700), (100, 100, 300), (129, 512, 256), (300, 640, 515)])
+def test_k_sliced_s32_accumulators_bit_exact(zo, env, M, K, N, slices):
+    env(ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=slices)
+    rng = np.random.default_rng(M + K + N)
+    a = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    w = H.gen_weights(rng, K, N)
+    zp = np.array([131], dtype=np.int32)
+    want = (a.astype(np.int64) - 131) @ w.astype(np.int64)
+    a_d, w_d = H.to_dev(a), H.to_dev(w)
+    for _ in range(2):   # the partial-tile scratch is reused call after call
+        p = lowoha.MatmulParams(src=capi.DT_U8, wei=capi.DT_S8, dst=capi.DT_S32)
+        p.src_zp = lowoha.QuantParam(zp.ctypes.data, capi.DT_S32, (1,))
+        dst = torch.zeros((M, N), dtype=torch.int32, device=H.DEV)
+        st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, a_d, K, w_d, N, None, 0.0, dst, N, False, p)
+        assert st == capi.SUCCESS, lowoha.last_error()
+        assert "ksliced" in lowoha.last_kernel()
+        assert np.array_equal(H.to_host(dst).astype(np.int64), want)
+
+
+@pytest.mark.parametrize("po", [None, capi.PO_SWISH, capi.PO_GELU_TANH])
+@pytest.mark.parametrize("M,K,N,ldc_pad", [(48, 512, 320, 0), (200, 384, 322, 3)])
+def test_k_sliced_bf16_epilogues(zo, env, po, M, K, N, ldc_pad):
+    env(ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=3)
+    rng = np.random.default_rng(M + N + (po or 0))
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    ss = rng.uniform(0.01, 0.03, M).astype(np.float32)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    ss_d, ws_d = H.to_dev(ss), H.to_dev(ws)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    if po is not None:
+        p.postop_ = [lowoha.PostOp(po)]
+    p.weight_cache_type = 0
+    got, want = _run_both(zo, p, a, w, M, N, K, bias=bias, host_bufs={"src_scale": ss, "wei_scale": ws}, ldc=N + ldc_pad)
+    assert "ksliced" in lowoha.last_kernel()
+    H.check_bf16(got[:, :N], want[:, :N], atol=1e-6 if po == capi.PO_GELU_TANH else 0.0, max_frac=5e-3)
+    assert np.all(got[:, N:] == 0)
+
+
+@pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_S8, capi.DT_U8])
+def test_k_sliced_f32_exact_and_quantized_destinations(zo, env, dst_dt):
+    env(ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=4)
+    rng = np.random.default_rng(100 + dst_dt)
+    M, K, N = 150, 320, 290
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    ss = np.array([0.02], dtype=np.float32)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    ws_d = H.to_dev(ws)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=dst_dt, bias=capi.DT_F32)
+    p.src_scale = lowoha.QuantParam(ss.ctypes.data, capi.DT_F32, (1,))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    bufs = {"src_scale": ss, "wei_scale": ws}
+    if dst_dt != capi.DT_F32:
+        ds = np.array([7.5], dtype=np.float32)
+        dz = np.array([3], dtype=np.int32)
+        p.dst_scale = lowoha.QuantParam(ds.ctypes.data, capi.DT_F32, (1,))
+        p.dst_zp = lowoha.QuantParam(dz.ctypes.data, capi.DT_S32, (1,))
+        bufs.update(dst_scale=ds, dst_zp=dz)
+    p.weight_cache_type = 0
+    got, want = _run_both(zo, p, a, w, M, N, K, bias=bias, host_bufs=bufs)
+    assert "ksliced" in lowoha.last_kernel()
+    assert np.array_equal(got, want)
+
+
+def test_k_slices_chosen_for_a_problem_with_few_tiles(zo):
+    """M = 128, N = 14336, K = 4096 (56 tiles): the launch plan slices K without being told to,
+    and the dynamic-quantization call agrees with the oracle."""
+    from tests.test_gpu_matmul import _oracle
+    rng = np.random.default_rng(5)
+    M, K, N = 128, 4096, 14336
+    x = H.gen_bf16_normal(rng, (M, K))
+    w = H.gen_weights(rng, K, N)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    x_d, w_d, ws_d = H.to_dev(x), H.to_dev(w), H.to_dev(ws)
+    blob = H.prepack(w_d, K, N)
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+    p.mem_format_b = "r"
+    p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, blob, N, None, 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert "ksliced" in lowoha.last_kernel()
+    sel = np.sort(rng.choice(M, 24, replace=False))
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    ph.mem_format_b = "n"
+    ph.src_scale = lowoha.QuantParam(None, capi.DT_F32, (len(sel), 1))
+    want, _, _ = _oracle(zo, ph, np.ascontiguousarray(x[sel]), w, len(sel), N, K)
+    H.check_bf16(H.to_host(dst)[sel], want)

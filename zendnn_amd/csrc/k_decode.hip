@@ -193,44 +193,8 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
     return s;
   };
 
-  if (!gated) {
-    const int32_t s = fetch(e_h);
-    const void *bias = p.bias;
-    const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
-    const bool has_bias = bias != nullptr;
-    const int64_t o = (int64_t)e_row * p.ldc + e_n;
-    const bool bf = epi.dst_dt == ZMI_DT_BF16;
-    switch (epi.fast_kind) {
-    case ZMI_EK_NONE: {
-      const float y = zmi_fast_value<ZMI_EK_NONE>(s, cc0, rs, has_rs, has_ws, has_bias);
-      if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
-      break;
-    }
-    case ZMI_EK_SWISH: {
-      const float y = zmi_fast_value<ZMI_EK_SWISH>(s, cc0, rs, has_rs, has_ws, has_bias);
-      if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
-      break;
-    }
-    case ZMI_EK_GELU_TANH: {
-      const float y = zmi_fast_value<ZMI_EK_GELU_TANH>(s, cc0, rs, has_rs, has_ws, has_bias);
-      if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
-      break;
-    }
-    default:
-      if (zmi_epilogue_is_raw_s32(epi, bias)) ((int32_t *)p.dst)[o] = s + cc0.comp;
-      else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, cc0, rs, e_row, e_n, p.dst, p.ldc));
-    }
-  } else {
-    const int half = N / 2;
-    const int32_t sg = fetch(0), su = fetch(1);
-    float gv = zmi_epilogue_value(epi, sg, cc0, rs, e_row, e_n, p.dst, p.ldc);
-    float uv = zmi_epilogue_value(epi, su, cc1, rs, e_row, e_n + half, p.dst, p.ldc);
-    if (epi.dst_dt == ZMI_DT_BF16) {
-      gv = zmi_bf16_to_f32(zmi_f32_to_bf16(gv));
-      uv = zmi_bf16_to_f32(zmi_f32_to_bf16(uv));
-    }
-    zmi_store(p.dst, epi.dst_dt, (int64_t)e_row * p.ldc + e_n, zmi_gated(epi.gated_act, gv, uv));
-  }
+  if (!gated) zmi_finish_element(p, epi, cc0, rs, fetch(e_h), e_row, e_n);
+  else zmi_finish_gated(p, epi, cc0, cc1, rs, fetch(0), fetch(1), e_row, e_n);
 }
 
 int zmi_decode_grid(const ZmiProblem &p, bool gated) {

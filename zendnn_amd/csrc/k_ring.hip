@@ -146,7 +146,7 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
                                                                                    const ZmiProblem *probs,
                                                                                    int n_prob, int n_items,
                                                                                    const int *tile_tab, int bm_idx, int top_flags,
-                                                                                   ZmiEpilogue epi) {
+                                                                                   ZmiRingSplit split, ZmiEpilogue epi) {
   using Cfg = RingCfg<BM, DEEP>;
   constexpr int MI = BM / 64, NI = 4;
   constexpr int AF = Cfg::AF, STAGE = Cfg::STAGE, NS = Cfg::NS, NPM = Cfg::NPAIR_MAX;
@@ -168,8 +168,11 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   if (tile_tab) n_items = tile_tab[bm_idx];
   const int b = blockIdx.x;
   const int per_xcd = (n_items + 7) / 8;
-  const int id = (b % 8) * per_xcd + b / 8;
-  if (b / 8 >= per_xcd || id >= n_items) return;
+  const int item = (b % 8) * per_xcd + b / 8;
+  if (b / 8 >= per_xcd || item >= n_items) return;
+  // K slices of one tile are neighbours (same XCD: their partial sums meet in one L2)
+  const int n_slice = split.slices;
+  const int id = item / n_slice, slice = item % n_slice;
   ZmiProblem p;
   int tm, tn, m0;
   {
@@ -224,7 +227,9 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
 
   const int M = p.M, N = p.N, K = p.K;
   const int K_pad = (int)zmi_blob_kpad(K);
-  const int nk = K_pad / 64;
+  const int nk_all = K_pad / 64;
+  const int k_first = (int)((int64_t)slice * nk_all / n_slice);           // this slice's stages of 64 k
+  const int nk = (int)((int64_t)(slice + 1) * nk_all / n_slice) - k_first;
   const int64_t frow_bytes = (int64_t)K_pad * 32;
   const uint8_t *Afr = (const uint8_t *)p.A;
   const uint8_t *Bfr = p.blob + zmi_blob_tiles_off(N);
@@ -268,8 +273,8 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   const int n_my = (Cfg::P - wave + 3) / 4;      // pairs this wavefront really loads
   const bool short_wave = n_my < NPM;
 
-  uint32_t voff = lane * 16;
-  const uint32_t voff_max = lane * 16 + (nk - 1) * 2048;
+  uint32_t voff = lane * 16 + k_first * 2048;
+  const uint32_t voff_max = lane * 16 + (k_first + nk - 1) * 2048;
   auto issue_all = [&](int slot) {
 #pragma unroll
     for (int j = 0; j < NPM; ++j)
@@ -323,17 +328,14 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
     }
   };
 
-  // ---- prologue: NS-1 stages in flight, the first one landed --------------------------
-#pragma unroll
-  for (int s = 0; s < NS - 1; ++s) issue_all(s);
-
-  // ---- epilogue constants, requested behind the first stages so their latency hides under the main loop:
-  // the row scales of the tile (LDS) and this lane's eight column contexts (registers)
+  // ---- epilogue constants: requested here, ahead of the first stages (so that the counted
+  // waits of the main loop cover them), as raw words that nothing touches before the main
+  // loop is over (a wait here would hold the loop back by a memory round trip per dependent
+  // load): the row scale of row `tid` of the tile and this lane's eight column constants
   float *row_scale = reinterpret_cast<float *>(smem + Cfg::ROWS_OFF);
-  for (int r = tid; r < BM; r += R_THREADS) {
-    const int m = m0 + r;
-    row_scale[r] = m < M ? zmi_row_scale(epi, p, m) : 1.0f;
-  }
+  const int rs_row = m0 + tid < M ? m0 + tid : M - 1;
+  const uint32_t rs_word = zmi_row_scale_raw(epi, p, colsum, rs_row);
+  const int32_t zp_word = zmi_zp_raw(p, colsum);
   const int hi = lane / 32, cl = lane % 32;
   const int c16 = lane % 16, r4 = lane / 16;
   const void *bias = p.bias;
@@ -343,30 +345,29 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
 
   // output columns of this lane: two runs of 4
   int n_run[2];
-  ZmiColCtx cc[2][4];
+  ZmiColRaw craw[2][4];
+  auto col_ok = [&](int n) { return n < N ? n : N - 1; };
   if (!gated) {
     n_run[0] = tn * 256 + wn * 128 + c16 * 4;
     n_run[1] = n_run[0] + 64;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) cc[h][j] = zmi_col_ctx(epi, p, colsum, n_run[h] + j, N);
   } else {
     // run 0: gate columns n, run 1: the matching up columns n + N/2; output column n
     n_run[0] = tn * 128 + wn * 64 + c16 * 4;
     n_run[1] = n_run[0] + half;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      cc[0][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j, half);
-      cc[1][j] = zmi_col_ctx(epi, p, colsum, n_run[0] + j < half ? n_run[1] + j : N, N);
-    }
   }
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) craw[h][j] = zmi_col_raw(epi, p, colsum, col_ok(n_run[h] + j));
   const int n_lim = gated ? half : N;
   // vector stores need every row start aligned
   const int es = dst_dt == ZMI_DT_BF16 ? 2 : (dst_dt == ZMI_DT_S8 || dst_dt == ZMI_DT_U8 ? 1 : 4);
   const bool vec_ok = (((uintptr_t)p.dst) % 16 == 0) && ((p.ldc * es) % 16 == 0);
   const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
 
+  // ---- prologue: NS-1 stages in flight, the first one landed --------------------------
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s) issue_all(s);
   if (short_wave) zmi_wait_vm<(NS - 2) * (NPM - 1) * 2>();
   else zmi_wait_vm<(NS - 2) * NPM * 2>();
   zmi_wg_barrier();
@@ -394,7 +395,40 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   zmi_wait_vm<0>();
   zmi_wg_barrier();
 
+  // ---- K slices: every slice leaves its int32 partial tile in the workspace, in register
+  // order (16 bytes per lane and store: whole cache lines), and is done;
+  // zmi_ring_reduce_kernel adds the slices of a tile and runs the epilogue on all CUs.
+  if (BM != 256 && n_slice > 1) {   // (256-row tiles are chosen only when they cover the CUs)
+    constexpr int CH = NI * MI * 4;   // 16-byte chunks per lane
+    int32_t *mine = split.partial + (((int64_t)id * n_slice + slice) * 4 + wave) * (CH * 256) + lane * 4;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const v4i o = {acc[ni][mi][g * 4], acc[ni][mi][g * 4 + 1], acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]};
+          *zmi_global<v4i>(mine + ((ni * MI + mi) * 4 + g) * 256) = o;
+        }
+    return;
+  }
+
   // ------------------------------------------------------------------------ epilogue
+  // decode the constants requested in the prologue
+  if (tid < BM) row_scale[tid] = m0 + tid < M ? zmi_row_scale_from_raw(epi, p, rs_word, rs_row) : 1.0f;
+  ZmiColCtx cc[2][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (!gated) {
+      cc[0][j] = zmi_col_ctx_raw(epi, p, craw[0][j], zp_word, n_run[0] + j, col_ok(n_run[0] + j), N);
+      cc[1][j] = zmi_col_ctx_raw(epi, p, craw[1][j], zp_word, n_run[1] + j, col_ok(n_run[1] + j), N);
+    } else {
+      cc[0][j] = zmi_col_ctx_raw(epi, p, craw[0][j], zp_word, n_run[0] + j, col_ok(n_run[0] + j), half);
+      cc[1][j] = zmi_col_ctx_raw(epi, p, craw[1][j], zp_word, n_run[0] + j < half ? n_run[1] + j : N,
+                                 col_ok(n_run[1] + j), N);
+    }
+  }
+  __syncthreads();
   int32_t *stage = reinterpret_cast<int32_t *>(smem) + wave * R_EPI_WAVE_WORDS;
   // the bf16 fast forms multiply / add unconditionally: absent scales are 1, an absent bias is -0
   if (dst_dt == ZMI_DT_BF16 && epi.fast_kind != ZMI_EK_GENERIC) {
@@ -592,6 +626,81 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   }
 }
 
+// Second step of a K-sliced launch: adds the partial tiles of the slices and finishes the
+// elements.  One wavefront per 16-byte chunk column of a tile: lane l of chunk (wave w,
+// ni, mi, g) holds row (w/2)*(BM/2) + mi*32 + l%32 and the four columns from
+// (w%2)*128 + ni*32 + g*8 + (l/32)*4 of the tile, as the MFMA left them.
+template <int BM>
+__global__ __launch_bounds__(R_THREADS) void zmi_ring_reduce_kernel(ZmiProblem p, int top_flags, ZmiRingSplit split,
+                                                                    ZmiEpilogue epi) {
+  constexpr int MI = BM / 64, NI = 4, CH = NI * MI * 4;
+  const int top = top_flags & 0xffff;
+  const int lane = threadIdx.x % 64;
+  const bool gated = epi.gated_act != 0;
+  const int NIU = gated ? 2 : NI;                         // gated: ni = 0, 1 pair with ni + 2
+  const int units_per_tile = 4 * NIU * MI * 4;            // wavefront units: (w, ni, mi, g)
+  const int unit = blockIdx.x * (R_THREADS / 64) + threadIdx.x / 64;
+  const int tile = unit / units_per_tile;
+  int full; bool rem;
+  zmi_ring_rows<BM>(p.M, top_flags, full, rem);
+  const int tiles_m = full + (rem ? 1 : 0);
+  const int ncols = gated ? p.N / 2 : p.N;
+  const int per = gated ? 128 : 256;
+  const int tiles_n = (ncols + per - 1) / per;
+  if (tile >= tiles_m * tiles_n) return;
+  // same tile numbering as the GEMM kernel
+  const int GM = tiles_m < 8 ? tiles_m : 8;
+  const int per_group = GM * tiles_n;
+  const int first_m = (tile / per_group) * GM;
+  const int gm = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+  const int r = tile % per_group;
+  const int tm = first_m + r % gm, tn = r / gm;
+  const int m0 = tm < full ? tm * top : (p.M / top) * top;
+
+  int u = unit % units_per_tile;
+  const int g = u % 4; u /= 4;
+  const int mi = u % MI; u /= MI;
+  const int ni = u % NIU; u /= NIU;
+  const int w = u, wm = w / 2, wn = w % 2;
+
+  const int m = m0 + wm * (BM / 2) + mi * 32 + lane % 32;
+  const int cin = ni * 32 + g * 8 + (lane / 32) * 4;      // column inside the wavefront's 128
+  v4i sum[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  for (int s = 0; s < split.slices; ++s) {
+    const int32_t *base = split.partial + (((int64_t)tile * split.slices + s) * 4 + w) * (CH * 256) + lane * 4;
+    const v4i a = *zmi_global<const v4i>(base + ((ni * MI + mi) * 4 + g) * 256);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum[0][j] += a[j];
+    if (gated) {
+      const v4i b = *zmi_global<const v4i>(base + (((ni + 2) * MI + mi) * 4 + g) * 256);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum[1][j] += b[j];
+    }
+  }
+  if (m >= p.M) return;
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+  const float rs = zmi_row_scale(epi, p, m);
+  if (!gated) {
+    const int n0 = tn * 256 + wn * 128 + cin;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + j;
+      if (n >= p.N) break;
+      zmi_finish_element(p, epi, zmi_col_ctx(epi, p, colsum, n, p.N), rs, sum[0][j], m, n);
+    }
+  } else {
+    const int half = p.N / 2;
+    const int n0 = tn * 128 + wn * 64 + cin;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + j;
+      if (n >= half) break;
+      zmi_finish_gated(p, epi, zmi_col_ctx(epi, p, colsum, n, half), zmi_col_ctx(epi, p, colsum, n + half, p.N), rs,
+                       sum[0][j], sum[1][j], m, n);
+    }
+  }
+}
+
 // Tile table of a problem set, computed where the row counts live: tab[0..2] = number of
 // tiles of the 256 / 128 / 64 row kernels, tab[4 + b * n_prob + e] = index of the first
 // tile of problem e in kernel b.  One wavefront, 64 problems per step.
@@ -626,9 +735,19 @@ __global__ __launch_bounds__(64) void zmi_ring_count_kernel(const ZmiProblem *pr
   if (lane == 0) { tab[0] = run[0]; tab[1] = run[1]; tab[2] = run[2]; }
 }
 
+static int ring_cu_count() {
+  static const int n_cu = [] {
+    int dev = 0, n = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    return n;
+  }();
+  return n_cu;
+}
+
 template <int BM, bool DEEP>
 static hipError_t ring_launch_cfg(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items,
-                                  const int *tile_tab, int top, const ZmiEpilogue &epi, hipStream_t stream) {
+                                  const int *tile_tab, int top, const ZmiRingSplit &split, const ZmiEpilogue &epi,
+                                  hipStream_t stream) {
   const size_t smem = RingCfg<BM, DEEP>::SMEM;
   static bool attr_done = false;
   if (!attr_done) {
@@ -639,24 +758,22 @@ static hipError_t ring_launch_cfg(const ZmiProblem &p0, const ZmiProblem *probs,
   }
   const int grid = (n_items + 7) / 8 * 8;   // a multiple of 8 so the XCD renumbering applies
   hipLaunchKernelGGL((zmi_gemm_ring_kernel<BM, DEEP>), dim3(grid), dim3(R_THREADS), smem, stream, p0, probs, n_prob,
-                     n_items, tile_tab, BM == 256 ? 0 : (BM == 128 ? 1 : 2), top, epi);
+                     n_items, tile_tab, BM == 256 ? 0 : (BM == 128 ? 1 : 2), top, split, epi);
   return hipGetLastError();
 }
 
 template <int BM>
 static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items, bool exact,
-                              const int *tile_tab, int top, const ZmiEpilogue &epi, hipStream_t stream) {
+                              const int *tile_tab, int top, const ZmiRingSplit &split, const ZmiEpilogue &epi,
+                              hipStream_t stream) {
   if (n_items <= 0) return hipSuccess;
+  n_items *= split.slices;
   // at most one workgroup per CU anyway: let it have the whole LDS for its ring
-  static const int n_cu = [] {
-    int dev = 0, n = 256;
-    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    return n;
-  }();
+  const int n_cu = ring_cu_count();
   (void)exact;   // a bound that fits one workgroup per CU is as good as the exact count
   if (BM != 256 && n_items <= n_cu)
-    return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, epi, stream);
-  return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, epi, stream);
+    return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
+  return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
 }
 
 // Largest tile height for a problem set: 256-row tiles once they fill the chip,
@@ -679,18 +796,65 @@ int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool
   return (avg <= 64 ? 64 : 128) | ZMI_RING_PAD;
 }
 
+// One problem: tile height and K slices.  A problem whose tiles cover only a fraction of
+// the CUs is bound by the latency of its few weight streams: each tile is then split over
+// K, at the price of a second launch that re-reads the int32 partial tiles.  Measured on
+// MI355X (K = 4096, N = 4096 / 14336, M = 32 .. 1024): four slices pay off up to a quarter
+// of the CUs' worth of tiles (16 .. 64 tiles: 42 -> 34 us, 50 -> 45 us per call); two or
+// eight slices, or slicing 112 and more tiles, lose to the unsliced launch.
+ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices) {
+  ZmiRingPlan plan;
+  plan.top = top_hint ? top_hint : zmi_ring_pick_top(M, N);
+  plan.slices = 1;
+  plan.partial_bytes = 0;
+  const int64_t tiles_n = (N + 255) / 256;
+  plan.tiles = (int)(((M + plan.top - 1) / plan.top) * tiles_n);
+  if (M <= 0) return plan;
+  const int n_cu = ring_cu_count();
+  const int nk = (int)(zmi_blob_kpad(K) / 64);
+  const int top = M <= 64 ? 64 : 128;
+  const int64_t tiles = ((M + top - 1) / top) * tiles_n;
+  int slices = 1;
+  if (force_slices > 0) slices = force_slices;
+  else if (tiles * 4 <= n_cu && nk >= 16) slices = 4;
+  if (slices > nk) slices = nk;
+  if (slices < 2) return plan;
+  plan.top = top | ZMI_RING_PAD;
+  plan.slices = slices;
+  plan.tiles = (int)tiles;
+  plan.partial_bytes = (size_t)tiles * slices * top * 256 * sizeof(int32_t);
+  return plan;
+}
+
 // One problem, M rows in fragment-major order at p.A.
-hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream) {
+hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, const ZmiRingSplit *split,
+                                hipStream_t stream) {
   if (p.M <= 0) return hipSuccess;
   const bool gated = epi.gated_act != 0;
+  ZmiRingSplit sp = {1, nullptr};
+  if (split && split->slices > 1) {
+    // sliced launches are one launch: the remainder rows stay with the top-height kernel
+    if (!(top & ZMI_RING_PAD) || (top & 0xffff) == 256 || !split->partial) return hipErrorInvalidValue;
+    if (split->slices > (int)(zmi_blob_kpad(p.K) / 64)) return hipErrorInvalidValue;
+    sp = *split;
+  }
   hipError_t e = hipSuccess;
   if ((top & 0xffff) == 256) {
-    e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), true, nullptr, top, epi, stream);
+    e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
     if (e != hipSuccess) return e;
   }
-  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, epi, stream);
+  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
   if (e != hipSuccess) return e;
-  return ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, epi, stream);
+  e = ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
+  if (e != hipSuccess || sp.slices == 1) return e;
+  // the slices' partial tiles -> finished elements
+  const int th = top & 0xffff;
+  const int tiles = th == 128 ? zmi_ring_items<128>(p.M, p.N, top, gated) : zmi_ring_items<64>(p.M, p.N, top, gated);
+  const int units = tiles * 4 * (gated ? 2 : 4) * (th / 64) * 4;
+  const int grid = (units + R_THREADS / 64 - 1) / (R_THREADS / 64);
+  if (th == 128) hipLaunchKernelGGL(zmi_ring_reduce_kernel<128>, dim3(grid), dim3(R_THREADS), 0, stream, p, top, sp, epi);
+  else hipLaunchKernelGGL(zmi_ring_reduce_kernel<64>, dim3(grid), dim3(R_THREADS), 0, stream, p, top, sp, epi);
+  return hipGetLastError();
 }
 
 // Every problem of the table.  probs_host mirrors probs_dev and sizes the grids; when it is
@@ -726,12 +890,13 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
   hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0, tab_dev);
   const bool exact = probs_host != nullptr;
   ZmiProblem dummy = {};
+  const ZmiRingSplit whole = {1, nullptr};
   hipError_t e = hipSuccess;
   if ((top & 0xffff) == 256) {
-    e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], exact, tab_dev, top, epi, stream);
+    e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], exact, tab_dev, top, whole, epi, stream);
     if (e != hipSuccess) return e;
   }
-  e = ring_launch<128>(dummy, probs_dev, n_prob, items[1], exact, tab_dev, top, epi, stream);
+  e = ring_launch<128>(dummy, probs_dev, n_prob, items[1], exact, tab_dev, top, whole, epi, stream);
   if (e != hipSuccess) return e;
-  return ring_launch<64>(dummy, probs_dev, n_prob, items[2], exact, tab_dev, top, epi, stream);
+  return ring_launch<64>(dummy, probs_dev, n_prob, items[2], exact, tab_dev, top, whole, epi, stream);
 }

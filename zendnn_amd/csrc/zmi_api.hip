@@ -225,38 +225,56 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
   return ZMI_SUCCESS;
 }
 
-static int pick_top(int M, int N) {
+// Tile height and K slices of a one-problem ring launch.  ZMI_GEMM_TOP (128 / 256) and
+// ZMI_RING_SPLITK (1 = never slice, n = n slices) override the choice; the tests use them
+// to reach every kernel configuration with small shapes.
+ZmiRingPlan plan_ring_gemm(int M, int N, int K) {
+  int top_hint = 0, force = 0;
   if (const char *env = std::getenv("ZMI_GEMM_TOP")) {
-    int v = std::atoi(env);
-    if (v == 128 || v == 256) return v;
+    const int v = std::atoi(env);
+    if (v == 128 || v == 256) top_hint = v;
   }
-  return zmi_ring_pick_top(M, N);
+  if (const char *env = std::getenv("ZMI_RING_SPLITK")) force = std::atoi(env);
+  return zmi_ring_plan(M, N, K, top_hint, force);
 }
 
-int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi) {
+int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
   if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
     set_kernel_name("decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
-  } else if (!use_ring_kernel(prob.M)) {
+  } else if (!use_ring_kernel(prob.M, prob.N)) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
   } else {
     // prob.A is fragment-major here (see use_ring_kernel)
-    const int top = pick_top(prob.M, epi.gated_act ? prob.N / 2 : prob.N);
-    set_kernel_name(top == 256 ? "ring_mfma32x32x32_top256" : "ring_mfma32x32x32_top128");
-    if (!hip_ok(zmi_launch_gemm_ring(prob, epi, top, stream()), "MFMA GEMM launch")) return ZMI_FAILURE;
+    if (!plan) { set_error("ring GEMM without a launch plan"); return ZMI_FAILURE; }
+    ZmiRingSplit split = {1, nullptr};
+    if (plan->slices > 1) {
+      // (the scratch arena was sized for the partial tiles by the caller)
+      split.slices = plan->slices;
+      split.partial = (int32_t *)arena().alloc(plan->partial_bytes);
+      if (!split.partial) { set_error("no scratch for the K-sliced GEMM"); return ZMI_FAILURE; }
+    }
+    const int th = plan->top & 0xffff;
+    set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")
+                                     : (th == 256 ? "ring_mfma32x32x32_top256" : "ring_mfma32x32x32_top128"));
+    if (!hip_ok(zmi_launch_gemm_ring(prob, epi, plan->top, &split, stream()), "MFMA GEMM launch")) return ZMI_FAILURE;
   }
   return ZMI_SUCCESS;
 }
 
 // Problems with more rows than the small-M kernels take run on the MFMA-bound
 // kernel, which reads the activations in fragment-major order.
-bool use_ring_kernel(int M) {
-  static const int min_m = [] {
-    const char *env = std::getenv("ZMI_RING_MIN_M");
-    return env ? std::atoi(env) : 129;
-  }();
-  return M >= min_m;
+bool use_ring_kernel(int M, int N) {
+  // ZMI_RING_MIN_M overrides the choice (the tests reach the 64-row tile through it)
+  if (const char *env = std::getenv("ZMI_RING_MIN_M")) {
+    const int min_m = std::atoi(env);
+    if (min_m > 0) return M >= min_m;
+  }
+  // Above 128 rows always.  From 65 rows the K-sliced ring launch beats the small-M kernel
+  // once the output is wide enough for that kernel's per-row cost to show (measured:
+  // M = 128: N = 4096 36 vs 34 us, N = 14336 74 vs 45 us per call).
+  return M > 128 || (M > 64 && (int64_t)M * N >= 96 * 8192);
 }
 
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
@@ -339,7 +357,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                          std::min(weight_cache_env(), p.weight_cache_type) > 0;
   const bool pack_in_arena = p.mem_format_b != 'r' && !use_cache;
   const int64_t K16 = zmi_round_up(K, 16);
-  const bool ring = use_ring_kernel(M);
+  const bool ring = use_ring_kernel(M, N);
   const int64_t frag_kpad = ring ? zmi_blob_kpad(K) : 0;
   const size_t a_bytes = ring ? (size_t)zmi_afrag_bytes(M, K) : (size_t)M * K16;
   const bool repack_a = !dyn && (ring || a_needs_repack(src, lda, K, transA != 0));
@@ -347,6 +365,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (pack_in_arena) need += Arena::padded((size_t)zmi_blob_bytes(K, N));
   if (dyn) need += Arena::padded(a_bytes) + Arena::padded(sizeof(float) * (size_t)M) + 256;
   if (repack_a) need += Arena::padded(a_bytes);
+  ZmiRingPlan plan = {};
+  if (ring) {
+    plan = plan_ring_gemm(M, N, K);
+    need += Arena::padded(plan.partial_bytes);
+  }
   if (!arena().begin(need)) return ZMI_FAILURE;
 
   // ---- weights ----
@@ -446,7 +469,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       st = hip_ok(zmi_launch_gemm_smallm_fused(prob, epi, fused, stream()), "fused small-M GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
     }
   } else {
-    st = run_single_gemm(prob, epi);
+    st = run_single_gemm(prob, epi, ring ? &plan : nullptr);
   }
   upload_fence();
   return st;

@@ -267,6 +267,84 @@ __device__ __forceinline__ ZmiColCtx zmi_col_ctx(const ZmiEpilogue &e, const Zmi
   return c;
 }
 
+// ---- the same constants, requested early and decoded late ------------------------------------
+// A kernel that must not wait in its prologue fetches the aligned 32-bit word that holds an
+// element (an aligned word never leaves the element's page) and picks the element out of it
+// when the epilogue starts.  The request is one instruction whatever the element type is and
+// is issued whether or not the array exists (then from `fallback`, any readable word), so
+// the requests form a branch-free run of loads that nothing waits on.
+__device__ __forceinline__ int zmi_log2_size(int dt) {
+  return dt == ZMI_DT_BF16 ? 1 : (dt == ZMI_DT_S8 || dt == ZMI_DT_U8) ? 0 : 2;
+}
+__device__ __forceinline__ uint32_t zmi_ld_word(const void *p, const void *fallback, int dt, int64_t i) {
+  const uintptr_t addr = p ? (uintptr_t)p + ((uintptr_t)i << zmi_log2_size(dt)) : (uintptr_t)fallback;
+  return *(ZMI_GLOBAL const uint32_t *)(addr & ~(uintptr_t)3);
+}
+__device__ __forceinline__ float zmi_word_f32(uint32_t word, const void *p, int dt, int64_t i) {
+  const uintptr_t addr = (uintptr_t)p + ((uintptr_t)i << zmi_log2_size(dt));
+  const uint32_t raw = word >> ((uint32_t)(addr & 3) * 8);
+  switch (dt) {
+  case ZMI_DT_BF16: return __uint_as_float(raw << 16);
+  case ZMI_DT_S32: return (float)(int32_t)raw;
+  case ZMI_DT_S8: return (float)(int8_t)raw;
+  case ZMI_DT_U8: return (float)(uint8_t)raw;
+  default: return __uint_as_float(raw);
+  }
+}
+
+struct ZmiColRaw {
+  uint32_t wscale, bias;
+  int32_t colsum;
+};
+// n_ok: a column index that exists (the caller clamps); the decode step below knows whether
+// the lane's real column does.
+__device__ __forceinline__ ZmiColRaw zmi_col_raw(const ZmiEpilogue &e, const ZmiProblem &p, const int32_t *colsum,
+                                                 int n_ok) {
+  ZmiColRaw r;
+  r.wscale = zmi_ld_word(p.wei_scale_ptr, colsum, e.wei_scale_dt, e.wei_scale_mode == 1 ? 0 : n_ok);
+  r.bias = zmi_ld_word(p.bias, colsum, e.bias_dt, n_ok);
+  r.colsum = *(ZMI_GLOBAL const int32_t *)(uintptr_t)(colsum + n_ok);
+  return r;
+}
+__device__ __forceinline__ int32_t zmi_zp_raw(const ZmiProblem &p, const int32_t *colsum) {
+  return *(ZMI_GLOBAL const int32_t *)(uintptr_t)(p.src_zp_ptr ? p.src_zp_ptr : colsum);
+}
+// Same result as zmi_col_ctx(e, p, colsum, n, N) from the words fetched for column n_ok.
+__device__ __forceinline__ ZmiColCtx zmi_col_ctx_raw(const ZmiEpilogue &e, const ZmiProblem &p, const ZmiColRaw &r,
+                                                     int32_t zp_raw, int n, int n_ok, int N) {
+  ZmiColCtx c;
+  c.wscale = 1.0f;
+  c.bias = 0.0f;
+  c.comp = 0;
+  c.shift = 0;
+  if (n < N) {
+    if (e.wei_scale_mode) {
+      c.wscale = p.wei_scale_ptr ? zmi_word_f32(r.wscale, p.wei_scale_ptr, e.wei_scale_dt, e.wei_scale_mode == 1 ? 0 : n_ok)
+                                 : p.wei_scale_val;
+    }
+    if (p.bias) c.bias = zmi_word_f32(r.bias, p.bias, e.bias_dt, n_ok);
+    int32_t k = p.a_is_u8 ? 128 : 0;
+    if (e.has_zp) k -= p.src_zp_ptr ? zp_raw : p.src_zp_val;
+    if (k) c.comp = k * r.colsum;
+    if (p.a_is_u8) c.shift = 128 * r.colsum;
+  }
+  return c;
+}
+__device__ __forceinline__ uint32_t zmi_row_scale_raw(const ZmiEpilogue &e, const ZmiProblem &p, const void *fallback,
+                                                      int m_ok) {
+  const bool have = e.src_scale_mode == ZMI_SS_TENSOR_PTR || e.src_scale_mode == ZMI_SS_TOKEN_PTR;
+  return zmi_ld_word(have ? p.src_scale_ptr : nullptr, fallback, e.src_scale_dt,
+                     e.src_scale_mode == ZMI_SS_TOKEN_PTR ? m_ok : 0);
+}
+__device__ __forceinline__ float zmi_row_scale_from_raw(const ZmiEpilogue &e, const ZmiProblem &p, uint32_t raw, int m_ok) {
+  switch (e.src_scale_mode) {
+  case ZMI_SS_VALUE: return p.src_scale_val;
+  case ZMI_SS_TENSOR_PTR: return zmi_word_f32(raw, p.src_scale_ptr, e.src_scale_dt, 0);
+  case ZMI_SS_TOKEN_PTR: return zmi_word_f32(raw, p.src_scale_ptr, e.src_scale_dt, m_ok);
+  default: return 1.0f;
+  }
+}
+
 __device__ __forceinline__ float zmi_row_scale(const ZmiEpilogue &e, const ZmiProblem &p, int m) {
   switch (e.src_scale_mode) {
   case ZMI_SS_VALUE: return p.src_scale_val;
@@ -392,5 +470,47 @@ __device__ __forceinline__ void zmi_store(void *dst, int dt, int64_t i, float y)
 __device__ __forceinline__ bool zmi_epilogue_is_raw_s32(const ZmiEpilogue &e, const void *bias) {
   return e.dst_dt == ZMI_DT_S32 && !e.src_scale_mode && !e.wei_scale_mode && !bias && !e.n_po &&
          !e.has_dst_q && e.alpha == 1.0f && e.beta == 0.0f;
+}
+
+// One finished output element: accumulator -> epilogue -> store at dst[m * ldc + n].  The
+// kernels that produce one element per thread (decode, the K-slice reduction) end here.
+__device__ __forceinline__ void zmi_finish_element(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &c,
+                                                   float rs, int32_t s, int m, int n) {
+  const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+  const bool has_bias = p.bias != nullptr;
+  const int64_t o = (int64_t)m * p.ldc + n;
+  const bool bf = epi.dst_dt == ZMI_DT_BF16;
+  switch (epi.fast_kind) {
+  case ZMI_EK_NONE: {
+    const float y = zmi_fast_value<ZMI_EK_NONE>(s, c, rs, has_rs, has_ws, has_bias);
+    if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+    break;
+  }
+  case ZMI_EK_SWISH: {
+    const float y = zmi_fast_value<ZMI_EK_SWISH>(s, c, rs, has_rs, has_ws, has_bias);
+    if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+    break;
+  }
+  case ZMI_EK_GELU_TANH: {
+    const float y = zmi_fast_value<ZMI_EK_GELU_TANH>(s, c, rs, has_rs, has_ws, has_bias);
+    if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
+    break;
+  }
+  default:
+    if (zmi_epilogue_is_raw_s32(epi, p.bias)) ((int32_t *)p.dst)[o] = s + c.comp;
+    else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, c, rs, m, n, p.dst, p.ldc));
+  }
+}
+// Gated pair: sg / su are the accumulators of weight columns n (gate) and n + N/2 (up);
+// the output column is n.
+__device__ __forceinline__ void zmi_finish_gated(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &cg,
+                                                 const ZmiColCtx &cu, float rs, int32_t sg, int32_t su, int m, int n) {
+  float gv = zmi_epilogue_value(epi, sg, cg, rs, m, n, p.dst, p.ldc);
+  float uv = zmi_epilogue_value(epi, su, cu, rs, m, n + p.N / 2, p.dst, p.ldc);
+  if (epi.dst_dt == ZMI_DT_BF16) {
+    gv = zmi_bf16_to_f32(zmi_f32_to_bf16(gv));
+    uv = zmi_bf16_to_f32(zmi_f32_to_bf16(uv));
+  }
+  zmi_store(p.dst, epi.dst_dt, (int64_t)m * p.ldc + n, zmi_gated(epi.gated_act, gv, uv));
 }
 #endif  // __HIPCC__

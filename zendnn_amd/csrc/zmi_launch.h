@@ -44,7 +44,25 @@ hipError_t zmi_launch_quant_tensor(const void *src, int32_t src_dt, int64_t M, i
 // k_ring.hip: A in fragment-major order; `top` is the largest tile height (128 or 256)
 int zmi_ring_pick_top(int64_t rows, int64_t out_cols);
 int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated);
-hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, hipStream_t stream);
+// K slices of a one-problem ring launch.  When a problem has fewer tiles than the device
+// has CUs, every tile is computed by `slices` workgroups, each over its own range of K;
+// they leave int32 partial tiles in `partial`, and a second kernel adds the slices of each
+// tile and runs the epilogue.
+struct ZmiRingSplit {
+  int slices;              // 1: no slicing, the pointer is unused
+  int32_t *partial;        // tiles * slices * tile rows * 256 words
+};
+struct ZmiRingPlan {
+  int top;                 // tile height (with ZMI_RING_PAD when slices > 1)
+  int slices;
+  int tiles;
+  size_t partial_bytes;    // 0 when slices == 1
+};
+// top_hint: tile height to use when the launch is not sliced (0: zmi_ring_pick_top);
+// force_slices: 0 = choose, n = that many slices where the shape allows it.
+ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices);
+hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, const ZmiRingSplit *split,
+                                hipStream_t stream);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev,
                                       const ZmiEpilogue &epi, hipStream_t stream);
