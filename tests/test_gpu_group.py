@@ -172,3 +172,28 @@ def test_device_routing_matches_host_scatter(zo):
     assert torch.equal(out2.view(torch.int16), d.out.view(torch.int16))
     want = MH.oracle_moe(zo, c, list(range(c.T)))
     check_moe_out(H.to_host(out2), want)
+
+
+@pytest.mark.parametrize("T,topk,E", [(7, 1, 3), (500, 2, 8), (4096, 6, 64),
+                                      (5000, 8, 64),                            # segments longer than the register window
+                                      (700, 4, 65), (3000, 8, 200)])
+def test_route_is_a_stable_counting_sort(zo, T, topk, E):
+    """zmi_moe_route: counts, offsets and slots are those of a stable sort of the (t, k) entries
+    by expert; ids outside [0, E) get slot -1 and are not counted."""
+    rng = np.random.default_rng(T + topk + E)
+    p = rng.dirichlet(np.full(E, 0.3))                       # skewed: some experts empty, some crowded
+    ids = rng.choice(E, size=(T, topk), p=p).astype(np.int32)
+    bad = rng.random((T, topk)) < 0.01
+    ids[bad] = rng.choice([-1, E, E + 5], size=int(bad.sum()))
+    st, counts, offsets, slot_of = lowoha.moe_route(H.to_dev(ids), E)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    flat = ids.reshape(-1)
+    ok = (flat >= 0) & (flat < E)
+    want_counts = np.bincount(flat[ok], minlength=E)
+    want_off = np.concatenate([[0], np.cumsum(want_counts)])
+    order = np.argsort(np.where(ok, flat, E), kind="stable")[: int(ok.sum())]
+    want_slot = np.full(flat.shape, -1, dtype=np.int64)
+    want_slot[order] = np.arange(order.size)
+    assert np.array_equal(H.to_host(counts), want_counts)
+    assert np.array_equal(H.to_host(offsets), want_off)
+    assert np.array_equal(H.to_host(slot_of), want_slot)

@@ -133,7 +133,7 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
 // ---------------------------------------------------------------------------
 // Routing.  One workgroup of 16 wavefronts; wavefront w owns the contiguous
 // segment w of the flat (t,k) index space.
-//   A: per-wavefront histograms hist[w][e] (LDS atomics);
+//   A: per-wavefront histograms hist[w][e];
 //   B: counts / exclusive offsets per expert, and cursor[w][e] = offsets[e] +
 //      sum of hist[w'][e] for w' < w;
 //   C: every wavefront walks its segment in order, 64 entries at a time; an
@@ -141,6 +141,7 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
 // The order inside an expert is therefore the (t,k) order: deterministic.
 // ---------------------------------------------------------------------------
 #define RT_WAVES 16
+#define RT_KEEP 24   // ids kept per lane: 24 x 64 x 16 = 24576 entries without a second read
 
 __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int32_t *topk_ids, int n, int E,
                                                                       int align, int32_t *counts,
@@ -150,16 +151,30 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
   int32_t *hist = sh;
   int32_t *off = sh + RT_WAVES * E;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  int ebits = 1;
+  while ((1 << ebits) < E) ++ebits;          // expert ids fit in ebits bits
   if (src_of)
     for (int i = tid; i < n_slots; i += blockDim.x) src_of[i] = -1;
   for (int i = tid; i < RT_WAVES * E; i += blockDim.x) hist[i] = 0;
   __syncthreads();
   const int seg = (n + RT_WAVES - 1) / RT_WAVES;
   const int s0 = wave * seg, s1 = (s0 + seg < n) ? s0 + seg : n;
-  for (int i = s0 + lane; i < s1; i += 64) {
-    const int e = topk_ids[i];
-    if (e >= 0 && e < E) atomicAdd(&hist[wave * E + e], 1);
+  // The segment's ids are read once, all loads in flight together, and kept in registers
+  // for both passes (RT_KEEP x 64 per wavefront; what a longer segment has beyond that is
+  // read again in pass C).
+  int keep[RT_KEEP];
+#pragma unroll
+  for (int it = 0; it < RT_KEEP; ++it) {
+    const int i = s0 + it * 64 + lane;
+    keep[it] = i < s1 ? topk_ids[i] : -1;
   }
+  auto count = [&](int e) {
+    if (e >= 0 && e < E) atomicAdd(&hist[wave * E + e], 1);
+  };
+#pragma unroll
+  for (int it = 0; it < RT_KEEP; ++it)
+    if (s0 + it * 64 < s1) count(keep[it]);
+  for (int i0 = s0 + RT_KEEP * 64; i0 < s1; i0 += 64) count(i0 + lane < s1 ? topk_ids[i0 + lane] : -1);
   __syncthreads();
   // per-expert totals and the per-wavefront running starts (thread e handles expert e)
   for (int e = tid; e < E; e += blockDim.x) {
@@ -180,12 +195,8 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
     offsets[E] = run;
   }
   __syncthreads();
-  int ebits = 1;
-  while ((1 << ebits) < E) ++ebits;          // expert ids fit in ebits bits
-  for (int i0 = s0; i0 < s1; i0 += 64) {
-    const int i = i0 + lane;
+  auto place = [&](int i, int e) {
     const bool live = i < s1;
-    int e = live ? topk_ids[i] : -1;
     const bool ok = live && e >= 0 && e < E;
     if (!ok) e = -1;
     // lanes holding the same expert as this lane
@@ -206,6 +217,13 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
       slot_of[i] = -1;
     }
     __builtin_amdgcn_wave_barrier();
+  };
+#pragma unroll
+  for (int it = 0; it < RT_KEEP; ++it)
+    if (s0 + it * 64 < s1) place(s0 + it * 64 + lane, keep[it]);
+  for (int i0 = s0 + RT_KEEP * 64; i0 < s1; i0 += 64) {
+    const int i = i0 + lane;
+    place(i, i < s1 ? topk_ids[i] : -1);
   }
 }
 

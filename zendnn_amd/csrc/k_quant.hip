@@ -146,7 +146,7 @@ __global__ __launch_bounds__(QT_THREADS) void zmi_quant_rows_kernel(ZmiQuantMat 
 // starting at 16 q + 1024 step, i.e. exactly one 16-byte chunk of the fragment
 // layout, and the 8 threads of one q write 8 consecutive chunks (128 bytes).
 // The rows are read twice (absmax, then quantize); the second read hits L2.
-template <bool BF16>
+template <bool BF16, int FR_STEPS>
 __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat mat0, const ZmiQuantMat *mats, int n_mat,
                                                               int scale_dt) {
   __shared__ float red[FR_THREADS / 64][8];
@@ -219,8 +219,9 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
     *(v4i *)(m.dst + zmi_afrag_off(r, k, m.frag_kpad)) = o;
   };
   // rows of up to FR_STEPS * FR_THREADS * 2 elements stay in registers between the two passes
-  // (bf16 only: 8 registers per step); longer rows are read twice, the second time from L2
-  constexpr int FR_STEPS = 8;
+  // (bf16 only: 8 registers per step; FR_STEPS is the smallest of 2 / 4 / 8 that holds the row,
+  // so that short rows leave registers for more workgroups per CU); longer rows are read
+  // twice, the second time from L2
   const bool in_regs = BF16 && K <= FR_STEPS * FR_THREADS * 2;
   v4i keep[FR_STEPS][2];
   float amax = 0.0f;
@@ -295,6 +296,18 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
   }
 }
 
+// launches the 8-row kernel with the smallest register window that holds a row
+template <bool BF16>
+static void zmi_quant_frag8_launch(unsigned grid, hipStream_t stream, const ZmiQuantMat &m0, const ZmiQuantMat *mats,
+                                   int n_mat, int scale_dt, int64_t k_max) {
+  if (k_max <= 2 * FR_THREADS * 2)
+    hipLaunchKernelGGL((zmi_quant_frag8_kernel<BF16, 2>), dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats, n_mat, scale_dt);
+  else if (k_max <= 4 * FR_THREADS * 2)
+    hipLaunchKernelGGL((zmi_quant_frag8_kernel<BF16, 4>), dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats, n_mat, scale_dt);
+  else
+    hipLaunchKernelGGL((zmi_quant_frag8_kernel<BF16, 8>), dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats, n_mat, scale_dt);
+}
+
 static bool zmi_quant_frag8_ok(const void *src, int64_t K, int64_t ld_src, int32_t src_dt) {
   const int64_t es = src_dt == ZMI_DT_BF16 ? 2 : 4;
   return K % 16 == 0 && ((uintptr_t)src) % 16 == 0 && (ld_src * es) % 16 == 0;
@@ -308,12 +321,14 @@ hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int
   m.src = src; m.dst = dst; m.scale = scales; m.ld_src = ld_src; m.ld_dst = ld_dst;
   m.M = (int32_t)M; m.K = (int32_t)K; m.row_start = 0; m.frag_kpad = (int32_t)frag_kpad;
   m.gather = nullptr; m.gather_div = 1;
-  if (frag_kpad && zmi_quant_frag8_ok(src, K, ld_src, src_dt)) {
+  // Up to a few thousand rows one workgroup per row wins, also for fragment-major output
+  // (measured on MI355X, K = 4096: 4 .. 5 us per call less at 128 .. 1024 rows, 1 us less at
+  // 2048); the wider stores of the 8-rows-per-workgroup kernel pay once the launch is large
+  // (26000 rows x 1408: 40 us against 63 us).
+  if (frag_kpad && M > 2048 && zmi_quant_frag8_ok(src, K, ld_src, src_dt)) {
     const unsigned grid = (unsigned)((M + 7) / 8);
-    if (src_dt == ZMI_DT_BF16)
-      hipLaunchKernelGGL(zmi_quant_frag8_kernel<true>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, scale_dt);
-    else
-      hipLaunchKernelGGL(zmi_quant_frag8_kernel<false>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, scale_dt);
+    if (src_dt == ZMI_DT_BF16) zmi_quant_frag8_launch<true>(grid, stream, m, nullptr, 1, scale_dt, K);
+    else zmi_quant_frag8_launch<false>(grid, stream, m, nullptr, 1, scale_dt, K);
     return hipGetLastError();
   }
   if (src_dt == ZMI_DT_BF16)
@@ -336,10 +351,9 @@ hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_
   if (rows8) {
     // every matrix is fragment-major, eligible for the 8-row kernel, and starts at a multiple of 8 rows
     const unsigned grid = (unsigned)((total_rows + 7) / 8);
-    if (src_dt == ZMI_DT_BF16)
-      hipLaunchKernelGGL(zmi_quant_frag8_kernel<true>, dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats_dev, n_mat, scale_dt);
-    else
-      hipLaunchKernelGGL(zmi_quant_frag8_kernel<false>, dim3(grid), dim3(FR_THREADS), 0, stream, m0, mats_dev, n_mat, scale_dt);
+    // (the row lengths live on the device: the widest register window serves them all)
+    if (src_dt == ZMI_DT_BF16) zmi_quant_frag8_launch<true>(grid, stream, m0, mats_dev, n_mat, scale_dt, 1 << 30);
+    else zmi_quant_frag8_launch<false>(grid, stream, m0, mats_dev, n_mat, scale_dt, 1 << 30);
     return hipGetLastError();
   }
   if (src_dt == ZMI_DT_BF16)
@@ -427,9 +441,7 @@ hipError_t zmi_launch_quant_gather(const void *x, int32_t x_dt, int64_t ldx, int
   m.M = (int32_t)n_rows; m.K = (int32_t)K; m.row_start = 0; m.frag_kpad = (int32_t)frag_kpad;
   m.gather = gather; m.gather_div = gather_div;
   const unsigned grid = (unsigned)((n_rows + 7) / 8);
-  if (x_dt == ZMI_DT_BF16)
-    hipLaunchKernelGGL(zmi_quant_frag8_kernel<true>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, ZMI_DT_F32);
-  else
-    hipLaunchKernelGGL(zmi_quant_frag8_kernel<false>, dim3(grid), dim3(FR_THREADS), 0, stream, m, (const ZmiQuantMat *)nullptr, 1, ZMI_DT_F32);
+  if (x_dt == ZMI_DT_BF16) zmi_quant_frag8_launch<true>(grid, stream, m, nullptr, 1, ZMI_DT_F32, K);
+  else zmi_quant_frag8_launch<false>(grid, stream, m, nullptr, 1, ZMI_DT_F32, K);
   return hipGetLastError();
 }
