@@ -30,3 +30,19 @@ def _fresh_weight_cache(request):
     if request.node.get_closest_marker("gpu") is not None:
         from zendnn_amd import capi
         capi.load().zmi_clear_weight_cache()
+
+
+@pytest.fixture(params=["decode", "smallm"])
+def small_m_kernel(request):
+    """Problems of 17 .. 128 rows run on the decode kernel (16-row groups) when K fits its LDS and
+    on the small-M kernel otherwise; tests that use this fixture run once on each."""
+    old = os.environ.get("ZMI_DECODE_MAX_M")
+    if request.param == "smallm":
+        os.environ["ZMI_DECODE_MAX_M"] = "16"
+    else:
+        os.environ.pop("ZMI_DECODE_MAX_M", None)
+    yield request.param
+    if old is None:
+        os.environ.pop("ZMI_DECODE_MAX_M", None)
+    else:
+        os.environ["ZMI_DECODE_MAX_M"] = old

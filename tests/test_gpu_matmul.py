@@ -22,7 +22,7 @@ def _oracle(zo, p_host, src, w, M, N, K, **kw):
 # ------------------------------------------------------------------ config 1
 @pytest.mark.parametrize("M,K,N", [(128, 4096, 4096), (32, 256, 128), (128, 512, 192)])
 @pytest.mark.parametrize("packed", [False, True])
-def test_u8s8_zero_point_s32_and_f32(zo, M, K, N, packed):
+def test_u8s8_zero_point_s32_and_f32(zo, small_m_kernel, M, K, N, packed):
     rng = np.random.default_rng(0x5EED0001)
     a = rng.integers(0, 256, (M, K), dtype=np.uint8)
     w = H.gen_weights(rng, K, N)
@@ -156,3 +156,51 @@ def test_prefill_dynamic_quant_bias_gelu(zo, M, K, N, rows):
         acc = np.empty((len(sel), N), dtype=np.int32)
         zo.lib().zo_gemm_s32_bt(q.ctypes.data, capi.DT_S8, K, Bt.ctypes.data, K, len(sel), N, K, acc.ctypes.data, N)
         assert np.array_equal(H.to_host(acc_d), acc)
+
+
+# ------------------------------------------------------------------ 17 .. 128 rows
+@pytest.mark.parametrize("M", [17, 40, 64, 100, 128])
+@pytest.mark.parametrize("K,N", [(4096, 1000), (520, 96)])
+def test_row_groups_dynamic_quant_bf16_silu(zo, small_m_kernel, M, K, N):
+    """More than one 16-row group: a partly filled last group, a column edge inside a block,
+    fused per-token quantization (scales bit-exact) and the bf16 SiLU epilogue."""
+    rng = np.random.default_rng(M * 31 + N)
+    x = H.gen_bf16_normal(rng, (M, K))
+    w = H.gen_weights(rng, K, N)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    x_d, w_d, ws_d = H.to_dev(x), H.to_dev(w), H.to_dev(ws)
+    blob = H.prepack(w_d, K, N)
+    scales_d = torch.zeros(M, dtype=torch.float32, device=H.DEV)
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(scales_d, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+    p.mem_format_b = "r"
+    p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+    for _ in range(2):
+        st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, blob, N, None, 0.0, dst, N, True, p)
+        assert st == capi.SUCCESS, lowoha.last_error()
+    assert small_m_kernel in lowoha.last_kernel() or "ring" in lowoha.last_kernel()
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    ph.mem_format_b = "n"
+    want, _, scales = _oracle(zo, ph, x, w, M, N, K, want_scales=True)
+    assert np.array_equal(H.to_host(scales_d), scales)
+    H.check_bf16(H.to_host(dst), want)
+
+
+@pytest.mark.parametrize("M,K,N", [(33, 1000, 300), (128, 4096, 512)])
+def test_row_groups_s32_accumulators_bit_exact(zo, small_m_kernel, M, K, N):
+    rng = np.random.default_rng(M + K + N)
+    a = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    w = H.gen_weights(rng, K, N)
+    zp = np.array([77], dtype=np.int32)
+    p = lowoha.MatmulParams(src=capi.DT_U8, wei=capi.DT_S8, dst=capi.DT_S32)
+    p.src_zp = lowoha.QuantParam(zp.ctypes.data, capi.DT_S32, (1,))
+    dst = torch.zeros((M, N), dtype=torch.int32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(a), K, H.to_dev(w), N, None, 0.0, dst, N, False, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert small_m_kernel in lowoha.last_kernel() or "ring" in lowoha.last_kernel()
+    want = (a.astype(np.int64) - 77) @ w.astype(np.int64)
+    assert np.array_equal(H.to_host(dst).astype(np.int64), want)

@@ -8,7 +8,7 @@ import torch
 from zendnn_amd import capi, lowoha
 from tests import gpu_helpers as H
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("small_m_kernel")]
 
 
 def _dq_params(M, K, src_dt, scale_buf, dims):

@@ -130,7 +130,7 @@ def env():
 @pytest.mark.parametrize("slices", [2, 3, 8])
 @pytest.mark.parametrize("M,K,N", [(20, 256, 256), (64, 1000, 700), (100, 100, 300), (129, 512, 256), (300, 640, 515)])
 def test_k_sliced_s32_accumulators_bit_exact(zo, env, M, K, N, slices):
-    env(ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=slices)
+    env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=slices)
     rng = np.random.default_rng(M + K + N)
     a = rng.integers(0, 256, (M, K), dtype=np.uint8)
     w = H.gen_weights(rng, K, N)
@@ -150,7 +150,7 @@ def test_k_sliced_s32_accumulators_bit_exact(zo, env, M, K, N, slices):
 @pytest.mark.parametrize("po", [None, capi.PO_SWISH, capi.PO_GELU_TANH])
 @pytest.mark.parametrize("M,K,N,ldc_pad", [(48, 512, 320, 0), (200, 384, 322, 3)])
 def test_k_sliced_bf16_epilogues(zo, env, po, M, K, N, ldc_pad):
-    env(ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=3)
+    env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=3)
     rng = np.random.default_rng(M + N + (po or 0))
     a = rng.integers(-128, 128, (M, K), dtype=np.int8)
     w = H.gen_weights(rng, K, N)
@@ -172,7 +172,7 @@ def test_k_sliced_bf16_epilogues(zo, env, po, M, K, N, ldc_pad):
 
 @pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_S8, capi.DT_U8])
 def test_k_sliced_f32_exact_and_quantized_destinations(zo, env, dst_dt):
-    env(ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=4)
+    env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=4)
     rng = np.random.default_rng(100 + dst_dt)
     M, K, N = 150, 320, 290
     a = rng.integers(-128, 128, (M, K), dtype=np.int8)
@@ -198,11 +198,11 @@ def test_k_sliced_f32_exact_and_quantized_destinations(zo, env, dst_dt):
 
 
 def test_k_slices_chosen_for_a_problem_with_few_tiles(zo):
-    """M = 128, N = 14336, K = 4096 (56 tiles): the launch plan slices K without being told to,
+    """M = 192, N = 4096, K = 4096 (32 tiles): the launch plan slices K without being told to,
     and the dynamic-quantization call agrees with the oracle."""
     from tests.test_gpu_matmul import _oracle
     rng = np.random.default_rng(5)
-    M, K, N = 128, 4096, 14336
+    M, K, N = 192, 4096, 4096
     x = H.gen_bf16_normal(rng, (M, K))
     w = H.gen_weights(rng, K, N)
     ws = rng.uniform(0.001, 0.01, N).astype(np.float32)

@@ -1,4 +1,4 @@
-// Decode int8 GEMM for gfx950: C[M<=16, N] = epilogue(A[M,K] x blob), K_pad <= 4096.
+// Decode int8 GEMM for gfx950: C[M<=128, N] = epilogue(A[M,K] x blob), K_pad <= 4096.
 //
 // Same call sites as k_smallm.hip (the aocl_gemm_s8s8s32o*_sym_quant call,
 // zendnnl/src/lowoha_operators/matmul/backends/aocl/aocl_kernel.cpp:1239-1257, and the
@@ -6,8 +6,11 @@
 // int8_microkernel.cpp:196-606), specialised for the one-to-sixteen-token case, where
 // the weights are streamed once from HBM and everything else has to stay out of
 // the way of that stream:
-//   * one workgroup (8 wavefronts) per 32 weight columns; wavefront w streams the
-//     w-th eighth of K with 16-byte-per-lane loads, all issued up front;
+//   * one workgroup (8 wavefronts) per 32 weight columns and up to RPW groups of 16 rows;
+//     wavefront w streams the w-th eighth of K with 16-byte-per-lane loads, all issued up
+//     front, and keeps its weights in registers for all its row groups; with more than
+//     RPW row groups the workgroups of one column block are neighbours on one XCD, so
+//     the weights leave HBM once and the others find them in that XCD's L2;
 //   * the activation rows are read from L2 with row-contiguous loads (consecutive
 //     lanes, consecutive bytes) BEFORE the weight loads, so they return first,
 //     and are laid out in LDS in MFMA operand order (bank-swizzled); the MFMA A
@@ -41,8 +44,9 @@ __device__ __forceinline__ int dec_lds_off(int cc, int g, int r) {
   return cc * 1024 + ((g * 16 + (r ^ ((g * 4 + (cc & 3)) & 15))) << 4);
 }
 
-__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProblem p, ZmiEpilogue epi,
-                                                                        ZmiFusedQuant fq) {
+template <int RPW>
+__global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_decode_kernel(ZmiProblem p, ZmiEpilogue epi,
+                                                                                       ZmiFusedQuant fq, int n_blk) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);   // scalar: slice bounds and addresses stay in SGPRs
@@ -59,7 +63,20 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
     if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
     return;
   }
-  const int blk = fq.x ? (int)blockIdx.x - M : (int)blockIdx.x;
+  // column block and rows: with at most RPW row groups the workgroup index is the column
+  // block; with more, the indices (dealt round robin to the 8 XCDs) are renumbered so that
+  // every XCD owns a contiguous range and the workgroups of a column block stay together
+  const int n_rg = (M + 16 * RPW - 1) / (16 * RPW);
+  int blk = fq.x ? (int)blockIdx.x - M : (int)blockIdx.x;
+  int rg = 0;
+  if (n_rg > 1) {
+    const int per_xcd = (n_blk * n_rg + 7) / 8;
+    const int id = (blk % 8) * per_xcd + blk / 8;
+    if (blk / 8 >= per_xcd || id >= n_blk * n_rg) return;
+    blk = id / n_rg;
+    rg = id % n_rg;
+  }
+  const int r0 = rg * 16 * RPW;   // first row of this workgroup; row group j starts at r0 + 16 j
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
 
@@ -80,27 +97,50 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
   const int e_h = gated ? 0 : (tid % 32) / 16;
   const int e_c = tid % 16;
   const int e_n = ocol[e_h] + e_c;
-  const bool e_live = e_row < M && e_row < 16 && (gated ? e_n < N / 2 : e_n < N);
-  ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_live ? e_n : N, N);
+  const bool e_col = e_row < 16 && (gated ? e_n < N / 2 : e_n < N);
+  ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_col ? e_n : N, N);
   ZmiColCtx cc1 = cc0;
-  if (gated) cc1 = zmi_col_ctx(epi, p, colsum, e_live ? e_n + N / 2 : N, N);
+  if (gated) cc1 = zmi_col_ctx(epi, p, colsum, e_col ? e_n + N / 2 : N, N);
   // (with fused quantization the row scales exist only after the wait below)
-  float rs = fq.x ? 1.0f : zmi_row_scale(epi, p, e_live ? e_row : 0);
+  float rs[RPW];
+  auto load_rs = [&]() {
+    #pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int m = r0 + j * 16 + e_row;
+      rs[j] = zmi_row_scale(epi, p, e_col && m < M ? m : 0);
+    }
+  };
+  if (!fq.x) load_rs();
 
-  // ---- activation loads (row-contiguous): 64 items (row, 1 KiB segment); wavefront w takes rows w and w + 8 ----
+  // ---- activation loads (row-contiguous): 64 items (row, 1 KiB segment) per row group; wavefront w takes rows w and w + 8 ----
   const int c16 = lane % 16, g = lane / 16;
   v4i araw[2][4];
-  auto load_rows = [&]() {
+  auto load_rows = [&](int j) {
     const int8_t *A = (const int8_t *)p.A;
     const int G = ((K + 15) & ~15) / 16;   // readable 16-byte granules per row
     #pragma unroll
     for (int i = 0; i < 2; ++i)
       #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const int row = wave + 8 * i, gran = s * 64 + lane;
+        const int row = r0 + j * 16 + wave + 8 * i, gran = s * 64 + lane;
         v4i v = {0, 0, 0, 0};
         if (row < M && gran < G) v = *(const v4i *)(A + (int64_t)row * p.lda + gran * 16);
         araw[i][s] = v;
+      }
+  };
+  // rows -> LDS in operand order
+  auto store_rows = [&](int j) {
+    const uint32_t xm = p.a_is_u8 ? 0x80808080u : 0u;
+    #pragma unroll
+    for (int i = 0; i < 2; ++i)
+      #pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int row = wave + 8 * i, gran = s * 64 + lane;
+        v4i v = araw[i][s];
+        v[0] ^= xm; v[1] ^= xm; v[2] ^= xm; v[3] ^= xm;
+        if (r0 + j * 16 + row >= M) v = (v4i){0, 0, 0, 0};
+        // granule s*64 + lane: chunk s*16 + lane/4, k group lane%4 (the swizzle does not depend on s)
+        if (gran * 16 < K_pad) *(v4i *)(lds + dec_lds_off(lane / 4, lane % 4, row) + s * 16384) = v;
       }
   };
 
@@ -124,7 +164,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
 
   if (!fq.x) {
     // rows first, so they return first; then the whole slice
-    load_rows();
+    load_rows(0);
     #pragma unroll
     for (int u = 0; u < 8; ++u) load_b(u);
   } else {
@@ -139,62 +179,62 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode_kernel(ZmiProb
     }
     __syncthreads();
     asm volatile("" ::: "memory");   // the loads below stay below the wait
-    rs = zmi_row_scale(epi, p, e_live ? e_row : 0);
-    load_rows();
+    load_rs();
+    load_rows(0);
     #pragma unroll
     for (int u = DEC_FQ_FIRST; u < 8; ++u) load_b(u);
   }
 
-  // ---- rows -> LDS in operand order ----
-  {
-    const uint32_t xm = p.a_is_u8 ? 0x80808080u : 0u;
-    #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int row = wave + 8 * i, gran = s * 64 + lane;
-        v4i v = araw[i][s];
-        v[0] ^= xm; v[1] ^= xm; v[2] ^= xm; v[3] ^= xm;
-        if (row >= M) v = (v4i){0, 0, 0, 0};
-        // granule s*64 + lane: chunk s*16 + lane/4, k group lane%4 (the swizzle does not depend on s)
-        if (gran * 16 < K_pad) *(v4i *)(lds + dec_lds_off(lane / 4, lane % 4, row) + s * 16384) = v;
-      }
-  }
-  __syncthreads();
-
-  // ---- MFMA: one 16x16x64 per chunk and column group ----
-  v4i acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  // ---- per row group: rows -> LDS, then one 16x16x64 MFMA per chunk and column group; the
+  // next group's rows are requested before the MFMAs of this one ----
+  v4i acc[RPW][2];
   #pragma unroll
-  for (int u = 0; u < 8; ++u) {
-    const bool live = c_begin + u < c_end;
-    const int c = live ? c_begin + u : c_begin;
-    v4i a = *(const v4i *)(lds + dec_lds_off(c, g, c16));
-    if (!live) a = (v4i){0, 0, 0, 0};   // whatever b holds then adds nothing
-    acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[0], 0, 0, 0);
-    acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[1], 0, 0, 0);
+  for (int j = 0; j < RPW; ++j) {
+    acc[j][0] = (v4i){0, 0, 0, 0};
+    acc[j][1] = (v4i){0, 0, 0, 0};
+    if (j > 0 && r0 + j * 16 >= M) continue;   // (uniform) no rows left for this group
+    if (j > 0) __syncthreads();                // every wavefront has read the previous group's rows
+    store_rows(j);
+    __syncthreads();
+    if (j + 1 < RPW && r0 + (j + 1) * 16 < M) load_rows(j + 1);
+    #pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const bool live = c_begin + u < c_end;
+      const int c = live ? c_begin + u : c_begin;
+      v4i a = *(const v4i *)(lds + dec_lds_off(c, g, c16));
+      if (!live) a = (v4i){0, 0, 0, 0};   // whatever b holds then adds nothing
+      acc[j][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[j][0], 0, 0, 0);
+      acc[j][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[j][1], 0, 0, 0);
+    }
   }
 
   // ---- cross-wavefront reduction through LDS (reuses the operand area) ----
   __syncthreads();
   int32_t *red = (int32_t *)lds;
   #pragma unroll
-  for (int h = 0; h < 2; ++h)
+  for (int j = 0; j < RPW; ++j)
     #pragma unroll
-    for (int j = 0; j < 4; ++j) red[wave * 512 + (h * 4 + j) * 64 + lane] = acc[h][j];
+    for (int h = 0; h < 2; ++h)
+      #pragma unroll
+      for (int q = 0; q < 4; ++q) red[(wave * RPW + j) * 512 + (h * 4 + q) * 64 + lane] = acc[j][h][q];
   __syncthreads();
-  if (!e_live) return;
+  if (!e_col) return;
 
-  // acc[h][j] of lane l is row (l/16)*4 + j, column h*16 + l%16
-  auto fetch = [&](int h) -> int32_t {
-    const int off = (h * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_c;
+  // acc[j][h][q] of lane l is row j*16 + (l/16)*4 + q, column h*16 + l%16
+  auto fetch = [&](int j, int h) -> int32_t {
+    const int off = j * 512 + (h * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_c;
     int32_t s = 0;
     #pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) s += red[w * 512 + off];
+    for (int w = 0; w < DEC_WAVES; ++w) s += red[w * RPW * 512 + off];
     return s;
   };
-
-  if (!gated) zmi_finish_element(p, epi, cc0, rs, fetch(e_h), e_row, e_n);
-  else zmi_finish_gated(p, epi, cc0, cc1, rs, fetch(0), fetch(1), e_row, e_n);
+  #pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const int m = r0 + j * 16 + e_row;
+    if (m >= M) break;
+    if (!gated) zmi_finish_element(p, epi, cc0, rs[j], fetch(j, e_h), m, e_n);
+    else zmi_finish_gated(p, epi, cc0, cc1, rs[j], fetch(j, 0), fetch(j, 1), m, e_n);
+  }
 }
 
 int zmi_decode_grid(const ZmiProblem &p, bool gated) {
@@ -202,26 +242,37 @@ int zmi_decode_grid(const ZmiProblem &p, bool gated) {
 }
 
 bool zmi_decode_kernel_fits(const ZmiProblem &p) {
-  return p.M > 0 && p.M <= 16 && zmi_blob_kpad(p.K) <= 4096;
+  return p.M > 0 && p.M <= 128 && zmi_blob_kpad(p.K) <= 4096;
 }
 
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
                                   hipStream_t stream) {
   if (!zmi_decode_kernel_fits(p)) return hipErrorInvalidValue;
   const bool gated = epi.gated_act != 0;
-  const int grid = gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
-  if (grid <= 0) return hipSuccess;
+  const int n_blk = zmi_decode_grid(p, gated);
+  if (n_blk <= 0) return hipSuccess;
+  // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at
+  // 32 / 64 rows, N = K = 4096, against 13 / 20 us with 64); above that, 64 rows per workgroup
+  // keep the weights in registers for four row groups (128 rows: 23 against 27 us)
+  const int rpw = p.M <= 64 ? 1 : 4;
+  const int n_rg = (p.M + 16 * rpw - 1) / (16 * rpw);
+  // (several workgroups per column block: a multiple of 8, for the renumbering over the XCDs)
+  const int grid = n_rg == 1 ? n_blk : (n_blk * n_rg + 7) / 8 * 8;
+  // the operand area (16 rows x K_pad) is reused by the partial tiles (16 KiB per row group)
   const size_t a_bytes = (size_t)zmi_blob_kpad(p.K) * 16;
-  const size_t smem = a_bytes > DEC_RED_BYTES ? a_bytes : (size_t)DEC_RED_BYTES;
+  const size_t r_bytes = (size_t)DEC_RED_BYTES * rpw;
+  const size_t smem = a_bytes > r_bytes ? a_bytes : r_bytes;
   static bool attr_done = false;
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_decode_kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * 16);
-    if (e != hipSuccess) return e;
+    for (const void *f : {(const void *)zmi_gemm_decode_kernel<1>, (const void *)zmi_gemm_decode_kernel<4>}) {
+      hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * 16);
+      if (e != hipSuccess) return e;
+    }
     attr_done = true;
   }
   ZmiFusedQuant none = {};
-  hipLaunchKernelGGL(zmi_gemm_decode_kernel, dim3(grid + (fq ? p.M : 0)), dim3(DEC_THREADS), smem, stream, p, epi,
-                     fq ? *fq : none);
+  const dim3 g3(grid + (fq ? p.M : 0)), b3(DEC_THREADS);
+  if (rpw == 1) hipLaunchKernelGGL(zmi_gemm_decode_kernel<1>, g3, b3, smem, stream, p, epi, fq ? *fq : none, n_blk);
+  else hipLaunchKernelGGL(zmi_gemm_decode_kernel<4>, g3, b3, smem, stream, p, epi, fq ? *fq : none, n_blk);
   return hipGetLastError();
 }

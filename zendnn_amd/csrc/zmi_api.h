@@ -10,5 +10,5 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
                        ZmiEpilogue *out, ZmiProblem *prob);
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan);
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA);
-bool use_ring_kernel(int M, int N);
+bool use_ring_kernel(int M, int N, int K);
 }  // namespace zmi

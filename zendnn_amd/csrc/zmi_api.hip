@@ -225,6 +225,27 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
   return ZMI_SUCCESS;
 }
 
+// Kernel choice for one problem.  Measured on MI355X with K = 4096 (us per call, bf16 rows
+// quantized per token, bf16 out), N = 4096 / 14336:
+//   rows   decode kernel   small-M kernel   ring (K-sliced)
+//     32     12 / 23         14 / 24          28 / 35
+//     64     17 / 34         21 / 35          28 / 36
+//    128     23 / 58         36 / 74          34 / 45
+// The decode kernel reads every row once per 32-column block (the rows cross L2 N / 32
+// times), the ring kernel once per 256 columns but needs three launches when it slices K:
+// up to 64 rows, and up to 128 rows while the output is narrow, the decode kernel wins.
+static bool wide_output(int M, int N) { return (int64_t)M * N >= 96 * 8192; }
+
+static bool decode_kernel_allowed(int M, int N, int K) {
+  // ZMI_DECODE_MAX_M (0 .. 128) caps the rows the decode kernel takes; the tests use it to
+  // reach the other kernels with few rows
+  int max_m = 128;
+  if (const char *env = std::getenv("ZMI_DECODE_MAX_M")) max_m = std::atoi(env);
+  if (std::getenv("ZMI_NO_DECODE_KERNEL")) max_m = 0;
+  if (M > max_m || M > 128 || zmi_blob_kpad(K) > 4096) return false;
+  return M <= 64 || !wide_output(M, N);
+}
+
 // Tile height and K slices of a one-problem ring launch.  ZMI_GEMM_TOP (128 / 256) and
 // ZMI_RING_SPLITK (1 = never slice, n = n slices) override the choice; the tests use them
 // to reach every kernel configuration with small shapes.
@@ -239,10 +260,10 @@ ZmiRingPlan plan_ring_gemm(int M, int N, int K) {
 }
 
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
-  if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
+  if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
     set_kernel_name("decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
-  } else if (!use_ring_kernel(prob.M, prob.N)) {
+  } else if (!use_ring_kernel(prob.M, prob.N, prob.K)) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
   } else {
@@ -265,16 +286,14 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
 
 // Problems with more rows than the small-M kernels take run on the MFMA-bound
 // kernel, which reads the activations in fragment-major order.
-bool use_ring_kernel(int M, int N) {
+bool use_ring_kernel(int M, int N, int K) {
+  if (decode_kernel_allowed(M, N, K)) return false;
   // ZMI_RING_MIN_M overrides the choice (the tests reach the 64-row tile through it)
   if (const char *env = std::getenv("ZMI_RING_MIN_M")) {
     const int min_m = std::atoi(env);
     if (min_m > 0) return M >= min_m;
   }
-  // Above 128 rows always.  From 65 rows the K-sliced ring launch beats the small-M kernel
-  // once the output is wide enough for that kernel's per-row cost to show (measured:
-  // M = 128: N = 4096 36 vs 34 us, N = 14336 74 vs 45 us per call).
-  return M > 128 || (M > 64 && (int64_t)M * N >= 96 * 8192);
+  return M > 128 || (M > 64 && wide_output(M, N));
 }
 
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
@@ -357,7 +376,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                          std::min(weight_cache_env(), p.weight_cache_type) > 0;
   const bool pack_in_arena = p.mem_format_b != 'r' && !use_cache;
   const int64_t K16 = zmi_round_up(K, 16);
-  const bool ring = use_ring_kernel(M, N);
+  const bool ring = use_ring_kernel(M, N, K);
   const int64_t frag_kpad = ring ? zmi_blob_kpad(K) : 0;
   const size_t a_bytes = ring ? (size_t)zmi_afrag_bytes(M, K) : (size_t)M * K16;
   const bool repack_a = !dyn && (ring || a_needs_repack(src, lda, K, transA != 0));
@@ -405,7 +424,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     prob.A = q; prob.lda = K16;
     const bool per_token = (dyn_scale_n == M && M > 1) || M == 1;
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
-    const bool decode_kernel = M <= 16 && zmi_blob_kpad(K) <= 4096 && !std::getenv("ZMI_NO_DECODE_KERNEL");
+    const bool decode_kernel = decode_kernel_allowed(M, N, K);
     // (the decode kernel's producers are its first workgroups and wait for nothing, so its grid need not be resident)
     if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob, false) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
@@ -461,7 +480,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (use_fused) {
     // a one-row scale in device memory reads like a per-token scale
     if (epi.src_scale_mode == ZMI_SS_TENSOR_PTR) epi.src_scale_mode = ZMI_SS_TOKEN_PTR;
-    if (zmi_decode_kernel_fits(prob) && !std::getenv("ZMI_NO_DECODE_KERNEL")) {
+    if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
       set_kernel_name("decode_lds_rows_mfma16x16x64 (fused per-token quant)");
       st = hip_ok(zmi_launch_gemm_decode(prob, epi, &fused, stream()), "fused decode GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
     } else {

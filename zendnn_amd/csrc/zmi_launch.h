@@ -86,7 +86,7 @@ hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &
                                         hipStream_t stream);
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
 
-// k_decode.hip: single problem, M <= 16, K_pad <= 4096
+// k_decode.hip: single problem, M <= 128, K_pad <= 4096
 bool zmi_decode_kernel_fits(const ZmiProblem &p);
 // fq != null: the launch also quantizes the M source rows (its grid must be resident at once)
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
