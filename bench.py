@@ -41,7 +41,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["decode_M1", "decode_M4", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
+                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
                              "moe_config4", "moe_config5"],
                     help="run one of the other configs alone and print its entry (for profiler runs)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -294,6 +294,10 @@ def main():
     extras = {
         "decode_M1": lambda: run_decode_m(1),
         "decode_M4": lambda: run_decode_m(4),
+        # the same call with more rows than a decode step proper: 16-row groups of the decode kernel
+        # (64 rows) and the K-sliced large-M kernel (128 rows)
+        "decode_M64": lambda: run_decode_m(64),
+        "decode_M128": lambda: run_decode_m(128),
         "prefill_N4096": lambda: run_prefill(4096),
         "prefill_N14336": lambda: run_prefill(14336),
         "config1_u8s8_M128": run_config1,

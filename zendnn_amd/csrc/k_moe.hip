@@ -131,68 +131,118 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
 }
 
 // ---------------------------------------------------------------------------
-// Routing.  One workgroup of 16 wavefronts; wavefront w owns the contiguous
-// segment w of the flat (t,k) index space.
-//   A: per-wavefront histograms hist[w][e];
-//   B: counts / exclusive offsets per expert, and cursor[w][e] = offsets[e] +
-//      sum of hist[w'][e] for w' < w;
+// Routing.  G workgroups of 16 wavefronts; wavefront u = 16 g + w owns the
+// contiguous segment u of the flat (t,k) index space.
+//   A: per-wavefront histograms hist[u][e] (LDS atomics);
+//   B: counts / exclusive offsets per expert, and cursor[u][e] = offsets[e] +
+//      sum of hist[u'][e] for u' < u;
 //   C: every wavefront walks its segment in order, 64 entries at a time; an
 //      entry's slot is cursor + (number of lower lanes with the same expert).
 // The order inside an expert is therefore the (t,k) order: deterministic.
+// One workgroup does A, B and C in one launch.  Several workgroups (long id lists: one
+// workgroup would walk them 1024 entries at a time) take two launches: `phase` 0 is pass A,
+// whose histograms go to ghist[16 G][E] in device memory; `phase` 1 reads all of them back
+// for pass B (every workgroup computes the offsets for itself) and runs pass C.
 // ---------------------------------------------------------------------------
 #define RT_WAVES 16
-#define RT_KEEP 24   // ids kept per lane: 24 x 64 x 16 = 24576 entries without a second read
+#define RT_KEEP 8    // ids kept per lane between the passes of one launch: 8 x 64 x 16 = 8192 entries per workgroup
 
 __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int32_t *topk_ids, int n, int E,
                                                                       int align, int32_t *counts,
                                                                       int32_t *offsets, int32_t *slot_of,
-                                                                      int32_t *src_of, int n_slots) {
-  extern __shared__ int32_t sh[];   // hist[RT_WAVES][E], then off[E+1]
+                                                                      int32_t *src_of, int n_slots, int32_t *ghist,
+                                                                      int phase) {
+  extern __shared__ int32_t sh[];   // hist[RT_WAVES][E], off[E+1], then (several workgroups) all histograms
   int32_t *hist = sh;
   int32_t *off = sh + RT_WAVES * E;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int G = gridDim.x, g = blockIdx.x;
+  const bool multi = G > 1;
   int ebits = 1;
   while ((1 << ebits) < E) ++ebits;          // expert ids fit in ebits bits
-  if (src_of)
-    for (int i = tid; i < n_slots; i += blockDim.x) src_of[i] = -1;
-  for (int i = tid; i < RT_WAVES * E; i += blockDim.x) hist[i] = 0;
-  __syncthreads();
-  const int seg = (n + RT_WAVES - 1) / RT_WAVES;
-  const int s0 = wave * seg, s1 = (s0 + seg < n) ? s0 + seg : n;
+  const int seg = (n + G * RT_WAVES - 1) / (G * RT_WAVES);
+  const int s0 = (g * RT_WAVES + wave) * seg < n ? (g * RT_WAVES + wave) * seg : n;
+  const int s1 = (s0 + seg < n) ? s0 + seg : n;
   // The segment's ids are read once, all loads in flight together, and kept in registers
-  // for both passes (RT_KEEP x 64 per wavefront; what a longer segment has beyond that is
-  // read again in pass C).
+  // (RT_KEEP x 64 per wavefront; what a longer segment has beyond that is read again).
   int keep[RT_KEEP];
 #pragma unroll
   for (int it = 0; it < RT_KEEP; ++it) {
     const int i = s0 + it * 64 + lane;
     keep[it] = i < s1 ? topk_ids[i] : -1;
   }
-  auto count = [&](int e) {
-    if (e >= 0 && e < E) atomicAdd(&hist[wave * E + e], 1);
-  };
+  if (!multi || phase == 0) {
+    if (src_of)
+      for (int i = g * blockDim.x + tid; i < n_slots; i += G * blockDim.x) src_of[i] = -1;
+    for (int i = tid; i < RT_WAVES * E; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    auto count = [&](int e) {
+      if (e >= 0 && e < E) atomicAdd(&hist[wave * E + e], 1);
+    };
 #pragma unroll
-  for (int it = 0; it < RT_KEEP; ++it)
-    if (s0 + it * 64 < s1) count(keep[it]);
-  for (int i0 = s0 + RT_KEEP * 64; i0 < s1; i0 += 64) count(i0 + lane < s1 ? topk_ids[i0 + lane] : -1);
-  __syncthreads();
-  // per-expert totals and the per-wavefront running starts (thread e handles expert e)
+    for (int it = 0; it < RT_KEEP; ++it)
+      if (s0 + it * 64 < s1) count(keep[it]);
+    for (int i0 = s0 + RT_KEEP * 64; i0 < s1; i0 += 64) count(i0 + lane < s1 ? topk_ids[i0 + lane] : -1);
+    __syncthreads();
+    if (multi) {
+      for (int i = tid; i < RT_WAVES * E; i += blockDim.x) ghist[(size_t)g * RT_WAVES * E + i] = hist[i];
+      return;
+    }
+  }
+  // per-expert totals and the per-wavefront running starts (thread e handles expert e);
+  // several workgroups: all their histograms come into LDS first, in one sweep of loads
+  int32_t *gh = off + E + 1;
+  if (multi) {
+    for (int i = tid; i < G * RT_WAVES * E; i += blockDim.x) gh[i] = ghist[i];
+    __syncthreads();
+  }
   for (int e = tid; e < E; e += blockDim.x) {
     int run = 0;
-    for (int w = 0; w < RT_WAVES; ++w) {
-      const int c = hist[w * E + e];
-      hist[w * E + e] = run;
-      run += c;
+    if (!multi) {
+      for (int w = 0; w < RT_WAVES; ++w) {
+        const int c = hist[w * E + e];
+        hist[w * E + e] = run;
+        run += c;
+      }
+    } else {
+      for (int u = 0; u < G * RT_WAVES; ++u) {
+        if (u == g * RT_WAVES) {
+          // this workgroup's wavefronts start here
+          int r2 = run;
+          for (int w = 0; w < RT_WAVES; ++w) {
+            hist[w * E + e] = r2;
+            r2 += gh[(u + w) * E + e];
+          }
+        }
+        run += gh[u * E + e];
+      }
     }
     off[e] = run;
-    counts[e] = run;
+    if (g == 0) counts[e] = run;
   }
   __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    for (int e = 0; e < E; ++e) { const int c = off[e]; off[e] = run; offsets[e] = run; run += (c + align - 1) / align * align; }
-    off[E] = run;
-    offsets[E] = run;
+  // exclusive offsets of the aligned counts: wavefront 0 scans 64 experts per step
+  if (wave == 0) {
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + lane;
+      const int c = e < E ? (off[e] + align - 1) / align * align : 0;
+      int x = c;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int y = __shfl_up(x, o);
+        if (lane >= o) x += y;
+      }
+      if (e < E) {
+        off[e] = carry + x - c;
+        if (g == 0) offsets[e] = carry + x - c;
+      }
+      carry += __shfl(x, 63);
+    }
+    if (lane == 0) {
+      off[E] = carry;
+      if (g == 0) offsets[E] = carry;
+    }
   }
   __syncthreads();
   auto place = [&](int i, int e) {
@@ -227,11 +277,30 @@ __global__ __launch_bounds__(RT_WAVES * 64) void zmi_moe_route_kernel(const int3
   }
 }
 
+// workgroups of a routing launch: 4096 entries each (4 steps of 64 per wavefront), at most 16,
+// and no more than keep all the per-wavefront histograms within 64 KiB of LDS
+static int zmi_moe_route_groups(int64_t n, int E) {
+  int64_t G = (n + 4095) / 4096;
+  if (G > 16) G = 16;
+  const int64_t cap = 16384 / ((int64_t)RT_WAVES * E);
+  if (G > cap) G = cap;
+  return G < 1 ? 1 : (int)G;
+}
+
+// hist_scratch: zmi_moe_route_scratch_ints(T * topk, E) ints of device memory for the
+// several-workgroup form (null: one workgroup whatever the size).
+size_t zmi_moe_route_scratch_ints(int64_t n, int E) {
+  const int G = zmi_moe_route_groups(n, E);
+  return G > 1 ? (size_t)G * RT_WAVES * E : 0;
+}
+
 hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
                                 int32_t *offsets, int32_t *slot_of, int32_t *src_of, int n_slots,
-                                hipStream_t stream) {
+                                int32_t *hist_scratch, hipStream_t stream) {
   if (E > 2047 || E <= 0) return hipErrorInvalidValue;
-  const size_t smem = ((size_t)RT_WAVES * E + E + 1) * sizeof(int32_t);
+  const int n = T * topk;
+  const int G = hist_scratch ? zmi_moe_route_groups(n, E) : 1;
+  const size_t smem = ((size_t)RT_WAVES * E + E + 1 + (G > 1 ? (size_t)G * RT_WAVES * E : 0)) * sizeof(int32_t);
   static size_t attr = 0;
   if (smem > attr) {
     hipError_t e = hipFuncSetAttribute((const void *)zmi_moe_route_kernel,
@@ -239,8 +308,12 @@ hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E,
     if (e != hipSuccess) return e;
     attr = smem;
   }
-  hipLaunchKernelGGL(zmi_moe_route_kernel, dim3(1), dim3(RT_WAVES * 64), smem, stream, topk_ids, T * topk, E,
-                     align < 1 ? 1 : align, counts, offsets, slot_of, src_of, n_slots);
+  const int al = align < 1 ? 1 : align;
+  if (G > 1)
+    hipLaunchKernelGGL(zmi_moe_route_kernel, dim3(G), dim3(RT_WAVES * 64), smem, stream, topk_ids, n, E, al, counts,
+                       offsets, slot_of, src_of, n_slots, hist_scratch, 0);
+  hipLaunchKernelGGL(zmi_moe_route_kernel, dim3(G), dim3(RT_WAVES * 64), smem, stream, topk_ids, n, E, al, counts,
+                     offsets, slot_of, src_of, n_slots, hist_scratch, 1);
   return hipGetLastError();
 }
 

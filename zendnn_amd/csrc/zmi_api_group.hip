@@ -585,7 +585,10 @@ int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk, int32_t 
   if (!topk_ids || !counts || !offsets || !slot_of || T <= 0 || topk <= 0 || E <= 0) { set_error("moe_route: bad arguments"); return ZMI_FAILURE; }
   if (E > 2047) { set_error("moe_route: at most 2047 experts"); return ZMI_UNIMPLEMENTED; }
   if (!ensure_device()) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, 1, counts, offsets, slot_of, nullptr, 0, stream()), "moe route launch")) return ZMI_FAILURE;
+  const size_t hist_ints = zmi_moe_route_scratch_ints((int64_t)T * topk, E);
+  if (!arena().begin(Arena::padded(hist_ints * sizeof(int32_t)))) return ZMI_FAILURE;
+  int32_t *hist = hist_ints ? (int32_t *)arena().alloc(hist_ints * sizeof(int32_t)) : nullptr;
+  if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, 1, counts, offsets, slot_of, nullptr, 0, hist, stream()), "moe route launch")) return ZMI_FAILURE;
   set_kernel_name("moe_route");
   return ZMI_SUCCESS;
 }
@@ -614,7 +617,10 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   need += Arena::padded((size_t)Rp * kpI) + Arena::padded(sizeof(float) * Rp);       // A2, s2
   need += Arena::padded((size_t)Rp * H * 2);                                         // Y bf16
   need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * (size_t)E));
+  const size_t hist_ints = zmi_moe_route_scratch_ints(R, E);
+  need += Arena::padded(hist_ints * sizeof(int32_t));
   if (!arena().begin(need)) return ZMI_FAILURE;
+  int32_t *route_hist = hist_ints ? (int32_t *)arena().alloc(hist_ints * sizeof(int32_t)) : nullptr;
   int32_t *counts = (int32_t *)arena().alloc(sizeof(int32_t) * E);
   int32_t *offsets = (int32_t *)arena().alloc(sizeof(int32_t) * (E + 1));
   int32_t *slot_of = (int32_t *)arena().alloc(sizeof(int32_t) * R);
@@ -646,7 +652,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   tb.w13_scale = (const float *const *)(tdev + 2 * E); tb.w2_scale = (const float *const *)(tdev + 3 * E);
 
   hipStream_t s = stream();
-  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, 32, counts, offsets, slot_of, src_of, (int)Rp, s), "moe route launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_route(d->topk_ids, T, topk, E, 32, counts, offsets, slot_of, src_of, (int)Rp, route_hist, s), "moe route launch")) return ZMI_FAILURE;
   // every slot quantizes its token's row itself (8 slots per workgroup, whole 128-byte lines of the
   // fragment layout); rows that do not allow 16-byte loads take the per-token scatter form
   if (hipSuccess != zmi_launch_quant_gather(d->x, ZMI_DT_BF16, d->ldx, H, src_of, topk, Rp, A1, kpH, s1, s)) {

@@ -108,9 +108,10 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
                                   hipStream_t stream);
 // align: every expert's first slot is rounded up to a multiple of it (1: dense numbering).
 // src_of (optional, n_slots entries): the flat (token, k) index that fills each slot, -1 for idle slots.
+size_t zmi_moe_route_scratch_ints(int64_t n, int E);
 hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
                                 int32_t *offsets, int32_t *slot_of, int32_t *src_of, int n_slots,
-                                hipStream_t stream);
+                                int32_t *hist_scratch, hipStream_t stream);
 // A1 is fragment-major over the slot numbering, K_pad = zmi_blob_kpad(H)
 hipError_t zmi_launch_moe_quant_scatter(const void *x, int64_t ldx, int T, int H, int topk,
                                         const int32_t *slot_of, int8_t *A1, float *s1, hipStream_t stream);
