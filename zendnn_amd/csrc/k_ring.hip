@@ -627,26 +627,23 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
 }
 
 // Second step of a K-sliced launch: adds the partial tiles of the slices and finishes the
-// elements.  One wavefront per 16-byte chunk column of a tile: lane l of chunk (wave w,
-// ni, mi, g) holds row (w/2)*(BM/2) + mi*32 + l%32 and the four columns from
-// (w%2)*128 + ni*32 + g*8 + (l/32)*4 of the tile, as the MFMA left them.
+// elements (plain epilogues only: gated launches are never sliced).  One wavefront per
+// 16-byte chunk column of a tile: lane l of chunk (wave w, ni, mi, g) holds row
+// (w/2)*(BM/2) + mi*32 + l%32 and the four columns from (w%2)*128 + ni*32 + g*8 + (l/32)*4
+// of the tile, as the MFMA left them.
 template <int BM>
 __global__ __launch_bounds__(R_THREADS) void zmi_ring_reduce_kernel(ZmiProblem p, int top_flags, ZmiRingSplit split,
                                                                     ZmiEpilogue epi) {
   constexpr int MI = BM / 64, NI = 4, CH = NI * MI * 4;
   const int top = top_flags & 0xffff;
   const int lane = threadIdx.x % 64;
-  const bool gated = epi.gated_act != 0;
-  const int NIU = gated ? 2 : NI;                         // gated: ni = 0, 1 pair with ni + 2
-  const int units_per_tile = 4 * NIU * MI * 4;            // wavefront units: (w, ni, mi, g)
+  constexpr int units_per_tile = 4 * CH;                  // wavefront units: (w, ni, mi, g)
   const int unit = blockIdx.x * (R_THREADS / 64) + threadIdx.x / 64;
   const int tile = unit / units_per_tile;
   int full; bool rem;
   zmi_ring_rows<BM>(p.M, top_flags, full, rem);
   const int tiles_m = full + (rem ? 1 : 0);
-  const int ncols = gated ? p.N / 2 : p.N;
-  const int per = gated ? 128 : 256;
-  const int tiles_n = (ncols + per - 1) / per;
+  const int tiles_n = (p.N + 255) / 256;
   if (tile >= tiles_m * tiles_n) return;
   // same tile numbering as the GEMM kernel
   const int GM = tiles_m < 8 ? tiles_m : 8;
@@ -660,44 +657,26 @@ __global__ __launch_bounds__(R_THREADS) void zmi_ring_reduce_kernel(ZmiProblem p
   int u = unit % units_per_tile;
   const int g = u % 4; u /= 4;
   const int mi = u % MI; u /= MI;
-  const int ni = u % NIU; u /= NIU;
+  const int ni = u % NI; u /= NI;
   const int w = u, wm = w / 2, wn = w % 2;
 
   const int m = m0 + wm * (BM / 2) + mi * 32 + lane % 32;
-  const int cin = ni * 32 + g * 8 + (lane / 32) * 4;      // column inside the wavefront's 128
-  v4i sum[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  const int n0 = tn * 256 + wn * 128 + ni * 32 + g * 8 + (lane / 32) * 4;
+  v4i sum = {0, 0, 0, 0};
   for (int s = 0; s < split.slices; ++s) {
     const int32_t *base = split.partial + (((int64_t)tile * split.slices + s) * 4 + w) * (CH * 256) + lane * 4;
     const v4i a = *zmi_global<const v4i>(base + ((ni * MI + mi) * 4 + g) * 256);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) sum[0][j] += a[j];
-    if (gated) {
-      const v4i b = *zmi_global<const v4i>(base + (((ni + 2) * MI + mi) * 4 + g) * 256);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) sum[1][j] += b[j];
-    }
+    for (int j = 0; j < 4; ++j) sum[j] += a[j];
   }
   if (m >= p.M) return;
   const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
   const float rs = zmi_row_scale(epi, p, m);
-  if (!gated) {
-    const int n0 = tn * 256 + wn * 128 + cin;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + j;
-      if (n >= p.N) break;
-      zmi_finish_element(p, epi, zmi_col_ctx(epi, p, colsum, n, p.N), rs, sum[0][j], m, n);
-    }
-  } else {
-    const int half = p.N / 2;
-    const int n0 = tn * 128 + wn * 64 + cin;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + j;
-      if (n >= half) break;
-      zmi_finish_gated(p, epi, zmi_col_ctx(epi, p, colsum, n, half), zmi_col_ctx(epi, p, colsum, n + half, p.N), rs,
-                       sum[0][j], sum[1][j], m, n);
-    }
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + j;
+    if (n >= p.N) break;
+    zmi_finish_element(p, epi, zmi_col_ctx(epi, p, colsum, n, p.N), rs, sum[j], m, n);
   }
 }
 
@@ -834,7 +813,7 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
   ZmiRingSplit sp = {1, nullptr};
   if (split && split->slices > 1) {
     // sliced launches are one launch: the remainder rows stay with the top-height kernel
-    if (!(top & ZMI_RING_PAD) || (top & 0xffff) == 256 || !split->partial) return hipErrorInvalidValue;
+    if (!(top & ZMI_RING_PAD) || (top & 0xffff) == 256 || !split->partial || gated) return hipErrorInvalidValue;
     if (split->slices > (int)(zmi_blob_kpad(p.K) / 64)) return hipErrorInvalidValue;
     sp = *split;
   }
@@ -850,7 +829,7 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
   // the slices' partial tiles -> finished elements
   const int th = top & 0xffff;
   const int tiles = th == 128 ? zmi_ring_items<128>(p.M, p.N, top, gated) : zmi_ring_items<64>(p.M, p.N, top, gated);
-  const int units = tiles * 4 * (gated ? 2 : 4) * (th / 64) * 4;
+  const int units = tiles * 4 * 4 * (th / 64) * 4;
   const int grid = (units + R_THREADS / 64 - 1) / (R_THREADS / 64);
   if (th == 128) hipLaunchKernelGGL(zmi_ring_reduce_kernel<128>, dim3(grid), dim3(R_THREADS), 0, stream, p, top, sp, epi);
   else hipLaunchKernelGGL(zmi_ring_reduce_kernel<64>, dim3(grid), dim3(R_THREADS), 0, stream, p, top, sp, epi);

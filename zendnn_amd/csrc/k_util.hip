@@ -23,15 +23,19 @@ hipError_t zmi_launch_pad_rows(const void *src, int64_t M, int64_t K, int64_t ld
   return hipGetLastError();
 }
 
-// Fragment-major copy for the large-M kernel: one workgroup per 32-row block,
-// one 16-byte chunk per thread and step, written in fragment order (coalesced).
+// Fragment-major copy for the large-M kernel: one workgroup per 32-row block and segment of
+// RF_SEG_KB fragments along K (so that a few hundred rows already fill the device), one
+// 16-byte chunk per thread and step, written in fragment order (coalesced).
+#define RF_SEG_KB 16
 __global__ __launch_bounds__(256) void zmi_repack_frag_kernel(const int8_t *src, int64_t M, int64_t K,
                                                               int64_t ld_src, int trans, int is_u8, int8_t *dst,
                                                               int64_t k_pad) {
   const int64_t fr = blockIdx.x;
-  const int64_t chunks = (k_pad / 32) * 64;
+  const int64_t kb_first = (int64_t)blockIdx.y * RF_SEG_KB;
+  const int64_t kb_left = k_pad / 32 - kb_first;
+  const int64_t chunks = (kb_left < RF_SEG_KB ? kb_left : RF_SEG_KB) * 64;
   for (int64_t idx = threadIdx.x; idx < chunks; idx += blockDim.x) {
-    const int64_t kb = idx / 64;
+    const int64_t kb = kb_first + idx / 64;
     const int l = (int)(idx % 64);
     const int64_t row = fr * 32 + l % 32;
     const int64_t k0 = kb * 32 + (l / 32) * 16;
@@ -56,7 +60,9 @@ __global__ __launch_bounds__(256) void zmi_repack_frag_kernel(const int8_t *src,
 hipError_t zmi_launch_repack_frag(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans, int is_u8,
                                   int8_t *dst, hipStream_t stream) {
   if (M <= 0) return hipSuccess;
-  hipLaunchKernelGGL(zmi_repack_frag_kernel, dim3((unsigned)((M + 31) / 32)), dim3(256), 0, stream,
-                     (const int8_t *)src, M, K, ld_src, trans, is_u8, dst, zmi_blob_kpad(K));
+  const int64_t k_pad = zmi_blob_kpad(K);
+  const unsigned segs = (unsigned)((k_pad / 32 + RF_SEG_KB - 1) / RF_SEG_KB);
+  hipLaunchKernelGGL(zmi_repack_frag_kernel, dim3((unsigned)((M + 31) / 32), segs), dim3(256), 0, stream,
+                     (const int8_t *)src, M, K, ld_src, trans, is_u8, dst, k_pad);
   return hipGetLastError();
 }
