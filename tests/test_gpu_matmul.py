@@ -1,6 +1,8 @@
 """GPU parity of matmul_direct (through the C ABI) against the CPU oracle on
 the same seeded inputs.  Bars: s32 accumulators bit-exact; f32 within 1e-5
 relative; bf16 within one bf16 ulp."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -159,9 +161,24 @@ def test_prefill_dynamic_quant_bias_gelu(zo, M, K, N, rows):
 
 
 # ------------------------------------------------------------------ 17 .. 128 rows
+@pytest.fixture(params=["fused", "separate"])
+def quant_launch(request):
+    """Per-token quantization inside the GEMM launch (the default where a kernel offers it) or in a launch of its own."""
+    old = os.environ.get("ZMI_NO_FUSED_QUANT")
+    if request.param == "separate":
+        os.environ["ZMI_NO_FUSED_QUANT"] = "1"
+    else:
+        os.environ.pop("ZMI_NO_FUSED_QUANT", None)
+    yield request.param
+    if old is None:
+        os.environ.pop("ZMI_NO_FUSED_QUANT", None)
+    else:
+        os.environ["ZMI_NO_FUSED_QUANT"] = old
+
+
 @pytest.mark.parametrize("M", [17, 40, 64, 100, 128])
 @pytest.mark.parametrize("K,N", [(4096, 1000), (520, 96)])
-def test_row_groups_dynamic_quant_bf16_silu(zo, small_m_kernel, M, K, N):
+def test_row_groups_dynamic_quant_bf16_silu(zo, small_m_kernel, quant_launch, M, K, N):
     """More than one 16-row group: a partly filled last group, a column edge inside a block,
     fused per-token quantization (scales bit-exact) and the bf16 SiLU epilogue."""
     rng = np.random.default_rng(M * 31 + N)
