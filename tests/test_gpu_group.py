@@ -12,15 +12,28 @@ from tests import moe_helpers as MH
 pytestmark = pytest.mark.gpu
 
 
-def check_moe_out(got_bits, want_bits):
+def check_moe_out(got_bits, want_bits, flipped_rows=0):
     """The fused block re-quantizes a bf16 intermediate, so a one-ulp flip of one
     activation (device exp vs libm) moves a few s32 accumulators of Op2 by a few
     counts: nearly all outputs are identical, a small fraction moves by one bf16
-    ulp, and none by more than two."""
+    ulp, and none by more than two.
+    flipped_rows > 0 additionally accepts that many output rows in which such a flip crossed a
+    rounding boundary of the re-quantization (one s8 count of one Op2 input, i.e. up to
+    absmax(row of activations) * max weight scale in every output of the row): there the bound
+    is 1 % of the row's largest output instead of two ulps.  With large activations (hundreds)
+    and small outputs that is many ulps of an output near zero; the main configurations do not
+    need it."""
     d = H.bf16_ulp_diff(got_bits, want_bits)
     g = (got_bits.astype(np.uint32) << 16).view(np.float32)
     w = (want_bits.astype(np.uint32) << 16).view(np.float32)
     d = np.where(np.abs(g.astype(np.float64) - w.astype(np.float64)) <= 1e-6, np.minimum(d, 1), d)
+    if flipped_rows > 0:
+        bad = np.where(d.max(axis=1) > 2)[0]
+        assert len(bad) <= flipped_rows, f"{len(bad)} rows differ by more than two bf16 ulps"
+        for r in bad:
+            lim = 0.01 * np.abs(w[r]).max()
+            assert np.abs(g[r].astype(np.float64) - w[r].astype(np.float64)).max() <= lim, f"row {r}"
+            d[r] = 0
     assert d.max() <= 2, f"max bf16 ulp diff {d.max()}"
     assert (d > 1).mean() <= 1e-4
     assert (d > 0).mean() <= 2e-2
@@ -197,3 +210,32 @@ def test_route_is_a_stable_counting_sort(zo, T, topk, E):
     assert np.array_equal(H.to_host(counts), want_counts)
     assert np.array_equal(H.to_host(offsets), want_off)
     assert np.array_equal(H.to_host(slot_of), want_slot)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_fused_moe_random_configuration(zo, seed):
+    """Seeded random MoE blocks (tokens, widths, experts, top-k, skew): every token against the oracle,
+    through group_matmul_direct with fused_moe and through the device-routed form."""
+    rng = np.random.default_rng(7000 + seed)
+    T = int(rng.choice([1, 5, 33, 130, 260]))
+    Hd = int(rng.choice([64, 128, 320, 512]))
+    I = int(rng.choice([16, 48, 96, 160, 352]))
+    E = int(rng.choice([1, 2, 3, 8, 16, 40, 70]))
+    topk = int(rng.integers(1, min(E, 6) + 1))
+    skew = bool(rng.integers(2))
+    c = MH.make_case(0x5EED1000 + seed, T, Hd, I, E, topk, skew)
+    d = MH.DeviceMoe(c, packed=bool(rng.integers(2)))
+    st = d.call_fused()
+    assert st == capi.SUCCESS, lowoha.last_error()
+    want = MH.oracle_moe(zo, c, list(range(T)))
+    check_moe_out(H.to_host(d.out), want, flipped_rows=max(1, T // 50))
+    w13b = [H.prepack(w, c.H, 2 * c.I) for w in d.w13]
+    w2b = [H.prepack(w, c.I, c.H) for w in d.w2]
+    out2 = torch.zeros((c.T, c.H), dtype=torch.bfloat16, device=H.DEV)
+    st = lowoha.moe_fused_device(d.x, H.to_dev(c.ids), d.topk_w, w13b, w2b, d.s13, d.s2, c.I, capi.ACT_SILU_AND_MUL, out2)
+    if I % 32 != 0:
+        # the device-routed form keeps every expert on fragment-row boundaries: documented limit
+        assert st == capi.UNIMPLEMENTED
+        return
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert torch.equal(out2.view(torch.int16), d.out.view(torch.int16))

@@ -347,8 +347,10 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     bool fuse_act = run_act && gated_act != ZMI_ACT_SWIGLU_OAI_MUL;
     for (size_t i = 0; i < num_ops && fuse_act; ++i)
       if (a.M[i] > 0 && (a.N[i] / 2) % 32 != 0) fuse_act = false;
-    // a caller-visible wide dst keeps the un-activated up half only in the unfused form
-    const bool tight_internal = op1_internal && run_act;
+    // internal Op1 scratch holds only the activated half when the epilogue produces it; with the
+    // stand-alone activation kernel it is as wide as a caller-visible dst ([gate | up], result in
+    // the first half)
+    const bool tight_internal = op1_internal && fuse_act;
 
     // ---- scratch plan ----
     size_t need = 0;
@@ -490,7 +492,6 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
         maxN = std::max(maxN, a.N[i]);
         mats.push_back(m);
       }
-      if (tight_internal) { set_error("internal: tight Op1 scratch needs the fused activation"); return ZMI_FAILURE; }
       const ZmiActMat *dev = (const ZmiActMat *)upload(mats.data(), mats.size() * sizeof(ZmiActMat));
       if (!dev) return ZMI_FAILURE;
       if (!hip_ok(zmi_launch_gated_act(dev, nullptr, (int)mats.size(), r0, maxN, gated_act, p0.dt_dst, stream()), "gated act launch")) return ZMI_FAILURE;
