@@ -239,3 +239,74 @@ def test_fused_moe_random_configuration(zo, seed):
         return
     assert st == capi.SUCCESS, lowoha.last_error()
     assert torch.equal(out2.view(torch.int16), d.out.view(torch.int16))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_group_of_unrelated_gemms_random_configuration(zo, seed):
+    """group_matmul_direct without MoE extras: experts with unrelated shapes (M = 0 included), static s8 / u8
+    sources with per-tensor scales and zero-points, f32 bias, one post-op, f32 / bf16 / s32 destinations with padded
+    leading dimensions.  Every expert is compared with the oracle's single matmul."""
+    rng = np.random.default_rng(9000 + seed)
+    E = int(rng.integers(1, 7))
+    u8 = bool(rng.integers(2))
+    dst_dt = [capi.DT_F32, capi.DT_BF16, capi.DT_S32][int(rng.integers(3))]
+    po = [None, capi.PO_RELU, capi.PO_SWISH][int(rng.integers(3))] if dst_dt != capi.DT_S32 else None
+    torch_dt = {capi.DT_F32: torch.float32, capi.DT_BF16: torch.bfloat16, capi.DT_S32: torch.int32}[dst_dt]
+    Ms = [int(rng.choice([0, 1, 9, 40, 128, 130, 300])) for _ in range(E)]
+    Ks = [int(rng.choice([16, 48, 200, 512, 1030])) for _ in range(E)]
+    Ns = [int(rng.choice([8, 33, 128, 260])) for _ in range(E)]
+    srcs, ws_, dsts, params, biases, keepalive, host = [], [], [], [], [], [], []
+    for e in range(E):
+        M, K, N = Ms[e], Ks[e], Ns[e]
+        a = rng.integers(0, 256, (max(M, 1), K), dtype=np.uint8)
+        if not u8:
+            a = a.view(np.int8)
+        w = H.gen_weights(rng, K, N)
+        p = lowoha.MatmulParams(src=capi.DT_U8 if u8 else capi.DT_S8, wei=capi.DT_S8, dst=dst_dt)
+        bufs = {}
+        bias = None
+        if u8:
+            zp = np.array([int(rng.integers(100, 156))], dtype=np.int32)
+            p.src_zp = lowoha.QuantParam(zp.ctypes.data, capi.DT_S32, (1,))
+            bufs["src_zp"] = zp
+        if dst_dt != capi.DT_S32:
+            ss = np.array([float(rng.uniform(0.005, 0.03))], dtype=np.float32)
+            ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+            ws_d = H.to_dev(ws)
+            p.src_scale = lowoha.QuantParam(ss.ctypes.data, capi.DT_F32, (1,))
+            p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+            bufs.update(src_scale=ss, wei_scale=ws)
+            keepalive.append(ws_d)
+            if rng.integers(2):
+                bias = rng.standard_normal(N).astype(np.float32)
+                p.dt_bias = capi.DT_F32
+            if po is not None:
+                p.postop_ = [lowoha.PostOp(po)]
+        p.weight_cache_type = 0
+        ldc = N + int(rng.integers(0, 5))
+        srcs.append(H.to_dev(a)); ws_.append(H.to_dev(w))
+        dsts.append(torch.zeros((max(M, 1), ldc), dtype=torch_dt, device=H.DEV))
+        biases.append(H.to_dev(bias)); params.append(p)
+        host.append((a, w, bias, bufs, ldc))
+    # a uniform bias dtype is part of the call's contract only per expert; experts without bias pass null
+    st = lowoha.group_matmul_direct(["r"] * E, [False] * E, [False] * E, Ms, Ns, Ks, [1.0] * E, srcs, Ks, ws_, Ns,
+                                    biases, [0.0] * E, dsts, [h[4] for h in host], [False] * E, params)
+    if st == capi.UNIMPLEMENTED and len({p.dt_bias for p in params}) > 1:
+        pytest.skip("experts that disagree on the bias type: " + lowoha.last_error())
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for e in range(E):
+        M, K, N = Ms[e], Ks[e], Ns[e]
+        if M == 0:
+            continue
+        a, w, bias, bufs, ldc = host[e]
+        keep = []
+        ph = H.host_params(params[e], **bufs)
+        _, want, _, _ = zo.matmul_int8(a, w, ph.flat(keep), M, N, K, bias=bias)
+        got = H.to_host(dsts[e])[:M, :N]
+        if dst_dt == capi.DT_BF16:
+            H.check_bf16(got, want, max_frac=1e-2)
+        elif dst_dt == capi.DT_F32 and po == capi.PO_SWISH:
+            H.check_f32(got, want)
+        else:
+            assert np.array_equal(got, want), f"seed {seed} expert {e}: M={M} K={K} N={N}"
+        assert np.all(H.to_host(dsts[e])[:, N:] == 0)
