@@ -361,15 +361,13 @@ __global__ __launch_bounds__(256) void zmi_moe_quant_scatter_kernel(const uint16
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
   for (int k = threadIdx.x * 8; k < H; k += blockDim.x * 8) {
     float v[8];
     load8(k, v);
     __attribute__((aligned(8))) int8_t q[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      q[j] = 0;
-      if ((__float_as_uint(v[j]) & 0x7f800000u) != 0x7f800000u) q[j] = (int8_t)(int32_t)rintf(__fdiv_rn(v[j], s));
-    }
+    for (int j = 0; j < 8; ++j) q[j] = zmi_quant_elem(v[j], s, inv);
     for (int j = 0; j < topk; ++j) {
       const int slot = slot_of[t * topk + j];
       // 8 consecutive k starting at a multiple of 8 are contiguous in fragment order

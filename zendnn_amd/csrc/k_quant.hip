@@ -26,11 +26,6 @@ __device__ __forceinline__ float zmi_block_max(float v, float *red) {
   return r;
 }
 
-__device__ __forceinline__ int8_t zmi_quant_one(float v, float scale) {
-  // isfinite
-  if ((__float_as_uint(v) & 0x7f800000u) == 0x7f800000u) return 0;
-  return (int8_t)(int32_t)rintf(__fdiv_rn(v, scale));
-}
 
 // dst + dst_off(k) is where element k of this row goes: k itself for K-contiguous
 // rows, the fragment-major position otherwise (8 consecutive k starting at a
@@ -74,6 +69,7 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, int
     if (amax < 1e-10f) amax = 1e-10f;
     float s = __fdiv_rn(amax, 127.0f);
     if (s < 1e-10f) s = 1e-10f;
+    const float inv = __fdiv_rn(1.0f, s);
     if (t == 0) {
       if (scale_dt == ZMI_DT_BF16) *(uint16_t *)scale = zmi_f32_to_bf16_rne(s);
       else *(float *)scale = s;
@@ -85,7 +81,7 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, int
       if (k < K) {
         __attribute__((aligned(8))) int8_t q[8];
         #pragma unroll
-        for (int j = 0; j < 8; ++j) q[j] = zmi_quant_one(v[c][j], s);
+        for (int j = 0; j < 8; ++j) q[j] = zmi_quant_elem(v[c][j], s, inv);
         *(uint2 *)(dst + dst_off(k)) = *(const uint2 *)q;
       }
     }
@@ -102,6 +98,7 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, int
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
   if (t == 0) {
     if (scale_dt == ZMI_DT_BF16) *(uint16_t *)scale = zmi_f32_to_bf16_rne(s);
     else *(float *)scale = s;
@@ -109,7 +106,7 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, int
   if (!dst) return;
   for (int k = t; k < K; k += QT_THREADS) {
     float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)srcv)[k]) : ((const float *)srcv)[k];
-    dst[dst_off(k)] = zmi_quant_one(x, s);
+    dst[dst_off(k)] = zmi_quant_elem(x, s, inv);
   }
 }
 
@@ -207,13 +204,13 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
     }
     return amax;
   };
-  auto quant_store = [&](const float (&v)[16], float s, int k) {
+  auto quant_store = [&](const float (&v)[16], float s, float inv, int k) {
     v4i o;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       uint32_t w = 0;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) w |= ((uint32_t)(uint8_t)zmi_quant_one(v[4 * j + b], s)) << (8 * b);
+      for (int b = 0; b < 4; ++b) w |= ((uint32_t)(uint8_t)zmi_quant_elem(v[4 * j + b], s, inv)) << (8 * b);
       o[j] = (int)w;
     }
     *(v4i *)(m.dst + zmi_afrag_off(r, k, m.frag_kpad)) = o;
@@ -267,6 +264,7 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
   if (!live) return;
   if (q == 0) {
     void *sc = (char *)m.scale + (size_t)r * (scale_dt == ZMI_DT_BF16 ? 2 : 4);
@@ -282,7 +280,7 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
         v4i w[4] = {keep[st][0], keep[st][1], keep[st][0], keep[st][1]};
         float v[16];
         unpack(w, v);
-        quant_store(v, s, k);
+        quant_store(v, s, inv, k);
       }
     }
   } else {
@@ -291,7 +289,7 @@ __global__ __launch_bounds__(FR_THREADS) void zmi_quant_frag8_kernel(ZmiQuantMat
       float v[16];
       load_raw(k, w);
       unpack(w, v);
-      quant_store(v, s, k);
+      quant_store(v, s, inv, k);
     }
   }
 }
@@ -397,11 +395,12 @@ __global__ __launch_bounds__(QT_THREADS) void zmi_quant_tensor_kernel(const void
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
   if (threadIdx.x == 0) scales[row] = s;
   if (!dst) return;
   for (int64_t k = threadIdx.x; k < K; k += QT_THREADS) {
     float x = BF16 ? zmi_bf16_to_f32(((const uint16_t *)src)[row * ld + k]) : ((const float *)src)[row * ld + k];
-    dst[frag_kpad ? zmi_afrag_off(row, k, frag_kpad) : row * ld_dst + k] = zmi_quant_one(x, s);
+    dst[frag_kpad ? zmi_afrag_off(row, k, frag_kpad) : row * ld_dst + k] = zmi_quant_elem(x, s, inv);
   }
 }
 

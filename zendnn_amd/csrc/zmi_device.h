@@ -186,6 +186,23 @@ __device__ __forceinline__ float zmi_ld_f32(const void *p, int dt, int64_t i) {
   }
 }
 
+// Per-token quantization of one element: (int8) rint(v / scale) with the division correctly
+// rounded, the reference's "true divide" (scalar twin: dynamic_per_token_ref_kernel.cpp:70-96);
+// non-finite inputs give 0.  The division is what the quantization kernels spend their time
+// on, so it is replaced by v * inv (inv = 1 / scale, correctly rounded, once per row) wherever
+// that provably rounds to the same integer: |v * inv - v / scale| <= 127 * 2^-23 < 1.6e-5 and
+// the rounded quotient is within 127 * 2^-24 of the true one, so the two can round to
+// different integers only when v * inv lies within 3.8e-5 of a half-integer; those elements
+// (about one in a thousand) take the division.
+__device__ __forceinline__ int8_t zmi_quant_elem(float v, float scale, float inv) {
+  const bool finite = (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u;
+  const float x = finite ? v : 0.0f;
+  const float t = __fmul_rn(x, inv);
+  float r = rintf(t);
+  if (fabsf(t - r) > 0.4999f) r = rintf(__fdiv_rn(x, scale));
+  return (int8_t)(int32_t)r;
+}
+
 // exp(x) from the hardware exp2 with a split product x*log2(e) so the argument
 // error does not grow with |x|; about 2 ulp over the range the activations use.
 __device__ __forceinline__ float zmi_expf(float x) {

@@ -7,11 +7,6 @@
 #include "zmi_device.h"
 #include "zmi_launch.h"
 
-__device__ __forceinline__ int8_t zmi_sq_quant(float v, float scale) {
-  if ((__float_as_uint(v) & 0x7f800000u) == 0x7f800000u) return 0;
-  return (int8_t)(int32_t)rintf(__fdiv_rn(v, scale));
-}
-
 // Quantizes one source row with the whole workgroup.  The s8 row and its scale
 // are written with device-scope (write-through) stores: the eight XCDs have
 // private, mutually non-coherent L2s, and a full release / acquire fence pair
@@ -59,6 +54,7 @@ static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
   if (t == 0) {
     __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (fq.user_scales) {
@@ -73,7 +69,7 @@ static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int
       for (int h = 0; h < 2; ++h) {
         unsigned int w = 0;
         #pragma unroll
-        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(v8[h * 4 + j], s)) << (8 * j);
+        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_quant_elem(v8[h * 4 + j], s, inv)) << (8 * j);
         __hip_atomic_store(&dst[t * 2 + h], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
@@ -82,7 +78,7 @@ static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int
   for (int k4 = t; k4 < K / 4; k4 += nt) {
     unsigned int w = 0;
     #pragma unroll
-    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(ld(k4 * 4 + j), s)) << (8 * j);
+    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_quant_elem(ld(k4 * 4 + j), s, inv)) << (8 * j);
     __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
@@ -127,6 +123,7 @@ static __device__ void zmi_fused_quant_row_wave(const ZmiFusedQuant &fq, int row
   if (amax < 1e-10f) amax = 1e-10f;
   float s = __fdiv_rn(amax, 127.0f);
   if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
   if (lane == 0) {
     __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (fq.user_scales) {
@@ -143,7 +140,7 @@ static __device__ void zmi_fused_quant_row_wave(const ZmiFusedQuant &fq, int row
       for (int h = 0; h < 2; ++h) {
         unsigned int w = 0;
         #pragma unroll
-        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(v[h * 4 + j], s)) << (8 * j);
+        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_quant_elem(v[h * 4 + j], s, inv)) << (8 * j);
         __hip_atomic_store(&dst[k / 4 + h], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
@@ -152,7 +149,7 @@ static __device__ void zmi_fused_quant_row_wave(const ZmiFusedQuant &fq, int row
   for (int k4 = lane; k4 < K / 4; k4 += 64) {
     unsigned int w = 0;
     #pragma unroll
-    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_sq_quant(ld(k4 * 4 + j), s)) << (8 * j);
+    for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_quant_elem(ld(k4 * 4 + j), s, inv)) << (8 * j);
     __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
