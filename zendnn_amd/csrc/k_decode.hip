@@ -3,9 +3,9 @@
 // Same call sites as k_smallm.hip (the aocl_gemm_s8s8s32o*_sym_quant call,
 // zendnnl/src/lowoha_operators/matmul/backends/aocl/aocl_kernel.cpp:1239-1257, and the
 // in-house decode microkernel, matmul/group_matmul/custom_kernel/ukernel/
-// int8_microkernel.cpp:196-606), specialised for the one-to-sixteen-token case, where
-// the weights are streamed once from HBM and everything else has to stay out of
-// the way of that stream:
+// int8_microkernel.cpp:196-606), specialised for K_pad <= 4096 and built around the
+// one-to-sixteen-token case, where the weights are streamed once from HBM and everything
+// else has to stay out of the way of that stream:
 //   * one workgroup (8 wavefronts) per 32 weight columns and up to RPW groups of 16 rows;
 //     wavefront w streams the w-th eighth of K with 16-byte-per-lane loads, all issued up
 //     front, and keeps its weights in registers for all its row groups; with more than
@@ -20,10 +20,10 @@
 //   * the per-column / per-row epilogue constants are fetched before anything
 //     else, so the tail after the last weight byte is LDS-only;
 //   * optionally the per-token quantization of the M source rows is part of the
-//     launch: M extra workgroups at the head of the grid quantize one row each and publish it, every
-//     workgroup puts the first half of its weight stream in flight, waits for the
+//     launch: M extra workgroups at the head of the grid quantize one row each and publish it,
+//     every workgroup puts three quarters of its weight stream in flight, waits for the
 //     rows (the wait is bounded, producers wait for nothing and are dispatched
-//     first), then requests the rows and the second half of the stream.
+//     first), then requests the rows and the rest of the stream.
 #include "zmi_device.h"
 #include "zmi_fused_quant.h"
 #include "zmi_launch.h"

@@ -1,5 +1,6 @@
-// Small-M (decode) int8 GEMM for gfx950 (HBM-bound weight streaming):
-// C[M<=128, N] = epilogue(A[M,K] x blob).
+// Small-M (decode) int8 GEMM for gfx950 (HBM-bound weight streaming), any K:
+// C[M<=128, N] = epilogue(A[M,K] x blob).  k_decode.hip takes these shapes when K_pad <= 4096
+// (its rows fit LDS); this kernel takes the longer K.
 //
 // Replaces, for decode shapes, the same aocl_gemm_s8s8s32o*_sym_quant call site
 // as the large-M kernel (zendnnl/src/lowoha_operators/matmul/backends/aocl/
