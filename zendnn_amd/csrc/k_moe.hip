@@ -3,6 +3,7 @@
 // quantize-and-scatter, and the per-expert problem table.  All HBM-bound.
 #include "zmi_device.h"
 #include "zmi_launch.h"
+#include "zmi_ring_table.h"
 
 // ---------------------------------------------------------------------------
 // Gated activation in place: buf[m, 0:dim] = act(gate) * up, dim = N/2.
@@ -392,30 +393,41 @@ hipError_t zmi_launch_moe_quant_scatter(const void *x, int64_t ldx, int T, int H
 // Per-expert problem tables for Op1 (gate|up) and Op2 (down) from the device
 // side counts / offsets.
 // ---------------------------------------------------------------------------
-__global__ void zmi_moe_build_problems_kernel(ZmiMoeTables tb, int E, int H, int I, const int32_t *counts,
-                                              const int32_t *offsets, const int8_t *A1, const float *s1,
-                                              uint16_t *act, const int8_t *A2, const float *s2, uint16_t *Y,
-                                              ZmiProblem *op1, ZmiProblem *op2) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= E) return;
-  const int64_t o = offsets[e];   // a multiple of 32: every expert starts on a fragment row
-  ZmiProblem a = {};
-  a.A = A1 + o * zmi_blob_kpad(H); a.lda = H; a.blob = (const uint8_t *)tb.w13_blob[e];
-  a.dst = act + o * I; a.ldc = I; a.M = counts[e]; a.N = 2 * I; a.K = H; a.a_is_u8 = 0;
-  a.src_scale_ptr = s1 + o; a.wei_scale_ptr = tb.w13_scale[e];
-  op1[e] = a;
-  ZmiProblem b = {};
-  b.A = A2 + o * zmi_blob_kpad(I); b.lda = I; b.blob = (const uint8_t *)tb.w2_blob[e];
-  b.dst = Y + o * H; b.ldc = H; b.M = counts[e]; b.N = H; b.K = I; b.a_is_u8 = 0;
-  b.src_scale_ptr = s2 + o; b.wei_scale_ptr = tb.w2_scale[e];
-  op2[e] = b;
+__global__ __launch_bounds__(256) void zmi_moe_build_problems_kernel(ZmiMoeTables tb, int E, int H, int I,
+                                                                     const int32_t *counts, const int32_t *offsets,
+                                                                     const int8_t *A1, const float *s1, uint16_t *act,
+                                                                     const int8_t *A2, const float *s2, uint16_t *Y,
+                                                                     ZmiProblem *op1, ZmiProblem *op2, int top1,
+                                                                     int top2, int *tab1, int *tab2) {
+  // one workgroup: the problem tables first, then (their rows are visible to the whole workgroup
+  // after the barrier) wavefronts 0 and 1 fill the tile tables of the two grouped GEMM launches
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    const int64_t o = offsets[e];   // a multiple of 32: every expert starts on a fragment row
+    ZmiProblem a = {};
+    a.A = A1 + o * zmi_blob_kpad(H); a.lda = H; a.blob = (const uint8_t *)tb.w13_blob[e];
+    a.dst = act + o * I; a.ldc = I; a.M = counts[e]; a.N = 2 * I; a.K = H; a.a_is_u8 = 0;
+    a.src_scale_ptr = s1 + o; a.wei_scale_ptr = tb.w13_scale[e];
+    op1[e] = a;
+    ZmiProblem b = {};
+    b.A = A2 + o * zmi_blob_kpad(I); b.lda = I; b.blob = (const uint8_t *)tb.w2_blob[e];
+    b.dst = Y + o * H; b.ldc = H; b.M = counts[e]; b.N = H; b.K = I; b.a_is_u8 = 0;
+    b.src_scale_ptr = s2 + o; b.wei_scale_ptr = tb.w2_scale[e];
+    op2[e] = b;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  if (wave == 0 && tab1) zmi_ring_fill_table(op1, E, top1, 1, tab1, lane);
+  if (wave == 1 && tab2) zmi_ring_fill_table(op2, E, top2, 0, tab2, lane);
 }
 
+// top1 / top2, tab1 / tab2: tile heights and tile tables of the Op1 (gated) and Op2 grouped launches
+// (zmi_launch_gemm_ring_group with tab_ready = true then skips its own table launch).
 hipError_t zmi_launch_moe_build_problems(ZmiMoeTables tb, int E, int H, int I, const int32_t *counts,
                                          const int32_t *offsets, const int8_t *A1, const float *s1, void *act,
                                          const int8_t *A2, const float *s2, void *Y, ZmiProblem *op1,
-                                         ZmiProblem *op2, hipStream_t stream) {
-  hipLaunchKernelGGL(zmi_moe_build_problems_kernel, dim3((E + 63) / 64), dim3(64), 0, stream, tb, E, H, I, counts,
-                     offsets, A1, s1, (uint16_t *)act, A2, s2, (uint16_t *)Y, op1, op2);
+                                         ZmiProblem *op2, int top1, int top2, int *tab1, int *tab2,
+                                         hipStream_t stream) {
+  hipLaunchKernelGGL(zmi_moe_build_problems_kernel, dim3(1), dim3(256), 0, stream, tb, E, H, I, counts, offsets, A1,
+                     s1, (uint16_t *)act, A2, s2, (uint16_t *)Y, op1, op2, top1, top2, tab1, tab2);
   return hipGetLastError();
 }

@@ -31,6 +31,7 @@
 
 #include "zmi_device.h"
 #include "zmi_launch.h"
+#include "zmi_ring_table.h"
 
 #ifndef ZMI_RING_EPI_UNROLL
 #define ZMI_RING_EPI_UNROLL 2
@@ -69,31 +70,6 @@ struct RingCfg {
   static constexpr int ROWS_OFF = RING > EPI ? RING : EPI;  // BM row scales, live during the main loop
   static constexpr int SMEM = ROWS_OFF + BM * 4;
 };
-
-// Row blocks of one problem for a launch whose largest tile has `top` rows:
-// floor(M / top) full blocks (handled by the BM == top kernel) and one remainder
-// block handled by the smallest of {64, 128, 256} that holds it.  `top` may carry
-// ZMI_RING_PAD: the remainder then stays with the BM == top kernel as a partly
-// filled block, so that the weights of a problem are streamed by one launch only
-// (the choice when the launch is bound by weight traffic, not by MFMA work).
-#define ZMI_RING_PAD 0x10000
-template <int BM>
-__device__ __host__ __forceinline__ void zmi_ring_rows(int M, int top_flags, int &full, bool &has_rem) {
-  const int top = top_flags & 0xffff;
-  full = BM == top ? M / top : 0;
-  const int r = M % top;
-  if (top_flags & ZMI_RING_PAD) has_rem = BM == top && r > 0;
-  else has_rem = r > 0 && r <= BM && (BM == 64 || r > BM / 2);
-}
-
-template <int BM>
-__host__ __device__ __forceinline__ int zmi_ring_items(int M, int N, int top, bool gated) {
-  int full; bool rem;
-  zmi_ring_rows<BM>(M, top, full, rem);
-  const int ncols = gated ? N / 2 : N;
-  const int per = gated ? 128 : 256;
-  return (full + (rem ? 1 : 0)) * ((ncols + per - 1) / per);
-}
 
 // Interior strips with a bf16 destination: every row and column of the strip is
 // valid and 8-byte stores are aligned, so the loop body is straight-line code.
@@ -680,38 +656,9 @@ __global__ __launch_bounds__(R_THREADS) void zmi_ring_reduce_kernel(ZmiProblem p
   }
 }
 
-// Tile table of a problem set, computed where the row counts live: tab[0..2] = number of
-// tiles of the 256 / 128 / 64 row kernels, tab[4 + b * n_prob + e] = index of the first
-// tile of problem e in kernel b.  One wavefront, 64 problems per step.
 __global__ __launch_bounds__(64) void zmi_ring_count_kernel(const ZmiProblem *probs, int n_prob, int top, int gated,
                                                              int *tab) {
-  const int lane = threadIdx.x;
-  int run[3] = {0, 0, 0};
-  for (int e0 = 0; e0 < n_prob; e0 += 64) {
-    const int e = e0 + lane;
-    int c[3] = {0, 0, 0};
-    if (e < n_prob) {
-      const int M = probs[e].M, N = probs[e].N;
-      if (M > 0) {
-        if ((top & 0xffff) == 256) c[0] = zmi_ring_items<256>(M, N, top, gated != 0);
-        c[1] = zmi_ring_items<128>(M, N, top, gated != 0);
-        c[2] = zmi_ring_items<64>(M, N, top, gated != 0);
-      }
-    }
-#pragma unroll
-    for (int b = 0; b < 3; ++b) {
-      // inclusive prefix over the wavefront
-      int x = c[b];
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int y = __shfl_up(x, o);
-        if (lane >= o) x += y;
-      }
-      if (e < n_prob) tab[4 + b * n_prob + e] = run[b] + x - c[b];
-      run[b] += __shfl(x, 63);
-    }
-  }
-  if (lane == 0) { tab[0] = run[0]; tab[1] = run[1]; tab[2] = run[2]; }
+  zmi_ring_fill_table(probs, n_prob, top, gated, tab, threadIdx.x);
 }
 
 static int ring_cu_count() {
@@ -838,9 +785,10 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
 
 // Every problem of the table.  probs_host mirrors probs_dev and sizes the grids; when it is
 // null (row counts known only on the device) worst_rows / worst_cols bound them and surplus
-// workgroups exit at once.  tab_dev is 4 + 3 * n_prob ints of scratch for the tile table.
+// workgroups exit at once.  tab_dev is 4 + 3 * n_prob ints of scratch for the tile table
+// (tab_ready: already filled for this table, tile height and epilogue kind by an earlier kernel).
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
-                                      int top, int64_t worst_rows, int worst_cols, int *tab_dev,
+                                      int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
                                       const ZmiEpilogue &epi, hipStream_t stream) {
   const bool gated = epi.gated_act != 0;
   if (!tab_dev) return hipErrorInvalidValue;
@@ -866,7 +814,8 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
     }
   }
   if (items[0] + items[1] + items[2] <= 0) return hipSuccess;
-  hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0, tab_dev);
+  if (!tab_ready)
+    hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0, tab_dev);
   const bool exact = probs_host != nullptr;
   ZmiProblem dummy = {};
   const ZmiRingSplit whole = {1, nullptr};

@@ -254,7 +254,7 @@ int32_t launch_stage(const Stage &st, const char *what) {
   const int top = group_top(rows, n, kmax, cols, st.epi.gated_act != 0);
   int *tab = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)n));
   if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
-  if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, st.epi, stream()), what)) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) return ZMI_FAILURE;
   return ZMI_SUCCESS;
 }
 
@@ -660,7 +660,10 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
     (void)hipGetLastError();
     if (!hip_ok(zmi_launch_moe_quant_scatter(d->x, d->ldx, T, H, topk, slot_of, A1, s1, s), "quant scatter launch")) return ZMI_FAILURE;
   }
-  if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, s), "problem table launch")) return ZMI_FAILURE;
+  // row counts live on the device: the grids are sized for the worst case, and the kernel that builds
+  // the per-expert problem tables fills the tile tables of both grouped launches as well
+  const int top1 = group_top(R, E, H, 2 * I, true), top2 = group_top(R, E, I, H, false);
+  if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, top1, top2, tile_tab1, tile_tab2, s), "problem table launch")) return ZMI_FAILURE;
 
   ZmiEpilogue e1;
   std::memset(&e1, 0, sizeof(e1));
@@ -669,12 +672,10 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   e1.bias_dt = ZMI_DT_F32; e1.alpha = 1.0f; e1.beta = 0.0f; e1.dst_dt = ZMI_DT_BF16; e1.fast_kind = ZMI_EK_NONE;
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
-  // row counts live on the device: the grids are sized for the worst case
-  const int top1 = group_top(R, E, H, 2 * I, true), top2 = group_top(R, E, I, H, false);
-  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, true, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;
   upload_fence();
   set_kernel_name("moe_fused_device");

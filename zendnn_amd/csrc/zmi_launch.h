@@ -64,7 +64,7 @@ ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices);
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, const ZmiRingSplit *split,
                                 hipStream_t stream);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
-                                      int top, int64_t worst_rows, int worst_cols, int *tab_dev,
+                                      int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
                                       const ZmiEpilogue &epi, hipStream_t stream);
 
 // k_smallm.hip
@@ -122,9 +122,10 @@ struct ZmiMoeTables {   // device arrays of E entries each
   const float *const *w2_scale;
 };
 hipError_t zmi_launch_moe_build_problems(ZmiMoeTables tb, int E, int H, int I, const int32_t *counts,
-                                         const int32_t *offsets, const int8_t *A1, const float *s1,
-                                         void *act, const int8_t *A2, const float *s2, void *Y,
-                                         ZmiProblem *op1, ZmiProblem *op2, hipStream_t stream);
+                                         const int32_t *offsets, const int8_t *A1, const float *s1, void *act,
+                                         const int8_t *A2, const float *s2, void *Y, ZmiProblem *op1,
+                                         ZmiProblem *op2, int top1, int top2, int *tab1, int *tab2,
+                                         hipStream_t stream);
 
 // k_util.hip
 hipError_t zmi_launch_pad_rows(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans,
