@@ -53,7 +53,6 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
   const int M = p.M, N = p.N, K = p.K;
   const int K_pad = (int)zmi_blob_kpad(K);
   const int nchunks = K_pad / 64;
-  const bool gated = epi.gated_act != 0;
   // With fused quantization the first M workgroups only quantize one source row each,
   // publish it and leave; the streaming workgroups follow them in dispatch order.
   if (fq.x && (int)blockIdx.x < M) {
@@ -80,27 +79,17 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
 
-  // the two 16-column groups h = 0, 1: weight column wcol[h], output column ocol[h]
-  // (gated: h = 0 gate, h = 1 up, one output column)
-  int wcol[2], ocol[2];
-  if (!gated) {
-    wcol[0] = blk * 32; wcol[1] = blk * 32 + 16;
-    ocol[0] = wcol[0]; ocol[1] = wcol[1];
-  } else {
-    wcol[0] = blk * 16; wcol[1] = blk * 16 + N / 2;
-    ocol[0] = blk * 16; ocol[1] = blk * 16;
-  }
+  // the two 16-column groups h = 0, 1 of the block
+  const int wcol[2] = {blk * 32, blk * 32 + 16};
 
   // ---- epilogue constants of this thread's output element, fetched first ----
-  // plain: element (row tid/32, column tid%32); gated: threads < 256, (row tid/16, column tid%16)
-  const int e_row = gated ? tid / 16 : tid / 32;
-  const int e_h = gated ? 0 : (tid % 32) / 16;
+  // element (row tid/32, column tid%32) of every row group
+  const int e_row = tid / 32;
+  const int e_h = (tid % 32) / 16;
   const int e_c = tid % 16;
-  const int e_n = ocol[e_h] + e_c;
-  const bool e_col = e_row < 16 && (gated ? e_n < N / 2 : e_n < N);
-  ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_col ? e_n : N, N);
-  ZmiColCtx cc1 = cc0;
-  if (gated) cc1 = zmi_col_ctx(epi, p, colsum, e_col ? e_n + N / 2 : N, N);
+  const int e_n = wcol[e_h] + e_c;
+  const bool e_col = e_n < N;
+  const ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_col ? e_n : N, N);
   // (with fused quantization the row scales exist only after the wait below)
   float rs[RPW];
   auto load_rs = [&]() {
@@ -232,14 +221,11 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
   for (int j = 0; j < RPW; ++j) {
     const int m = r0 + j * 16 + e_row;
     if (m >= M) break;
-    if (!gated) zmi_finish_element(p, epi, cc0, rs[j], fetch(j, e_h), m, e_n);
-    else zmi_finish_gated(p, epi, cc0, cc1, rs[j], fetch(j, 0), fetch(j, 1), m, e_n);
+    zmi_finish_element(p, epi, cc0, rs[j], fetch(j, e_h), m, e_n);
   }
 }
 
-int zmi_decode_grid(const ZmiProblem &p, bool gated) {
-  return gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
-}
+int zmi_decode_grid(const ZmiProblem &p) { return (int)(zmi_blob_npad(p.N) / 32); }
 
 bool zmi_decode_kernel_fits(const ZmiProblem &p) {
   return p.M > 0 && p.M <= 128 && zmi_blob_kpad(p.K) <= 4096;
@@ -248,8 +234,8 @@ bool zmi_decode_kernel_fits(const ZmiProblem &p) {
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
                                   hipStream_t stream) {
   if (!zmi_decode_kernel_fits(p)) return hipErrorInvalidValue;
-  const bool gated = epi.gated_act != 0;
-  const int n_blk = zmi_decode_grid(p, gated);
+  if (epi.gated_act != 0) return hipErrorInvalidValue;   // gated GEMMs are grouped launches: the large-M kernel
+  const int n_blk = zmi_decode_grid(p);
   if (n_blk <= 0) return hipSuccess;
   // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at
   // 32 / 64 rows, N = K = 4096, against 13 / 20 us with 64); above that, 64 rows per workgroup

@@ -31,45 +31,19 @@
 // The wait is bounded; producers never wait for anything, and the host only
 // uses this form when the whole grid is resident at once.
 template <int MB, int UNROLL>
-__global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, const ZmiProblem *probs,
-                                                               int n_prob, int m_lo, int m_hi,
-                                                               ZmiEpilogue epi, ZmiFusedQuant fq) {
+__global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p, ZmiEpilogue epi, ZmiFusedQuant fq) {
   extern __shared__ __attribute__((aligned(16))) int32_t red[];   // [W][MB*2*4*64]
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int W = blockDim.x / 64;
-  const bool gated = epi.gated_act != 0;
-
-  // ---- which problem / column block ----
-  ZmiProblem p = p0;
-  int blk = blockIdx.x;
-  if (probs) {
-    int base = 0, e = 0;
-    for (; e < n_prob; ++e) {
-      const int M = probs[e].M;
-      if (!(M > m_lo && M <= m_hi)) continue;
-      const int cnt = gated ? probs[e].N / 2 / 16 : (int)(zmi_blob_npad(probs[e].N) / 32);
-      if (blk < base + cnt) break;
-      base += cnt;
-    }
-    if (e == n_prob) return;
-    p = probs[e];
-    blk -= base;
-  }
+  const int blk = blockIdx.x;   // one 32-column block of the blob
   const int M = p.M, N = p.N, K = p.K;
   const int64_t K_pad = zmi_blob_kpad(K);
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
 
-  // the two 16-column groups h = 0, 1 this workgroup multiplies: weight column
-  // wcol[h], stored to output column ocol[h] (gated: h=0 gate, h=1 up, one output)
-  int wcol[2], ocol[2];
-  if (!gated) {
-    wcol[0] = blk * 32; wcol[1] = blk * 32 + 16;
-    ocol[0] = wcol[0]; ocol[1] = wcol[1];
-  } else {
-    wcol[0] = blk * 16; wcol[1] = blk * 16 + N / 2;
-    ocol[0] = blk * 16; ocol[1] = blk * 16;
-  }
+  // the two 16-column groups h = 0, 1 this workgroup multiplies
+  const int wcol[2] = {blk * 32, blk * 32 + 16};
+  const int *ocol = wcol;
 
   // lane role inside a 16x16x64 operand: column / row c16, k group g (16 bytes each)
   const int c16 = lane % 16, g = lane / 16;
@@ -173,7 +147,6 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
       for (int j = 0; j < 4; ++j) red[wave * PER_WAVE + ((mb * 2 + h) * 4 + j) * 64 + lane] = acc[mb][h][j];
   __syncthreads();
 
-  const void *bias = p.bias;
   const int rows = M < MB * 16 ? M : MB * 16;
 
   // acc[mb][h][j] of lane l is row mb*16 + (l/16)*4 + j, column h*16 + l%16
@@ -185,66 +158,17 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p0, co
     return s;
   };
 
-  if (!gated) {
-    const bool raw = zmi_epilogue_is_raw_s32(epi, bias);
-    const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
-    const bool has_bias = bias != nullptr;
-    for (int e = tid; e < rows * 32; e += blockDim.x) {
-      const int row = e / 32, col = e % 32;
-      const int h = col / 16, cidx = col % 16;
-      const int n = ocol[h] + cidx;
-      if (n >= N) continue;
-      const int32_t s = fetch(row, h, cidx);
-      const ZmiColCtx cc = zmi_col_ctx(epi, p, colsum, n, N);
-      const int64_t o = (int64_t)row * p.ldc + n;
-      const float rs = zmi_row_scale(epi, p, row);
-      const bool bf = epi.dst_dt == ZMI_DT_BF16;
-      // straight-line variants for the common epilogues, interpreter otherwise
-      switch (epi.fast_kind) {
-      case ZMI_EK_NONE: {
-        const float y = zmi_fast_value<ZMI_EK_NONE>(s, cc, rs, has_rs, has_ws, has_bias);
-        if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
-        break;
-      }
-      case ZMI_EK_SWISH: {
-        const float y = zmi_fast_value<ZMI_EK_SWISH>(s, cc, rs, has_rs, has_ws, has_bias);
-        if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
-        break;
-      }
-      case ZMI_EK_GELU_TANH: {
-        const float y = zmi_fast_value<ZMI_EK_GELU_TANH>(s, cc, rs, has_rs, has_ws, has_bias);
-        if (bf) zmi_fast_store<true>(p.dst, o, y); else zmi_fast_store<false>(p.dst, o, y);
-        break;
-      }
-      default:
-        if (raw) ((int32_t *)p.dst)[o] = s + cc.comp;
-        else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, cc, rs, row, n, p.dst, p.ldc));
-      }
-    }
-  } else {
-    const int half = N / 2;
-    for (int e = tid; e < rows * 16; e += blockDim.x) {
-      const int row = e / 16, cidx = e % 16;
-      const int n = ocol[0] + cidx;
-      if (n >= half) continue;
-      const int32_t sg = fetch(row, 0, cidx), su = fetch(row, 1, cidx);
-      ZmiColCtx cg = zmi_col_ctx(epi, p, colsum, n, N);
-      ZmiColCtx cu = zmi_col_ctx(epi, p, colsum, n + half, N);
-      const float rs = zmi_row_scale(epi, p, row);
-      float gv = zmi_epilogue_value(epi, sg, cg, rs, row, n, p.dst, p.ldc);
-      float uv = zmi_epilogue_value(epi, su, cu, rs, row, n + half, p.dst, p.ldc);
-      if (epi.dst_dt == ZMI_DT_BF16) {
-        gv = zmi_bf16_to_f32(zmi_f32_to_bf16(gv));
-        uv = zmi_bf16_to_f32(zmi_f32_to_bf16(uv));
-      }
-      zmi_store(p.dst, epi.dst_dt, (int64_t)row * p.ldc + n, zmi_gated(epi.gated_act, gv, uv));
-    }
+  for (int e = tid; e < rows * 32; e += blockDim.x) {
+    const int row = e / 32, col = e % 32;
+    const int h = col / 16, cidx = col % 16;
+    const int n = ocol[h] + cidx;
+    if (n >= N) continue;
+    zmi_finish_element(p, epi, zmi_col_ctx(epi, p, colsum, n, N), zmi_row_scale(epi, p, row), fetch(row, h, cidx), row, n);
   }
 }
 
 template <int MB, int UNROLL>
-static hipError_t launch_small(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int m_lo, int m_hi,
-                               int grid, int W, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
+static hipError_t launch_small(const ZmiProblem &p, int grid, int W, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
                                hipStream_t stream) {
   size_t smem = (size_t)W * MB * 2 * 4 * 64 * sizeof(int32_t);
   if (smem < 256) smem = 256;
@@ -255,8 +179,7 @@ static hipError_t launch_small(const ZmiProblem &p0, const ZmiProblem *probs, in
     if (e != hipSuccess) return e;
     attr_smem = smem;
   }
-  hipLaunchKernelGGL((zmi_gemm_smallm_kernel<MB, UNROLL>), dim3(grid), dim3(W * 64), smem, stream, p0, probs,
-                     n_prob, m_lo, m_hi, epi, fq);
+  hipLaunchKernelGGL((zmi_gemm_smallm_kernel<MB, UNROLL>), dim3(grid), dim3(W * 64), smem, stream, p, epi, fq);
   return hipGetLastError();
 }
 
@@ -272,30 +195,28 @@ static int pick_waves(int grid, int MB, int64_t K_pad) {
   return W;
 }
 
-static hipError_t dispatch_small(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int m_lo,
-                                 int m_hi, int grid, int64_t K_pad, const ZmiEpilogue &epi,
-                                 const ZmiFusedQuant &fq, hipStream_t stream) {
+static hipError_t dispatch_small(const ZmiProblem &p, int grid, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
+                                 hipStream_t stream) {
   if (grid <= 0) return hipSuccess;
-  const int mb = (m_hi + 15) / 16;
-  if (mb <= 1) return launch_small<1, 8>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 1, K_pad), epi, fq, stream);
-  if (mb <= 2) return launch_small<2, 4>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 2, K_pad), epi, fq, stream);
-  if (mb <= 4) return launch_small<4, 2>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 4, K_pad), epi, fq, stream);
-  return launch_small<8, 1>(p0, probs, n_prob, m_lo, m_hi, grid, pick_waves(grid, 8, K_pad), epi, fq, stream);
+  if (epi.gated_act != 0) return hipErrorInvalidValue;   // gated GEMMs are grouped launches: the large-M kernel
+  const int64_t K_pad = zmi_blob_kpad(p.K);
+  const int mb = (p.M + 15) / 16;
+  if (mb <= 1) return launch_small<1, 8>(p, grid, pick_waves(grid, 1, K_pad), epi, fq, stream);
+  if (mb <= 2) return launch_small<2, 4>(p, grid, pick_waves(grid, 2, K_pad), epi, fq, stream);
+  if (mb <= 4) return launch_small<4, 2>(p, grid, pick_waves(grid, 4, K_pad), epi, fq, stream);
+  return launch_small<8, 1>(p, grid, pick_waves(grid, 8, K_pad), epi, fq, stream);
 }
 
-static int small_blocks(const ZmiProblem &p, bool gated) {
-  return gated ? p.N / 2 / 16 : (int)(zmi_blob_npad(p.N) / 32);
-}
+static int small_blocks(const ZmiProblem &p) { return (int)(zmi_blob_npad(p.N) / 32); }
 
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
   if (p.M <= 0) return hipSuccess;
   if (p.M > 128) return hipErrorInvalidValue;
   ZmiFusedQuant none = {};
-  return dispatch_small(p, nullptr, 1, 0, p.M, small_blocks(p, epi.gated_act != 0), zmi_blob_kpad(p.K), epi,
-                        none, stream);
+  return dispatch_small(p, small_blocks(p), epi, none, stream);
 }
 
-int zmi_smallm_grid(const ZmiProblem &p, bool gated) { return small_blocks(p, gated); }
+int zmi_smallm_grid(const ZmiProblem &p) { return small_blocks(p); }
 
 // Same, with the per-token quantization of the source rows fused into the launch.
 // Only valid when the whole grid is resident at once (zmi_smallm_grid(p) <= 2 * #CUs).
@@ -303,6 +224,5 @@ hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &
                                         hipStream_t stream) {
   if (p.M <= 0) return hipSuccess;
   if (p.M > 128) return hipErrorInvalidValue;
-  return dispatch_small(p, nullptr, 1, 0, p.M, small_blocks(p, epi.gated_act != 0), zmi_blob_kpad(p.K), epi,
-                        fq, stream);
+  return dispatch_small(p, small_blocks(p), epi, fq, stream);
 }

@@ -426,7 +426,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
     const bool decode_kernel = decode_kernel_allowed(M, N, K);
     // (the decode kernel's producers are its first workgroups and wait for nothing, so its grid need not be resident)
-    if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob, false) <= 512) &&
+    if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
       if (!ctr) return ZMI_FAILURE;

@@ -518,16 +518,4 @@ __device__ __forceinline__ void zmi_finish_element(const ZmiProblem &p, const Zm
     else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, c, rs, m, n, p.dst, p.ldc));
   }
 }
-// Gated pair: sg / su are the accumulators of weight columns n (gate) and n + N/2 (up);
-// the output column is n.
-__device__ __forceinline__ void zmi_finish_gated(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &cg,
-                                                 const ZmiColCtx &cu, float rs, int32_t sg, int32_t su, int m, int n) {
-  float gv = zmi_epilogue_value(epi, sg, cg, rs, m, n, p.dst, p.ldc);
-  float uv = zmi_epilogue_value(epi, su, cu, rs, m, n + p.N / 2, p.dst, p.ldc);
-  if (epi.dst_dt == ZMI_DT_BF16) {
-    gv = zmi_bf16_to_f32(zmi_f32_to_bf16(gv));
-    uv = zmi_bf16_to_f32(zmi_f32_to_bf16(uv));
-  }
-  zmi_store(p.dst, epi.dst_dt, (int64_t)m * p.ldc + n, zmi_gated(epi.gated_act, gv, uv));
-}
 #endif  // __HIPCC__

@@ -81,7 +81,7 @@ struct ZmiFusedQuant {
   unsigned int target;    // value the counter reaches when all M rows of this launch are published
 };
 
-int zmi_smallm_grid(const ZmiProblem &p, bool gated);
+int zmi_smallm_grid(const ZmiProblem &p);
 hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant &fq,
                                         hipStream_t stream);
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
@@ -91,7 +91,7 @@ bool zmi_decode_kernel_fits(const ZmiProblem &p);
 // fq != null: the launch also quantizes the M source rows (its grid must be resident at once)
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
                                   hipStream_t stream);
-int zmi_decode_grid(const ZmiProblem &p, bool gated);
+int zmi_decode_grid(const ZmiProblem &p);
 
 // k_moe.hip
 struct ZmiActMat {
