@@ -103,7 +103,10 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
 
   // ---- activation loads (row-contiguous): 64 items (row, 1 KiB segment) per row group; wavefront w takes rows w and w + 8 ----
   const int c16 = lane % 16, g = lane / 16;
-  v4i araw[2][4];
+  // (two register sets when a workgroup has several row groups: the rows of group j + 2 are
+  // requested while group j is multiplied, which covers their L2 latency)
+  constexpr int NSET = RPW > 1 ? 2 : 1;
+  v4i araw[NSET][2][4];
   auto load_rows = [&](int j) {
     const int8_t *A = (const int8_t *)p.A;
     const int G = ((K + 15) & ~15) / 16;   // readable 16-byte granules per row
@@ -114,7 +117,7 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
         const int row = r0 + j * 16 + wave + 8 * i, gran = s * 64 + lane;
         v4i v = {0, 0, 0, 0};
         if (row < M && gran < G) v = *(const v4i *)(A + (int64_t)row * p.lda + gran * 16);
-        araw[i][s] = v;
+        araw[j % NSET][i][s] = v;
       }
   };
   // rows -> LDS in operand order
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
       #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const int row = wave + 8 * i, gran = s * 64 + lane;
-        v4i v = araw[i][s];
+        v4i v = araw[j % NSET][i][s];
         v[0] ^= xm; v[1] ^= xm; v[2] ^= xm; v[3] ^= xm;
         if (r0 + j * 16 + row >= M) v = (v4i){0, 0, 0, 0};
         // granule s*64 + lane: chunk s*16 + lane/4, k group lane%4 (the swizzle does not depend on s)
@@ -156,6 +159,7 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
     load_rows(0);
     #pragma unroll
     for (int u = 0; u < 8; ++u) load_b(u);
+    if (RPW > 1 && r0 + 16 < M) load_rows(1);
   } else {
     #pragma unroll
     for (int u = 0; u < DEC_FQ_FIRST; ++u) load_b(u);
@@ -172,10 +176,11 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
     load_rows(0);
     #pragma unroll
     for (int u = DEC_FQ_FIRST; u < 8; ++u) load_b(u);
+    if (RPW > 1 && r0 + 16 < M) load_rows(1);
   }
 
   // ---- per row group: rows -> LDS, then one 16x16x64 MFMA per chunk and column group; the
-  // next group's rows are requested before the MFMAs of this one ----
+  // rows of the group after the next are requested before the MFMAs of this one ----
   v4i acc[RPW][2];
   #pragma unroll
   for (int j = 0; j < RPW; ++j) {
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
     if (j > 0) __syncthreads();                // every wavefront has read the previous group's rows
     store_rows(j);
     __syncthreads();
-    if (j + 1 < RPW && r0 + (j + 1) * 16 < M) load_rows(j + 1);
+    if (j + 2 < RPW && r0 + (j + 2) * 16 < M) load_rows(j + 2);
     #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const bool live = c_begin + u < c_end;
