@@ -220,7 +220,7 @@ def test_fused_moe_random_configuration(zo, seed):
     T = int(rng.choice([1, 5, 33, 130, 260]))
     Hd = int(rng.choice([64, 128, 320, 512]))
     I = int(rng.choice([16, 48, 96, 160, 352]))
-    E = int(rng.choice([1, 2, 3, 8, 16, 40, 70]))
+    E = int(rng.choice([2, 3, 8, 16, 40, 70]))     # (one expert would be the reference's sequential-chain form: src.size() == 1)
     topk = int(rng.integers(1, min(E, 6) + 1))
     skew = bool(rng.integers(2))
     c = MH.make_case(0x5EED1000 + seed, T, Hd, I, E, topk, skew)
@@ -247,7 +247,7 @@ def test_group_of_unrelated_gemms_random_configuration(zo, seed):
     sources with per-tensor scales and zero-points, f32 bias, one post-op, f32 / bf16 / s32 destinations with padded
     leading dimensions.  Every expert is compared with the oracle's single matmul."""
     rng = np.random.default_rng(9000 + seed)
-    E = int(rng.integers(1, 7))
+    E = int(rng.integers(2, 7))                    # (src.size() == 1 is the sequential-chain form)
     u8 = bool(rng.integers(2))
     dst_dt = [capi.DT_F32, capi.DT_BF16, capi.DT_S32][int(rng.integers(3))]
     po = [None, capi.PO_RELU, capi.PO_SWISH][int(rng.integers(3))] if dst_dt != capi.DT_S32 else None

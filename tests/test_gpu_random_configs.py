@@ -77,7 +77,10 @@ def test_static_quant_random_configuration(zo, seed):
     what = f"seed {seed}: M={M} K={K} N={N} u8={u8} tA={transA} tB={transB} dst={dst_dt} po={po} [{lowoha.last_kernel()}]"
     g, wv = got[:, :N], want[:, :N]
     if dst_dt == capi.DT_BF16:
-        H.check_bf16(g, wv, atol=1e-6 if po == capi.PO_GELU_TANH else 0.0, max_frac=1e-2)
+        if po is None or po == capi.PO_RELU:
+            assert np.array_equal(g, wv), what         # every step of the chain is a correctly rounded f32 operation
+        else:
+            H.check_bf16(g, wv, atol=1e-6 if po == capi.PO_GELU_TANH else 0.0, max_frac=1e-2)
     elif dst_dt == capi.DT_F32:
         if po is None or po == capi.PO_RELU:
             assert np.array_equal(g, wv), what
@@ -134,7 +137,9 @@ def test_dynamic_quant_random_configuration(zo, seed):
     what = f"seed {seed}: M={M} K={K} N={N} src={src_dt} dst={dst_dt} per_token={per_token} po={po} [{lowoha.last_kernel()}]"
     got_sc = H.to_host(scales_d)
     assert np.array_equal(got_sc, np.asarray(scales, dtype=np.float32).reshape(-1)[:n_sc]), what
-    if dst_dt == capi.DT_BF16:
+    if po is None or po == capi.PO_RELU:
+        assert np.array_equal(H.to_host(dst), want), what   # exact scales, exact quantization, correctly rounded f32 chain
+    elif dst_dt == capi.DT_BF16:
         H.check_bf16(H.to_host(dst), want, atol=1e-6 if po == capi.PO_GELU_TANH else 0.0, max_frac=1e-2)
     else:
         H.check_f32(H.to_host(dst), want, rtol=1e-5, atol=1e-6)

@@ -89,8 +89,8 @@ __device__ __forceinline__ void zmi_ring_strip_bf16(const int32_t *stage, const 
     float y0[4], y1[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      y0[j] = __builtin_fmaf((float)(a0[j] + cc[0][j].comp) * rs, cc[0][j].wscale, cc[0][j].bias);
-      y1[j] = __builtin_fmaf((float)(a1[j] + cc[1][j].comp) * rs, cc[1][j].wscale, cc[1][j].bias);
+      y0[j] = __fadd_rn(__fmul_rn(__fmul_rn((float)(a0[j] + cc[0][j].comp), rs), cc[0][j].wscale), cc[0][j].bias);
+      y1[j] = __fadd_rn(__fmul_rn(__fmul_rn((float)(a1[j] + cc[1][j].comp), rs), cc[1][j].wscale), cc[1][j].bias);
     }
     if (!GATED) {
 #pragma unroll
@@ -447,11 +447,11 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
         if (m >= M) continue;
         float y0[4], y1[4];
         if (DT == 1) {
-          // bf16 store: scale chain with one fused multiply-add (absent scales are 1, absent bias -0)
+          // bf16 store: the reference's separately rounded scale chain (absent scales are 1, absent bias -0)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            y0[j] = __builtin_fmaf((float)(a0[j] + cc[0][j].comp) * rs, cc[0][j].wscale, cc[0][j].bias);
-            y1[j] = __builtin_fmaf((float)(a1[j] + cc[1][j].comp) * rs, cc[1][j].wscale, cc[1][j].bias);
+            y0[j] = __fadd_rn(__fmul_rn(__fmul_rn((float)(a0[j] + cc[0][j].comp), rs), cc[0][j].wscale), cc[0][j].bias);
+            y1[j] = __fadd_rn(__fmul_rn(__fmul_rn((float)(a1[j] + cc[1][j].comp), rs), cc[1][j].wscale), cc[1][j].bias);
             if (!gated) { y0[j] = zmi_act_bf16<EK>(y0[j]); y1[j] = zmi_act_bf16<EK>(y1[j]); }
           }
         } else {
