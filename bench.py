@@ -41,7 +41,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
+                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
                              "moe_config4", "moe_config5"],
                     help="run one of the other configs alone and print its entry (for profiler runs)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -214,6 +214,36 @@ def main():
                 "gemm_only_GBps": round((K_DEC * N_DEC + m * K_DEC + m * 4 + N_DEC * 4 + m * N_DEC * 2) / (tk * 1e-3) / 1e9, 1),
                 "kernel": lowoha.last_kernel()}
 
+    def run_decode_per_group(m, gs):
+        # the decode call with per-group scales: {M,G} source scales computed by the library, {G,N} weight scales,
+        # G = K / gs; two launches (per-group quantization, per-group GEMM); bytes = the per-token call's + the scales
+        G = K_DEC // gs
+        blobs = [prepack(rand_w(K_DEC, N_DEC), K_DEC, N_DEC) for _ in range(n_sets)]
+        ws = torch.rand((G, N_DEC), device=dev, generator=g) * 0.009 + 0.001
+        x = torch.randn((m, K_DEC), device=dev, generator=g).to(torch.bfloat16)
+        dst = torch.zeros((m, N_DEC), dtype=torch.bfloat16, device=dev)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (m, G))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (G, N_DEC))
+        p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        calls = [lowoha.prepared_matmul("r", False, False, m, N_DEC, K_DEC, 1.0, x, K_DEC, blob, N_DEC, None, 0.0,
+                                        dst, N_DEC, True, p)[0] for blob in blobs]
+        state = {"i": 0}
+
+        def step():
+            st = calls[state["i"] % n_sets]()
+            state["i"] += 1
+            if st != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+
+        t = ev_time(step, 100, 10)
+        nbytes = K_DEC * N_DEC + m * K_DEC * 2 + G * N_DEC * 4 + m * G * 4 + m * N_DEC * 2
+        return {"GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2), "group_size": gs,
+                "kernel": lowoha.last_kernel()}
+
     def run_prefill(N):
         # config 3: whole call = per-token quantization launch (rows written in MFMA fragment order) + GEMM launch;
         # the per-kernel split is in the rocprofv3 summaries under profiles/
@@ -298,6 +328,8 @@ def main():
         # (64 rows) and the K-sliced large-M kernel (128 rows)
         "decode_M64": lambda: run_decode_m(64),
         "decode_M128": lambda: run_decode_m(128),
+        "decode_M16_per_group128": lambda: run_decode_per_group(16, 128),
+        "decode_M16_per_group32": lambda: run_decode_per_group(16, 32),
         "prefill_N4096": lambda: run_prefill(4096),
         "prefill_N14336": lambda: run_prefill(14336),
         "config1_u8s8_M128": run_config1,

@@ -43,6 +43,9 @@ def lib():
         L.zo_quant_per_token.restype = None
         L.zo_quant_per_token.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64,
                                          C.c_void_p, C.c_int64, C.c_void_p]
+        L.zo_quant_per_group.restype = None
+        L.zo_quant_per_group.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                         C.c_void_p, C.c_int64, C.c_void_p]
         L.zo_gemm_s32.restype = C.c_int64
         L.zo_gemm_s32.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
                                   C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
@@ -102,6 +105,16 @@ def quant_per_token(src, src_dt):
     return q, s
 
 
+def quant_per_group(src, src_dt, G):
+    """src [M,K] (float32, or uint16 bf16 bits) -> (q int8 [M,K], scales f32 [M,G]); K % G == 0."""
+    src = np.ascontiguousarray(src)
+    M, K = src.shape
+    q = np.empty((M, K), dtype=np.int8)
+    s = np.empty((M, G), dtype=np.float32)
+    lib().zo_quant_per_group(_p(src), src_dt, M, K, G, K, _p(q), K, _p(s))
+    return q, s
+
+
 def gemm_s32(A, B, transA=False, transB=False):
     """Exact s32 accumulator; A u8/s8 [M,K] (or [K,M] if transA), B s8 [K,N]
     (or [N,K] if transB).  Returns (acc [M,N] int32, overflow_count)."""
@@ -118,7 +131,7 @@ def gemm_s32(A, B, transA=False, transB=False):
 
 def matmul_int8(src, weight, params, M, N, K, *, bias=None, dst=None, lda=None, ldb=None,
                 ldc=None, transA=False, transB=False, alpha=1.0, beta=0.0, want_acc=False,
-                want_scales=False):
+                want_scales=False, n_scales=None):
     """Runs the oracle's matmul_direct on host arrays.  params is a
     capi.MatmulParamsT whose buff pointers reference host memory.  Returns
     (status, dst array, acc or None, scales or None)."""
@@ -130,7 +143,7 @@ def matmul_int8(src, weight, params, M, N, K, *, bias=None, dst=None, lda=None, 
     if dst is None:
         dst = np.zeros((M, ldc), dtype=NP_OF_DT[params.dt_dst])
     acc = np.empty((M, N), dtype=np.int32) if want_acc else None
-    scales = np.empty((M,), dtype=np.float32) if want_scales else None
+    scales = np.empty((n_scales or M,), dtype=np.float32) if want_scales else None   # (M * G with per-group scales)
     call = MatmulCall()
     call.layout = b"r"
     call.transA, call.transB = int(transA), int(transB)

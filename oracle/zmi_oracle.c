@@ -26,6 +26,11 @@
  *   dequant chain / bias         special cases (unit scales, equal per-channel
  *                                scales == per-tensor), op order from source
  *   post-ops                     libm double evaluation within 2 f32 ulp
+ *   per-group scales             closed form (all-ones operands, power-of-two scales: every step exact),
+ *                                equal power-of-two group scales == per-token chain bit for bit,
+ *                                numpy float32 brute force on small random cases
+ *   zo_quant_per_group           per-group constants (closed form), == zo_quant_per_token on the
+ *                                [M*G, K/G] view
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
  *   prepack layout, weight_prepack_size values: parity unpinned (opaque by the
  *     reference's contract; only the round trip matmul(prepack(B)) == matmul(B)
@@ -148,6 +153,38 @@ ZO_EXPORT void zo_quant_per_token(const void *src, int32_t src_dt, int64_t M, in
       if (!isfinite(v)) { dst[m * ld_dst + j] = 0; continue; }
       int32_t q = (int32_t)nearbyintf(v / scale);
       dst[m * ld_dst + j] = (int8_t)q;
+    }
+  }
+}
+
+/* Per-group dynamic quantization, symmetric: the per-token rule applied to each of the G
+ * slices of a row (lowoha_operators/reorder/reorder_data_type/dynamic_quant_impl/
+ * per_group_avx512_f32_fma_kernel.cpp:78-86 for the scale, :276-292 for q = nearbyint(v / scale)
+ * with the true division; dispatch by the {M,G} scale dims, lowoha_reorder.cpp:167-171).
+ * scales is {M,G} row-major. */
+ZO_EXPORT void zo_quant_per_group(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t G,
+                                  int64_t ld_src, int8_t *dst, int64_t ld_dst, float *scales) {
+  const int64_t gs = K / G;
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t g = 0; g < G; ++g) {
+      float absmax = 0.0f;
+      for (int64_t j = 0; j < gs; ++j) {
+        float v = zo_read_f32(src, src_dt, m * ld_src + g * gs + j);
+        if (isfinite(v)) {
+          float a = fabsf(v);
+          if (a > absmax) absmax = a;
+        }
+      }
+      if (absmax < 1e-10f) absmax = 1e-10f;
+      float scale = absmax / 127.0f;
+      if (scale < 1e-10f) scale = 1e-10f;
+      scales[m * G + g] = scale;
+      if (!dst) continue;
+      for (int64_t j = 0; j < gs; ++j) {
+        float v = zo_read_f32(src, src_dt, m * ld_src + g * gs + j);
+        dst[m * ld_dst + g * gs + j] = isfinite(v) ? (int8_t)(int32_t)nearbyintf(v / scale) : 0;
+      }
     }
   }
 }
@@ -346,7 +383,11 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
     sbuf = (float *)malloc(sizeof(float) * (size_t)M);
     int64_t dn = 1;
     for (int i = 0; i < p->src_scale.ndims; ++i) dn *= p->src_scale.dims[i];
-    if (dn == M && M > 1) {
+    if (dn > M && dn % M == 0 && K % (dn / M) == 0) {
+      free(sbuf);
+      sbuf = (float *)malloc(sizeof(float) * (size_t)dn);
+      zo_quant_per_group(A, a_dt, M, K, dn / M, lda, qbuf, K, sbuf);
+    } else if (dn == M && M > 1) {
       zo_quant_per_token(A, a_dt, M, K, lda, qbuf, K, sbuf);
     } else {
       /* per-tensor dynamic scale: same formula over the whole tensor,
@@ -369,13 +410,66 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
       }
       dn = 1;
     }
-    if (c->scale_out) memcpy(c->scale_out, sbuf, sizeof(float) * (size_t)(dn == 1 ? 1 : M));
+    if (c->scale_out) memcpy(c->scale_out, sbuf, sizeof(float) * (size_t)dn);
     A = qbuf; a_dt = ZMI_DT_S8; lda = K;
-    src_scale = sbuf; src_scale_n = dn == 1 ? 1 : M; src_scale_dt = ZMI_DT_F32;
+    src_scale = sbuf; src_scale_n = dn; src_scale_dt = ZMI_DT_F32;
   } else if (a_dt != ZMI_DT_S8 && a_dt != ZMI_DT_U8) {
     return ZMI_UNIMPLEMENTED;
   } else {
     src_scale = (const float *)p->src_scale.buff;
+  }
+
+  /* Per-group source scales ({M,G}, with {G,N} weight scales): per-group branch of
+   * compute_quantized_matmul, operators/matmul/matmul_ref_kernel.cpp:917-1001 --
+   *   sum = 0; for g: grp = float(sum_{k in g} a*w) * ss[m*G+g]; grp *= ws[g*N+n]; sum += grp
+   * then alpha, beta, bias, post-ops (the source / weight scale multiplications of the
+   * plain chain are skipped, :1041-1048).  The validator admits it for symmetric
+   * s8 / bf16 / f32 sources and f32 / bf16 destinations only
+   * (lowoha_operators/matmul/lowoha_matmul_utils.cpp:253-301). */
+  if (src_scale_n > M && src_scale_n % M == 0) {
+    const int64_t G = src_scale_n / M;
+    const int64_t wn = p->wei_scale.buff ? zo_nelems(&p->wei_scale) : 0;
+    if (K % G != 0 || wn != G * N || p->src_zp.buff || a_dt != ZMI_DT_S8 ||
+        !(p->dt_dst == ZMI_DT_F32 || p->dt_dst == ZMI_DT_BF16)) {
+      free(qbuf); free(sbuf);
+      return ZMI_FAILURE;
+    }
+    const int64_t gs = K / G;
+    const int8_t *W = (const int8_t *)c->weight;
+    #pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+      for (int64_t n = 0; n < N; ++n) {
+        float sum = 0.0f;
+        for (int64_t g = 0; g < G; ++g) {
+          int32_t group_sum = 0;
+          for (int64_t k = g * gs; k < (g + 1) * gs; ++k) {
+            int32_t a = ((const int8_t *)A)[transA ? k * lda + m : m * lda + k];
+            group_sum += a * (int32_t)W[c->transB ? n * c->ldb + k : k * c->ldb + n];
+          }
+          float grp = (float)group_sum * zo_read_f32(src_scale, src_scale_dt, m * G + g);
+          grp *= zo_read_f32(p->wei_scale.buff, p->wei_scale.dt, g * N + n);
+          sum += grp;
+        }
+        float y = sum;
+        if (c->alpha != 1.0f) y *= c->alpha;
+        if (c->beta != 0.0f) y += zo_read_f32(c->dst, p->dt_dst, m * (int64_t)c->ldc + n) * c->beta;
+        if (c->bias) y += zo_read_f32(c->bias, p->dt_bias == ZMI_DT_NONE ? ZMI_DT_F32 : p->dt_bias, n);
+        for (int i = 0; i < p->n_postops; ++i) {
+          const zmi_post_op_t *po = &p->postops[i];
+          if (po->po_type == ZMI_PO_BINARY_ADD || po->po_type == ZMI_PO_BINARY_MUL) {
+            int64_t ld = po->leading_dim > 0 ? po->leading_dim : N;
+            int rowb = (po->ndims == 2 && po->dims[0] == 1) || po->ndims == 1;
+            float t = zo_read_f32(po->buff, po->dtype, rowb ? n : m * ld + n);
+            y = po->po_type == ZMI_PO_BINARY_ADD ? y + t : y * t;
+          } else {
+            y = zo_eltwise(po->po_type, y, po->alpha, po->beta);
+          }
+        }
+        zo_store(c->dst, p->dt_dst, m * (int64_t)c->ldc + n, y);
+      }
+    }
+    free(qbuf); free(sbuf);
+    return ZMI_SUCCESS;
   }
 
   int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)M * N);

@@ -1,0 +1,157 @@
+"""GPU parity of matmul_direct with per-group symmetric scales: source scales {M,G}, weight scales {G,N}
+(reference: validation lowoha_operators/matmul/lowoha_matmul_utils.cpp:253-301, arithmetic
+operators/matmul/matmul_ref_kernel.cpp:917-1001).  The kernel adds the group terms in the reference's order
+with one rounding per step, so f32 results without an activation are compared bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from zendnn_amd import capi, lowoha
+from tests import gpu_helpers as H
+from tests.test_gpu_reorder_edges import _run_both
+
+pytestmark = pytest.mark.gpu
+
+
+def _scales(rng, M, N, G):
+    ss = rng.uniform(0.005, 0.03, (M, G)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    return ss, ws
+
+
+# (M, K, N, G): group sizes 64, 128, 256, 32 and 16; one row .. several 64-row blocks; ragged N
+SHAPES = [(1, 128, 32, 2), (5, 256, 33, 4), (16, 4096, 512, 32), (16, 1024, 100, 4), (40, 512, 100, 16),
+          (70, 192, 64, 12), (17, 64, 16, 4), (300, 1024, 260, 8), (130, 2048, 48, 32), (3, 32, 5, 2)]
+
+
+@pytest.mark.parametrize("M,K,N,G", SHAPES)
+def test_static_per_group_f32_bit_exact(zo, M, K, N, G):
+    rng = np.random.default_rng(M * 7 + K + N + G)
+    ss, ws = _scales(rng, M, N, G)
+    bias = rng.standard_normal(N).astype(np.float32)
+    for transA, transB, pad, with_bias in ((False, False, 0, True), (False, True, 3, False), (True, False, 5, True)):
+        a = rng.integers(-128, 128, (K, M + pad) if transA else (M, K + pad), dtype=np.int8)
+        w = rng.integers(-127, 128, (N, K + pad) if transB else (K, N + pad), dtype=np.int8)
+        ss_d, ws_d = H.to_dev(ss), H.to_dev(ws)
+        p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32,
+                                bias=capi.DT_F32 if with_bias else capi.DT_NONE)
+        p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, G))
+        p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (G, N))
+        p.weight_cache_type = 0
+        got, want = _run_both(zo, p, a, w, M, N, K, bias=bias if with_bias else None,
+                              host_bufs={"src_scale": ss, "wei_scale": ws}, lda=a.shape[1], ldb=w.shape[1],
+                              ldc=N + 3, transA=transA, transB=transB)
+        assert lowoha.last_kernel() == "pergroup_mfma16x16x64"
+        assert np.array_equal(got[:, :N], want[:, :N]), (M, K, N, G, transA, transB)
+        assert np.all(got[:, N:] == 0)
+
+
+@pytest.mark.parametrize("M,K,N,G", [(16, 4096, 512, 32), (40, 512, 100, 16), (200, 256, 64, 2)])
+@pytest.mark.parametrize("po", [capi.PO_SWISH, capi.PO_GELU_TANH, capi.PO_RELU])
+def test_static_per_group_bf16_post_ops_prepacked_bf16_scales(zo, M, K, N, G, po):
+    """bf16 destination, one activation, prepacked weights, scales stored as bf16."""
+    rng = np.random.default_rng(po * 100 + M)
+    ss, ws = _scales(rng, M, N, G)
+    ss_b, ws_b = H.bf16_bits(ss), H.bf16_bits(ws)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    a_d, w_d = H.to_dev(a), H.to_dev(w)
+    ss_d, ws_d = H.to_dev(ss_b), H.to_dev(ws_b)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_BF16, (M, G))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_BF16, (G, N))
+    p.postop_ = [lowoha.PostOp(po)]
+    p.mem_format_b = "r"
+    p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, a_d, K, H.prepack(w_d, K, N), N, None, 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    ph = H.host_params(p, src_scale=ss_b, wei_scale=ws_b)
+    ph.mem_format_b = "n"
+    keep = []
+    st, want, _, _ = zo.matmul_int8(a, w, ph.flat(keep), M, N, K)
+    assert st == capi.SUCCESS
+    if po == capi.PO_RELU:
+        assert np.array_equal(H.to_host(dst), want)
+    else:
+        H.check_bf16(H.to_host(dst), want, atol=1e-6 if po == capi.PO_GELU_TANH else 0.0, max_frac=1e-2)
+
+
+def test_static_per_group_alpha_beta(zo):
+    rng = np.random.default_rng(77)
+    M, K, N, G = 20, 256, 40, 4
+    ss, ws = _scales(rng, M, N, G)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    c0 = rng.standard_normal((M, N)).astype(np.float32)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
+    ss_d, ws_d = H.to_dev(ss), H.to_dev(ws)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, G))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (G, N))
+    p.weight_cache_type = 0
+    got, want = _run_both(zo, p, a, w, M, N, K, host_bufs={"src_scale": ss, "wei_scale": ws}, dst_np=c0,
+                          alpha=0.5, beta=1.5)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("M,K,N,G", [(16, 4096, 14336, 32), (4, 4096, 1024, 64), (1, 512, 64, 8), (33, 256, 40, 16),
+                                     (150, 1024, 96, 8)])
+@pytest.mark.parametrize("src_dt", [capi.DT_BF16, capi.DT_F32])
+def test_dynamic_per_group(zo, M, K, N, G, src_dt):
+    """bf16 / f32 rows quantized per (row, group) by the library: the {M,G} scales it writes are bit-exact, and so
+    is the f32 output (exact scales, exact s8 rows, the reference's order of additions).  The first case has
+    the shape of the headline decode configuration."""
+    if src_dt == capi.DT_F32 and N > 2000:
+        pytest.skip("one full-size case is enough")
+    rng = np.random.default_rng(M + K + G)
+    x32 = (rng.standard_normal((M, K)) * rng.uniform(0.2, 3.0, (M, 1))).astype(np.float32)
+    x32[0, 3] = np.nan
+    x = H.bf16_bits(x32) if src_dt == capi.DT_BF16 else x32
+    w = H.gen_weights(rng, K, N)
+    ws = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    x_d, w_d, ws_d = H.to_dev(x), H.to_dev(w), H.to_dev(ws)
+    scales_d = torch.zeros(M * G, dtype=torch.float32, device=H.DEV)
+    p = lowoha.MatmulParams(src=src_dt, wei=capi.DT_S8, dst=capi.DT_F32, compute=capi.DT_S8, bias=capi.DT_F32)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(scales_d, capi.DT_F32, (M, G))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (G, N))
+    p.weight_cache_type = 0
+    dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, w_d, N, H.to_dev(bias), 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert lowoha.last_kernel() == "pergroup_mfma16x16x64"
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    keep = []
+    st, want, _, scales = zo.matmul_int8(x, w, ph.flat(keep), M, N, K, bias=bias, want_scales=True, n_scales=M * G)
+    assert st == capi.SUCCESS
+    assert np.array_equal(H.to_host(scales_d), scales)
+    assert np.array_equal(H.to_host(dst), want)
+
+
+def test_per_group_rejections(zo):
+    M, K, N = 4, 192, 16
+    a_d = H.to_dev(np.ones((M, K), dtype=np.int8))
+    w_d = H.to_dev(np.ones((K, N), dtype=np.int8))
+    dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+
+    def call(G, wei_dims, src=capi.DT_S8, dst_dt=capi.DT_F32, zp=False):
+        ss_d = torch.ones(M * G, dtype=torch.float32, device=H.DEV)
+        ws_d = torch.ones(int(np.prod(wei_dims)), dtype=torch.float32, device=H.DEV)
+        p = lowoha.MatmulParams(src=src, wei=capi.DT_S8, dst=dst_dt)
+        p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, G))
+        p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, wei_dims)
+        if zp:
+            z = np.array([3], dtype=np.int32)
+            p.src_zp = lowoha.QuantParam(z.ctypes.data, capi.DT_S32, (1,))
+        p.weight_cache_type = 0
+        return lowoha.matmul_direct("r", False, False, M, N, K, 1.0, a_d, K, w_d, N, None, 0.0, dst, N, False, p)
+
+    assert call(3, (3, N)) == capi.SUCCESS                       # group size 64
+    assert call(4, (4, N)) == capi.UNIMPLEMENTED                 # group size 48: documented limit of this build
+    assert call(3, (1, N)) == capi.FAILURE                       # per-channel weight scale (reference: failure)
+    assert call(3, (2, N)) == capi.FAILURE                       # group counts differ
+    assert call(5, (5, N)) == capi.FAILURE                       # K % G != 0
+    assert call(3, (3, N), zp=True) == capi.FAILURE              # symmetric only
+    assert call(3, (3, N), src=capi.DT_U8) == capi.FAILURE       # s8 / bf16 / f32 sources only
+    assert call(3, (3, N), dst_dt=capi.DT_S8) == capi.FAILURE    # f32 / bf16 destinations only

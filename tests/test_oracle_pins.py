@@ -262,6 +262,132 @@ def test_chain_dynamic_quant_per_token(zo):
     assert np.abs(dst - full).max() < 0.02 * np.abs(full).max()
 
 
+# ------------------------------------------------------- per-group scales
+def _pg_params(ss, ws, M, N, G, dst=capi.DT_F32, **kw):
+    return _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=dst,
+                   src_scale=capi.quant(ss.ctypes.data, capi.DT_F32, (M, G)),
+                   wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, (G, N)), **kw)
+
+
+def test_per_group_closed_form_with_power_of_two_scales(zo):
+    """All-ones operands: every group sum is K/G; with scales 2^-(..) every product and every partial sum
+    is exact, so the result is the closed form sum_g (K/G) ss[m,g] ws[g,n].  The scale patterns differ
+    along every axis, so a transposed or mis-strided scale index changes the answer."""
+    M, K, N, G = 3, 64, 5, 4
+    A = np.ones((M, K), dtype=np.int8)
+    B = np.ones((K, N), dtype=np.int8)
+    ss = np.array([[2.0 ** -(m + 2 * g) for g in range(G)] for m in range(M)], dtype=np.float32)
+    ws = np.array([[2.0 ** -(3 * g + n) for n in range(N)] for g in range(G)], dtype=np.float32)
+    st, dst, _, _ = zo.matmul_int8(A, B, _pg_params(ss, ws, M, N, G), M, N, K)
+    assert st == capi.SUCCESS
+    want = np.array([[sum((K // G) * float(ss[m, g]) * float(ws[g, n]) for g in range(G)) for n in range(N)]
+                     for m in range(M)])
+    assert np.array_equal(dst[:, :N].astype(np.float64), want)
+
+
+def test_per_group_with_equal_power_of_two_group_scales_is_the_per_token_chain(zo):
+    """ss[m,g] = s_m and ws[g,n] = w_n (powers of two, so nothing rounds): the group terms add up to
+    float(acc) s_m w_n exactly, i.e. the per-token / per-channel result bit for bit."""
+    rng = np.random.default_rng(21)
+    M, K, N, G = 4, 96, 7, 3
+    A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    sm = (2.0 ** -rng.integers(2, 8, M)).astype(np.float32)
+    wn = (2.0 ** -rng.integers(4, 10, N)).astype(np.float32)
+    ss = np.repeat(sm[:, None], G, axis=1).copy()
+    ws = np.repeat(wn[None, :], G, axis=0).copy()
+    bias = rng.standard_normal(N).astype(np.float32)
+    st, got, _, _ = zo.matmul_int8(A, B, _pg_params(ss, ws, M, N, G, dt_bias=capi.DT_F32), M, N, K, bias=bias)
+    assert st == capi.SUCCESS
+    p = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32, dt_bias=capi.DT_F32,
+                src_scale=capi.quant(sm.ctypes.data, capi.DT_F32, (M, 1)),
+                wei_scale=capi.quant(wn.ctypes.data, capi.DT_F32, (1, N)))
+    st, want, _, _ = zo.matmul_int8(A, B, p, M, N, K, bias=bias)
+    assert st == capi.SUCCESS
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("transB", [False, True])
+def test_per_group_numpy_float32_brute_force(zo, transB):
+    """Independent statement on a small random case: integer group sums by numpy, then one float32
+    rounding per step in the reference's order (scale by ss, scale by ws, add in group order, bias)."""
+    rng = np.random.default_rng(22)
+    M, K, N, G = 5, 128, 9, 8
+    A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    ss = rng.uniform(0.005, 0.03, (M, G)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    Bw = np.ascontiguousarray(B.T) if transB else B
+    st, got, _, _ = zo.matmul_int8(A, Bw, _pg_params(ss, ws, M, N, G, dt_bias=capi.DT_F32), M, N, K, bias=bias,
+                                   transB=transB)
+    assert st == capi.SUCCESS
+    gs = K // G
+    gsum = np.einsum("mgk,gkn->mgn", A.reshape(M, G, gs).astype(np.int64), B.reshape(G, gs, N).astype(np.int64))
+    y = np.zeros((M, N), dtype=np.float32)
+    for g in range(G):
+        t = (gsum[:, g, :].astype(np.float32) * ss[:, g][:, None]).astype(np.float32)
+        t = (t * ws[g][None, :]).astype(np.float32)
+        y = (y + t).astype(np.float32)
+    y = (y + bias[None, :]).astype(np.float32)
+    assert np.array_equal(got[:, :N], y)
+    # a wrong group order would still pass the closed forms above; it fails here unless float addition commuted
+    exact = np.einsum("mgn,mg,gn->mn", gsum.astype(np.float64), ss.astype(np.float64), ws.astype(np.float64)) + bias
+    assert np.allclose(got[:, :N], exact, rtol=1e-5, atol=1e-5)
+
+
+def test_per_group_rejects_what_the_reference_validator_rejects(zo):
+    M, K, N, G = 2, 64, 4, 2
+    A = np.ones((M, K), dtype=np.int8)
+    B = np.ones((K, N), dtype=np.int8)
+    ss = np.ones((M, G), dtype=np.float32)
+    ws_bad = np.ones((1, N), dtype=np.float32)           # per-channel weight scale with a per-group source scale
+    p = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32,
+                src_scale=capi.quant(ss.ctypes.data, capi.DT_F32, (M, G)),
+                wei_scale=capi.quant(ws_bad.ctypes.data, capi.DT_F32, (1, N)))
+    st, _, _, _ = zo.matmul_int8(A, B, p, M, N, K)
+    assert st == capi.FAILURE
+
+
+def test_quant_per_group_closed_form_and_per_token_view(zo):
+    """Every group of a row holds its own constant: scale = |c| / 127 and q = +-127 per group; and the whole
+    thing equals the per-token rule on the [M*G, K/G] view of the rows."""
+    M, K, G = 3, 96, 6
+    gs = K // G
+    c = np.array([[(-1.0) ** (m + g) * (0.25 + m + 3 * g) for g in range(G)] for m in range(M)], dtype=np.float32)
+    x = np.repeat(c, gs, axis=1)
+    q, s = zo.quant_per_group(x, capi.DT_F32, G)
+    assert np.array_equal(s, (np.abs(c) / np.float32(127.0)).astype(np.float32))
+    assert np.array_equal(q, np.repeat(np.where(c > 0, 127, -127).astype(np.int8), gs, axis=1))
+    rng = np.random.default_rng(23)
+    x = (rng.standard_normal((M, K)) * rng.uniform(0.1, 5.0, (M, K))).astype(np.float32)
+    x[1, 40] = np.nan
+    x[2, 3] = np.inf
+    q, s = zo.quant_per_group(x, capi.DT_F32, G)
+    qv, sv = zo.quant_per_token(x.reshape(M * G, gs), capi.DT_F32)
+    assert np.array_equal(q.reshape(M * G, gs), qv) and np.array_equal(s.reshape(-1), sv)
+    assert q[1, 40] == 0 and q[2, 3] == 0
+
+
+def test_chain_dynamic_quant_per_group(zo):
+    rng = np.random.default_rng(24)
+    M, K, N, G = 4, 128, 6, 4
+    x = zo.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    p = _params(dt_src=capi.DT_BF16, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32, dt_compute=capi.DT_S8, dynamic_quant=1,
+                src_scale=capi.quant(None, capi.DT_F32, (M, G)),
+                wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, (G, N)))
+    st, dst, _, scales = zo.matmul_int8(x, B, p, M, N, K, want_scales=True, n_scales=M * G)
+    assert st == capi.SUCCESS
+    q, s = zo.quant_per_group(x, capi.DT_BF16, G)
+    assert np.array_equal(s.reshape(-1), scales)
+    st, want, _, _ = zo.matmul_int8(q, B, _pg_params(s, ws, M, N, G), M, N, K)
+    assert np.array_equal(dst, want)
+    full = zo.bf16_to_f32(x).astype(np.float64) @ (B.astype(np.float64) * np.repeat(ws, K // G, axis=0))
+    assert np.abs(dst - full).max() < 0.02 * np.abs(full).max()
+
+
 # ------------------------------------------------------------- post-ops
 def test_eltwise_against_libm_double(zo):
     xs = np.concatenate([np.linspace(-12, 12, 4001), [0.0, -0.0, 1e-6, -1e-6, 30.0, -30.0]]).astype(np.float32)

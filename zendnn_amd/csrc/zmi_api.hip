@@ -130,9 +130,14 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
     } else if (n == M) {
       prob->src_scale_ptr = p.src_scale.buff;
       e.src_scale_mode = ZMI_SS_TOKEN_PTR;
+    } else if (n > M && n % M == 0) {
+      // {M, G}: one scale per row and K group (lowoha_matmul_utils.cpp:262-270)
+      prob->src_scale_ptr = p.src_scale.buff;
+      e.src_scale_mode = ZMI_SS_GROUP_PTR;
+      e.n_groups = (int32_t)(n / M);
     } else {
-      set_error("per-group source scales are not implemented");
-      return ZMI_UNIMPLEMENTED;
+      set_error("source scale must be per-tensor, per-token {M,1} or per-group {M,G}");
+      return ZMI_FAILURE;
     }
   }
   // weight scale
@@ -148,13 +153,24 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
       if (!scalar_param_f32(p.wei_scale.buff, e.wei_scale_dt, &prob->wei_scale_val, &dp)) return ZMI_FAILURE;
       prob->wei_scale_ptr = dp;
       e.wei_scale_mode = 1;
-    } else if (n == N) {
+    } else if (n == N && e.n_groups == 0) {
       prob->wei_scale_ptr = p.wei_scale.buff;
       e.wei_scale_mode = 2;
+    } else if (e.n_groups > 0 && n == (int64_t)e.n_groups * N) {
+      prob->wei_scale_ptr = p.wei_scale.buff;
+      e.wei_scale_mode = 3;
+    } else if (e.n_groups > 0) {
+      // lowoha_matmul_utils.cpp:292-301
+      set_error("per-group source scale requires a per-group weight scale of G * N elements");
+      return ZMI_FAILURE;
     } else {
-      set_error("per-group weight scales are not implemented");
+      set_error("per-group weight scales need a per-group source scale ({M,G} with the same G)");
       return ZMI_UNIMPLEMENTED;
     }
+  }
+  if (e.n_groups > 0 && e.wei_scale_mode != 3) {
+    set_error("per-group source scale requires a per-group weight scale of G * N elements");
+    return ZMI_FAILURE;
   }
   if (p.wei_zp.buff) {
     set_error("weight zero-points are not implemented (symmetric s8 weights only)");
@@ -365,9 +381,34 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (dyn) {
     dyn_scale_n = 1;
     for (int i = 0; i < p.src_scale.ndims; ++i) dyn_scale_n *= p.src_scale.dims[i];
-    if (!(dyn_scale_n == 1 || dyn_scale_n == M)) { set_error("dynamic per-group source scales are not implemented"); return ZMI_UNIMPLEMENTED; }
+    if (!(dyn_scale_n == 1 || dyn_scale_n == M || (dyn_scale_n > M && dyn_scale_n % M == 0 && K % (dyn_scale_n / M) == 0))) {
+      set_error("dynamic source scale dims must be {1}, {M,1} or {M,G} with K divisible by G");
+      return ZMI_FAILURE;
+    }
     if (p.src_zp.buff) { set_error("dynamic quantization is symmetric: no source zero-point"); return ZMI_FAILURE; }
     if (transA) { set_error("dynamic quantization of a transposed source is not implemented"); return ZMI_UNIMPLEMENTED; }
+  }
+  // per-group scales ({M,G} source, {G,N} weights): G slices of K (lowoha_matmul_utils.cpp:262-301)
+  int64_t pg_groups = 0;
+  if (dyn) {
+    if (dyn_scale_n > M) pg_groups = dyn_scale_n / M;
+  } else if (p.src_scale.buff) {
+    const int64_t n = nelems(p.src_scale);
+    if (n > M && n % M == 0) pg_groups = n / M;
+  }
+  if (pg_groups) {
+    if (K % pg_groups != 0) { set_error("per-group source scale: K must be divisible by the number of groups"); return ZMI_FAILURE; }
+    if (p.src_zp.buff) { set_error("per-group source scales are symmetric: no source zero-point"); return ZMI_FAILURE; }
+    if (p.dt_src == ZMI_DT_U8) { set_error("per-group source scales need an s8 / bf16 / f32 source"); return ZMI_FAILURE; }
+    if (p.dt_dst != ZMI_DT_F32 && p.dt_dst != ZMI_DT_BF16) { set_error("per-group source scales need an f32 / bf16 destination"); return ZMI_FAILURE; }
+    if (!p.wei_scale.buff || nelems(p.wei_scale) != pg_groups * N) {
+      set_error("per-group source scale requires a per-group weight scale of G * N elements");
+      return ZMI_FAILURE;
+    }
+    if (!zmi_pergroup_group_size_ok(K / pg_groups)) {
+      set_error("per-group scales: group sizes of 16, 32 or a multiple of 64 are implemented");
+      return ZMI_UNIMPLEMENTED;
+    }
   }
   if (!ensure_device()) return ZMI_FAILURE;
 
@@ -376,13 +417,13 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                          std::min(weight_cache_env(), p.weight_cache_type) > 0;
   const bool pack_in_arena = p.mem_format_b != 'r' && !use_cache;
   const int64_t K16 = zmi_round_up(K, 16);
-  const bool ring = use_ring_kernel(M, N, K);
+  const bool ring = !pg_groups && use_ring_kernel(M, N, K);
   const int64_t frag_kpad = ring ? zmi_blob_kpad(K) : 0;
   const size_t a_bytes = ring ? (size_t)zmi_afrag_bytes(M, K) : (size_t)M * K16;
   const bool repack_a = !dyn && (ring || a_needs_repack(src, lda, K, transA != 0));
   size_t need = 0;
   if (pack_in_arena) need += Arena::padded((size_t)zmi_blob_bytes(K, N));
-  if (dyn) need += Arena::padded(a_bytes) + Arena::padded(sizeof(float) * (size_t)M) + 256;
+  if (dyn) need += Arena::padded(a_bytes) + Arena::padded(sizeof(float) * (size_t)M * (size_t)(pg_groups ? pg_groups : 1)) + 256;
   if (repack_a) need += Arena::padded(a_bytes);
   ZmiRingPlan plan = {};
   if (ring) {
@@ -416,7 +457,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
     int8_t *q = (int8_t *)arena().alloc(a_bytes);
-    float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M);
+    float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M * (size_t)(pg_groups ? pg_groups : 1));
     unsigned int *amax = (unsigned int *)arena().alloc(256);
     // bytes of q between K and K16 stay unwritten: the blob's rows beyond K are zero
     int32_t sdt = p.src_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p.src_scale.dt;
@@ -426,7 +467,16 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
     const bool decode_kernel = decode_kernel_allowed(M, N, K);
     // (the decode kernel's producers are its first workgroups and wait for nothing, so its grid need not be resident)
-    if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
+    if (pg_groups) {
+      // reference: the per-group dynamic reorder in front of the sym-quant GEMM
+      // (matmul/quantization/reorder_quantization.cpp:43-280 with {M,G} scale dims)
+      if (!hip_ok(zmi_launch_quant_groups(src, p.dt_src, M, K, lda, pg_groups, q, K16, sc, (void *)p.src_scale.buff, sdt,
+                                          stream()), "per-group quant launch"))
+        return ZMI_FAILURE;
+      ep.src_scale.buff = sc;
+      ep.src_scale.dt = ZMI_DT_F32;
+      ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
+    } else if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
       if (!ctr) return ZMI_FAILURE;
@@ -477,7 +527,10 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   ZmiEpilogue epi;
   int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
   if (st != ZMI_SUCCESS) return st;
-  if (use_fused) {
+  if (epi.n_groups > 0) {
+    set_kernel_name("pergroup_mfma16x16x64");
+    st = hip_ok(zmi_launch_gemm_pergroup(prob, epi, stream()), "per-group GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+  } else if (use_fused) {
     // a one-row scale in device memory reads like a per-token scale
     if (epi.src_scale_mode == ZMI_SS_TENSOR_PTR) epi.src_scale_mode = ZMI_SS_TOKEN_PTR;
     if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {

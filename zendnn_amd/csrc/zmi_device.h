@@ -91,7 +91,8 @@ struct ZmiPostOp {
   float alpha, beta;   // clip bounds
 };
 
-enum { ZMI_SS_NONE = 0, ZMI_SS_VALUE = 1, ZMI_SS_TENSOR_PTR = 2, ZMI_SS_TOKEN_PTR = 3 };
+// (ZMI_SS_GROUP_PTR: one scale per row and K group, {M, G} row-major; only the per-group kernel reads it)
+enum { ZMI_SS_NONE = 0, ZMI_SS_VALUE = 1, ZMI_SS_TENSOR_PTR = 2, ZMI_SS_TOKEN_PTR = 3, ZMI_SS_GROUP_PTR = 4 };
 
 // Straight-line epilogue variants: alpha == 1, beta == 0, no destination
 // quantization, bf16 or f32 destination, at most one element-wise post-op of
@@ -101,7 +102,7 @@ enum { ZMI_EK_GENERIC = 0, ZMI_EK_NONE = 1, ZMI_EK_SWISH = 2, ZMI_EK_GELU_TANH =
 struct ZmiEpilogue {
   int32_t src_scale_mode;  // ZMI_SS_*
   int32_t src_scale_dt;
-  int32_t wei_scale_mode;  // 0: none; 1: per tensor; 2: per channel (indexed by n)
+  int32_t wei_scale_mode;  // 0: none; 1: per tensor; 2: per channel (indexed by n); 3: per K group and channel, {G, N}
   int32_t wei_scale_dt;
   int32_t has_zp;
   int32_t bias_dt;
@@ -118,6 +119,7 @@ struct ZmiEpilogue {
   int32_t dst_dt;
   int32_t gated_act;      // enum zmi_gated_act; != 0: columns are [gate | up] halves
   int32_t fast_kind;      // ZMI_EK_*: straight-line epilogue variant, 0 = generic interpreter
+  int32_t n_groups;       // > 0: per-group source and weight scales over G = n_groups slices of K
 };
 
 // One GEMM problem: C[M,N] = epilogue(A[M,K] x blob), with the operands the
@@ -371,6 +373,28 @@ __device__ __forceinline__ float zmi_row_scale(const ZmiEpilogue &e, const ZmiPr
   }
 }
 
+// What follows the scaled accumulator: bias, post-ops in order, destination quantization
+// (reference: operators/matmul/matmul_ref_kernel.cpp:1049-1053 and the post-op loop after it).
+// The per-group kernel enters here with its f32 sum of group terms.
+__device__ __forceinline__ float zmi_epilogue_tail(const ZmiEpilogue &e, float y, float bias, int m, int n) {
+  y = __fadd_rn(y, bias);
+  for (int i = 0; i < e.n_po; ++i) {
+    const ZmiPostOp &po = e.po[i];
+    if (po.type == ZMI_PO_BINARY_ADD || po.type == ZMI_PO_BINARY_MUL) {
+      float t = zmi_ld_f32(po.buff, po.dtype, po.rowb ? (int64_t)n : (int64_t)m * po.ld + n);
+      y = po.type == ZMI_PO_BINARY_ADD ? __fadd_rn(y, t) : __fmul_rn(y, t);
+    } else {
+      y = zmi_eltwise(po.type, y, po.alpha, po.beta);
+    }
+  }
+  if (e.has_dst_q) {
+    float ds = e.dst_scale_ptr ? zmi_ld_f32(e.dst_scale_ptr, e.dst_scale_dt, 0) : e.dst_scale_val;
+    float dz = e.dst_zp_ptr ? zmi_ld_f32(e.dst_zp_ptr, e.dst_zp_dt, 0) : e.dst_zp_val;
+    y = __fadd_rn(__fmul_rn(y, ds), dz);
+  }
+  return y;
+}
+
 // acc -> f32 value before the store conversion (all steps separately rounded,
 // in the reference's order).
 __device__ __forceinline__ float zmi_epilogue_value(const ZmiEpilogue &e, int32_t acc, const ZmiColCtx &c,
@@ -388,22 +412,7 @@ __device__ __forceinline__ float zmi_epilogue_value(const ZmiEpilogue &e, int32_
   }
   if (e.src_scale_mode) y = __fmul_rn(y, rscale);
   if (e.wei_scale_mode) y = __fmul_rn(y, c.wscale);
-  y = __fadd_rn(y, c.bias);
-  for (int i = 0; i < e.n_po; ++i) {
-    const ZmiPostOp &po = e.po[i];
-    if (po.type == ZMI_PO_BINARY_ADD || po.type == ZMI_PO_BINARY_MUL) {
-      float t = zmi_ld_f32(po.buff, po.dtype, po.rowb ? (int64_t)n : (int64_t)m * po.ld + n);
-      y = po.type == ZMI_PO_BINARY_ADD ? __fadd_rn(y, t) : __fmul_rn(y, t);
-    } else {
-      y = zmi_eltwise(po.type, y, po.alpha, po.beta);
-    }
-  }
-  if (e.has_dst_q) {
-    float ds = e.dst_scale_ptr ? zmi_ld_f32(e.dst_scale_ptr, e.dst_scale_dt, 0) : e.dst_scale_val;
-    float dz = e.dst_zp_ptr ? zmi_ld_f32(e.dst_zp_ptr, e.dst_zp_dt, 0) : e.dst_zp_val;
-    y = __fadd_rn(__fmul_rn(y, ds), dz);
-  }
-  return y;
+  return zmi_epilogue_tail(e, y, c.bias, m, n);
 }
 
 // Straight-line form of zmi_epilogue_value + zmi_store for the ZMI_EK_* variants:

@@ -86,6 +86,15 @@ hipError_t zmi_launch_gemm_smallm_fused(const ZmiProblem &p, const ZmiEpilogue &
                                         hipStream_t stream);
 hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
 
+// k_pergroup.hip: per-group symmetric scales ({M,G} source, {G,N} weights), any M; s8 rows with a
+// 16-byte aligned leading dimension; group sizes 16, 32 or a multiple of 64
+bool zmi_pergroup_group_size_ok(int64_t gs);
+hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+// per (row, group) dynamic quantization of bf16 / f32 rows: s8 rows (ld ldq), f32 scales {M,G} and an
+// optional copy of the scales in the caller's buffer (f32 or bf16)
+hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
+                                   int64_t ldq, float *scales, void *user_scales, int32_t user_dt, hipStream_t stream);
+
 // k_decode.hip: single problem, M <= 128, K_pad <= 4096
 bool zmi_decode_kernel_fits(const ZmiProblem &p);
 // fq != null: the launch also quantizes the M source rows (its grid must be resident at once)
