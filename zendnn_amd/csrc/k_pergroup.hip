@@ -12,15 +12,18 @@
 // v_mfma_i32_16x16x64_i8, folding the integer accumulator into the f32 sum at every group
 // boundary.  Weights are read once per row block straight from the prepacked blob (a
 // 16-column half of a 1 KiB fragment is 256 contiguous bytes per 16 k), D chunks of 64 k
-// ahead; the scales of the next group are requested one group ahead.  Groups of 16 or 32 k
-// share a 64-k chunk: the chunk is multiplied once per group with the other groups' lanes
-// of the row operand zeroed.
+// ahead; the scales of the wavefront's rows and columns are staged in LDS up to 128 groups
+// at a time.  Groups of 16 or 32 k share a 64-k chunk: the chunk is multiplied once per group
+// with the other groups' lanes of the row operand zeroed.
 #include "zmi_device.h"
 #include "zmi_launch.h"
 
 #define PG_WAVES 4
 
-template <int RB, int D>
+// RB: 16-row blocks per wavefront; D: chunks per operand set; SUB: groups per 64-k chunk (1: groups of whole
+// chunks); CPG: chunks per group when that is 1 or 2 (groups of 64 / 128), 0: any other multiple of 64,
+// taken from gs at run time
+template <int RB, int D, int SUB, int CPG>
 __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiProblem p, ZmiEpilogue epi, int n_cb,
                                                                           int n_items, int gs) {
   const int lane = threadIdx.x % 64;
@@ -35,36 +38,66 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
   const int row0 = rbk * 16 * RB;
   const uint8_t *bsrc = p.blob + zmi_blob_tiles_off(N) + (int64_t)(cb / 2) * zmi_blob_nb_stride(K) + (g4 / 2) * 1024 +
                         ((g4 % 2) * 32 + (cb % 2) * 16 + c16) * 16;
-  const int8_t *A = (const int8_t *)p.A;
-
-  // ---- operand ring: D chunks of 64 k in flight ----
-  v4i b[D], a[D][RB];
-  auto request = [&](int slot, int c) {
-    const bool in = c < nch;                       // (uniform) past the end: nothing is read
-    b[slot] = in ? *(const v4i *)(bsrc + (int64_t)c * 2048) : (v4i){0, 0, 0, 0};
+  // rows past M repeat row M - 1 (their results are never stored); k past K reads k = 0 (the blob's
+  // rows past K are zero): every request is unconditional and the loop has no divergent branch
+  const int8_t *arow[RB];
 #pragma unroll
-    for (int j = 0; j < RB; ++j) {
-      const int row = row0 + j * 16 + c16;
-      const int k = c * 64 + g4 * 16;
-      a[slot][j] = (in && row < M && k < K) ? *(const v4i *)(A + (int64_t)row * p.lda + k) : (v4i){0, 0, 0, 0};
+  for (int j = 0; j < RB; ++j) {
+    const int row = row0 + j * 16 + c16;
+    arow[j] = (const int8_t *)p.A + (int64_t)(row < M ? row : M - 1) * p.lda;
+  }
+
+  // ---- operands: two sets of D chunks of 64 k; one set is multiplied while the other set's requests
+  // (issued before it) are in flight.  (A ring refilled chunk by chunk ends up with all its requests
+  // at the end of the loop body and a wait for all of them at the top: one memory latency per D chunks.) ----
+  v4i b[2][D], a[2][D][RB];
+  auto request_set = [&](int set, int c_first) {
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+      const int c = c_first + s;
+      const int cc = c < nch ? c : nch - 1;          // (uniform) past the end: a valid chunk, never used
+      b[set][s] = *(const v4i *)(bsrc + (int64_t)cc * 2048);
+      const int k = cc * 64 + g4 * 16;
+      const int ka = k < K ? k : 0;
+#pragma unroll
+      for (int j = 0; j < RB; ++j) a[set][s][j] = *(const v4i *)(arow[j] + ka);
     }
   };
-#pragma unroll
-  for (int s = 0; s < D; ++s) request(s, s);
+  request_set(0, 0);
+  request_set(1, D);
 
-  // ---- scales of the next group to be folded ----
-  float wsn, ssn[RB][4];
-  auto request_scales = [&](int gi) {
-    wsn = col < N ? zmi_ld_f32(p.wei_scale_ptr, epi.wei_scale_dt, (int64_t)gi * N + col) : 0.0f;
-#pragma unroll
-    for (int j = 0; j < RB; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int row = row0 + j * 16 + g4 * 4 + q;   // accumulator element q of this lane
-        ssn[j][q] = row < M ? zmi_ld_f32(p.src_scale_ptr, epi.src_scale_dt, (int64_t)row * G + gi) : 0.0f;
+  // ---- scales: this wavefront's slices ({G,16} weight scales, {16 RB, G} source scales) are staged in its own
+  // LDS area GB groups at a time, all requests in flight at once; a fold then needs no global load.  (Fetching
+  // them one group ahead from global memory made every fold wait for a full memory latency.) ----
+  constexpr int GB = RB == 1 ? 128 : 32;           // groups per staged block: 16 KiB / 10 KiB per wavefront
+  __shared__ float scale_lds[PG_WAVES][(16 + 16 * RB) * GB];
+  float *ws_l = scale_lds[wave], *ss_l = scale_lds[wave] + 16 * GB;
+  auto stage_scales = [&](int gb0) {
+    const int ng = G - gb0 < GB ? G - gb0 : GB;
+    // (other lanes of this wavefront may still read the previous block; its LDS accesses are served in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // (no divergent branch and no type switch inside the loops, so that eight requests go out per wait;
+    // columns past N and rows past M read the last valid one, their results are never stored)
+    auto fill = [&](float *dst_l, const void *src, bool bf16, int count, auto index, auto slot) {
+      if (bf16) {
+#pragma unroll 8
+        for (int i = lane; i < count; i += 64) dst_l[slot(i)] = zmi_bf16_to_f32(((const uint16_t *)src)[index(i)]);
+      } else {
+#pragma unroll 8
+        for (int i = lane; i < count; i += 64) dst_l[slot(i)] = ((const float *)src)[index(i)];
       }
+    };
+    fill(ws_l, p.wei_scale_ptr, epi.wei_scale_dt == ZMI_DT_BF16, ng * 16,
+         [&](int i) { const int n = cb * 16 + i % 16; return (int64_t)(gb0 + i / 16) * N + (n < N ? n : N - 1); },
+         [&](int i) { return i; });
+    fill(ss_l, p.src_scale_ptr, epi.src_scale_dt == ZMI_DT_BF16, ng * 16 * RB,
+         [&](int i) { const int r = row0 + i / ng; return (int64_t)(r < M ? r : M - 1) * G + gb0 + i % ng; },
+         [&](int i) { return (i / ng) * GB + i % ng; });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
-  request_scales(0);
 
   v4i acc[RB];
   float sum[RB][4];
@@ -74,20 +107,15 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
 #pragma unroll
     for (int q = 0; q < 4; ++q) sum[j][q] = 0.0f;
   }
-  // group gi is complete in acc: sum += (float(acc) * ss[m, gi]) * ws[gi, n], each step rounded
-  auto fold = [&](int gi) {
-    const float wsv = wsn;
-    float ssv[RB][4];
-#pragma unroll
-    for (int j = 0; j < RB; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) ssv[j][q] = ssn[j][q];
-    if (gi + 1 < G) request_scales(gi + 1);
+  // group gi (gl within the staged block) is complete in acc:
+  // sum += (float(acc) * ss[m, gi]) * ws[gi, n], each step rounded
+  auto fold = [&](int gl) {
+    const float wsv = ws_l[gl * 16 + c16];
 #pragma unroll
     for (int j = 0; j < RB; ++j) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        float t = __fmul_rn((float)acc[j][q], ssv[j][q]);
+        float t = __fmul_rn((float)acc[j][q], ss_l[(j * 16 + g4 * 4 + q) * GB + gl]);
         t = __fmul_rn(t, wsv);
         sum[j][q] = __fadd_rn(sum[j][q], t);
       }
@@ -95,33 +123,54 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
     }
   };
 
-  const int cpg = gs >= 64 ? gs / 64 : 1;   // chunks per group
-  const int sub = gs >= 64 ? 1 : 64 / gs;   // groups per chunk
-  for (int c0 = 0; c0 < nch; c0 += D) {
+  const int cpg = SUB != 1 ? 1 : CPG ? CPG : gs / 64;             // chunks per group
+  const int blk_chunks = SUB == 1 ? GB * cpg : GB / SUB;        // chunks per staged block (a multiple of 2 D)
+  // one chunk: multiply, fold where a group ends.  s is the chunk's position in its block of D (c % D):
+  // with CPG known the fold positions are fixed at compile time and a block of D chunks is straight-line
+  // code
+  auto step = [&](int c, int set, int s, int gb0) {
+    if (SUB == 1) {
 #pragma unroll
-    for (int s = 0; s < D; ++s) {
-      const int c = c0 + s;
-      if (c < nch) {
-        if (sub == 1) {
+      for (int j = 0; j < RB; ++j)
+        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[set][s][j], b[set][s], acc[j], 0, 0, 0);
+      if (CPG ? (s + 1) % (CPG ? CPG : 1) == 0 : (c + 1) % cpg == 0) fold(c / cpg - gb0);
+    } else {
 #pragma unroll
-          for (int j = 0; j < RB; ++j) acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[s][j], b[s], acc[j], 0, 0, 0);
-          if ((c + 1) % cpg == 0) fold(c / cpg);
-        } else {
-          for (int t = 0; t < sub; ++t) {
-            const int gi = c * sub + t;
-            if (gi >= G) break;   // (K_pad beyond K)
-            const bool mine = (g4 * 16) / gs == t;   // this lane's 16 k belong to group t of the chunk
+      for (int t = 0; t < SUB; ++t) {
+        const int gi = c * SUB + t;
+        if (gi < G) {   // (uniform; K_pad may reach past K)
+          const bool mine = g4 / (4 / SUB) == t;   // this lane's 16 k belong to group t of the chunk
 #pragma unroll
-            for (int j = 0; j < RB; ++j) {
-              const v4i am = mine ? a[s][j] : (v4i){0, 0, 0, 0};
-              acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(am, b[s], acc[j], 0, 0, 0);
-            }
-            fold(gi);
+          for (int j = 0; j < RB; ++j) {
+            const v4i am = mine ? a[set][s][j] : (v4i){0, 0, 0, 0};
+            acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(am, b[set][s], acc[j], 0, 0, 0);
           }
+          fold(gi - gb0);
         }
       }
-      request(s, c + D);
     }
+  };
+  for (int cb0 = 0; cb0 < nch; cb0 += blk_chunks) {
+    const int gb0 = SUB == 1 ? cb0 / cpg : cb0 * SUB;           // first group of the block
+    stage_scales(gb0);
+    const int cend = cb0 + blk_chunks < nch ? cb0 + blk_chunks : nch;
+    int c0 = cb0;
+    for (; c0 + 2 * D <= cend; c0 += 2 * D) {
+#pragma unroll
+      for (int set = 0; set < 2; ++set) {
+#pragma unroll
+        for (int s = 0; s < D; ++s) step(c0 + set * D + s, set, s, gb0);
+        __builtin_amdgcn_sched_barrier(0);   // the set's next requests stay between its use and the other set's
+        request_set(set, c0 + set * D + 2 * D);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // (only the last block can end with fewer than 2 D chunks; nothing is requested after them)
+#pragma unroll
+    for (int set = 0; set < 2; ++set)
+#pragma unroll
+      for (int s = 0; s < D; ++s)
+        if (c0 + set * D + s < cend) step(c0 + set * D + s, set, s, gb0);
   }
 
   // ---- alpha / beta, then the common tail; acc element q of lane l is row (l / 16) * 4 + q, column l % 16 ----
@@ -157,8 +206,18 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
   const int n_rb = (p.M + 16 * rb - 1) / (16 * rb);
   const int n_items = n_cb * n_rb;
   const dim3 grid((n_items + PG_WAVES - 1) / PG_WAVES), block(PG_WAVES * 64);
-  if (rb == 1) hipLaunchKernelGGL((zmi_gemm_pergroup_kernel<1, 8>), grid, block, 0, stream, p, epi, n_cb, n_items, gs);
-  else hipLaunchKernelGGL((zmi_gemm_pergroup_kernel<4, 4>), grid, block, 0, stream, p, epi, n_cb, n_items, gs);
+  const int sub = gs >= 64 ? 1 : 64 / gs;
+#define PG_LAUNCH(RB_, D_, SUB_, CPG_) \
+  hipLaunchKernelGGL((zmi_gemm_pergroup_kernel<RB_, D_, SUB_, CPG_>), grid, block, 0, stream, p, epi, n_cb, n_items, gs)
+  const int cpg = sub == 1 ? (gs == 64 ? 1 : gs == 128 ? 2 : 0) : 1;
+  if (rb == 1) {
+    if (sub == 2) PG_LAUNCH(1, 8, 2, 1); else if (sub == 4) PG_LAUNCH(1, 8, 4, 1);
+    else if (cpg == 1) PG_LAUNCH(1, 8, 1, 1); else if (cpg == 2) PG_LAUNCH(1, 8, 1, 2); else PG_LAUNCH(1, 8, 1, 0);
+  } else {
+    if (sub == 2) PG_LAUNCH(4, 2, 2, 1); else if (sub == 4) PG_LAUNCH(4, 2, 4, 1);
+    else if (cpg == 1) PG_LAUNCH(4, 2, 1, 1); else if (cpg == 2) PG_LAUNCH(4, 2, 1, 2); else PG_LAUNCH(4, 2, 1, 0);
+  }
+#undef PG_LAUNCH
   return hipGetLastError();
 }
 
@@ -168,48 +227,64 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
 // per_group_avx512_f32_fma_kernel.cpp:78-86 scale, :276-292 quantization): per (row, group)
 // absmax over finite values, scale = max(absmax, 1e-10) / 127 clamped to >= 1e-10,
 // q = (int8) nearbyint(v / scale) with the true division, non-finite -> 0; i.e. the per-token
-// rule applied to every group of a row.  One workgroup per row, one wavefront per group in turn.
+// rule applied to every group of a row.  One wavefront per (row, group).
 template <bool BF16>
-__global__ __launch_bounds__(256) void zmi_quant_groups_kernel(const void *x, int64_t ldx, int K, int G, int8_t *q,
+__global__ __launch_bounds__(256) void zmi_quant_groups_kernel(const void *x, int64_t ldx, int M, int K, int G, int8_t *q,
                                                                int64_t ldq, float *scales, void *user_scales,
                                                                int32_t user_dt) {
-  const int m = blockIdx.x, lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int lane = threadIdx.x % 64;
+  const int64_t item = (int64_t)blockIdx.x * 4 + threadIdx.x / 64;   // one wavefront per (row, group)
+  if (item >= (int64_t)M * G) return;
+  const int m = (int)(item / G), g = (int)(item % G);
   const int gs = K / G;
-  for (int g = wave; g < G; g += 4) {
-    const int64_t base = (int64_t)m * ldx + (int64_t)g * gs;
-    auto ld = [&](int k) { return BF16 ? zmi_bf16_to_f32(((const uint16_t *)x)[base + k]) : ((const float *)x)[base + k]; };
-    float amax = 0.0f;
-    for (int k = lane; k < gs; k += 64) {
-      const float a = fabsf(ld(k));
-      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
-    }
+  const int64_t base = (int64_t)m * ldx + (int64_t)g * gs;
+  auto ld = [&](int k) { return BF16 ? zmi_bf16_to_f32(((const uint16_t *)x)[base + k]) : ((const float *)x)[base + k]; };
+  // (groups of up to 256 elements stay in registers between the two passes)
+  float keep[4];
+  float amax = 0.0f;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    if (amax < 1e-10f) amax = 1e-10f;
-    float s = __fdiv_rn(amax, 127.0f);
-    if (s < 1e-10f) s = 1e-10f;
-    const float inv = __fdiv_rn(1.0f, s);
-    if (lane == 0) {
-      scales[(int64_t)m * G + g] = s;
-      if (user_scales) {
-        if (user_dt == ZMI_DT_BF16) ((uint16_t *)user_scales)[(int64_t)m * G + g] = zmi_f32_to_bf16_rne(s);
-        else ((float *)user_scales)[(int64_t)m * G + g] = s;
-      }
-    }
-    int8_t *dst = q + (int64_t)m * ldq + (int64_t)g * gs;
-    for (int k = lane; k < gs; k += 64) dst[k] = zmi_quant_elem(ld(k), s, inv);
+  for (int i = 0; i < 4; ++i) {
+    const int k = lane + 64 * i;
+    keep[i] = k < gs ? ld(k) : 0.0f;
+    const float a = fabsf(keep[i]);
+    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
   }
+  for (int k = lane + 256; k < gs; k += 64) {
+    const float a = fabsf(ld(k));
+    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
+  if (lane == 0) {
+    scales[item] = s;
+    if (user_scales) {
+      if (user_dt == ZMI_DT_BF16) ((uint16_t *)user_scales)[item] = zmi_f32_to_bf16_rne(s);
+      else ((float *)user_scales)[item] = s;
+    }
+  }
+  int8_t *dst = q + (int64_t)m * ldq + (int64_t)g * gs;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = lane + 64 * i;
+    if (k < gs) dst[k] = zmi_quant_elem(keep[i], s, inv);
+  }
+  for (int k = lane + 256; k < gs; k += 64) dst[k] = zmi_quant_elem(ld(k), s, inv);
 }
 
 hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
                                    int64_t ldq, float *scales, void *user_scales, int32_t user_dt, hipStream_t stream) {
   if (M <= 0) return hipSuccess;
   if (G <= 0 || K % G != 0 || (x_dt != ZMI_DT_BF16 && x_dt != ZMI_DT_F32)) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((M * G + 3) / 4));
   if (x_dt == ZMI_DT_BF16)
-    hipLaunchKernelGGL(zmi_quant_groups_kernel<true>, dim3((unsigned)M), dim3(256), 0, stream, x, ldx, (int)K, (int)G, q,
+    hipLaunchKernelGGL(zmi_quant_groups_kernel<true>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q,
                        ldq, scales, user_scales, user_dt);
   else
-    hipLaunchKernelGGL(zmi_quant_groups_kernel<false>, dim3((unsigned)M), dim3(256), 0, stream, x, ldx, (int)K, (int)G, q,
+    hipLaunchKernelGGL(zmi_quant_groups_kernel<false>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q,
                        ldq, scales, user_scales, user_dt);
   return hipGetLastError();
 }
