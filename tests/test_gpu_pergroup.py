@@ -155,3 +155,99 @@ def test_per_group_rejections(zo):
     assert call(3, (3, N), zp=True) == capi.FAILURE              # symmetric only
     assert call(3, (3, N), src=capi.DT_U8) == capi.FAILURE       # s8 / bf16 / f32 sources only
     assert call(3, (3, N), dst_dt=capi.DT_S8) == capi.FAILURE    # f32 / bf16 destinations only
+
+
+# ---------------------------------------------------------------- the quantization entry points
+@pytest.mark.parametrize("M,K,G", [(1, 64, 2), (7, 512, 16), (33, 4096, 32), (5, 20000, 4), (300, 1408, 11)])
+@pytest.mark.parametrize("src_dt", [capi.DT_BF16, capi.DT_F32])
+def test_reorder_direct_dynamic_per_group_bit_exact(zo, M, K, G, src_dt):
+    """reorder_direct with {M,G} scale dims (lowoha_reorder.cpp:167-171): s8 rows and scales equal the oracle's,
+    with zero groups, NaN and infinities; scales as f32 and as bf16; scales only (dst == nullptr)."""
+    rng = np.random.default_rng(M * 131 + K + G)
+    xf = (rng.standard_normal((M, K)) * rng.uniform(0.01, 30, (M, 1))).astype(np.float32)
+    gs = K // G
+    xf[0, :gs] = 0.0                        # a zero group: scale clamps to 1e-10
+    xf[M - 1, K - 1] = np.inf
+    xf[M // 2, 1] = np.nan
+    x = H.bf16_bits(xf) if src_dt == capi.DT_BF16 else xf
+    x_d = H.to_dev(x)
+    q, s = zo.quant_per_group(x, src_dt, G)
+
+    def params(scale_buf, scale_dt):
+        rp = lowoha.ReorderParams()
+        rp.src_dtype, rp.dst_dtype = src_dt, capi.DT_S8
+        rp.dynamic_quant = True
+        rp.algo = 1
+        rp.src_shape = rp.dst_shape = (M, K)
+        rp.scale = lowoha.QuantParam(scale_buf, scale_dt, (M, G))
+        return rp
+
+    q_d = torch.zeros((M, K), dtype=torch.int8, device=H.DEV)
+    s_d = torch.zeros(M * G, dtype=torch.float32, device=H.DEV)
+    st = lowoha.reorder_direct(x_d, q_d, params(s_d, capi.DT_F32))
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert lowoha.last_kernel() == "quant_groups"
+    assert np.array_equal(H.to_host(s_d).reshape(M, G), s)
+    assert np.array_equal(H.to_host(q_d), q)
+    # bf16 scales: the f32 scale rounded to nearest even; the rows are quantized with the f32 scale
+    sb_d = torch.zeros(M * G, dtype=torch.bfloat16, device=H.DEV)
+    q2_d = torch.zeros((M, K), dtype=torch.int8, device=H.DEV)
+    st = lowoha.reorder_direct(x_d, q2_d, params(sb_d, capi.DT_BF16))
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert np.array_equal(H.to_host(sb_d).reshape(M, G), H.bf16_bits(s))
+    assert torch.equal(q2_d, q_d)
+    # scales only
+    s2 = torch.zeros(M * G, dtype=torch.float32, device=H.DEV)
+    st = lowoha.reorder_direct(x_d, None, params(s2, capi.DT_F32))
+    assert st == capi.SUCCESS and torch.equal(s2, s_d)
+
+
+def test_reorder_direct_per_group_needs_divisible_k(zo):
+    M, K = 4, 100
+    x_d = torch.zeros((M, K), dtype=torch.float32, device=H.DEV)
+    q_d = torch.zeros((M, K), dtype=torch.int8, device=H.DEV)
+    s_d = torch.zeros(M * 3, dtype=torch.float32, device=H.DEV)
+    rp = lowoha.ReorderParams()
+    rp.src_dtype, rp.dst_dtype = capi.DT_F32, capi.DT_S8
+    rp.dynamic_quant = True
+    rp.algo = 1
+    rp.src_shape = rp.dst_shape = (M, K)
+    rp.scale = lowoha.QuantParam(s_d, capi.DT_F32, (M, 3))
+    assert lowoha.reorder_direct(x_d, q_d, rp) == capi.FAILURE
+
+
+@pytest.mark.parametrize("G", [1, 8])
+def test_group_dynamic_quant_per_token_and_per_group(zo, G):
+    """group_dynamic_quant (lowoha_reorder.cpp:279-404) through the C ABI: several matrices, one with no rows, padded
+    row strides; num_groups <= 1 is per token, > 1 per group."""
+    import ctypes as C
+    rng = np.random.default_rng(40 + G)
+    shapes = [(5, 64), (0, 128), (33, 512), (2, 1024)]
+    lib = capi.load()
+    n = len(shapes)
+    keep, want = [], []
+    srcs, dsts, scales = (C.c_void_p * n)(), (C.c_void_p * n)(), (C.c_void_p * n)()
+    Ms, Ks = (C.c_int32 * n)(), (C.c_int32 * n)()
+    lds, ldd = (C.c_int64 * n)(), (C.c_int64 * n)()
+    for i, (M, K) in enumerate(shapes):
+        pad = 8 * (i % 2)
+        xf = (rng.standard_normal((max(M, 1), K + pad)) * 3).astype(np.float32)
+        x = H.bf16_bits(xf)
+        x_d = H.to_dev(x)
+        q_d = torch.zeros((max(M, 1), K + pad), dtype=torch.int8, device=H.DEV)
+        s_d = torch.zeros(max(M, 1) * G, dtype=torch.float32, device=H.DEV)
+        keep += [x_d, q_d, s_d]
+        srcs[i], dsts[i], scales[i] = x_d.data_ptr(), q_d.data_ptr(), s_d.data_ptr()
+        Ms[i], Ks[i], lds[i], ldd[i] = M, K, K + pad, K + pad
+        xs = np.ascontiguousarray(x[:, :K])
+        want.append(zo.quant_per_group(xs, capi.DT_BF16, G) if G > 1 else zo.quant_per_token(xs, capi.DT_BF16))
+    gp = capi.GroupDqParamsT(capi.DT_BF16, capi.DT_S8, capi.DT_F32, 0, G)
+    st = lib.zmi_group_dynamic_quant(n, srcs, Ms, Ks, lds, dsts, ldd, scales, C.byref(gp))
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for i, (M, K) in enumerate(shapes):
+        if M == 0:
+            continue
+        q, s = want[i]
+        assert np.array_equal(H.to_host(keep[3 * i + 1])[:M, :K], q[:M])
+        assert np.array_equal(H.to_host(keep[3 * i + 2])[:M * G], np.asarray(s).reshape(-1)[:M * G])
+        assert np.all(H.to_host(keep[3 * i + 1])[:, K:] == 0)          # padding bytes of dst are left alone

@@ -266,6 +266,7 @@ __global__ __launch_bounds__(256) void zmi_quant_groups_kernel(const void *x, in
       else ((float *)user_scales)[item] = s;
     }
   }
+  if (!q) return;   // scales only
   int8_t *dst = q + (int64_t)m * ldq + (int64_t)g * gs;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {

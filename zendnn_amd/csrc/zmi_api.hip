@@ -617,7 +617,25 @@ static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t 
     set_kernel_name("quant_tensor");
     return ZMI_SUCCESS;
   }
-  set_error("dynamic quantization: only per-token {M,1} and per-tensor scales are implemented");
+  // per-group along K: scale dims {M, G}, 1 < G < K, K % G == 0 (reference: is_per_group_col_dims and the
+  // fused per-group dispatch, reorder/lowoha_reorder.cpp:167-171; dims rule lowoha_reorder_utils.cpp:180-211)
+  if (rp.scale.ndims == 2 && rp.scale.dims[0] == M && rp.scale.dims[1] > 1 && rp.scale.dims[1] != K) {
+    const int64_t G = rp.scale.dims[1];
+    if (K % G != 0) { set_error("dynamic quantization: per-group scale needs K divisible by the number of groups"); return ZMI_FAILURE; }
+    float *sc = (float *)rp.scale.buff;
+    void *user = nullptr;
+    if (sdt != ZMI_DT_F32) {
+      if (!arena().begin(Arena::padded(sizeof(float) * (size_t)(M * G)))) return ZMI_FAILURE;
+      sc = (float *)arena().alloc(sizeof(float) * (size_t)(M * G));
+      user = (void *)rp.scale.buff;
+    }
+    if (!hip_ok(zmi_launch_quant_groups(src, rp.src_dtype, M, K, ld, G, (int8_t *)dst, K, sc, user, sdt, stream()),
+                "per-group quant launch"))
+      return ZMI_FAILURE;
+    set_kernel_name("quant_groups");
+    return ZMI_SUCCESS;
+  }
+  set_error("dynamic quantization: scale dims must be {1}, {M,1} or {M,G}");
   return ZMI_UNIMPLEMENTED;
 }
 
@@ -652,9 +670,36 @@ int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src, const int32_t
     set_error("group_dynamic_quant: only bf16/f32 -> s8");
     return ZMI_FAILURE;
   }
-  if (params->num_groups > 1) { set_error("group_dynamic_quant: per-group scales are not implemented"); return ZMI_UNIMPLEMENTED; }
   const int32_t sdt = params->scale_dtype == ZMI_DT_NONE ? ZMI_DT_F32 : params->scale_dtype;
   if (sdt != ZMI_DT_F32 && sdt != ZMI_DT_BF16) { set_error("group_dynamic_quant: scale must be f32 or bf16"); return ZMI_FAILURE; }
+  if (params->num_groups > 1) {
+    // per-group: every matrix gets {M[i], num_groups} scales (lowoha_reorder.cpp:318-393); one launch per matrix
+    const int64_t G = params->num_groups;
+    size_t need = 0;
+    for (int i = 0; i < n; ++i) {
+      if (M[i] < 0 || K[i] <= 0) { set_error("group_dynamic_quant: bad shape"); return ZMI_FAILURE; }
+      if (M[i] == 0) continue;
+      if (K[i] % G != 0) { set_error("group_dynamic_quant: per-group requires K % num_groups == 0"); return ZMI_FAILURE; }
+      if (!src[i] || !dst[i] || !scale[i]) { set_error("group_dynamic_quant: null buffer for an active matrix"); return ZMI_FAILURE; }
+      if (sdt != ZMI_DT_F32) need += Arena::padded(sizeof(float) * (size_t)(M[i] * G));
+    }
+    if (!ensure_device()) return ZMI_FAILURE;
+    if (!arena().begin(need)) return ZMI_FAILURE;
+    for (int i = 0; i < n; ++i) {
+      if (M[i] == 0) continue;
+      const int64_t lds_ = src_row_stride && src_row_stride[i] ? src_row_stride[i] : K[i];
+      const int64_t ldd = dst_row_stride && dst_row_stride[i] ? dst_row_stride[i] : K[i];
+      if (lds_ < K[i] || ldd < K[i]) { set_error("group_dynamic_quant: row stride smaller than K"); return ZMI_FAILURE; }
+      float *sc = (float *)scale[i];
+      void *user = nullptr;
+      if (sdt != ZMI_DT_F32) { sc = (float *)arena().alloc(sizeof(float) * (size_t)(M[i] * G)); user = scale[i]; }
+      if (!hip_ok(zmi_launch_quant_groups(src[i], params->src_dtype, M[i], K[i], lds_, G, (int8_t *)dst[i], ldd, sc, user, sdt,
+                                          stream()), "per-group quant launch"))
+        return ZMI_FAILURE;
+    }
+    set_kernel_name("quant_groups");
+    return ZMI_SUCCESS;
+  }
   std::vector<ZmiQuantMat> mats;
   int64_t rows = 0;
   for (int i = 0; i < n; ++i) {
