@@ -21,7 +21,11 @@ def _scales(rng, M, N, G):
 
 # (M, K, N, G): group sizes 64, 128, 256, 32 and 16; one row .. several 64-row blocks; ragged N
 SHAPES = [(1, 128, 32, 2), (5, 256, 33, 4), (16, 4096, 512, 32), (16, 1024, 100, 4), (40, 512, 100, 16),
-          (70, 192, 64, 12), (17, 64, 16, 4), (300, 1024, 260, 8), (130, 2048, 48, 32), (3, 32, 5, 2)]
+          (70, 192, 64, 12), (17, 64, 16, 4), (300, 1024, 260, 8), (130, 2048, 48, 32), (3, 32, 5, 2),
+          # up to 16 rows with K = 512 .. 4096 and whole groups per eighth of K: the decode-shaped kernel, every
+          # (chunks, groups) per wavefront pair it is built for
+          (16, 4096, 40, 64), (9, 4096, 33, 16), (2, 4096, 64, 8), (16, 2048, 96, 32), (5, 2048, 32, 16),
+          (1, 2048, 70, 8), (16, 1024, 64, 16), (3, 1024, 31, 8), (12, 512, 50, 8)]
 
 
 @pytest.mark.parametrize("M,K,N,G", SHAPES)
@@ -41,7 +45,7 @@ def test_static_per_group_f32_bit_exact(zo, M, K, N, G):
         got, want = _run_both(zo, p, a, w, M, N, K, bias=bias if with_bias else None,
                               host_bufs={"src_scale": ss, "wei_scale": ws}, lda=a.shape[1], ldb=w.shape[1],
                               ldc=N + 3, transA=transA, transB=transB)
-        assert lowoha.last_kernel() == "pergroup_mfma16x16x64"
+        assert lowoha.last_kernel().startswith("pergroup_")
         assert np.array_equal(got[:, :N], want[:, :N]), (M, K, N, G, transA, transB)
         assert np.all(got[:, N:] == 0)
 
@@ -75,6 +79,24 @@ def test_static_per_group_bf16_post_ops_prepacked_bf16_scales(zo, M, K, N, G, po
         assert np.array_equal(H.to_host(dst), want)
     else:
         H.check_bf16(H.to_host(dst), want, atol=1e-6 if po == capi.PO_GELU_TANH else 0.0, max_frac=1e-2)
+
+
+def test_generic_kernel_on_a_decode_shaped_problem(zo, monkeypatch):
+    """The one-wavefront-per-column-block kernel on a shape the decode-shaped kernel would take (env switch)."""
+    monkeypatch.setenv("ZMI_PERGROUP_GENERIC", "1")
+    rng = np.random.default_rng(5)
+    M, K, N, G = 16, 2048, 96, 16
+    ss, ws = _scales(rng, M, N, G)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
+    ss_d, ws_d = H.to_dev(ss), H.to_dev(ws)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, G))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (G, N))
+    p.weight_cache_type = 0
+    got, want = _run_both(zo, p, a, w, M, N, K, host_bufs={"src_scale": ss, "wei_scale": ws})
+    assert lowoha.last_kernel() == "pergroup_mfma16x16x64"
+    assert np.array_equal(got, want)
 
 
 def test_static_per_group_alpha_beta(zo):
@@ -120,7 +142,7 @@ def test_dynamic_per_group(zo, M, K, N, G, src_dt):
     dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
     st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, w_d, N, H.to_dev(bias), 0.0, dst, N, True, p)
     assert st == capi.SUCCESS, lowoha.last_error()
-    assert lowoha.last_kernel() == "pergroup_mfma16x16x64"
+    assert lowoha.last_kernel().startswith("pergroup_")
     ph = H.host_params(p, src_scale=None, wei_scale=ws)
     keep = []
     st, want, _, scales = zo.matmul_int8(x, w, ph.flat(keep), M, N, K, bias=bias, want_scales=True, n_scales=M * G)

@@ -17,8 +17,9 @@
 // with the other groups' lanes of the row operand zeroed.
 #include "zmi_device.h"
 #include "zmi_launch.h"
+#include <cstdlib>
 
-#define PG_WAVES 4
+#define PG_WAVES 2
 
 // RB: 16-row blocks per wavefront; D: chunks per operand set; SUB: groups per 64-k chunk (1: groups of whole
 // chunks); CPG: chunks per group when that is 1 or 2 (groups of 64 / 128), 0: any other multiple of 64,
@@ -38,30 +39,60 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
   const int row0 = rbk * 16 * RB;
   const uint8_t *bsrc = p.blob + zmi_blob_tiles_off(N) + (int64_t)(cb / 2) * zmi_blob_nb_stride(K) + (g4 / 2) * 1024 +
                         ((g4 % 2) * 32 + (cb % 2) * 16 + c16) * 16;
-  // rows past M repeat row M - 1 (their results are never stored); k past K reads k = 0 (the blob's
-  // rows past K are zero): every request is unconditional and the loop has no divergent branch
-  const int8_t *arow[RB];
-#pragma unroll
-  for (int j = 0; j < RB; ++j) {
-    const int row = row0 + j * 16 + c16;
-    arow[j] = (const int8_t *)p.A + (int64_t)(row < M ? row : M - 1) * p.lda;
-  }
-
   // ---- operands: two sets of D chunks of 64 k; one set is multiplied while the other set's requests
   // (issued before it) are in flight.  (A ring refilled chunk by chunk ends up with all its requests
-  // at the end of the loop body and a wait for all of them at the top: one memory latency per D chunks.) ----
-  v4i b[2][D], a[2][D][RB];
+  // at the end of the loop body and a wait for all of them at the top: one memory latency per D chunks.)
+  // The activation rows are requested row-contiguously (D * 4 consecutive lanes, D * 64 consecutive bytes:
+  // in operand order a request touches 16 rows and takes the address unit four times as long), RB * D = 8
+  // requests per set, and go through this wavefront's LDS area into operand order just before they are used.
+  // Rows past M repeat row M - 1 (their results are never stored); k past K reads k = 0 (the blob's rows
+  // past K are zero): every request is unconditional and the loop has no divergent branch. ----
+  static_assert(RB * D == 8, "eight row requests per lane and set");
+  constexpr int LPR = D * 4;                      // lanes (16-byte granules) per row and set
+  constexpr int RPI = 64 / LPR;                   // rows per request
+  const int a_q = lane % LPR, a_s = a_q / 4, a_g = a_q % 4;
+  const int8_t *arow[8];
+  int a_lds[8];                                   // byte offset of this lane's granule in the staging area
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int rl = i * RPI + lane / LPR;          // row within the wavefront's 16 RB rows
+    const int row = row0 + rl;
+    arow[i] = (const int8_t *)p.A + (int64_t)(row < M ? row : M - 1) * p.lda;
+    a_lds[i] = ((((rl / 16) * D + a_s) * 64 + a_g * 16 + ((rl % 16) ^ ((a_g * 4 + (a_s & 3)) & 15))) << 4);
+  }
+  __shared__ __attribute__((aligned(16))) uint8_t a_stage[PG_WAVES][RB * D * 1024];
+  uint8_t *a_l = a_stage[wave];
+  v4i b[2][D], raw[2][8];
   auto request_set = [&](int set, int c_first) {
+    {
+      const int c = c_first + a_s;
+      const int cc = c < nch ? c : nch - 1;        // past the end: a valid chunk, never used
+      const int k = cc * 64 + a_g * 16;
+      const int ka = k < K ? k : 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) raw[set][i] = *(const v4i *)(arow[i] + ka);
+    }
 #pragma unroll
     for (int s = 0; s < D; ++s) {
       const int c = c_first + s;
-      const int cc = c < nch ? c : nch - 1;          // (uniform) past the end: a valid chunk, never used
+      const int cc = c < nch ? c : nch - 1;        // (uniform)
       b[set][s] = *(const v4i *)(bsrc + (int64_t)cc * 2048);
-      const int k = cc * 64 + g4 * 16;
-      const int ka = k < K ? k : 0;
-#pragma unroll
-      for (int j = 0; j < RB; ++j) a[set][s][j] = *(const v4i *)(arow[j] + ka);
     }
+  };
+  // the set's rows -> LDS in operand order (bank-swizzled like the decode kernel's staging); only this
+  // wavefront's lanes touch the area and a wavefront's LDS accesses are served in order, so wavefront-scope
+  // fences (no instruction) are all the synchronisation there is
+  auto stage_rows = [&](int set) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *(v4i *)(a_l + a_lds[i]) = raw[set][i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto operand = [&](int s, int j) {
+    return *(const v4i *)(a_l + (((j * D + s) * 64 + g4 * 16 + (c16 ^ ((g4 * 4 + (s & 3)) & 15))) << 4));
   };
   request_set(0, 0);
   request_set(1, D);
@@ -132,7 +163,7 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
     if (SUB == 1) {
 #pragma unroll
       for (int j = 0; j < RB; ++j)
-        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[set][s][j], b[set][s], acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(operand(s, j), b[set][s], acc[j], 0, 0, 0);
       if (CPG ? (s + 1) % (CPG ? CPG : 1) == 0 : (c + 1) % cpg == 0) fold(c / cpg - gb0);
     } else {
 #pragma unroll
@@ -142,7 +173,7 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
           const bool mine = g4 / (4 / SUB) == t;   // this lane's 16 k belong to group t of the chunk
 #pragma unroll
           for (int j = 0; j < RB; ++j) {
-            const v4i am = mine ? a[set][s][j] : (v4i){0, 0, 0, 0};
+            const v4i am = mine ? operand(s, j) : (v4i){0, 0, 0, 0};
             acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(am, b[set][s], acc[j], 0, 0, 0);
           }
           fold(gi - gb0);
@@ -158,6 +189,7 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
     for (; c0 + 2 * D <= cend; c0 += 2 * D) {
 #pragma unroll
       for (int set = 0; set < 2; ++set) {
+        stage_rows(set);
 #pragma unroll
         for (int s = 0; s < D; ++s) step(c0 + set * D + s, set, s, gb0);
         __builtin_amdgcn_sched_barrier(0);   // the set's next requests stay between its use and the other set's
@@ -167,10 +199,13 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
     }
     // (only the last block can end with fewer than 2 D chunks; nothing is requested after them)
 #pragma unroll
-    for (int set = 0; set < 2; ++set)
+    for (int set = 0; set < 2; ++set) {
+      if (c0 + set * D >= cend) break;   // (uniform)
+      stage_rows(set);
 #pragma unroll
       for (int s = 0; s < D; ++s)
         if (c0 + set * D + s < cend) step(c0 + set * D + s, set, s, gb0);
+    }
   }
 
   // ---- alpha / beta, then the common tail; acc element q of lane l is row (l / 16) * 4 + q, column l % 16 ----
@@ -190,6 +225,163 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
     }
 }
 
+// ---- up to 16 rows: the decode kernel's shape with per-group partial tiles ---------------------
+// One workgroup of 8 wavefronts per 32 weight columns, wavefront w streams the w-th eighth of K with all
+// its requests in flight at once (k_decode.hip).  K may be split across wavefronts after all because what
+// crosses them is INTEGER: every wavefront keeps one accumulator per group of its slice (GPW whole groups
+// in CPW chunks of 64 k), the G = 8 GPW integer tiles meet in LDS, and one thread per output element then
+// adds float(acc_g) * ss[m, g] * ws[g, n] in group order -- the reference's additions, in its order, with
+// the weight stream of the per-token kernel.  Needs K a multiple of 512, whole groups per wavefront,
+// G <= 64 (2 KiB of LDS per group).
+#define PGD_WAVES 8
+#define PGD_THREADS (PGD_WAVES * 64)
+
+__device__ __forceinline__ int pgd_lds_off(int cc, int g, int r) {   // operand granule of chunk cc, k group g, row r
+  return cc * 1024 + ((g * 16 + (r ^ ((g * 4 + (cc & 3)) & 15))) << 4);
+}
+
+template <int CPW, int GPW>
+__global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(ZmiProblem p, ZmiEpilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr int CPG = CPW / GPW;                 // chunks per group
+  constexpr int G = PGD_WAVES * GPW;
+  constexpr int NCH = PGD_WAVES * CPW;           // K / 64
+  constexpr int MAIN = NCH * 1024 > G * 2048 ? NCH * 1024 : G * 2048;   // operand area, reused by the integer tiles
+  float *ws_l = reinterpret_cast<float *>(lds + MAIN);                  // [G][32]
+  float *ss_l = ws_l + G * 32;                                          // [16][G]
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int M = p.M, N = p.N, K = p.K;
+  const int blk = blockIdx.x;
+  const int c16 = lane % 16, g4 = lane / 16;
+  const int c_begin = wave * CPW;
+
+  // rows of this wavefront's slice: lanes 0..31 one row, lanes 32..63 the next (CPW * 64 bytes each)
+  const int a_q = lane % 32;
+  const bool a_live = a_q < CPW * 4;
+  v4i araw[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = 2 * i + lane / 32;
+    v4i v = {0, 0, 0, 0};
+    if (a_live && row < M) v = *(const v4i *)((const int8_t *)p.A + (int64_t)row * p.lda + (c_begin * 4 + a_q) * 16);
+    araw[i] = v;
+  }
+  // scales of this column block and of the rows, requested before the weight stream so that they are back
+  // first (columns past N / rows past M: never stored, read as the last valid one)
+  constexpr int WS_PT = (G * 32 + PGD_THREADS - 1) / PGD_THREADS;    // weight scales per thread
+  constexpr int SS_PT = (16 * G + PGD_THREADS - 1) / PGD_THREADS;    // source scales per thread
+  float ws_r[WS_PT], ss_r[SS_PT];
+#pragma unroll
+  for (int i = 0; i < WS_PT; ++i) {
+    const int e0 = tid + i * PGD_THREADS, e = e0 < G * 32 ? e0 : G * 32 - 1, n = blk * 32 + e % 32;
+    ws_r[i] = zmi_ld_f32(p.wei_scale_ptr, epi.wei_scale_dt, (int64_t)(e / 32) * N + (n < N ? n : N - 1));
+  }
+#pragma unroll
+  for (int i = 0; i < SS_PT; ++i) {
+    const int e0 = tid + i * PGD_THREADS, e = e0 < 16 * G ? e0 : 16 * G - 1, r = e / G;
+    ss_r[i] = zmi_ld_f32(p.src_scale_ptr, epi.src_scale_dt, (int64_t)(r < M ? r : M - 1) * G + e % G);
+  }
+  // the whole weight slice
+  const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
+  v4i b[CPW][2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint8_t *bsrc = tiles + (int64_t)blk * zmi_blob_nb_stride(K) + (g4 / 2) * 1024 + ((g4 % 2) * 32 + h * 16 + c16) * 16;
+#pragma unroll
+    for (int u = 0; u < CPW; ++u) b[u][h] = *(const v4i *)(bsrc + (int64_t)(c_begin + u) * 2048);
+  }
+  // (the scales requested ahead of the weights are parked in LDS only now, so nothing waited for them)
+#pragma unroll
+  for (int i = 0; i < WS_PT; ++i)
+    if (tid + i * PGD_THREADS < G * 32) ws_l[tid + i * PGD_THREADS] = ws_r[i];
+#pragma unroll
+  for (int i = 0; i < SS_PT; ++i)
+    if (tid + i * PGD_THREADS < 16 * G) ss_l[tid + i * PGD_THREADS] = ss_r[i];
+  // rows -> LDS in operand order; the wavefront reads back only its own slice (wavefront-scope fences, no barrier)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = 2 * i + lane / 32;
+    const int gran = c_begin * 4 + a_q;
+    if (a_live) *(v4i *)(lds + pgd_lds_off(gran / 4, gran % 4, row)) = araw[i];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  v4i acc[GPW][2];
+#pragma unroll
+  for (int gi = 0; gi < GPW; ++gi) {
+    acc[gi][0] = (v4i){0, 0, 0, 0};
+    acc[gi][1] = (v4i){0, 0, 0, 0};
+#pragma unroll
+    for (int u = gi * CPG; u < (gi + 1) * CPG; ++u) {
+      const v4i a = *(const v4i *)(lds + pgd_lds_off(c_begin + u, g4, c16));
+      acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[gi][0], 0, 0, 0);
+      acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[gi][1], 0, 0, 0);
+    }
+  }
+  // ---- the integer tiles of all groups meet in LDS (the operand area is done with) ----
+  __syncthreads();
+  int32_t *red = (int32_t *)lds;
+#pragma unroll
+  for (int gi = 0; gi < GPW; ++gi)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) red[(wave * GPW + gi) * 512 + (h * 4 + q) * 64 + lane] = acc[gi][h][q];
+  __syncthreads();
+  // ---- one thread per output element: the group terms in order, each step rounded ----
+  const int e_row = tid / 32, e_h = (tid % 32) / 16, e_c = tid % 16;
+  const int e_n = blk * 32 + e_h * 16 + e_c;
+  if (e_n >= N || e_row >= M) return;
+  // acc[h][q] of lane l is row (l / 16) * 4 + q, column h * 16 + l % 16
+  const int off = (e_h * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_c;
+  float sum = 0.0f;
+#pragma unroll 8
+  for (int g = 0; g < G; ++g) {
+    float t = __fmul_rn((float)red[g * 512 + off], ss_l[e_row * G + g]);
+    t = __fmul_rn(t, ws_l[g * 32 + e_h * 16 + e_c]);
+    sum = __fadd_rn(sum, t);
+  }
+  const int64_t o = (int64_t)e_row * p.ldc + e_n;
+  float y = sum;
+  if (epi.alpha != 1.0f) y = __fmul_rn(y, epi.alpha);
+  if (epi.beta != 0.0f) y = __fadd_rn(y, __fmul_rn(zmi_ld_f32(p.dst, epi.dst_dt, o), epi.beta));
+  const float bias = p.bias ? zmi_ld_f32(p.bias, epi.bias_dt, e_n) : 0.0f;
+  zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_tail(epi, y, bias, e_row, e_n));
+}
+
+template <int CPW, int GPW>
+static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
+  constexpr int G = PGD_WAVES * GPW, NCH = PGD_WAVES * CPW;
+  constexpr size_t main_bytes = NCH * 1024 > G * 2048 ? NCH * 1024 : G * 2048;
+  constexpr size_t smem = main_bytes + (size_t)G * 32 * 4 + (size_t)16 * G * 4;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_decode_pergroup_kernel<CPW, GPW>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  const dim3 grid((unsigned)(zmi_blob_npad(p.N) / 32)), block(PGD_THREADS);
+  hipLaunchKernelGGL((zmi_gemm_decode_pergroup_kernel<CPW, GPW>), grid, block, smem, stream, p, epi);
+  return hipGetLastError();
+}
+
+// the decode-shaped kernel serves: up to 16 rows, K = 512 * CPW (CPW in 1, 2, 4, 8), whole groups per wavefront
+static bool pgd_fits(const ZmiProblem &p, int G, int *cpw, int *gpw) {
+  if (p.M > 16 || p.K % 512 != 0 || p.K > 4096 || G % PGD_WAVES != 0 || G > 64) return false;
+  const int c = p.K / 512, g = G / PGD_WAVES;
+  if (!(c == 1 || c == 2 || c == 4 || c == 8) || c % g != 0) return false;
+  *cpw = c; *gpw = g;
+  return true;
+}
+
+bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G) {
+  int cpw, gpw;
+  return pgd_fits(p, G, &cpw, &gpw) && !getenv("ZMI_PERGROUP_GENERIC");
+}
+
 bool zmi_pergroup_group_size_ok(int64_t gs) { return gs > 0 && (gs % 64 == 0 || gs == 32 || gs == 16); }
 
 hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
@@ -201,6 +393,22 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
     return hipErrorInvalidValue;
   if (p.a_is_u8 || epi.has_zp || epi.gated_act) return hipErrorInvalidValue;   // symmetric s8 rows only
   if (p.lda % 16 != 0 || ((uintptr_t)p.A) % 16 != 0 || p.lda < p.K) return hipErrorInvalidValue;   // 16-byte row loads
+  int cpw = 0, gpw = 0;
+  if (pgd_fits(p, G, &cpw, &gpw) && !getenv("ZMI_PERGROUP_GENERIC")) {
+    switch (cpw * 16 + gpw) {
+    case 8 * 16 + 8: return pgd_launch<8, 8>(p, epi, stream);
+    case 8 * 16 + 4: return pgd_launch<8, 4>(p, epi, stream);
+    case 8 * 16 + 2: return pgd_launch<8, 2>(p, epi, stream);
+    case 8 * 16 + 1: return pgd_launch<8, 1>(p, epi, stream);
+    case 4 * 16 + 4: return pgd_launch<4, 4>(p, epi, stream);
+    case 4 * 16 + 2: return pgd_launch<4, 2>(p, epi, stream);
+    case 4 * 16 + 1: return pgd_launch<4, 1>(p, epi, stream);
+    case 2 * 16 + 2: return pgd_launch<2, 2>(p, epi, stream);
+    case 2 * 16 + 1: return pgd_launch<2, 1>(p, epi, stream);
+    case 1 * 16 + 1: return pgd_launch<1, 1>(p, epi, stream);
+    default: break;
+    }
+  }
   const int n_cb = (int)(zmi_blob_npad(p.N) / 16);
   const int rb = p.M <= 16 ? 1 : 4;
   const int n_rb = (p.M + 16 * rb - 1) / (16 * rb);

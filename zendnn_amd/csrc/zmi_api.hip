@@ -528,7 +528,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
   if (st != ZMI_SUCCESS) return st;
   if (epi.n_groups > 0) {
-    set_kernel_name("pergroup_mfma16x16x64");
+    set_kernel_name(zmi_pergroup_decode_shape(prob, epi.n_groups) ? "pergroup_decode_mfma16x16x64" : "pergroup_mfma16x16x64");
     st = hip_ok(zmi_launch_gemm_pergroup(prob, epi, stream()), "per-group GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
   } else if (use_fused) {
     // a one-row scale in device memory reads like a per-token scale

@@ -90,6 +90,8 @@ hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, h
 // 16-byte aligned leading dimension; group sizes 16, 32 or a multiple of 64
 bool zmi_pergroup_group_size_ok(int64_t gs);
 hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+// true when the launch above takes the decode-shaped kernel (up to 16 rows, K = 512 .. 4096 in whole eighths, G <= 64)
+bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G);
 // per (row, group) dynamic quantization of bf16 / f32 rows: s8 rows (ld ldq), f32 scales {M,G} and an
 // optional copy of the scales in the caller's buffer (f32 or bf16)
 hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
