@@ -16,6 +16,7 @@
 // at a time.  Groups of 16 or 32 k share a 64-k chunk: the chunk is multiplied once per group
 // with the other groups' lanes of the row operand zeroed.
 #include "zmi_device.h"
+#include "zmi_fused_quant.h"
 #include "zmi_launch.h"
 #include <cstdlib>
 
@@ -241,7 +242,8 @@ __device__ __forceinline__ int pgd_lds_off(int cc, int g, int r) {   // operand 
 }
 
 template <int CPW, int GPW>
-__global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(ZmiProblem p, ZmiEpilogue epi) {
+__global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(ZmiProblem p, ZmiEpilogue epi,
+                                                                               ZmiFusedQuant fq) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int CPG = CPW / GPW;                 // chunks per group
   constexpr int G = PGD_WAVES * GPW;
@@ -252,7 +254,17 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int M = p.M, N = p.N, K = p.K;
-  const int blk = blockIdx.x;
+  // With fused quantization the first M workgroups quantize one source row each (per group), publish it and
+  // leave; the streaming workgroups follow them in dispatch order and wait (bounded) for the M rows only after
+  // their weight requests are out.  Producers wait for nothing, so the wait cannot deadlock.
+  if (fq.x && (int)blockIdx.x < M) {
+    zmi_fused_quant_row_groups(fq, blockIdx.x, K, G);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
+    __syncthreads();
+    if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
+    return;
+  }
+  const int blk = fq.x ? (int)blockIdx.x - M : (int)blockIdx.x;
   const int c16 = lane % 16, g4 = lane / 16;
   const int c_begin = wave * CPW;
 
@@ -260,13 +272,16 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   const int a_q = lane % 32;
   const bool a_live = a_q < CPW * 4;
   v4i araw[8];
+  auto load_rows = [&]() {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = 2 * i + lane / 32;
-    v4i v = {0, 0, 0, 0};
-    if (a_live && row < M) v = *(const v4i *)((const int8_t *)p.A + (int64_t)row * p.lda + (c_begin * 4 + a_q) * 16);
-    araw[i] = v;
-  }
+    for (int i = 0; i < 8; ++i) {
+      const int row = 2 * i + lane / 32;
+      v4i v = {0, 0, 0, 0};
+      if (a_live && row < M) v = *(const v4i *)((const int8_t *)p.A + (int64_t)row * p.lda + (c_begin * 4 + a_q) * 16);
+      araw[i] = v;
+    }
+  };
+  if (!fq.x) load_rows();
   // scales of this column block and of the rows, requested before the weight stream so that they are back
   // first (columns past N / rows past M: never stored, read as the last valid one)
   constexpr int WS_PT = (G * 32 + PGD_THREADS - 1) / PGD_THREADS;    // weight scales per thread
@@ -277,19 +292,48 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
     const int e0 = tid + i * PGD_THREADS, e = e0 < G * 32 ? e0 : G * 32 - 1, n = blk * 32 + e % 32;
     ws_r[i] = zmi_ld_f32(p.wei_scale_ptr, epi.wei_scale_dt, (int64_t)(e / 32) * N + (n < N ? n : N - 1));
   }
+  auto load_ss = [&]() {
 #pragma unroll
-  for (int i = 0; i < SS_PT; ++i) {
-    const int e0 = tid + i * PGD_THREADS, e = e0 < 16 * G ? e0 : 16 * G - 1, r = e / G;
-    ss_r[i] = zmi_ld_f32(p.src_scale_ptr, epi.src_scale_dt, (int64_t)(r < M ? r : M - 1) * G + e % G);
-  }
+    for (int i = 0; i < SS_PT; ++i) {
+      const int e0 = tid + i * PGD_THREADS, e = e0 < 16 * G ? e0 : 16 * G - 1, r = e / G;
+      ss_r[i] = zmi_ld_f32(p.src_scale_ptr, epi.src_scale_dt, (int64_t)(r < M ? r : M - 1) * G + e % G);
+    }
+  };
+  if (!fq.x) load_ss();
   // the whole weight slice
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   v4i b[CPW][2];
+  const uint8_t *bsrc[2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const uint8_t *bsrc = tiles + (int64_t)blk * zmi_blob_nb_stride(K) + (g4 / 2) * 1024 + ((g4 % 2) * 32 + h * 16 + c16) * 16;
+  for (int h = 0; h < 2; ++h)
+    bsrc[h] = tiles + (int64_t)blk * zmi_blob_nb_stride(K) + (g4 / 2) * 1024 + ((g4 % 2) * 32 + h * 16 + c16) * 16;
+  // (with fused quantization three quarters of the slice go out before the wait for the rows, the rest
+  // after the row requests, like the per-token decode kernel)
+  constexpr int FIRST = CPW >= 4 ? CPW * 3 / 4 : CPW;
 #pragma unroll
-    for (int u = 0; u < CPW; ++u) b[u][h] = *(const v4i *)(bsrc + (int64_t)(c_begin + u) * 2048);
+  for (int u = 0; u < CPW; ++u)
+    if (u < FIRST || !fq.x) {
+      b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)(c_begin + u) * 2048);
+      b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(c_begin + u) * 2048);
+    }
+  if (fq.x) {
+    // the quantized rows and their scales exist once the counter says so
+    if (tid == 0) {
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        const unsigned int v = __hip_atomic_load(fq.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((int)(v - fq.target) >= 0) break;
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    __syncthreads();
+    asm volatile("" ::: "memory");   // the loads below stay below the wait
+    load_rows();
+    load_ss();
+#pragma unroll
+    for (int u = FIRST; u < CPW; ++u) {
+      b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)(c_begin + u) * 2048);
+      b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(c_begin + u) * 2048);
+    }
   }
   // (the scales requested ahead of the weights are parked in LDS only now, so nothing waited for them)
 #pragma unroll
@@ -352,7 +396,7 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
 }
 
 template <int CPW, int GPW>
-static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
+static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq, hipStream_t stream) {
   constexpr int G = PGD_WAVES * GPW, NCH = PGD_WAVES * CPW;
   constexpr size_t main_bytes = NCH * 1024 > G * 2048 ? NCH * 1024 : G * 2048;
   constexpr size_t smem = main_bytes + (size_t)G * 32 * 4 + (size_t)16 * G * 4;
@@ -363,8 +407,9 @@ static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, hipStr
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  const dim3 grid((unsigned)(zmi_blob_npad(p.N) / 32)), block(PGD_THREADS);
-  hipLaunchKernelGGL((zmi_gemm_decode_pergroup_kernel<CPW, GPW>), grid, block, smem, stream, p, epi);
+  ZmiFusedQuant none = {};
+  const dim3 grid((unsigned)(zmi_blob_npad(p.N) / 32) + (fq ? p.M : 0)), block(PGD_THREADS);
+  hipLaunchKernelGGL((zmi_gemm_decode_pergroup_kernel<CPW, GPW>), grid, block, smem, stream, p, epi, fq ? *fq : none);
   return hipGetLastError();
 }
 
@@ -384,7 +429,8 @@ bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G) {
 
 bool zmi_pergroup_group_size_ok(int64_t gs) { return gs > 0 && (gs % 64 == 0 || gs == 32 || gs == 16); }
 
-hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
+hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
+                                    hipStream_t stream) {
   const int G = epi.n_groups;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || G <= 0 || p.K % G != 0) return hipErrorInvalidValue;
   const int gs = p.K / G;
@@ -396,19 +442,20 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
   int cpw = 0, gpw = 0;
   if (pgd_fits(p, G, &cpw, &gpw) && !getenv("ZMI_PERGROUP_GENERIC")) {
     switch (cpw * 16 + gpw) {
-    case 8 * 16 + 8: return pgd_launch<8, 8>(p, epi, stream);
-    case 8 * 16 + 4: return pgd_launch<8, 4>(p, epi, stream);
-    case 8 * 16 + 2: return pgd_launch<8, 2>(p, epi, stream);
-    case 8 * 16 + 1: return pgd_launch<8, 1>(p, epi, stream);
-    case 4 * 16 + 4: return pgd_launch<4, 4>(p, epi, stream);
-    case 4 * 16 + 2: return pgd_launch<4, 2>(p, epi, stream);
-    case 4 * 16 + 1: return pgd_launch<4, 1>(p, epi, stream);
-    case 2 * 16 + 2: return pgd_launch<2, 2>(p, epi, stream);
-    case 2 * 16 + 1: return pgd_launch<2, 1>(p, epi, stream);
-    case 1 * 16 + 1: return pgd_launch<1, 1>(p, epi, stream);
+    case 8 * 16 + 8: return pgd_launch<8, 8>(p, epi, fq, stream);
+    case 8 * 16 + 4: return pgd_launch<8, 4>(p, epi, fq, stream);
+    case 8 * 16 + 2: return pgd_launch<8, 2>(p, epi, fq, stream);
+    case 8 * 16 + 1: return pgd_launch<8, 1>(p, epi, fq, stream);
+    case 4 * 16 + 4: return pgd_launch<4, 4>(p, epi, fq, stream);
+    case 4 * 16 + 2: return pgd_launch<4, 2>(p, epi, fq, stream);
+    case 4 * 16 + 1: return pgd_launch<4, 1>(p, epi, fq, stream);
+    case 2 * 16 + 2: return pgd_launch<2, 2>(p, epi, fq, stream);
+    case 2 * 16 + 1: return pgd_launch<2, 1>(p, epi, fq, stream);
+    case 1 * 16 + 1: return pgd_launch<1, 1>(p, epi, fq, stream);
     default: break;
     }
   }
+  if (fq) return hipErrorInvalidValue;   // fused quantization exists for the decode-shaped kernel only
   const int n_cb = (int)(zmi_blob_npad(p.N) / 16);
   const int rb = p.M <= 16 ? 1 : 4;
   const int n_rb = (p.M + 16 * rb - 1) / (16 * rb);

@@ -470,9 +470,19 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     if (pg_groups) {
       // reference: the per-group dynamic reorder in front of the sym-quant GEMM
       // (matmul/quantization/reorder_quantization.cpp:43-280 with {M,G} scale dims)
-      if (!hip_ok(zmi_launch_quant_groups(src, p.dt_src, M, K, lda, pg_groups, q, K16, sc, (void *)p.src_scale.buff, sdt,
-                                          stream()), "per-group quant launch"))
+      if (zmi_pergroup_decode_shape(prob, (int)pg_groups) && !std::getenv("ZMI_NO_FUSED_QUANT")) {
+        // decode shapes: the quantization is part of the GEMM launch (its first M workgroups)
+        unsigned int *ctr = fused_counter();
+        if (!ctr) return ZMI_FAILURE;
+        fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
+        fused.q = q; fused.ldq = K16; fused.scales = sc;
+        fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
+        fused.counter = ctr; fused.target = fused_next_target(M);
+        use_fused = true;
+      } else if (!hip_ok(zmi_launch_quant_groups(src, p.dt_src, M, K, lda, pg_groups, q, K16, sc, (void *)p.src_scale.buff,
+                                                 sdt, stream()), "per-group quant launch")) {
         return ZMI_FAILURE;
+      }
       ep.src_scale.buff = sc;
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
@@ -528,8 +538,10 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
   if (st != ZMI_SUCCESS) return st;
   if (epi.n_groups > 0) {
-    set_kernel_name(zmi_pergroup_decode_shape(prob, epi.n_groups) ? "pergroup_decode_mfma16x16x64" : "pergroup_mfma16x16x64");
-    st = hip_ok(zmi_launch_gemm_pergroup(prob, epi, stream()), "per-group GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+    set_kernel_name(use_fused ? "pergroup_decode_mfma16x16x64 (fused per-group quant)"
+                    : zmi_pergroup_decode_shape(prob, epi.n_groups) ? "pergroup_decode_mfma16x16x64" : "pergroup_mfma16x16x64");
+    st = hip_ok(zmi_launch_gemm_pergroup(prob, epi, use_fused ? &fused : nullptr, stream()), "per-group GEMM launch")
+             ? ZMI_SUCCESS : ZMI_FAILURE;
   } else if (use_fused) {
     // a one-row scale in device memory reads like a per-token scale
     if (epi.src_scale_mode == ZMI_SS_TENSOR_PTR) epi.src_scale_mode = ZMI_SS_TOKEN_PTR;

@@ -153,3 +153,103 @@ static __device__ void zmi_fused_quant_row_wave(const ZmiFusedQuant &fq, int row
     __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
+
+
+// Per-group form: one source row, G groups of K / G elements, every wavefront of the workgroup takes the
+// groups w, w + n_waves, ... (same arithmetic as zmi_quant_groups_kernel; K / G must be a multiple of 4).
+// Scales go to fq.scales[row * G + g]; published like the rows, with device-scope stores.
+static __device__ void zmi_fused_quant_row_groups(const ZmiFusedQuant &fq, int row, int K, int G) {
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, n_waves = blockDim.x / 64;
+  const bool bf16 = fq.x_dt == ZMI_DT_BF16;
+  const int gs = K / G;
+  // Fast form: the row fits the workgroup at 8 elements per thread and a group is a power-of-two run of
+  // lanes inside one wavefront (groups of 64 .. 512): one 16-byte request per thread (two for f32), the
+  // group maximum by lane exchanges, one 8-byte store -- a single trip to memory.
+  const int es = bf16 ? 2 : 4;
+  const char *rowp = (const char *)fq.x + (size_t)row * fq.ldx * es;
+  if (K % 8 == 0 && K <= (int)blockDim.x * 8 && gs >= 64 && gs <= 512 && (gs & (gs - 1)) == 0 &&
+      ((uintptr_t)rowp % 16) == 0) {
+    const int t = threadIdx.x;
+    float v8[8];
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) v8[j] = 0.0f;
+    if (t * 8 < K) {
+      if (bf16) {
+        const v4i raw = *(const v4i *)(rowp + (size_t)t * 16);
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v8[2 * j] = __uint_as_float(((uint32_t)raw[j]) << 16);
+          v8[2 * j + 1] = __uint_as_float(((uint32_t)raw[j]) & 0xffff0000u);
+        }
+      } else {
+        const v4i r0 = *(const v4i *)(rowp + (size_t)t * 32), r1 = *(const v4i *)(rowp + (size_t)t * 32 + 16);
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) { v8[j] = __int_as_float(r0[j]); v8[4 + j] = __int_as_float(r1[j]); }
+      }
+    }
+    float amax = 0.0f;
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = fabsf(v8[j]);
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+    const int lpg = gs / 8;   // lanes per group: 8 .. 64
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+      if (o < lpg) amax = fmaxf(amax, __shfl_xor(amax, o));
+    if (amax < 1e-10f) amax = 1e-10f;
+    float s = __fdiv_rn(amax, 127.0f);
+    if (s < 1e-10f) s = 1e-10f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (t * 8 < K) {
+      const int g = t * 8 / gs;
+      if (t % lpg == 0) {
+        __hip_atomic_store((unsigned int *)&fq.scales[(int64_t)row * G + g], __float_as_uint(s), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        if (fq.user_scales) {
+          if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[(int64_t)row * G + g] = zmi_f32_to_bf16_rne(s);
+          else ((float *)fq.user_scales)[(int64_t)row * G + g] = s;
+        }
+      }
+      unsigned int *dst = (unsigned int *)(fq.q + (int64_t)row * fq.ldq);
+      #pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        unsigned int w = 0;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_quant_elem(v8[h * 4 + j], s, inv)) << (8 * j);
+        __hip_atomic_store(&dst[t * 2 + h], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    return;
+  }
+  for (int g = wave; g < G; g += n_waves) {
+    const int64_t base = (int64_t)row * fq.ldx + (int64_t)g * gs;
+    auto ld = [&](int k) { return bf16 ? zmi_bf16_to_f32(((const uint16_t *)fq.x)[base + k]) : ((const float *)fq.x)[base + k]; };
+    float amax = 0.0f;
+    for (int k = lane; k < gs; k += 64) {
+      const float a = fabsf(ld(k));
+      if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+    }
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    if (amax < 1e-10f) amax = 1e-10f;
+    float s = __fdiv_rn(amax, 127.0f);
+    if (s < 1e-10f) s = 1e-10f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (lane == 0) {
+      __hip_atomic_store((unsigned int *)&fq.scales[(int64_t)row * G + g], __float_as_uint(s), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      if (fq.user_scales) {
+        if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[(int64_t)row * G + g] = zmi_f32_to_bf16_rne(s);
+        else ((float *)fq.user_scales)[(int64_t)row * G + g] = s;
+      }
+    }
+    unsigned int *dst = (unsigned int *)(fq.q + (int64_t)row * fq.ldq + (int64_t)g * gs);
+    for (int k4 = lane; k4 < gs / 4; k4 += 64) {
+      unsigned int w = 0;
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) w |= ((unsigned int)(uint8_t)zmi_quant_elem(ld(k4 * 4 + j), s, inv)) << (8 * j);
+      __hip_atomic_store(&dst[k4], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}

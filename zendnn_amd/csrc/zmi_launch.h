@@ -89,7 +89,10 @@ hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, h
 // k_pergroup.hip: per-group symmetric scales ({M,G} source, {G,N} weights), any M; s8 rows with a
 // 16-byte aligned leading dimension; group sizes 16, 32 or a multiple of 64
 bool zmi_pergroup_group_size_ok(int64_t gs);
-hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+struct ZmiFusedQuant;
+// fq != null (decode-shaped problems only): the per-group quantization of the M rows is part of the launch
+hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
+                                    hipStream_t stream);
 // true when the launch above takes the decode-shaped kernel (up to 16 rows, K = 512 .. 4096 in whole eighths, G <= 64)
 bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G);
 // per (row, group) dynamic quantization of bf16 / f32 rows: s8 rows (ld ldq), f32 scales {M,G} and an
