@@ -120,7 +120,8 @@ typedef struct zmi_matmul_params_t {
   int32_t lowoha_algo;        /* enum zmi_matmul_algo */
   int32_t num_threads;        /* accepted and ignored: the GPU grid replaces OpenMP */
   int32_t dynamic_quant;
-  int32_t pack_format_b;      /* 0 only; 1 (GGML Q8_0) => ZMI_UNIMPLEMENTED */
+  int32_t pack_format_b;      /* 0: plain weights; 1: GGML Q8_0 blocks [N][K/32] x {fp16 d, int8 qs[32]}
+                               * (transB and constant weights required; source scales {M, K/32}) */
   uint32_t total_matmul;
   uint32_t active_matmul;
   int32_t weight_cache_type;  /* 0 none, 1/2 keep a packed copy keyed by pointer */

@@ -46,6 +46,10 @@ def lib():
         L.zo_quant_per_group.restype = None
         L.zo_quant_per_group.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                                          C.c_void_p, C.c_int64, C.c_void_p]
+        L.zo_fp16_to_f32.restype = C.c_float
+        L.zo_fp16_to_f32.argtypes = [C.c_uint16]
+        L.zo_ggml_q8_0_unpack.restype = None
+        L.zo_ggml_q8_0_unpack.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.zo_gemm_s32.restype = C.c_int64
         L.zo_gemm_s32.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
                                   C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
@@ -113,6 +117,15 @@ def quant_per_group(src, src_dt, G):
     s = np.empty((M, G), dtype=np.float32)
     lib().zo_quant_per_group(_p(src), src_dt, M, K, G, K, _p(q), K, _p(s))
     return q, s
+
+
+def ggml_q8_0_unpack(blocks, N, K):
+    """blocks: uint8 [N * (K/32) * 34] -> (rows int8 [N,K], scales bf16 bits uint16 [K/32, N])."""
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    rows = np.empty((N, K), dtype=np.int8)
+    scales = np.empty((K // 32, N), dtype=np.uint16)
+    lib().zo_ggml_q8_0_unpack(_p(blocks), N, K, _p(rows), _p(scales))
+    return rows, scales
 
 
 def gemm_s32(A, B, transA=False, transB=False):

@@ -29,6 +29,8 @@
  *   per-group scales             closed form (all-ones operands, power-of-two scales: every step exact),
  *                                equal power-of-two group scales == per-token chain bit for bit,
  *                                numpy float32 brute force on small random cases
+ *   zo_fp16_to_f32, Q8_0 unpack  all 65536 half values against numpy float16; block layout by construction
+ *                                of the packed buffer from known rows and scales (numpy), bf16 via torch
  *   zo_quant_per_group           per-group constants (closed form), == zo_quant_per_token on the
  *                                [M*G, K/G] view
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
@@ -350,6 +352,50 @@ static void zo_store(void *dst, int32_t dt, int64_t i, float val) {
   }
 }
 
+/* ---- GGML Q8_0 packed weights ------------------------------------------------------------ */
+
+/* fp16_to_fp32 of lowoha_operators/matmul/ggml_weight_unpack.cpp:54-65 (llama.cpp's), restated on the bit
+ * fields: exact conversion of every half value, subnormals included. */
+ZO_EXPORT float zo_fp16_to_f32(uint16_t h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+  uint32_t u;
+  if (e == 0x1f) u = sign | 0x7f800000u | (m << 13);              /* inf / NaN */
+  else if (e != 0) u = sign | ((e + 112u) << 23) | (m << 13);     /* normal: rebias 15 -> 127 */
+  else if (m == 0) u = sign;                                      /* zero */
+  else {                                                          /* subnormal: m * 2^-24 */
+    float f = (float)m * 5.9604644775390625e-08f;
+    memcpy(&u, &f, 4);
+    u |= sign;
+  }
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* fp32_to_bf16 of ggml_weight_unpack.cpp:66-73: NaN quieted, else round to nearest even (no flush). */
+static uint16_t zo_ggml_f32_to_bf16(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 64u);
+  return (uint16_t)((u + (0x7fffu + ((u >> 16) & 1u))) >> 16);
+}
+
+/* ggml_unpack_weight_buffer, Q8_0 branch with bf16 scales (ggml_weight_unpack.cpp:190-236): blocks
+ * [N][K/32] of { fp16 d; int8 qs[32] } -> rows[n*K + g*32 + i] = qs[i], scales[g*N + n] = bf16(f32(d)). */
+ZO_EXPORT void zo_ggml_q8_0_unpack(const void *blocks, int64_t N, int64_t K, int8_t *rows, uint16_t *scales) {
+  const int64_t ng = K / 32;
+  const uint8_t *b = (const uint8_t *)blocks;
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t g = 0; g < ng; ++g) {
+      const uint8_t *blk = b + (n * ng + g) * 34;
+      uint16_t d;
+      memcpy(&d, blk, 2);
+      scales[g * N + n] = zo_ggml_f32_to_bf16(zo_fp16_to_f32(d));
+      memcpy(rows + n * K + g * 32, blk + 2, 32);
+    }
+}
+
 /* matmul_direct for the int8 path.  Pipeline of lowoha_operators/matmul/
  * lowoha_matmul.cpp:278-510: optional dynamic per-token quantization of a
  * bf16/f32 source (matmul/quantization/reorder_quantization.cpp:43-280), then
@@ -361,9 +407,26 @@ static void zo_store(void *dst, int32_t dt, int64_t i, float val) {
  *   store with the dtype's rounding.
  * Returns a ZMI_* status. */
 ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
-  const zmi_matmul_params_t *p = c->params;
+  zmi_matmul_params_t pl = *c->params;   /* working copy: the GGML unpack sets the weight scales */
+  const zmi_matmul_params_t *p = &pl;
   const int64_t M = c->M, N = c->N, K = c->K;
   if (p->dt_wei != ZMI_DT_S8) return ZMI_UNIMPLEMENTED;
+  const void *weight = c->weight;
+  int64_t ldb = c->ldb;
+  int8_t *ggml_rows = NULL;
+  uint16_t *ggml_scales = NULL;
+  if (p->pack_format_b == 1) {
+    /* validate_ggml_packed_inputs + unpack_ggml_weights_and_cache,
+     * lowoha_operators/matmul/ggml_weight_unpack.cpp:155-183, 367-420: transB required, the unpacked
+     * rows are [N, K], the scales become the bf16 {K/32, N} weight scales */
+    if (!c->transB || K % 32 != 0) return ZMI_FAILURE;
+    ggml_rows = (int8_t *)malloc((size_t)N * K);
+    ggml_scales = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(K / 32) * N);
+    zo_ggml_q8_0_unpack(weight, N, K, ggml_rows, ggml_scales);
+    weight = ggml_rows; ldb = K;
+    pl.wei_scale.buff = ggml_scales; pl.wei_scale.dt = ZMI_DT_BF16;
+    pl.wei_scale.ndims = 2; pl.wei_scale.dims[0] = K / 32; pl.wei_scale.dims[1] = N;
+  }
 
   const void *A = c->src;
   int32_t a_dt = p->dt_src;
@@ -431,11 +494,11 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
     const int64_t wn = p->wei_scale.buff ? zo_nelems(&p->wei_scale) : 0;
     if (K % G != 0 || wn != G * N || p->src_zp.buff || a_dt != ZMI_DT_S8 ||
         !(p->dt_dst == ZMI_DT_F32 || p->dt_dst == ZMI_DT_BF16)) {
-      free(qbuf); free(sbuf);
+      free(qbuf); free(sbuf); free(ggml_rows); free(ggml_scales);
       return ZMI_FAILURE;
     }
     const int64_t gs = K / G;
-    const int8_t *W = (const int8_t *)c->weight;
+    const int8_t *W = (const int8_t *)weight;
     #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m) {
       for (int64_t n = 0; n < N; ++n) {
@@ -444,7 +507,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
           int32_t group_sum = 0;
           for (int64_t k = g * gs; k < (g + 1) * gs; ++k) {
             int32_t a = ((const int8_t *)A)[transA ? k * lda + m : m * lda + k];
-            group_sum += a * (int32_t)W[c->transB ? n * c->ldb + k : k * c->ldb + n];
+            group_sum += a * (int32_t)W[c->transB ? n * ldb + k : k * ldb + n];
           }
           float grp = (float)group_sum * zo_read_f32(src_scale, src_scale_dt, m * G + g);
           grp *= zo_read_f32(p->wei_scale.buff, p->wei_scale.dt, g * N + n);
@@ -468,24 +531,24 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
         zo_store(c->dst, p->dt_dst, m * (int64_t)c->ldc + n, y);
       }
     }
-    free(qbuf); free(sbuf);
+    free(qbuf); free(sbuf); free(ggml_rows); free(ggml_scales);
     return ZMI_SUCCESS;
   }
 
   int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)M * N);
   if (!transA && M * N * K > (1 << 22)) {
-    int8_t *Bt = (int8_t *)c->weight;
-    int64_t ldbt = c->ldb;
+    int8_t *Bt = (int8_t *)weight;
+    int64_t ldbt = ldb;
     int8_t *tmp = NULL;
     if (!c->transB) {
       tmp = (int8_t *)malloc((size_t)N * K);
-      zo_transpose_s8((const int8_t *)c->weight, K, N, c->ldb, tmp);
+      zo_transpose_s8((const int8_t *)weight, K, N, ldb, tmp);
       Bt = tmp; ldbt = K;
     }
     zo_gemm_s32_bt(A, a_dt, lda, Bt, ldbt, M, N, K, acc, N);
     free(tmp);
   } else {
-    zo_gemm_s32(A, a_dt, transA, lda, (const int8_t *)c->weight, c->transB, c->ldb, M, N, K, acc, N);
+    zo_gemm_s32(A, a_dt, transA, lda, (const int8_t *)weight, c->transB, ldb, M, N, K, acc, N);
   }
   if (c->acc_out) memcpy(c->acc_out, acc, sizeof(int32_t) * (size_t)M * N);
 
@@ -493,7 +556,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
   int32_t *comp = NULL;
   if (src_zp) {
     comp = (int32_t *)malloc(sizeof(int32_t) * (size_t)N);
-    zo_zp_comp((const int8_t *)c->weight, c->transB, c->ldb, K, N, src_zp, comp);
+    zo_zp_comp((const int8_t *)weight, c->transB, ldb, K, N, src_zp, comp);
   }
   const int per_token = (src_scale_n == M && M > 1);
   const int64_t wei_scale_n = p->wei_scale.buff ? zo_nelems(&p->wei_scale) : 0;
@@ -529,7 +592,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
       zo_store(c->dst, p->dt_dst, m * (int64_t)c->ldc + n, y);
     }
   }
-  free(acc); free(comp); free(qbuf); free(sbuf);
+  free(acc); free(comp); free(qbuf); free(sbuf); free(ggml_rows); free(ggml_scales);
   return ZMI_SUCCESS;
 }
 

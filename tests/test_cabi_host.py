@@ -89,7 +89,9 @@ def test_matmul_validation_status_codes():
     assert _mm(p) == capi.FAILURE
     # outside the implemented path: status unimplemented, not failure
     assert _mm(lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_BF16, dst=capi.DT_BF16)) == capi.UNIMPLEMENTED
-    assert _mm(_int8_params(pack_format_b=1)) == capi.UNIMPLEMENTED
+    # GGML-packed weights: transB = true is required (the packed layout is N x K), as in the reference
+    assert _mm(_int8_params(pack_format_b=1)) == capi.FAILURE
+    assert _mm(_int8_params(pack_format_b=2)) == capi.FAILURE
     assert _mm(lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16)) == capi.UNIMPLEMENTED
     assert lowoha.matmul_direct("c", False, False, 4, 8, 16, 1.0, FAKE, 16, FAKE, 8, None, 0.0, FAKE, 8, True,
                                 _int8_params()) == capi.UNIMPLEMENTED

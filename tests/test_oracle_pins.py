@@ -388,6 +388,67 @@ def test_chain_dynamic_quant_per_group(zo):
     assert np.abs(dst - full).max() < 0.02 * np.abs(full).max()
 
 
+# ------------------------------------------------------------- GGML Q8_0
+def _q8_0_pack(rows, d16):
+    """rows int8 [N,K], d16 float16 [N, K/32] -> the packed buffer: [N][K/32] blocks of {fp16 d, int8 qs[32]}."""
+    N, K = rows.shape
+    blk = np.zeros((N, K // 32, 34), dtype=np.uint8)
+    blk[:, :, :2] = d16.view(np.uint16).reshape(N, K // 32, 1).view(np.uint8)
+    blk[:, :, 2:] = rows.reshape(N, K // 32, 32).view(np.uint8)
+    return blk.reshape(-1)
+
+
+def test_fp16_conversion_against_numpy_for_every_half_value(zo):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([zo.lib().zo_fp16_to_f32(int(v)) for v in h], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_ggml_q8_0_unpack_layout_and_bf16_scales(zo):
+    rng = np.random.default_rng(31)
+    N, K = 7, 96
+    rows = rng.integers(-128, 128, (N, K), dtype=np.int8)
+    d16 = rng.uniform(1e-4, 0.05, (N, K // 32)).astype(np.float16)
+    d16[0, 0] = np.float16(6e-8)               # an fp16 subnormal
+    got_rows, got_scales = zo.ggml_q8_0_unpack(_q8_0_pack(rows, d16), N, K)
+    assert np.array_equal(got_rows, rows)
+    want = torch.from_numpy(d16.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got_scales, want.T)  # scales[g, n] = bf16(f32(d[n, g]))
+
+
+def test_ggml_matmul_is_the_per_group_matmul_on_the_unpacked_weights(zo):
+    rng = np.random.default_rng(32)
+    M, K, N = 5, 128, 9
+    G = K // 32
+    A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    rows = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    d16 = rng.uniform(1e-3, 0.02, (N, G)).astype(np.float16)
+    ss = rng.uniform(0.005, 0.03, (M, G)).astype(np.float32)
+    packed = _q8_0_pack(rows, d16)
+    p = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32, pack_format_b=1,
+                src_scale=capi.quant(ss.ctypes.data, capi.DT_F32, (M, G)))
+    st, got, _, _ = zo.matmul_int8(A, packed, p, M, N, K, transB=True, ldb=K)
+    assert st == capi.SUCCESS
+    ws = zo.ggml_q8_0_unpack(packed, N, K)[1]
+    p2 = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32,
+                 src_scale=capi.quant(ss.ctypes.data, capi.DT_F32, (M, G)),
+                 wei_scale=capi.quant(ws.ctypes.data, capi.DT_BF16, (G, N)))
+    st, want, _, _ = zo.matmul_int8(A, rows, p2, M, N, K, transB=True, ldb=K)
+    assert st == capi.SUCCESS
+    assert np.array_equal(got, want)
+    # and it is the dequantised product to the scales' accuracy
+    wf = zo.bf16_to_f32(ws)                                             # [G, N]
+    full = np.einsum("mgk,ngk,mg,gn->mn", A.reshape(M, G, 32).astype(np.float64), rows.reshape(N, G, 32).astype(np.float64),
+                     ss.astype(np.float64), wf.astype(np.float64))
+    assert np.allclose(got, full, rtol=1e-5, atol=1e-5)
+    # transB = false is refused (the packed layout is N x K)
+    st, _, _, _ = zo.matmul_int8(A, packed, p, M, N, K, transB=False, ldb=K)
+    assert st == capi.FAILURE
+
+
 # ------------------------------------------------------------- post-ops
 def test_eltwise_against_libm_double(zo):
     xs = np.concatenate([np.linspace(-12, 12, 4001), [0.0, -0.0, 1e-6, -1e-6, 30.0, -30.0]]).astype(np.float32)

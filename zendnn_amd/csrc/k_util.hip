@@ -66,3 +66,35 @@ hipError_t zmi_launch_repack_frag(const void *src, int64_t M, int64_t K, int64_t
                      (const int8_t *)src, M, K, ld_src, trans, is_u8, dst, k_pad);
   return hipGetLastError();
 }
+
+// ---- GGML Q8_0 weights -> s8 rows [N, K] + bf16 scales {K / 32, N} ---------------------------------
+// Reference: ggml_unpack_weight_buffer, Q8_0 branch
+// (zendnnl/src/lowoha_operators/matmul/ggml_weight_unpack.cpp:190-236): the packed buffer is
+// N * (K / 32) blocks of { fp16 d; int8 qs[32] } (34 bytes, row-major over [N][K / 32]); the int8 values are
+// copied as they are and the scale of block (n, g) goes to scales[g * N + n], converted fp16 -> f32 -> bf16
+// (round to nearest even, NaN quieted; :66-73) -- unpack_ggml_weights_and_cache asks for bf16 scales (:412-420).
+__global__ __launch_bounds__(256) void zmi_ggml_q8_0_unpack_kernel(const uint8_t *blocks, int64_t N, int64_t K,
+                                                                   int8_t *rows, uint16_t *scales) {
+  const int64_t ng = K / 32;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // block index n * ng + g
+  if (i >= N * ng) return;
+  const int64_t n = i / ng, g = i % ng;
+  const uint16_t *b = (const uint16_t *)(blocks + i * 34);     // 34-byte blocks: 2-byte aligned
+  const uint16_t hb = b[0];
+  const float d = (float)__builtin_bit_cast(_Float16, hb);   // exact (fp16 subnormals included)
+  const uint32_t u = __float_as_uint(d);
+  scales[g * N + n] = (u & 0x7fffffffu) > 0x7f800000u ? (uint16_t)((u >> 16) | 64u)
+                                                       : (uint16_t)((u + (0x7fffu + ((u >> 16) & 1u))) >> 16);
+  uint16_t *dst = (uint16_t *)(rows + n * K + g * 32);         // K % 32 == 0: even offsets
+#pragma unroll
+  for (int j = 0; j < 16; ++j) dst[j] = b[1 + j];
+}
+
+hipError_t zmi_launch_ggml_q8_0_unpack(const void *blocks, int64_t N, int64_t K, int8_t *rows, uint16_t *scales,
+                                       hipStream_t stream) {
+  if (N <= 0 || K <= 0 || K % 32 != 0) return hipErrorInvalidValue;
+  const int64_t nb = N * (K / 32);
+  hipLaunchKernelGGL(zmi_ggml_q8_0_unpack_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, stream,
+                     (const uint8_t *)blocks, N, K, rows, scales);
+  return hipGetLastError();
+}

@@ -36,11 +36,12 @@ int32_t validate_matmul(const void *src, const void *weight, const void *dst, in
         return ZMI_FAILURE;
       }
       const int64_t wn = p.wei_scale.buff ? nelems(p.wei_scale) : 0;
-      if (per_token && wn != N) {
+      if (per_token && p.pack_format_b != 1 && wn != N) {
         set_error("per-token source scale requires a per-channel weight scale of N elements");
         return ZMI_FAILURE;
       }
-      if (per_group && wn != (n / M) * N) {
+      // (GGML-packed weights carry their per-group scales inside the packed buffer: lowoha_matmul_utils.cpp:276-283)
+      if (per_group && p.pack_format_b != 1 && wn != (n / M) * N) {
         set_error("per-group source scale requires a per-group weight scale");
         return ZMI_FAILURE;
       }
@@ -362,7 +363,15 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (p.dt_wei != ZMI_DT_S8) { set_error("only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
   if (layout != 'r' && layout != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
   if (Batch_A != 1 || Batch_B != 1) { set_error("batched matmul is not implemented"); return ZMI_UNIMPLEMENTED; }
-  if (p.pack_format_b != 0) { set_error("GGML-packed weights are not implemented"); return ZMI_UNIMPLEMENTED; }
+  const bool ggml = p.pack_format_b == 1;
+  if (p.pack_format_b != 0 && !ggml) { set_error("unknown pack_format_b"); return ZMI_FAILURE; }
+  if (ggml) {
+    // reference: validate_ggml_packed_inputs, matmul/ggml_weight_unpack.cpp:155-183
+    if (!is_weights_const) { set_error("GGML packed weights require constant weights"); return ZMI_FAILURE; }
+    if (!transB) { set_error("GGML packed weights require transB = true (the packed layout is N x K)"); return ZMI_FAILURE; }
+    if (K % 32 != 0) { set_error("GGML packed weights: K must be a multiple of 32"); return ZMI_FAILURE; }
+    if (p.mem_format_b == 'r') { set_error("GGML packed weights are unpacked and reordered by the library (mem_format_b must be 'n')"); return ZMI_FAILURE; }
+  }
   if (p.mem_format_b == 'r' && p.lowoha_algo != ZMI_ALGO_AOCL_DLP_BLOCKED) {
     // contract of the reference: prepacked weights require the blocked algo
     set_error("mem_format_b == 'r' requires lowoha_algo == aocl_dlp_blocked");
@@ -396,12 +405,27 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     const int64_t n = nelems(p.src_scale);
     if (n > M && n % M == 0) pg_groups = n / M;
   }
+  if (ggml) {
+    // reference: ggml_is_sym_quant (ggml_weight_unpack.cpp:142-153), checked after the source was quantized:
+    // s8 (or dynamically quantized) source, symmetric, more than one source scale, f32 / bf16 destination
+    const bool src_ok = dyn || p.dt_src == ZMI_DT_S8;
+    const int64_t sn = dyn ? dyn_scale_n : (p.src_scale.buff ? nelems(p.src_scale) : 0);
+    if (!src_ok || p.src_zp.buff || sn <= 1 || !(p.dt_dst == ZMI_DT_F32 || p.dt_dst == ZMI_DT_BF16)) {
+      set_error("GGML packed weights are supported only for symmetric per-group int8 matmul");
+      return ZMI_FAILURE;
+    }
+    if (pg_groups != K / 32) {
+      // (the packed scales are one per 32 k: the source scales must be {M, K / 32})
+      set_error("GGML packed weights: source scale dims must be {M, K / 32}");
+      return pg_groups ? ZMI_FAILURE : ZMI_UNIMPLEMENTED;
+    }
+  }
   if (pg_groups) {
     if (K % pg_groups != 0) { set_error("per-group source scale: K must be divisible by the number of groups"); return ZMI_FAILURE; }
     if (p.src_zp.buff) { set_error("per-group source scales are symmetric: no source zero-point"); return ZMI_FAILURE; }
     if (p.dt_src == ZMI_DT_U8) { set_error("per-group source scales need an s8 / bf16 / f32 source"); return ZMI_FAILURE; }
     if (p.dt_dst != ZMI_DT_F32 && p.dt_dst != ZMI_DT_BF16) { set_error("per-group source scales need an f32 / bf16 destination"); return ZMI_FAILURE; }
-    if (!p.wei_scale.buff || nelems(p.wei_scale) != pg_groups * N) {
+    if (!ggml && (!p.wei_scale.buff || nelems(p.wei_scale) != pg_groups * N)) {
       set_error("per-group source scale requires a per-group weight scale of G * N elements");
       return ZMI_FAILURE;
     }
@@ -413,9 +437,9 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (!ensure_device()) return ZMI_FAILURE;
 
   // ---- scratch plan ----
-  const bool use_cache = p.mem_format_b != 'r' && is_weights_const &&
+  const bool use_cache = !ggml && p.mem_format_b != 'r' && is_weights_const &&
                          std::min(weight_cache_env(), p.weight_cache_type) > 0;
-  const bool pack_in_arena = p.mem_format_b != 'r' && !use_cache;
+  const bool pack_in_arena = !ggml && p.mem_format_b != 'r' && !use_cache;
   const int64_t K16 = zmi_round_up(K, 16);
   const bool ring = !pg_groups && use_ring_kernel(M, N, K);
   const int64_t frag_kpad = ring ? zmi_blob_kpad(K) : 0;
@@ -434,7 +458,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
 
   // ---- weights ----
   const uint8_t *blob;
-  if (p.mem_format_b == 'r') {
+  const void *ggml_scales = nullptr;
+  if (ggml) {
+    blob = packed_ggml_q8_0(weight, K, N, &ggml_scales);
+    if (!blob) return ZMI_FAILURE;
+  } else if (p.mem_format_b == 'r') {
     if (!blob_matches(weight, K, N)) return ZMI_FAILURE;
     blob = (const uint8_t *)weight;
   } else {
@@ -445,6 +473,12 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
 
   // ---- source ----
   zmi_matmul_params_t ep = p;   // working copy: the caller's struct is never modified
+  if (ggml) {
+    // the unpack sets the weight scales: bf16, {K / 32, N} (ggml_weight_unpack.cpp:412-420)
+    ep.wei_scale.buff = ggml_scales;
+    ep.wei_scale.dt = ZMI_DT_BF16;
+    ep.wei_scale.ndims = 2; ep.wei_scale.dims[0] = K / 32; ep.wei_scale.dims[1] = N;
+  }
   ZmiProblem prob;
   std::memset(&prob, 0, sizeof(prob));
   prob.blob = blob;

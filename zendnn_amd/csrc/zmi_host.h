@@ -69,6 +69,8 @@ bool scalar_param_s32(const void *buff, int32_t dt, int32_t *value, const int32_
 // been reserved by the caller with blob_bytes).
 const uint8_t *packed_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB,
                               int32_t src_dtype, bool use_cache, void *arena_slot);
+// GGML Q8_0 packed weights [N][K/32] blocks: cached blob + bf16 scales {K/32, N} (null on failure)
+const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const void **scales);
 void clear_weight_cache();
 
 // Checks (once per pointer) that a caller-supplied blob carries the header of a

@@ -288,6 +288,42 @@ const uint8_t *packed_weights(const void *weight, int64_t K, int64_t N, int64_t 
   return (const uint8_t *)blob;
 }
 
+// GGML Q8_0 weights: unpacked and prepacked once per weight pointer (reference: unpack_ggml_weights_and_cache,
+// matmul/ggml_weight_unpack.cpp:367-480: cache keyed by pointer, K, N, ldb, trans; the cached buffer holds the
+// reordered weights followed by the bf16 scales).  One device allocation: blob, then the {K/32, N} scales.
+const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const void **scales) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  CacheKey key{weight, K, N, /*ldb (marks the packed format)*/ -34, true};
+  const size_t blob_bytes = (size_t)zmi_round_up(zmi_blob_bytes(K, N), 256);
+  auto it = g_cache.find(key);
+  if (it != g_cache.end()) {
+    g_lru.splice(g_lru.begin(), g_lru, it->second.lru);
+    *scales = it->second.blob + blob_bytes;
+    return it->second.blob;
+  }
+  void *buf = nullptr, *rows = nullptr;
+  if (!hip_ok(hipMalloc(&buf, blob_bytes + (size_t)(K / 32) * N * 2), "hipMalloc(GGML weights)")) return nullptr;
+  if (!hip_ok(hipMalloc(&rows, (size_t)N * K), "hipMalloc(GGML unpack)")) { (void)hipFree(buf); return nullptr; }
+  bool ok = hip_ok(zmi_launch_ggml_q8_0_unpack(weight, N, K, (int8_t *)rows, (uint16_t *)((uint8_t *)buf + blob_bytes),
+                                               stream()), "GGML unpack launch") &&
+            hip_ok(zmi_launch_prepack((const int8_t *)rows, K, N, K, /*transposed*/ 1, ZMI_DT_S8, 0, (uint8_t *)buf,
+                                      stream()), "prepack launch") &&
+            hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize");   // the unpacked rows are freed next
+  (void)hipFree(rows);
+  if (!ok) { (void)hipFree(buf); return nullptr; }
+  g_lru.push_front(key);
+  g_cache[key] = CacheVal{(uint8_t *)buf, g_lru.begin()};
+  while (g_cache.size() > cache_capacity()) {
+    (void)hipDeviceSynchronize();
+    CacheKey old = g_lru.back();
+    g_lru.pop_back();
+    (void)hipFree(g_cache[old].blob);
+    g_cache.erase(old);
+  }
+  *scales = (uint8_t *)buf + blob_bytes;
+  return (const uint8_t *)buf;
+}
+
 void clear_weight_cache() {
   std::lock_guard<std::mutex> lk(g_mu);
   if (!g_cache.empty()) (void)hipDeviceSynchronize();

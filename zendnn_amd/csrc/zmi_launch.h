@@ -144,6 +144,9 @@ hipError_t zmi_launch_moe_build_problems(ZmiMoeTables tb, int E, int H, int I, c
 // k_util.hip
 hipError_t zmi_launch_pad_rows(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans,
                                int8_t *dst, int64_t ld_dst, hipStream_t stream);
+// GGML Q8_0 blocks ([N][K/32] x {fp16 d, int8 qs[32]}) -> s8 rows [N, K] and bf16 scales {K/32, N}
+hipError_t zmi_launch_ggml_q8_0_unpack(const void *blocks, int64_t N, int64_t K, int8_t *rows, uint16_t *scales,
+                                       hipStream_t stream);
 // u8 / s8 rows (or their transpose) -> fragment-major s8; u8 values are shifted by -128
 hipError_t zmi_launch_repack_frag(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans, int is_u8,
                                   int8_t *dst, hipStream_t stream);
