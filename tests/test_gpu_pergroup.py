@@ -25,7 +25,9 @@ SHAPES = [(1, 128, 32, 2), (5, 256, 33, 4), (16, 4096, 512, 32), (16, 1024, 100,
           # up to 16 rows with K = 512 .. 4096 and whole groups per eighth of K: the decode-shaped kernel, every
           # (chunks, groups) per wavefront pair it is built for
           (16, 4096, 40, 64), (9, 4096, 33, 16), (2, 4096, 64, 8), (16, 2048, 96, 32), (5, 2048, 32, 16),
-          (1, 2048, 70, 8), (16, 1024, 64, 16), (3, 1024, 31, 8), (12, 512, 50, 8)]
+          (1, 2048, 70, 8), (16, 1024, 64, 16), (3, 1024, 31, 8), (12, 512, 50, 8),
+          # groups of 32 on it (two per chunk, 16 integer tiles per round)
+          (16, 4096, 64, 128), (7, 2048, 40, 64), (16, 1024, 33, 32), (2, 512, 96, 16)]
 
 
 @pytest.mark.parametrize("M,K,N,G", SHAPES)
@@ -117,6 +119,7 @@ def test_static_per_group_alpha_beta(zo):
 
 
 @pytest.mark.parametrize("M,K,N,G", [(16, 4096, 14336, 32), (4, 4096, 1024, 64), (1, 512, 64, 8), (33, 256, 40, 16),
+                                     (16, 4096, 320, 128), (9, 1024, 64, 32),
                                      (150, 1024, 96, 8)])
 @pytest.mark.parametrize("src_dt", [capi.DT_BF16, capi.DT_F32])
 def test_dynamic_per_group(zo, M, K, N, G, src_dt):

@@ -232,8 +232,8 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
 // crosses them is INTEGER: every wavefront keeps one accumulator per group of its slice (GPW whole groups
 // in CPW chunks of 64 k), the G = 8 GPW integer tiles meet in LDS, and one thread per output element then
 // adds float(acc_g) * ss[m, g] * ws[g, n] in group order -- the reference's additions, in its order, with
-// the weight stream of the per-token kernel.  Needs K a multiple of 512, whole groups per wavefront,
-// G <= 64 (2 KiB of LDS per group).
+// the weight stream of the per-token kernel.  Needs K = 512 * CPW (CPW in 1, 2, 4, 8) and whole groups of
+// 64 .. 512 k per wavefront slice, or groups of 32 k (two per chunk); 16 tiles of 2 KiB meet in LDS at a time.
 #define PGD_WAVES 8
 #define PGD_THREADS (PGD_WAVES * 64)
 
@@ -245,12 +245,18 @@ template <int CPW, int GPW>
 __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(ZmiProblem p, ZmiEpilogue epi,
                                                                                ZmiFusedQuant fq) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  constexpr int CPG = CPW / GPW;                 // chunks per group
+  constexpr int SUB = GPW > CPW ? GPW / CPW : 1;  // groups per chunk (2: groups of 32 k)
+  constexpr int CPG = GPW > CPW ? 1 : CPW / GPW;  // chunks per group
   constexpr int G = PGD_WAVES * GPW;
-  constexpr int NCH = PGD_WAVES * CPW;           // K / 64
-  constexpr int MAIN = NCH * 1024 > G * 2048 ? NCH * 1024 : G * 2048;   // operand area, reused by the integer tiles
-  float *ws_l = reinterpret_cast<float *>(lds + MAIN);                  // [G][32]
-  float *ss_l = ws_l + G * 32;                                          // [16][G]
+  constexpr int RT = G <= 32 ? G : 16;            // integer tiles (groups) that meet in LDS per round
+  constexpr int WPR = RT / GPW;                   // wavefronts whose tiles make one round
+  // LDS: the operand area (K * 16 bytes), which holds RT tiles of 2 KiB once the MFMAs are done; behind both,
+  // the scales: [G][32] weight scales, [16][G] source scales.  (They are parked there as soon as the weight
+  // requests are out: parking them only after the MFMAs, inside the freed operand area, cost 4 us -- their
+  // requests end up next to the parking, a full memory latency after the last weight byte.)
+  constexpr int MAIN = PGD_WAVES * CPW * 1024 > RT * 2048 ? PGD_WAVES * CPW * 1024 : RT * 2048;
+  float *ws_l = reinterpret_cast<float *>(lds + MAIN);
+  float *ss_l = ws_l + G * 32;
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int M = p.M, N = p.N, K = p.K;
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
       b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(c_begin + u) * 2048);
     }
   }
-  // (the scales requested ahead of the weights are parked in LDS only now, so nothing waited for them)
+  // scales -> LDS
 #pragma unroll
   for (int i = 0; i < WS_PT; ++i)
     if (tid + i * PGD_THREADS < G * 32) ws_l[tid + i * PGD_THREADS] = ws_r[i];
@@ -357,36 +363,54 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   for (int gi = 0; gi < GPW; ++gi) {
     acc[gi][0] = (v4i){0, 0, 0, 0};
     acc[gi][1] = (v4i){0, 0, 0, 0};
+    if (SUB == 1) {
 #pragma unroll
-    for (int u = gi * CPG; u < (gi + 1) * CPG; ++u) {
-      const v4i a = *(const v4i *)(lds + pgd_lds_off(c_begin + u, g4, c16));
+      for (int u = gi * CPG; u < (gi + 1) * CPG; ++u) {
+        const v4i a = *(const v4i *)(lds + pgd_lds_off(c_begin + u, g4, c16));
+        acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[gi][0], 0, 0, 0);
+        acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[gi][1], 0, 0, 0);
+      }
+    } else {
+      // two groups share a chunk: the chunk is multiplied once per group with the other group's lanes
+      // (k groups of 16) of the row operand zeroed
+      const int u = gi / SUB, t = gi % SUB;
+      v4i a = *(const v4i *)(lds + pgd_lds_off(c_begin + u, g4, c16));
+      if (g4 / (4 / SUB) != t) a = (v4i){0, 0, 0, 0};
       acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[gi][0], 0, 0, 0);
       acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[gi][1], 0, 0, 0);
     }
   }
-  // ---- the integer tiles of all groups meet in LDS (the operand area is done with) ----
+  // ---- the operand area is done with ----
   __syncthreads();
+  // ---- RT integer tiles at a time meet in LDS, in group order; one thread per output element adds the
+  // group terms in order, each step rounded ----
   int32_t *red = (int32_t *)lds;
-#pragma unroll
-  for (int gi = 0; gi < GPW; ++gi)
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) red[(wave * GPW + gi) * 512 + (h * 4 + q) * 64 + lane] = acc[gi][h][q];
-  __syncthreads();
-  // ---- one thread per output element: the group terms in order, each step rounded ----
   const int e_row = tid / 32, e_h = (tid % 32) / 16, e_c = tid % 16;
   const int e_n = blk * 32 + e_h * 16 + e_c;
-  if (e_n >= N || e_row >= M) return;
+  const bool e_live = e_n < N && e_row < M;
   // acc[h][q] of lane l is row (l / 16) * 4 + q, column h * 16 + l % 16
   const int off = (e_h * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_c;
   float sum = 0.0f;
+  for (int r = 0; r < G / RT; ++r) {
+    if (r > 0) __syncthreads();                    // the previous round's tiles have been read
+    if (wave / WPR == r) {
+#pragma unroll
+      for (int gi = 0; gi < GPW; ++gi)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) red[((wave % WPR) * GPW + gi) * 512 + (h * 4 + q) * 64 + lane] = acc[gi][h][q];
+    }
+    __syncthreads();
 #pragma unroll 8
-  for (int g = 0; g < G; ++g) {
-    float t = __fmul_rn((float)red[g * 512 + off], ss_l[e_row * G + g]);
-    t = __fmul_rn(t, ws_l[g * 32 + e_h * 16 + e_c]);
-    sum = __fadd_rn(sum, t);
+    for (int t = 0; t < RT; ++t) {
+      const int g = r * RT + t;
+      float v = __fmul_rn((float)red[t * 512 + off], ss_l[e_row * G + g]);
+      v = __fmul_rn(v, ws_l[g * 32 + e_h * 16 + e_c]);
+      sum = __fadd_rn(sum, v);
+    }
   }
+  if (!e_live) return;
   const int64_t o = (int64_t)e_row * p.ldc + e_n;
   float y = sum;
   if (epi.alpha != 1.0f) y = __fmul_rn(y, epi.alpha);
@@ -397,8 +421,8 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
 
 template <int CPW, int GPW>
 static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq, hipStream_t stream) {
-  constexpr int G = PGD_WAVES * GPW, NCH = PGD_WAVES * CPW;
-  constexpr size_t main_bytes = NCH * 1024 > G * 2048 ? NCH * 1024 : G * 2048;
+  constexpr int G = PGD_WAVES * GPW, NCH = PGD_WAVES * CPW, RT = G <= 32 ? G : 16;
+  constexpr size_t main_bytes = (size_t)NCH * 1024 > (size_t)RT * 2048 ? (size_t)NCH * 1024 : (size_t)RT * 2048;
   constexpr size_t smem = main_bytes + (size_t)G * 32 * 4 + (size_t)16 * G * 4;
   static bool attr_done = false;
   if (!attr_done) {
@@ -415,9 +439,10 @@ static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const 
 
 // the decode-shaped kernel serves: up to 16 rows, K = 512 * CPW (CPW in 1, 2, 4, 8), whole groups per wavefront
 static bool pgd_fits(const ZmiProblem &p, int G, int *cpw, int *gpw) {
-  if (p.M > 16 || p.K % 512 != 0 || p.K > 4096 || G % PGD_WAVES != 0 || G > 64) return false;
+  if (p.M > 16 || p.K % 512 != 0 || p.K > 4096 || G % PGD_WAVES != 0) return false;
   const int c = p.K / 512, g = G / PGD_WAVES;
-  if (!(c == 1 || c == 2 || c == 4 || c == 8) || c % g != 0) return false;
+  // whole groups of 64 .. 512 k per wavefront slice, or groups of 32 (two per chunk)
+  if (!(c == 1 || c == 2 || c == 4 || c == 8) || !((g <= c && c % g == 0) || g == 2 * c)) return false;
   *cpw = c; *gpw = g;
   return true;
 }
@@ -452,6 +477,10 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
     case 2 * 16 + 2: return pgd_launch<2, 2>(p, epi, fq, stream);
     case 2 * 16 + 1: return pgd_launch<2, 1>(p, epi, fq, stream);
     case 1 * 16 + 1: return pgd_launch<1, 1>(p, epi, fq, stream);
+    case 8 * 16 + 16: return pgd_launch<8, 16>(p, epi, fq, stream);
+    case 4 * 16 + 8: return pgd_launch<4, 8>(p, epi, fq, stream);
+    case 2 * 16 + 4: return pgd_launch<2, 4>(p, epi, fq, stream);
+    case 1 * 16 + 2: return pgd_launch<1, 2>(p, epi, fq, stream);
     default: break;
     }
   }

@@ -167,7 +167,7 @@ static __device__ void zmi_fused_quant_row_groups(const ZmiFusedQuant &fq, int r
   // group maximum by lane exchanges, one 8-byte store -- a single trip to memory.
   const int es = bf16 ? 2 : 4;
   const char *rowp = (const char *)fq.x + (size_t)row * fq.ldx * es;
-  if (K % 8 == 0 && K <= (int)blockDim.x * 8 && gs >= 64 && gs <= 512 && (gs & (gs - 1)) == 0 &&
+  if (K % 8 == 0 && K <= (int)blockDim.x * 8 && gs >= 8 && gs <= 512 && (gs & (gs - 1)) == 0 &&
       ((uintptr_t)rowp % 16) == 0) {
     const int t = threadIdx.x;
     float v8[8];
@@ -193,7 +193,7 @@ static __device__ void zmi_fused_quant_row_groups(const ZmiFusedQuant &fq, int r
       const float a = fabsf(v8[j]);
       if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
     }
-    const int lpg = gs / 8;   // lanes per group: 8 .. 64
+    const int lpg = gs / 8;   // lanes per group: 1 .. 64
     #pragma unroll
     for (int o = 32; o > 0; o >>= 1)
       if (o < lpg) amax = fmaxf(amax, __shfl_xor(amax, o));
