@@ -50,6 +50,8 @@ def lib():
         L.zo_fp16_to_f32.argtypes = [C.c_uint16]
         L.zo_ggml_q8_0_unpack.restype = None
         L.zo_ggml_q8_0_unpack.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
+        L.zo_s4_to_s8.restype = None
+        L.zo_s4_to_s8.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
         L.zo_gemm_s32.restype = C.c_int64
         L.zo_gemm_s32.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
                                   C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
@@ -126,6 +128,16 @@ def ggml_q8_0_unpack(blocks, N, K):
     scales = np.empty((K // 32, N), dtype=np.uint16)
     lib().zo_ggml_q8_0_unpack(_p(blocks), N, K, _p(rows), _p(scales))
     return rows, scales
+
+
+def s4_to_s8(packed, K, N, ldb=None, transposed=False):
+    """packed: uint8 nibble pairs of a [K, ldb] (or [N, ldb] when transposed) s4 matrix -> int8 [K, N]."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    if ldb is None:
+        ldb = K if transposed else N
+    out = np.empty((K, N), dtype=np.int8)
+    lib().zo_s4_to_s8(_p(packed), K, N, ldb, int(transposed), _p(out))
+    return out
 
 
 def gemm_s32(A, B, transA=False, transB=False):

@@ -31,6 +31,8 @@
  *                                numpy float32 brute force on small random cases
  *   zo_fp16_to_f32, Q8_0 unpack  all 65536 half values against numpy float16; block layout by construction
  *                                of the packed buffer from known rows and scales (numpy), bf16 via torch
+ *   zo_s4_to_s8 (W4A8 widening)  every nibble value in both positions (known answers), numpy shift/mask
+ *                                restatement on random buffers, both orientations with padded ldb
  *   zo_quant_per_group           per-group constants (closed form), == zo_quant_per_token on the
  *                                [M*G, K/G] view
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
@@ -396,6 +398,22 @@ ZO_EXPORT void zo_ggml_q8_0_unpack(const void *blocks, int64_t N, int64_t K, int
     }
 }
 
+/* cvt_s4_to_s8 with extract_4bit_nibble, lowoha_operators/matmul/backends/aocl/aocl_kernel.cpp:33-41, 144-163:
+ * element (row, col) of the K x N weight matrix sits at physical index row * ldb + col (col * ldb + row when
+ * transposed) of a nibble array, two per byte, even index = low nibble; the nibble is sign-extended from bit 3
+ * (-8 .. 7).  The result is a contiguous row-major [K, N] s8 matrix. */
+ZO_EXPORT void zo_s4_to_s8(const void *packed, int64_t K, int64_t N, int64_t ldb, int32_t transposed, int8_t *out) {
+  const uint8_t *w = (const uint8_t *)packed;
+  for (int64_t row = 0; row < K; ++row)
+    for (int64_t col = 0; col < N; ++col) {
+      const int64_t idx = transposed ? col * ldb + row : row * ldb + col;
+      const uint8_t byte = w[idx / 2];
+      int32_t v = (idx % 2 == 0) ? (byte & 0x0F) : (byte >> 4);
+      if (v & 0x08) v -= 16;
+      out[row * N + col] = (int8_t)v;
+    }
+}
+
 /* matmul_direct for the int8 path.  Pipeline of lowoha_operators/matmul/
  * lowoha_matmul.cpp:278-510: optional dynamic per-token quantization of a
  * bf16/f32 source (matmul/quantization/reorder_quantization.cpp:43-280), then
@@ -410,16 +428,43 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
   zmi_matmul_params_t pl = *c->params;   /* working copy: the GGML unpack sets the weight scales */
   const zmi_matmul_params_t *p = &pl;
   const int64_t M = c->M, N = c->N, K = c->K;
-  if (p->dt_wei != ZMI_DT_S8) return ZMI_UNIMPLEMENTED;
+  if (p->dt_wei != ZMI_DT_S8 && p->dt_wei != ZMI_DT_S4) return ZMI_UNIMPLEMENTED;
   const void *weight = c->weight;
   int64_t ldb = c->ldb;
+  int32_t transB = c->transB;
   int8_t *ggml_rows = NULL;
   uint16_t *ggml_scales = NULL;
+  int64_t w4a8_groups = 0;
+  if (p->dt_wei == ZMI_DT_S4) {
+    /* W4A8: validate_w4a8_inputs, lowoha_operators/matmul/lowoha_matmul_utils.cpp:72-176 (bf16 source with
+     * dynamic_quant and s8 compute, bf16 destination, symmetric, {G,N} f32 / bf16 weight scales, K/G a multiple
+     * of 4, source scale dims {1,1}, {M,1} or {M,G}); anything else with s4 weights is the weight-only path,
+     * which is not restated here.  The weights are widened once to [K,N] s8
+     * (w4a8ReorderAndCacheWeightsAocl, backends/aocl/aocl_kernel.cpp:704-793). */
+    if (p->dt_src == ZMI_DT_S8) return ZMI_FAILURE;
+    if (p->dynamic_quant && (p->dt_src == ZMI_DT_F32 || p->dt_dst == ZMI_DT_F32)) return ZMI_FAILURE;
+    if (p->dt_src == ZMI_DT_U8 && (p->src_scale.buff || p->dynamic_quant)) return ZMI_FAILURE;
+    if (!(p->dynamic_quant && p->dt_src == ZMI_DT_BF16)) return ZMI_UNIMPLEMENTED;
+    if (p->dt_compute != ZMI_DT_S8 || p->dt_dst != ZMI_DT_BF16) return ZMI_FAILURE;
+    if (p->wei_zp.buff || p->src_zp.buff || !p->wei_scale.buff) return ZMI_FAILURE;
+    if (p->wei_scale.dt != ZMI_DT_F32 && p->wei_scale.dt != ZMI_DT_BF16) return ZMI_FAILURE;
+    if (p->wei_scale.ndims != 2) return ZMI_FAILURE;
+    const int64_t G = p->wei_scale.dims[0];
+    if (G <= 0 || p->wei_scale.dims[1] != N || K % G != 0 || (K / G) % 4 != 0) return ZMI_FAILURE;
+    if (p->src_scale.dt != ZMI_DT_F32 && p->src_scale.dt != ZMI_DT_BF16) return ZMI_FAILURE;
+    if (p->src_scale.ndims != 2) return ZMI_FAILURE;
+    const int64_t sr = p->src_scale.dims[0], sc = p->src_scale.dims[1];
+    if (!((sr == 1 && sc == 1) || (sr == M && sc == 1) || (sr == M && sc == G))) return ZMI_FAILURE;
+    ggml_rows = (int8_t *)malloc((size_t)N * K);
+    zo_s4_to_s8(weight, K, N, ldb, transB, ggml_rows);
+    weight = ggml_rows; ldb = N; transB = 0;
+    w4a8_groups = G;
+  }
   if (p->pack_format_b == 1) {
     /* validate_ggml_packed_inputs + unpack_ggml_weights_and_cache,
      * lowoha_operators/matmul/ggml_weight_unpack.cpp:155-183, 367-420: transB required, the unpacked
      * rows are [N, K], the scales become the bf16 {K/32, N} weight scales */
-    if (!c->transB || K % 32 != 0) return ZMI_FAILURE;
+    if (!transB || K % 32 != 0) return ZMI_FAILURE;
     ggml_rows = (int8_t *)malloc((size_t)N * K);
     ggml_scales = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(K / 32) * N);
     zo_ggml_q8_0_unpack(weight, N, K, ggml_rows, ggml_scales);
@@ -474,6 +519,16 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
       dn = 1;
     }
     if (c->scale_out) memcpy(c->scale_out, sbuf, sizeof(float) * (size_t)dn);
+    if (w4a8_groups > 1 && dn <= M) {
+      /* broadcast_w4a8_src_scale, backends/aocl/aocl_kernel.cpp:167-236: compact per-tensor / per-token
+       * scales are repeated over the G groups, and the per-group GEMM follows */
+      float *wide = (float *)malloc(sizeof(float) * (size_t)M * w4a8_groups);
+      for (int64_t m = 0; m < M; ++m)
+        for (int64_t g = 0; g < w4a8_groups; ++g) wide[m * w4a8_groups + g] = sbuf[dn == 1 ? 0 : m];
+      free(sbuf);
+      sbuf = wide;
+      dn = M * w4a8_groups;
+    }
     A = qbuf; a_dt = ZMI_DT_S8; lda = K;
     src_scale = sbuf; src_scale_n = dn; src_scale_dt = ZMI_DT_F32;
   } else if (a_dt != ZMI_DT_S8 && a_dt != ZMI_DT_U8) {
@@ -507,7 +562,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
           int32_t group_sum = 0;
           for (int64_t k = g * gs; k < (g + 1) * gs; ++k) {
             int32_t a = ((const int8_t *)A)[transA ? k * lda + m : m * lda + k];
-            group_sum += a * (int32_t)W[c->transB ? n * ldb + k : k * ldb + n];
+            group_sum += a * (int32_t)W[transB ? n * ldb + k : k * ldb + n];
           }
           float grp = (float)group_sum * zo_read_f32(src_scale, src_scale_dt, m * G + g);
           grp *= zo_read_f32(p->wei_scale.buff, p->wei_scale.dt, g * N + n);
@@ -540,7 +595,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
     int8_t *Bt = (int8_t *)weight;
     int64_t ldbt = ldb;
     int8_t *tmp = NULL;
-    if (!c->transB) {
+    if (!transB) {
       tmp = (int8_t *)malloc((size_t)N * K);
       zo_transpose_s8((const int8_t *)weight, K, N, ldb, tmp);
       Bt = tmp; ldbt = K;
@@ -548,7 +603,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
     zo_gemm_s32_bt(A, a_dt, lda, Bt, ldbt, M, N, K, acc, N);
     free(tmp);
   } else {
-    zo_gemm_s32(A, a_dt, transA, lda, (const int8_t *)weight, c->transB, ldb, M, N, K, acc, N);
+    zo_gemm_s32(A, a_dt, transA, lda, (const int8_t *)weight, transB, ldb, M, N, K, acc, N);
   }
   if (c->acc_out) memcpy(c->acc_out, acc, sizeof(int32_t) * (size_t)M * N);
 
@@ -556,7 +611,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
   int32_t *comp = NULL;
   if (src_zp) {
     comp = (int32_t *)malloc(sizeof(int32_t) * (size_t)N);
-    zo_zp_comp((const int8_t *)weight, c->transB, ldb, K, N, src_zp, comp);
+    zo_zp_comp((const int8_t *)weight, transB, ldb, K, N, src_zp, comp);
   }
   const int per_token = (src_scale_n == M && M > 1);
   const int64_t wei_scale_n = p->wei_scale.buff ? zo_nelems(&p->wei_scale) : 0;

@@ -1,0 +1,131 @@
+"""GPU parity of matmul_direct for W4A8: bf16 rows quantized at run time to s8 (one scale per tensor, per row or
+per (row, group)), packed s4 weights with {G, N} scales, bf16 out.  The library widens the s4 codes to s8, reorders
+and caches them per weight pointer, repeats compact source scales over the groups and runs the per-group symmetric
+GEMM (reference: lowoha_operators/matmul/lowoha_matmul_utils.cpp:72-176 for the contract,
+matmul/backends/aocl/aocl_kernel.cpp:144-236, 704-793 for the widening, the scale broadcast and the cache)."""
+import numpy as np
+import pytest
+import torch
+
+from zendnn_amd import capi, lowoha
+from tests import gpu_helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _s4_pack(codes, ld):
+    R, C = codes.shape
+    full = np.full((R, ld), 5, dtype=np.int64)
+    full[:, :C] = codes
+    flat = full.reshape(-1) & 15
+    if flat.size % 2:
+        flat = np.append(flat, 0)
+    return (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)
+
+
+def _case(rng, M, K, N, G, transB, pad=0):
+    x = H.bf16_bits((rng.standard_normal((M, K)) * 2).astype(np.float32))
+    w = rng.integers(-8, 8, (K, N), dtype=np.int8)
+    ldb = (K if transB else N) + pad
+    packed = _s4_pack(w.T.copy(), ldb) if transB else _s4_pack(w, ldb)
+    ws = rng.uniform(0.01, 0.1, (G, N)).astype(np.float32)
+    return x, packed, ldb, ws
+
+
+def _run(zo, M, K, N, G, sdims, *, transB=False, const=True, postop=None, bias=False, ws_bf16=False, pad=0, calls=1,
+         want_kernel=None):
+    rng = np.random.default_rng(M * 7 + K + N * 3 + G)
+    x, packed, ldb, ws = _case(rng, M, K, N, G, transB, pad)
+    if ws_bf16:
+        ws_h = H.bf16_bits(ws)
+        ws_dt = capi.DT_BF16
+    else:
+        ws_h, ws_dt = ws, capi.DT_F32
+    b = rng.standard_normal(N).astype(np.float32) if bias else None
+    n_sc = int(np.prod(sdims))
+    x_d, w_d, ws_d = H.to_dev(x), H.to_dev(packed), H.to_dev(ws_h)
+    sc_d = torch.zeros(n_sc, dtype=torch.float32, device=H.DEV)
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S4, dst=capi.DT_BF16, compute=capi.DT_S8,
+                            bias=capi.DT_F32 if bias else capi.DT_NONE)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(sc_d, capi.DT_F32, sdims)
+    p.wei_scale = lowoha.QuantParam(ws_d, ws_dt, (G, N))
+    if postop is not None:
+        p.postop_ = [lowoha.PostOp(postop)]
+    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+    b_d = H.to_dev(b) if bias else None
+    for _ in range(calls):                       # a second call finds the widened weights in the cache
+        dst.zero_()
+        st = lowoha.matmul_direct("r", False, transB, M, N, K, 1.0, x_d, K, w_d, ldb, b_d, 0.0, dst, N, const, p)
+        assert st == capi.SUCCESS, lowoha.last_error()
+        if want_kernel:
+            assert lowoha.last_kernel().startswith(want_kernel), lowoha.last_kernel()
+    ph = H.host_params(p, src_scale=None, wei_scale=ws_h)
+    keep = []
+    st, want, _, scales = zo.matmul_int8(x, packed, ph.flat(keep), M, N, K, bias=b, transB=transB, ldb=ldb,
+                                         want_scales=True, n_scales=max(n_sc, M))
+    assert st == capi.SUCCESS
+    assert np.array_equal(H.to_host(sc_d), scales[:n_sc])
+    if postop is None:
+        assert np.array_equal(H.to_host(dst), want)     # every step is a correctly rounded f32 operation
+    else:
+        H.check_bf16(H.to_host(dst), want, max_frac=1e-2)
+    capi.load().zmi_clear_weight_cache()
+
+
+@pytest.mark.parametrize("M,K,N,G", [(16, 4096, 512, 32), (4, 4096, 14336, 32), (1, 4096, 96, 128), (16, 1024, 100, 16),
+                                     (5, 256, 33, 4), (40, 512, 70, 8), (130, 1024, 48, 32), (3, 128, 16, 8)])
+@pytest.mark.parametrize("kind", ["tensor", "token", "group"])
+def test_w4a8_scale_granularities(zo, M, K, N, G, kind):
+    sdims = {"tensor": (1, 1), "token": (M, 1), "group": (M, G)}[kind]
+    _run(zo, M, K, N, G, sdims, want_kernel="pergroup_", calls=2)
+
+
+@pytest.mark.parametrize("transB", [False, True])
+@pytest.mark.parametrize("const", [False, True])
+def test_w4a8_orientations_padding_and_uncached_weights(zo, transB, const):
+    _run(zo, 7, 512, 45, 8, (7, 1), transB=transB, const=const, pad=3 if transB else 1, bias=True)
+    _run(zo, 16, 2048, 64, 16, (16, 16), transB=transB, const=const, bias=True, ws_bf16=True)
+
+
+@pytest.mark.parametrize("postop", [capi.PO_SWISH, capi.PO_GELU_TANH, capi.PO_RELU])
+def test_w4a8_post_ops(zo, postop):
+    _run(zo, 16, 4096, 320, 32, (16, 1), postop=postop, bias=True)
+    _run(zo, 9, 1024, 64, 32, (9, 32), postop=postop)
+
+
+def test_w4a8_one_group_is_the_per_channel_chain(zo):
+    # G = 1: {1, N} weight scales, the plain per-token chain on the widened weights
+    _run(zo, 8, 512, 64, 1, (8, 1))
+    _run(zo, 200, 256, 300, 1, (200, 1))
+
+
+def test_w4a8_rejections(zo):
+    M, K, N, G = 4, 64, 8, 2
+    x_d = H.to_dev(np.zeros((M, K), dtype=np.uint16))
+    w_d = H.to_dev(np.zeros(K * N // 2, dtype=np.uint8))
+    ws_d = torch.ones(G * N, dtype=torch.float32, device=H.DEV)
+
+    def call(src=capi.DT_BF16, dst_dt=capi.DT_BF16, compute=capi.DT_S8, dyn=True, sdims=(M, 1), wdims=(G, N), fmt="n"):
+        p = lowoha.MatmulParams(src=src, wei=capi.DT_S4, dst=dst_dt, compute=compute)
+        p.dynamic_quant = dyn
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, sdims)
+        p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, wdims)
+        p.mem_format_b = fmt
+        if fmt == "r":
+            p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        dst = torch.zeros((M, N), dtype=torch.bfloat16 if dst_dt == capi.DT_BF16 else torch.float32, device=H.DEV)
+        return lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, w_d, N, None, 0.0, dst, N, True, p)
+
+    assert call() == capi.SUCCESS
+    assert call(src=capi.DT_S8) == capi.FAILURE
+    assert call(src=capi.DT_F32) == capi.FAILURE
+    assert call(dst_dt=capi.DT_F32) == capi.FAILURE
+    assert call(compute=capi.DT_BF16) == capi.FAILURE
+    assert call(dyn=False) == capi.UNIMPLEMENTED           # weight-only quantization is another path
+    assert call(sdims=(M, 3)) == capi.FAILURE
+    assert call(wdims=(G, N - 1)) == capi.FAILURE
+    assert call(wdims=(3, N)) == capi.FAILURE
+    assert call(wdims=(32, N)) == capi.FAILURE             # groups of 2
+    assert call(fmt="r") == capi.FAILURE                   # no prepacked form of s4 weights
+    capi.load().zmi_clear_weight_cache()

@@ -449,6 +449,97 @@ def test_ggml_matmul_is_the_per_group_matmul_on_the_unpacked_weights(zo):
     assert st == capi.FAILURE
 
 
+# ------------------------------------------------------------- W4A8 (s4 weights)
+def _s4_pack(codes, ld):
+    """codes int8 [R, C] in -8..7 -> packed nibbles of a [R, ld] matrix (pad columns hold 5): element i of the
+    flattened matrix is the low nibble of byte i // 2 when i is even, else the high nibble."""
+    R, C = codes.shape
+    full = np.full((R, ld), 5, dtype=np.int64)
+    full[:, :C] = codes
+    flat = full.reshape(-1) & 15
+    if flat.size % 2:
+        flat = np.append(flat, 0)
+    return (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)
+
+
+def test_s4_widening_known_answers_and_numpy_restatement(zo):
+    # every code in both nibble positions: byte (hi << 4 | lo) -> [lo, hi], sign-extended from bit 3
+    for lo in range(16):
+        for hi in range(16):
+            got = zo.s4_to_s8(np.array([(hi << 4) | lo], dtype=np.uint8), 1, 2)
+            assert got.tolist() == [[lo - 16 if lo >= 8 else lo, hi - 16 if hi >= 8 else hi]]
+    assert zo.s4_to_s8(np.array([0x87, 0xF0, 0x1E], dtype=np.uint8), 2, 3).tolist() == [[7, -8, 0], [-1, -2, 1]]
+    # random matrices, both orientations, padded (odd) leading dimension: the layout by construction
+    rng = np.random.default_rng(41)
+    for K, N, pad in [(8, 6, 0), (12, 5, 3), (7, 9, 1)]:
+        w = rng.integers(-8, 8, (K, N), dtype=np.int8)
+        assert np.array_equal(zo.s4_to_s8(_s4_pack(w, N + pad), K, N, ldb=N + pad), w)
+        assert np.array_equal(zo.s4_to_s8(_s4_pack(w.T.copy(), K + pad), K, N, ldb=K + pad, transposed=True), w)
+
+
+@pytest.mark.parametrize("scale_dims", ["tensor", "token", "group"])
+@pytest.mark.parametrize("transB", [False, True])
+def test_w4a8_is_the_per_group_matmul_on_the_widened_weights(zo, scale_dims, transB):
+    rng = np.random.default_rng(42)
+    M, K, N, G = 5, 128, 10, 4
+    x = zo.f32_to_bf16((rng.standard_normal((M, K)) * 3).astype(np.float32))
+    w = rng.integers(-8, 8, (K, N), dtype=np.int8)
+    packed = _s4_pack(w.T.copy(), K) if transB else _s4_pack(w, N)
+    ws = rng.uniform(0.01, 0.1, (G, N)).astype(np.float32)
+    dims = {"tensor": (1, 1), "token": (M, 1), "group": (M, G)}[scale_dims]
+    p = _params(dt_src=capi.DT_BF16, dt_wei=capi.DT_S4, dt_dst=capi.DT_BF16, dt_compute=capi.DT_S8, dynamic_quant=1,
+                src_scale=capi.quant(None, capi.DT_F32, dims),
+                wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, (G, N)))
+    st, got, _, scales = zo.matmul_int8(x, packed, p, M, N, K, transB=transB, ldb=K if transB else N,
+                                        want_scales=True, n_scales=M * G)
+    assert st == capi.SUCCESS
+    # the same source quantization as the s8-weight path, its scales repeated over the groups, then the per-group GEMM
+    if scale_dims == "group":
+        q, s = zo.quant_per_group(x, capi.DT_BF16, G)
+    elif scale_dims == "token":
+        q, s1 = zo.quant_per_token(x, capi.DT_BF16)
+        s = np.repeat(s1.reshape(M, 1), G, axis=1)
+    else:
+        xf = zo.bf16_to_f32(x)
+        s0 = np.float32(np.abs(xf).max()) / np.float32(127.0)
+        q = np.rint(xf / s0).astype(np.int8)
+        s = np.full((M, G), s0, dtype=np.float32)
+    s = np.ascontiguousarray(s, dtype=np.float32)
+    p2 = _params(dt_src=capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_BF16,
+                 src_scale=capi.quant(s.ctypes.data, capi.DT_F32, (M, G)),
+                 wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, (G, N)))
+    st, want, _, _ = zo.matmul_int8(q, w, p2, M, N, K)
+    assert st == capi.SUCCESS
+    assert np.array_equal(got, want)
+    # and it is the dequantised product to the quantization's accuracy
+    full = zo.bf16_to_f32(x).astype(np.float64) @ (w.astype(np.float64) * np.repeat(ws, K // G, axis=0))
+    assert np.abs(zo.bf16_to_f32(got) - full).max() < 0.03 * np.abs(full).max()
+
+
+def test_w4a8_rejections_follow_the_reference_validator(zo):
+    M, K, N, G = 4, 64, 8, 2
+    x = np.zeros((M, K), dtype=np.uint16)
+    packed = np.zeros(K * N // 2, dtype=np.uint8)
+    ws = np.ones((G, N), dtype=np.float32)
+
+    def call(src=capi.DT_BF16, dst=capi.DT_BF16, compute=capi.DT_S8, dyn=1, sdims=(M, 1), wdims=(G, N), K_=K):
+        p = _params(dt_src=src, dt_wei=capi.DT_S4, dt_dst=dst, dt_compute=compute, dynamic_quant=dyn,
+                    src_scale=capi.quant(None, capi.DT_F32, sdims),
+                    wei_scale=capi.quant(ws.ctypes.data, capi.DT_F32, wdims))
+        return zo.matmul_int8(x, packed, p, M, N, K_)[0]
+
+    assert call() == capi.SUCCESS
+    assert call(src=capi.DT_S8) == capi.FAILURE                 # pre-quantized sources are not W4A8
+    assert call(src=capi.DT_F32) == capi.FAILURE
+    assert call(dst=capi.DT_F32) == capi.FAILURE
+    assert call(compute=capi.DT_BF16) == capi.FAILURE
+    assert call(dyn=0) == capi.UNIMPLEMENTED                    # weight-only quantization: another path
+    assert call(sdims=(M, 3)) == capi.FAILURE
+    assert call(wdims=(G, N - 1)) == capi.FAILURE
+    assert call(wdims=(3, N)) == capi.FAILURE                   # K not divisible by G
+    assert call(wdims=(32, N)) == capi.FAILURE                  # groups of 2: not a multiple of 4
+
+
 # ------------------------------------------------------------- post-ops
 def test_eltwise_against_libm_double(zo):
     xs = np.concatenate([np.linspace(-12, 12, 4001), [0.0, -0.0, 1e-6, -1e-6, 30.0, -30.0]]).astype(np.float32)

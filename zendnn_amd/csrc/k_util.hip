@@ -98,3 +98,47 @@ hipError_t zmi_launch_ggml_q8_0_unpack(const void *blocks, int64_t N, int64_t K,
                      (const uint8_t *)blocks, N, K, rows, scales);
   return hipGetLastError();
 }
+
+// ---- packed s4 weights -> s8, same orientation ------------------------------------------------------
+// Reference: cvt_s4_to_s8 with extract_4bit_nibble
+// (zendnnl/src/lowoha_operators/matmul/backends/aocl/aocl_kernel.cpp:33-41, 144-163): nibble i of the packed
+// buffer (two per byte, even index = low nibble) is element i of a [rows, ld] matrix of 4-bit codes,
+// sign-extended from bit 3.  The orientation is kept (rows x cols out of rows x ld), so consecutive threads
+// read consecutive nibbles whichever way the weights lie; the prepack kernel transposes if it has to.
+__global__ __launch_bounds__(256) void zmi_s4_widen_kernel(const uint8_t *packed, int64_t rows, int64_t cols, int64_t ld,
+                                                           int8_t *out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // output element r * cols + c
+  if (i >= rows * cols) return;
+  const int64_t r = i / cols, c = i % cols;
+  const int64_t idx = r * ld + c;
+  const uint32_t byte = packed[idx >> 1];
+  const int32_t nib = (idx & 1) ? (int32_t)(byte >> 4) : (int32_t)(byte & 15u);
+  out[i] = (int8_t)((nib ^ 8) - 8);
+}
+
+hipError_t zmi_launch_s4_widen(const void *packed, int64_t rows, int64_t cols, int64_t ld, int8_t *out, hipStream_t stream) {
+  if (rows <= 0 || cols <= 0 || ld < cols) return hipErrorInvalidValue;
+  const int64_t n = rows * cols;
+  hipLaunchKernelGGL(zmi_s4_widen_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                     (const uint8_t *)packed, rows, cols, ld, out);
+  return hipGetLastError();
+}
+
+// ---- one scale per tensor / per row -> {M, G} f32 ---------------------------------------------------
+// Reference: broadcast_w4a8_src_scale (backends/aocl/aocl_kernel.cpp:167-236): compact source scales are
+// repeated over the G groups before the per-group GEMM.
+__global__ __launch_bounds__(256) void zmi_broadcast_scales_kernel(const void *src, int32_t dt, int per_tensor, int64_t M,
+                                                                  int64_t G, float *out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * G) return;
+  const int64_t m = per_tensor ? 0 : i / G;
+  out[i] = dt == ZMI_DT_BF16 ? __uint_as_float((uint32_t)((const uint16_t *)src)[m] << 16) : ((const float *)src)[m];
+}
+
+hipError_t zmi_launch_broadcast_scales(const void *src, int32_t dt, int per_tensor, int64_t M, int64_t G, float *out,
+                                       hipStream_t stream) {
+  if (M <= 0 || G <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(zmi_broadcast_scales_kernel, dim3((unsigned)((M * G + 255) / 256)), dim3(256), 0, stream, src, dt,
+                     per_tensor, M, G, out);
+  return hipGetLastError();
+}

@@ -317,6 +317,38 @@ bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
   return transA || (K % 16) != 0 || (lda % 16) != 0 || (((uintptr_t)A) % 16) != 0;
 }
 
+
+// W4A8 (bf16 source quantized at run time, packed s4 weights with {G,N} scales, bf16 destination):
+// validate_w4a8_inputs, matmul/lowoha_matmul_utils.cpp:72-176, in its order.  Other uses of s4 weights
+// (weight-only quantization with bf16 compute) are not part of this library.
+int32_t validate_w4a8(const zmi_matmul_params_t &p, int M, int N, int K) {
+  if (p.dt_src == ZMI_DT_S8) { set_error("W4A8 requires a bf16 source with dynamic_quant (a pre-quantized s8 source is not supported)"); return ZMI_FAILURE; }
+  if (p.dynamic_quant && (p.dt_src == ZMI_DT_F32 || p.dt_dst == ZMI_DT_F32)) { set_error("W4A8 supports bf16 source and bf16 output only"); return ZMI_FAILURE; }
+  if (p.dt_src == ZMI_DT_U8 && (p.src_scale.buff || p.dynamic_quant)) { set_error("s4 weights do not support a u8 source"); return ZMI_FAILURE; }
+  const bool entry = p.dynamic_quant && p.dt_src == ZMI_DT_BF16;
+  if (entry && p.dt_compute != ZMI_DT_S8) { set_error("W4A8 dynamic quantization requires s8 compute"); return ZMI_FAILURE; }
+  if (!entry) { set_error("s4 weights: only W4A8 (bf16 source, dynamic_quant, s8 compute) is implemented, not weight-only quantization"); return ZMI_UNIMPLEMENTED; }
+  if (p.dt_dst != ZMI_DT_BF16) { set_error("W4A8 dynamic quantization requires bf16 output"); return ZMI_FAILURE; }
+  if (p.wei_zp.buff || p.src_zp.buff) { set_error("W4A8 supports symmetric quantization only"); return ZMI_FAILURE; }
+  const zmi_quant_t &ws = p.wei_scale;
+  if (!ws.buff) { set_error("W4A8 requires a weight scale"); return ZMI_FAILURE; }
+  if (ws.dt != ZMI_DT_F32 && ws.dt != ZMI_DT_BF16) { set_error("W4A8 weight scale supports only f32 or bf16"); return ZMI_FAILURE; }
+  if (ws.ndims != 2) { set_error("W4A8 requires weight scale dims {G,N}"); return ZMI_FAILURE; }
+  const int64_t G = ws.dims[0];
+  if (G <= 0 || ws.dims[1] != N) { set_error("W4A8 requires weight scale dims {G,N}"); return ZMI_FAILURE; }
+  if (K % G != 0) { set_error("W4A8 requires K divisible by the weight group count"); return ZMI_FAILURE; }
+  if ((K / G) % 4 != 0) { set_error("W4A8 requires K/G to be a multiple of 4"); return ZMI_FAILURE; }
+  const zmi_quant_t &ss = p.src_scale;
+  if (ss.dt != ZMI_DT_F32 && ss.dt != ZMI_DT_BF16) { set_error("W4A8 source scale supports only f32 or bf16"); return ZMI_FAILURE; }
+  if (ss.ndims != 2) { set_error("W4A8 requires source scale dims {1,1}, {M,1}, or {M,G}"); return ZMI_FAILURE; }
+  const int64_t r = ss.dims[0], c = ss.dims[1];
+  if (!((r == 1 && c == 1) || (r == M && c == 1) || (r == M && c == G))) {
+    set_error("W4A8 requires source scale dims {1,1}, {M,1}, or {M,G}");
+    return ZMI_FAILURE;
+  }
+  return ZMI_SUCCESS;
+}
+
 }  // namespace zmi
 
 using namespace zmi;
@@ -352,7 +384,14 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   const zmi_matmul_params_t &p = *params;
   const int Batch_A = batch_params ? batch_params->Batch_A : 1;
   const int Batch_B = batch_params ? batch_params->Batch_B : 1;
-  if (diagnostics_enabled()) {
+  const bool w4a8 = p.dt_wei == ZMI_DT_S4;
+  if (w4a8) {
+    // (the shape rules of this path keep the kernels inside their buffers: checked whatever the diagnostics switch says)
+    if (!src || !weight || !dst || M <= 0 || N <= 0 || K <= 0) { set_error("null pointer or non-positive dimension"); return ZMI_FAILURE; }
+    int32_t st = validate_w4a8(p, M, N, K);
+    if (st != ZMI_SUCCESS) return st;
+    if (p.pack_format_b != 0 || p.mem_format_b == 'r') { set_error("s4 weights are passed as plain packed nibbles (mem_format_b 'n', no pack format)"); return ZMI_FAILURE; }
+  } else if (diagnostics_enabled()) {
     int32_t st = validate_matmul(src, weight, dst, M, N, K, Batch_A, Batch_B, p, is_weights_const != 0);
     if (st != ZMI_SUCCESS) return st;
   } else if (!src || !weight || !dst || M <= 0 || N <= 0 || K <= 0) {
@@ -360,7 +399,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     return ZMI_FAILURE;
   }
   // ---- what this library implements of matmul_direct: the int8 path ----
-  if (p.dt_wei != ZMI_DT_S8) { set_error("only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+  if (p.dt_wei != ZMI_DT_S8 && !w4a8) { set_error("only s8 and (W4A8) s4 weights are implemented"); return ZMI_UNIMPLEMENTED; }
   if (layout != 'r' && layout != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
   if (Batch_A != 1 || Batch_B != 1) { set_error("batched matmul is not implemented"); return ZMI_UNIMPLEMENTED; }
   const bool ggml = p.pack_format_b == 1;
@@ -377,7 +416,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     set_error("mem_format_b == 'r' requires lowoha_algo == aocl_dlp_blocked");
     return ZMI_FAILURE;
   }
-  const bool dyn = is_dynamic_quant_config(p);
+  const bool dyn = w4a8 || is_dynamic_quant_config(p);
   if (!dyn && p.dt_src != ZMI_DT_S8 && p.dt_src != ZMI_DT_U8) {
     set_error("source must be u8 / s8, or bf16 / f32 with dynamic_quant and an s8 compute type");
     return ZMI_UNIMPLEMENTED;
@@ -405,6 +444,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     const int64_t n = nelems(p.src_scale);
     if (n > M && n % M == 0) pg_groups = n / M;
   }
+  // W4A8 with one source scale per tensor or per row: the source is quantized that way, then the scales are
+  // repeated over the weights' G groups and the per-group GEMM follows (broadcast_w4a8_src_scale,
+  // matmul/backends/aocl/aocl_kernel.cpp:167-236).  G == 1 is the plain per-channel chain.
+  const bool bcast_src = w4a8 && pg_groups == 0 && p.wei_scale.dims[0] > 1;
+  if (bcast_src) pg_groups = p.wei_scale.dims[0];
   if (ggml) {
     // reference: ggml_is_sym_quant (ggml_weight_unpack.cpp:142-153), checked after the source was quantized:
     // s8 (or dynamically quantized) source, symmetric, more than one source scale, f32 / bf16 destination
@@ -440,6 +484,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   const bool use_cache = !ggml && p.mem_format_b != 'r' && is_weights_const &&
                          std::min(weight_cache_env(), p.weight_cache_type) > 0;
   const bool pack_in_arena = !ggml && p.mem_format_b != 'r' && !use_cache;
+  const size_t widen_bytes = w4a8 && pack_in_arena ? (size_t)K * (size_t)N : 0;
   const int64_t K16 = zmi_round_up(K, 16);
   const bool ring = !pg_groups && use_ring_kernel(M, N, K);
   const int64_t frag_kpad = ring ? zmi_blob_kpad(K) : 0;
@@ -447,6 +492,8 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   const bool repack_a = !dyn && (ring || a_needs_repack(src, lda, K, transA != 0));
   size_t need = 0;
   if (pack_in_arena) need += Arena::padded((size_t)zmi_blob_bytes(K, N));
+  if (widen_bytes) need += Arena::padded(widen_bytes);
+  if (bcast_src) need += Arena::padded(sizeof(float) * (size_t)M * (size_t)pg_groups);
   if (dyn) need += Arena::padded(a_bytes) + Arena::padded(sizeof(float) * (size_t)M * (size_t)(pg_groups ? pg_groups : 1)) + 256;
   if (repack_a) need += Arena::padded(a_bytes);
   ZmiRingPlan plan = {};
@@ -465,6 +512,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   } else if (p.mem_format_b == 'r') {
     if (!blob_matches(weight, K, N)) return ZMI_FAILURE;
     blob = (const uint8_t *)weight;
+  } else if (w4a8) {
+    void *wide = widen_bytes ? arena().alloc(widen_bytes) : nullptr;
+    void *slot = pack_in_arena ? arena().alloc((size_t)zmi_blob_bytes(K, N)) : nullptr;
+    blob = packed_s4_weights(weight, K, N, ldb, transB != 0, use_cache, wide, slot);
+    if (!blob) return ZMI_FAILURE;
   } else {
     void *slot = pack_in_arena ? arena().alloc((size_t)zmi_blob_bytes(K, N)) : nullptr;
     blob = packed_weights(weight, K, N, ldb, transB != 0, p.dt_src, use_cache, slot);
@@ -491,7 +543,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
     int8_t *q = (int8_t *)arena().alloc(a_bytes);
-    float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M * (size_t)(pg_groups ? pg_groups : 1));
+    float *sc = (float *)arena().alloc(sizeof(float) * (size_t)M * (size_t)(pg_groups && !bcast_src ? pg_groups : 1));
     unsigned int *amax = (unsigned int *)arena().alloc(256);
     // bytes of q between K and K16 stay unwritten: the blob's rows beyond K are zero
     int32_t sdt = p.src_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p.src_scale.dt;
@@ -501,7 +553,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     // decode shapes: quantization fused into the GEMM launch when its whole grid is resident at once
     const bool decode_kernel = decode_kernel_allowed(M, N, K);
     // (the decode kernel's producers are its first workgroups and wait for nothing, so its grid need not be resident)
-    if (pg_groups) {
+    if (pg_groups && !bcast_src) {
       // reference: the per-group dynamic reorder in front of the sym-quant GEMM
       // (matmul/quantization/reorder_quantization.cpp:43-280 with {M,G} scale dims)
       if (zmi_pergroup_decode_shape(prob, (int)pg_groups) && !std::getenv("ZMI_NO_FUSED_QUANT")) {
@@ -520,7 +572,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       ep.src_scale.buff = sc;
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
-    } else if (per_token && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
+    } else if (per_token && !bcast_src && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
       if (!ctr) return ZMI_FAILURE;
@@ -554,8 +606,18 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 1; ep.src_scale.dims[0] = 1;
     }
+    if (bcast_src) {
+      float *wide = (float *)arena().alloc(sizeof(float) * (size_t)M * (size_t)pg_groups);
+      if (!hip_ok(zmi_launch_broadcast_scales(ep.src_scale.buff, ep.src_scale.dt, ep.src_scale.ndims == 1, M, pg_groups,
+                                              wide, stream()), "scale broadcast launch"))
+        return ZMI_FAILURE;
+      ep.src_scale.buff = wide;
+      ep.src_scale.dt = ZMI_DT_F32;
+      ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
+    }
     prob.A = q; prob.lda = K16; prob.a_is_u8 = 0;
     ep.dt_src = ZMI_DT_S8;
+    ep.dt_wei = ZMI_DT_S8;   // (the s4 codes were widened)
   } else if (repack_a) {
     int8_t *a2 = (int8_t *)arena().alloc(a_bytes);
     if (ring) {

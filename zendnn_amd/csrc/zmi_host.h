@@ -71,6 +71,11 @@ const uint8_t *packed_weights(const void *weight, int64_t K, int64_t N, int64_t 
                               int32_t src_dtype, bool use_cache, void *arena_slot);
 // GGML Q8_0 packed weights [N][K/32] blocks: cached blob + bf16 scales {K/32, N} (null on failure)
 const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const void **scales);
+// packed s4 weights ([K, ldb] nibbles, or [N, ldb] when transB): widened to s8 and reordered.  With use_cache the
+// blob is kept per (pointer, shape, layout); otherwise widen_slot (K * N bytes) and arena_slot (blob_bytes) must
+// have been reserved in the arena by the caller.
+const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
+                                 void *widen_slot, void *arena_slot);
 void clear_weight_cache();
 
 // Checks (once per pointer) that a caller-supplied blob carries the header of a

@@ -324,6 +324,47 @@ const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const 
   return (const uint8_t *)buf;
 }
 
+// W4A8 weights: widened s4 -> s8 and reordered (reference: w4a8ReorderAndCacheWeightsAocl,
+// matmul/backends/aocl/aocl_kernel.cpp:704-793: a cache of its own keyed like the int8 one; here the key's
+// leading dimension is stored negated, which no s8 entry has).
+const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
+                                 void *widen_slot, void *arena_slot) {
+  const int64_t rows = transB ? N : K, cols = transB ? K : N;
+  if (!use_cache) {
+    if (!hip_ok(zmi_launch_s4_widen(weight, rows, cols, ldb, (int8_t *)widen_slot, stream()), "s4 widen launch") ||
+        !hip_ok(zmi_launch_prepack((const int8_t *)widen_slot, K, N, cols, transB, ZMI_DT_S8, 0, (uint8_t *)arena_slot,
+                                   stream()), "prepack launch"))
+      return nullptr;
+    return (const uint8_t *)arena_slot;
+  }
+  std::lock_guard<std::mutex> lk(g_mu);
+  CacheKey key{weight, K, N, -ldb - 1000, transB};
+  auto it = g_cache.find(key);
+  if (it != g_cache.end()) {
+    g_lru.splice(g_lru.begin(), g_lru, it->second.lru);
+    return it->second.blob;
+  }
+  void *blob = nullptr, *wide = nullptr;
+  if (!hip_ok(hipMalloc(&blob, (size_t)zmi_blob_bytes(K, N)), "hipMalloc(W4A8 weights)")) return nullptr;
+  if (!hip_ok(hipMalloc(&wide, (size_t)K * N), "hipMalloc(s4 widen)")) { (void)hipFree(blob); return nullptr; }
+  bool ok = hip_ok(zmi_launch_s4_widen(weight, rows, cols, ldb, (int8_t *)wide, stream()), "s4 widen launch") &&
+            hip_ok(zmi_launch_prepack((const int8_t *)wide, K, N, cols, transB, ZMI_DT_S8, 0, (uint8_t *)blob, stream()),
+                   "prepack launch") &&
+            hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize");   // the widened copy is freed next
+  (void)hipFree(wide);
+  if (!ok) { (void)hipFree(blob); return nullptr; }
+  g_lru.push_front(key);
+  g_cache[key] = CacheVal{(uint8_t *)blob, g_lru.begin()};
+  while (g_cache.size() > cache_capacity()) {
+    (void)hipDeviceSynchronize();
+    CacheKey old = g_lru.back();
+    g_lru.pop_back();
+    (void)hipFree(g_cache[old].blob);
+    g_cache.erase(old);
+  }
+  return (const uint8_t *)blob;
+}
+
 void clear_weight_cache() {
   std::lock_guard<std::mutex> lk(g_mu);
   if (!g_cache.empty()) (void)hipDeviceSynchronize();

@@ -147,6 +147,11 @@ hipError_t zmi_launch_pad_rows(const void *src, int64_t M, int64_t K, int64_t ld
 // GGML Q8_0 blocks ([N][K/32] x {fp16 d, int8 qs[32]}) -> s8 rows [N, K] and bf16 scales {K/32, N}
 hipError_t zmi_launch_ggml_q8_0_unpack(const void *blocks, int64_t N, int64_t K, int8_t *rows, uint16_t *scales,
                                        hipStream_t stream);
+// packed s4 codes of a [rows, ld] matrix (two per byte, even index = low nibble) -> s8 [rows, cols]
+hipError_t zmi_launch_s4_widen(const void *packed, int64_t rows, int64_t cols, int64_t ld, int8_t *out, hipStream_t stream);
+// one f32 / bf16 scale per tensor or per row -> f32 {M, G}
+hipError_t zmi_launch_broadcast_scales(const void *src, int32_t dt, int per_tensor, int64_t M, int64_t G, float *out,
+                                       hipStream_t stream);
 // u8 / s8 rows (or their transpose) -> fragment-major s8; u8 values are shifted by -128
 hipError_t zmi_launch_repack_frag(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans, int is_u8,
                                   int8_t *dst, hipStream_t stream);
