@@ -41,7 +41,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
+                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "decode_M16_w4a8_group128", "decode_M16_w4a8_group128_per_token_rows", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
                              "moe_config4", "moe_config5"],
                     help="run one of the other configs alone and print its entry (for profiler runs)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -244,6 +244,38 @@ def main():
         return {"GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2), "group_size": gs,
                 "kernel": lowoha.last_kernel()}
 
+    def run_decode_w4a8(m, gs, per_token):
+        # W4A8 decode: bf16 rows quantized by the library ({M,G} scales, or one per row repeated over the groups),
+        # packed s4 weights (K*N/2 bytes) with {G,N} scales; the library widens, reorders and caches them on the
+        # first call per weight pointer (outside the timed region) and then streams the 4-bit tiles.
+        # bytes = the 4-bit weights + rows + scales + output.
+        G = K_DEC // gs
+        ws4 = [torch.randint(0, 256, (K_DEC * N_DEC // 2,), dtype=torch.uint8, device=dev, generator=g) for _ in range(n_sets)]
+        ws = torch.rand((G, N_DEC), device=dev, generator=g) * 0.009 + 0.001
+        x = torch.randn((m, K_DEC), device=dev, generator=g).to(torch.bfloat16)
+        dst = torch.zeros((m, N_DEC), dtype=torch.bfloat16, device=dev)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S4, dst=capi.DT_BF16, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (m, 1) if per_token else (m, G))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (G, N_DEC))
+        p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+        calls = [lowoha.prepared_matmul("r", False, False, m, N_DEC, K_DEC, 1.0, x, K_DEC, w4, N_DEC, None, 0.0,
+                                        dst, N_DEC, True, p)[0] for w4 in ws4]
+        state = {"i": 0}
+
+        def step():
+            st = calls[state["i"] % n_sets]()
+            state["i"] += 1
+            if st != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+
+        t = ev_time(step, 100, 2 * n_sets)
+        nbytes = K_DEC * N_DEC // 2 + m * K_DEC * 2 + G * N_DEC * 4 + m * G * 4 + m * N_DEC * 2
+        out = {"GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2), "group_size": gs,
+               "source_scales": "per token" if per_token else "per group", "kernel": lowoha.last_kernel()}
+        capi.load().zmi_clear_weight_cache()
+        return out
+
     def run_prefill(N):
         # config 3: whole call = per-token quantization launch (rows written in MFMA fragment order) + GEMM launch;
         # the per-kernel split is in the rocprofv3 summaries under profiles/
@@ -330,6 +362,8 @@ def main():
         "decode_M128": lambda: run_decode_m(128),
         "decode_M16_per_group128": lambda: run_decode_per_group(16, 128),
         "decode_M16_per_group32": lambda: run_decode_per_group(16, 32),
+        "decode_M16_w4a8_group128": lambda: run_decode_w4a8(16, 128, False),
+        "decode_M16_w4a8_group128_per_token_rows": lambda: run_decode_w4a8(16, 128, True),
         "prefill_N4096": lambda: run_prefill(4096),
         "prefill_N14336": lambda: run_prefill(14336),
         "config1_u8s8_M128": run_config1,

@@ -94,6 +94,18 @@ def test_w4a8_post_ops(zo, postop):
     _run(zo, 9, 1024, 64, 32, (9, 32), postop=postop)
 
 
+@pytest.mark.parametrize("kind", ["tensor", "token", "group"])
+@pytest.mark.parametrize("M,K,N,G", [(16, 4096, 200, 32), (16, 4096, 64, 128), (7, 2048, 40, 8), (2, 1024, 96, 32),
+                                     (16, 1024, 33, 8)])
+def test_w4a8_decode_shapes_stream_the_4_bit_tiles(zo, M, K, N, G, kind):
+    # up to 16 rows, K = 1024 / 2048 / 4096, cached weights: the decode-shaped kernel reads 4-bit tiles; with one
+    # scale per row or per (row, group) the quantization is part of the same launch
+    sdims = {"tensor": (1, 1), "token": (M, 1), "group": (M, G)}[kind]
+    name = "pergroup_decode_s4_mfma16x16x64" + {"tensor": "", "token": " (fused per-token quant)",
+                                                "group": " (fused per-group quant)"}[kind]
+    _run(zo, M, K, N, G, sdims, want_kernel=name, calls=2, postop=capi.PO_SWISH if N == 200 else None, bias=N == 64)
+
+
 def test_w4a8_one_group_is_the_per_channel_chain(zo):
     # G = 1: {1, N} weight scales, the plain per-token chain on the widened weights
     _run(zo, 8, 512, 64, 1, (8, 1))

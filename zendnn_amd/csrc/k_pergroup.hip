@@ -241,10 +241,18 @@ __device__ __forceinline__ int pgd_lds_off(int cc, int g, int r) {   // operand 
   return cc * 1024 + ((g * 16 + (r ^ ((g * 4 + (cc & 3)) & 15))) << 4);
 }
 
-template <int CPW, int GPW>
+//
+// S4: the weights are streamed as 4-bit codes, half the bytes.  tiles_s4 holds, per 32-column block, one 2 KiB
+// piece per PAIR of 64-k chunks in the blob's lane order: every byte carries the code of the even chunk in its
+// high nibble and the code of the odd chunk in its low nibble.  (w & 0xf0f0f0f0) and ((w << 4) & 0xf0f0f0f0) are
+// then the two chunks' operands with every weight multiplied by 16 (a code in the high nibble of a byte IS
+// 16 * code as a signed byte: no sign extension to compute), the integer tiles are exact multiples of 16 and
+// are shifted back when they are folded.  |16 * code| <= 128, so the accumulators stay where s8 weights keep them.
+template <int CPW, int GPW, bool S4>
 __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(ZmiProblem p, ZmiEpilogue epi,
-                                                                               ZmiFusedQuant fq) {
+                                                                               ZmiFusedQuant fq, const uint8_t *tiles_s4) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  static_assert(!S4 || CPW % 2 == 0, "4-bit weights come in pairs of chunks");
   constexpr int SUB = GPW > CPW ? GPW / CPW : 1;  // groups per chunk (2: groups of 32 k)
   constexpr int CPG = GPW > CPW ? 1 : CPW / GPW;  // chunks per group
   constexpr int G = PGD_WAVES * GPW;
@@ -264,7 +272,8 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   // leave; the streaming workgroups follow them in dispatch order and wait (bounded) for the M rows only after
   // their weight requests are out.  Producers wait for nothing, so the wait cannot deadlock.
   if (fq.x && (int)blockIdx.x < M) {
-    zmi_fused_quant_row_groups(fq, blockIdx.x, K, G);
+    if (fq.per_row) zmi_fused_quant_row(fq, blockIdx.x, K, reinterpret_cast<float *>(lds));
+    else zmi_fused_quant_row_groups(fq, blockIdx.x, K, G);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
     __syncthreads();
     if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
@@ -302,26 +311,39 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
 #pragma unroll
     for (int i = 0; i < SS_PT; ++i) {
       const int e0 = tid + i * PGD_THREADS, e = e0 < 16 * G ? e0 : 16 * G - 1, r = e / G;
-      ss_r[i] = zmi_ld_f32(p.src_scale_ptr, epi.src_scale_dt, (int64_t)(r < M ? r : M - 1) * G + e % G);
+      const int64_t rr = r < M ? r : M - 1;
+      ss_r[i] = zmi_ld_f32(p.src_scale_ptr, epi.src_scale_dt, fq.x && fq.per_row ? rr : rr * G + e % G);
     }
   };
   if (!fq.x) load_ss();
-  // the whole weight slice
-  const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
-  v4i b[CPW][2];
+  // the whole weight slice: NL loads of 2 KiB pieces per column group (a piece is a chunk, or a pair of chunks
+  // of 4-bit codes)
+  constexpr int NL = S4 ? CPW / 2 : CPW;
+  const uint8_t *tiles = S4 ? tiles_s4 : p.blob + zmi_blob_tiles_off(N);
+  const int64_t nb_stride = S4 ? zmi_s4_nb_stride(K) : zmi_blob_nb_stride(K);
+  const int l_begin = S4 ? c_begin / 2 : c_begin;
+  v4i braw[NL][2];
   const uint8_t *bsrc[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h)
-    bsrc[h] = tiles + (int64_t)blk * zmi_blob_nb_stride(K) + (g4 / 2) * 1024 + ((g4 % 2) * 32 + h * 16 + c16) * 16;
+    bsrc[h] = tiles + (int64_t)blk * nb_stride + (g4 / 2) * 1024 + ((g4 % 2) * 32 + h * 16 + c16) * 16;
   // (with fused quantization three quarters of the slice go out before the wait for the rows, the rest
   // after the row requests, like the per-token decode kernel)
-  constexpr int FIRST = CPW >= 4 ? CPW * 3 / 4 : CPW;
+  constexpr int FIRST = NL >= 4 ? NL * 3 / 4 : NL;
 #pragma unroll
-  for (int u = 0; u < CPW; ++u)
+  for (int u = 0; u < NL; ++u)
     if (u < FIRST || !fq.x) {
-      b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)(c_begin + u) * 2048);
-      b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(c_begin + u) * 2048);
+      braw[u][0] = *(const v4i *)(bsrc[0] + (int64_t)(l_begin + u) * 2048);
+      braw[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(l_begin + u) * 2048);
     }
+  // operand of chunk u, column group h
+  auto bop = [&](int u, int h) -> v4i {
+    if (!S4) return braw[u][h];
+    const v4i w = braw[u / 2][h];
+    const int sh = (u % 2) * 4;
+    return (v4i){(int)(((uint32_t)w[0] << sh) & 0xf0f0f0f0u), (int)(((uint32_t)w[1] << sh) & 0xf0f0f0f0u),
+                 (int)(((uint32_t)w[2] << sh) & 0xf0f0f0f0u), (int)(((uint32_t)w[3] << sh) & 0xf0f0f0f0u)};
+  };
   if (fq.x) {
     // the quantized rows and their scales exist once the counter says so
     if (tid == 0) {
@@ -336,9 +358,9 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
     load_rows();
     load_ss();
 #pragma unroll
-    for (int u = FIRST; u < CPW; ++u) {
-      b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)(c_begin + u) * 2048);
-      b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(c_begin + u) * 2048);
+    for (int u = FIRST; u < NL; ++u) {
+      braw[u][0] = *(const v4i *)(bsrc[0] + (int64_t)(l_begin + u) * 2048);
+      braw[u][1] = *(const v4i *)(bsrc[1] + (int64_t)(l_begin + u) * 2048);
     }
   }
   // scales -> LDS
@@ -367,8 +389,8 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
 #pragma unroll
       for (int u = gi * CPG; u < (gi + 1) * CPG; ++u) {
         const v4i a = *(const v4i *)(lds + pgd_lds_off(c_begin + u, g4, c16));
-        acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[gi][0], 0, 0, 0);
-        acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[gi][1], 0, 0, 0);
+        acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bop(u, 0), acc[gi][0], 0, 0, 0);
+        acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bop(u, 1), acc[gi][1], 0, 0, 0);
       }
     } else {
       // two groups share a chunk: the chunk is multiplied once per group with the other group's lanes
@@ -376,8 +398,8 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
       const int u = gi / SUB, t = gi % SUB;
       v4i a = *(const v4i *)(lds + pgd_lds_off(c_begin + u, g4, c16));
       if (g4 / (4 / SUB) != t) a = (v4i){0, 0, 0, 0};
-      acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[gi][0], 0, 0, 0);
-      acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[gi][1], 0, 0, 0);
+      acc[gi][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bop(u, 0), acc[gi][0], 0, 0, 0);
+      acc[gi][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bop(u, 1), acc[gi][1], 0, 0, 0);
     }
   }
   // ---- the operand area is done with ----
@@ -405,7 +427,7 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
 #pragma unroll 8
     for (int t = 0; t < RT; ++t) {
       const int g = r * RT + t;
-      float v = __fmul_rn((float)red[t * 512 + off], ss_l[e_row * G + g]);
+      float v = __fmul_rn((float)(S4 ? red[t * 512 + off] >> 4 : red[t * 512 + off]), ss_l[e_row * G + g]);
       v = __fmul_rn(v, ws_l[g * 32 + e_h * 16 + e_c]);
       sum = __fadd_rn(sum, v);
     }
@@ -419,21 +441,23 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_tail(epi, y, bias, e_row, e_n));
 }
 
-template <int CPW, int GPW>
-static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq, hipStream_t stream) {
+template <int CPW, int GPW, bool S4 = false>
+static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq, hipStream_t stream,
+                             const uint8_t *tiles_s4 = nullptr) {
   constexpr int G = PGD_WAVES * GPW, NCH = PGD_WAVES * CPW, RT = G <= 32 ? G : 16;
   constexpr size_t main_bytes = (size_t)NCH * 1024 > (size_t)RT * 2048 ? (size_t)NCH * 1024 : (size_t)RT * 2048;
   constexpr size_t smem = main_bytes + (size_t)G * 32 * 4 + (size_t)16 * G * 4;
   static bool attr_done = false;
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_decode_pergroup_kernel<CPW, GPW>,
+    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_decode_pergroup_kernel<CPW, GPW, S4>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
   ZmiFusedQuant none = {};
   const dim3 grid((unsigned)(zmi_blob_npad(p.N) / 32) + (fq ? p.M : 0)), block(PGD_THREADS);
-  hipLaunchKernelGGL((zmi_gemm_decode_pergroup_kernel<CPW, GPW>), grid, block, smem, stream, p, epi, fq ? *fq : none);
+  hipLaunchKernelGGL((zmi_gemm_decode_pergroup_kernel<CPW, GPW, S4>), grid, block, smem, stream, p, epi, fq ? *fq : none,
+                     tiles_s4);
   return hipGetLastError();
 }
 
@@ -454,8 +478,13 @@ bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G) {
 
 bool zmi_pergroup_group_size_ok(int64_t gs) { return gs > 0 && (gs % 64 == 0 || gs == 32 || gs == 16); }
 
+bool zmi_pergroup_s4_shape(const ZmiProblem &p, int G) {
+  int cpw, gpw;
+  return pgd_fits(p, G, &cpw, &gpw) && cpw % 2 == 0 && !getenv("ZMI_PERGROUP_GENERIC") && !getenv("ZMI_NO_S4_STREAM");
+}
+
 hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
-                                    hipStream_t stream) {
+                                    hipStream_t stream, const uint8_t *tiles_s4) {
   const int G = epi.n_groups;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || G <= 0 || p.K % G != 0) return hipErrorInvalidValue;
   const int gs = p.K / G;
@@ -465,6 +494,24 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
   if (p.a_is_u8 || epi.has_zp || epi.gated_act) return hipErrorInvalidValue;   // symmetric s8 rows only
   if (p.lda % 16 != 0 || ((uintptr_t)p.A) % 16 != 0 || p.lda < p.K) return hipErrorInvalidValue;   // 16-byte row loads
   int cpw = 0, gpw = 0;
+  if (tiles_s4 && zmi_pergroup_s4_shape(p, G) && pgd_fits(p, G, &cpw, &gpw)) {
+    // 4-bit codes streamed as they are (W4A8 decode shapes)
+    switch (cpw * 16 + gpw) {
+    case 8 * 16 + 8: return pgd_launch<8, 8, true>(p, epi, fq, stream, tiles_s4);
+    case 8 * 16 + 4: return pgd_launch<8, 4, true>(p, epi, fq, stream, tiles_s4);
+    case 8 * 16 + 2: return pgd_launch<8, 2, true>(p, epi, fq, stream, tiles_s4);
+    case 8 * 16 + 1: return pgd_launch<8, 1, true>(p, epi, fq, stream, tiles_s4);
+    case 4 * 16 + 4: return pgd_launch<4, 4, true>(p, epi, fq, stream, tiles_s4);
+    case 4 * 16 + 2: return pgd_launch<4, 2, true>(p, epi, fq, stream, tiles_s4);
+    case 4 * 16 + 1: return pgd_launch<4, 1, true>(p, epi, fq, stream, tiles_s4);
+    case 2 * 16 + 2: return pgd_launch<2, 2, true>(p, epi, fq, stream, tiles_s4);
+    case 2 * 16 + 1: return pgd_launch<2, 1, true>(p, epi, fq, stream, tiles_s4);
+    case 8 * 16 + 16: return pgd_launch<8, 16, true>(p, epi, fq, stream, tiles_s4);
+    case 4 * 16 + 8: return pgd_launch<4, 8, true>(p, epi, fq, stream, tiles_s4);
+    case 2 * 16 + 4: return pgd_launch<2, 4, true>(p, epi, fq, stream, tiles_s4);
+    default: break;
+    }
+  }
   if (pgd_fits(p, G, &cpw, &gpw) && !getenv("ZMI_PERGROUP_GENERIC")) {
     switch (cpw * 16 + gpw) {
     case 8 * 16 + 8: return pgd_launch<8, 8>(p, epi, fq, stream);
@@ -571,5 +618,28 @@ hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64
   else
     hipLaunchKernelGGL(zmi_quant_groups_kernel<false>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q,
                        ldq, scales, user_scales, user_dt);
+  return hipGetLastError();
+}
+
+// ---- 4-bit tiles for the decode-shaped kernel --------------------------------------------------
+// From the blob of widened s8 weights (every byte a code in -8 .. 7): per 32-column block, the 2 KiB of chunk
+// 2c and of chunk 2c + 1 become one 2 KiB piece, high nibble = even chunk, low nibble = odd chunk.
+__global__ __launch_bounds__(256) void zmi_s4_tiles_kernel(const uint8_t *blob, int64_t K, int64_t N, uint8_t *out) {
+  const int64_t pairs = zmi_blob_kpad(K) / 128;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;      // 16-byte granule of the output
+  const int64_t per_nb = pairs * 128;
+  if (i >= per_nb * (zmi_blob_npad(N) / 32)) return;
+  const int64_t nb = i / per_nb, r = i % per_nb, cp = r / 128, gq = r % 128;
+  const uint8_t *src = blob + zmi_blob_tiles_off(N) + nb * zmi_blob_nb_stride(K) + cp * 4096 + gq * 16;
+  const v4i hi = *(const v4i *)src, lo = *(const v4i *)(src + 2048);
+  v4i o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = (int)((((uint32_t)hi[j] << 4) & 0xf0f0f0f0u) | ((uint32_t)lo[j] & 0x0f0f0f0fu));
+  *(v4i *)(out + nb * zmi_s4_nb_stride(K) + cp * 2048 + gq * 16) = o;
+}
+
+hipError_t zmi_launch_s4_tiles(const uint8_t *blob, int64_t K, int64_t N, uint8_t *out, hipStream_t stream) {
+  const int64_t n = (zmi_blob_kpad(K) / 128) * 128 * (zmi_blob_npad(N) / 32);
+  hipLaunchKernelGGL(zmi_s4_tiles_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, blob, K, N, out);
   return hipGetLastError();
 }

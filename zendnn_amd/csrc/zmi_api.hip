@@ -506,6 +506,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   // ---- weights ----
   const uint8_t *blob;
   const void *ggml_scales = nullptr;
+  const uint8_t *tiles_s4 = nullptr;
   if (ggml) {
     blob = packed_ggml_q8_0(weight, K, N, &ggml_scales);
     if (!blob) return ZMI_FAILURE;
@@ -515,7 +516,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   } else if (w4a8) {
     void *wide = widen_bytes ? arena().alloc(widen_bytes) : nullptr;
     void *slot = pack_in_arena ? arena().alloc((size_t)zmi_blob_bytes(K, N)) : nullptr;
-    blob = packed_s4_weights(weight, K, N, ldb, transB != 0, use_cache, wide, slot);
+    blob = packed_s4_weights(weight, K, N, ldb, transB != 0, use_cache, wide, slot, &tiles_s4);
     if (!blob) return ZMI_FAILURE;
   } else {
     void *slot = pack_in_arena ? arena().alloc((size_t)zmi_blob_bytes(K, N)) : nullptr;
@@ -572,6 +573,21 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       ep.src_scale.buff = sc;
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
+    } else if (bcast_src && per_token && K % 4 == 0 && zmi_pergroup_decode_shape(prob, (int)pg_groups) &&
+               !std::getenv("ZMI_NO_FUSED_QUANT")) {
+      // W4A8 decode shapes with one scale per row: the per-token quantization is part of the per-group GEMM
+      // launch, whose workgroups read the row's scale for every group (no broadcast copy)
+      unsigned int *ctr = fused_counter();
+      if (!ctr) return ZMI_FAILURE;
+      fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
+      fused.q = q; fused.ldq = K16; fused.scales = sc;
+      fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
+      fused.counter = ctr; fused.target = fused_next_target(M);
+      fused.per_row = 1;
+      use_fused = true;
+      ep.src_scale.buff = sc;
+      ep.src_scale.dt = ZMI_DT_F32;
+      ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
     } else if (per_token && !bcast_src && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
       unsigned int *ctr = fused_counter();
@@ -606,7 +622,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 1; ep.src_scale.dims[0] = 1;
     }
-    if (bcast_src) {
+    if (bcast_src && !use_fused) {
       float *wide = (float *)arena().alloc(sizeof(float) * (size_t)M * (size_t)pg_groups);
       if (!hip_ok(zmi_launch_broadcast_scales(ep.src_scale.buff, ep.src_scale.dt, ep.src_scale.ndims == 1, M, pg_groups,
                                               wide, stream()), "scale broadcast launch"))
@@ -634,9 +650,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
   if (st != ZMI_SUCCESS) return st;
   if (epi.n_groups > 0) {
-    set_kernel_name(use_fused ? "pergroup_decode_mfma16x16x64 (fused per-group quant)"
+    const bool s4_stream = tiles_s4 && zmi_pergroup_s4_shape(prob, epi.n_groups);
+    set_kernel_name(s4_stream ? (use_fused ? (fused.per_row ? "pergroup_decode_s4_mfma16x16x64 (fused per-token quant)" : "pergroup_decode_s4_mfma16x16x64 (fused per-group quant)") : "pergroup_decode_s4_mfma16x16x64")
+                    : use_fused ? "pergroup_decode_mfma16x16x64 (fused per-group quant)"
                     : zmi_pergroup_decode_shape(prob, epi.n_groups) ? "pergroup_decode_mfma16x16x64" : "pergroup_mfma16x16x64");
-    st = hip_ok(zmi_launch_gemm_pergroup(prob, epi, use_fused ? &fused : nullptr, stream()), "per-group GEMM launch")
+    st = hip_ok(zmi_launch_gemm_pergroup(prob, epi, use_fused ? &fused : nullptr, stream(), tiles_s4), "per-group GEMM launch")
              ? ZMI_SUCCESS : ZMI_FAILURE;
   } else if (use_fused) {
     // a one-row scale in device memory reads like a per-token scale

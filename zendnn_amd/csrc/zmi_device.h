@@ -59,6 +59,11 @@ static inline __host__ __device__ int64_t zmi_blob_tiles_off(int64_t N) {
 static inline __host__ __device__ int64_t zmi_blob_nb_stride(int64_t K) {
   return zmi_blob_kpad(K) * 32 + ZMI_NB_SKEW;
 }
+// 4-bit tiles (W4A8 decode shapes): per 32-column block one 2 KiB piece per pair of 64-k chunks
+static inline __host__ __device__ int64_t zmi_s4_nb_stride(int64_t K) { return zmi_blob_kpad(K) * 16 + ZMI_NB_SKEW; }
+static inline __host__ __device__ int64_t zmi_s4_tiles_bytes(int64_t K, int64_t N) {
+  return zmi_s4_nb_stride(K) * (zmi_blob_npad(N) / 32);
+}
 static inline __host__ __device__ int64_t zmi_blob_bytes(int64_t K, int64_t N) {
   return zmi_blob_tiles_off(N) + zmi_blob_nb_stride(K) * (zmi_blob_npad(N) / 32);
 }

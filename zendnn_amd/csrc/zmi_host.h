@@ -74,8 +74,9 @@ const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const 
 // packed s4 weights ([K, ldb] nibbles, or [N, ldb] when transB): widened to s8 and reordered.  With use_cache the
 // blob is kept per (pointer, shape, layout); otherwise widen_slot (K * N bytes) and arena_slot (blob_bytes) must
 // have been reserved in the arena by the caller.
+// *tiles_s4 receives the 4-bit tiles kept behind a cached blob (null when not cached: a one-off pack streams s8).
 const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
-                                 void *widen_slot, void *arena_slot);
+                                 void *widen_slot, void *arena_slot, const uint8_t **tiles_s4);
 void clear_weight_cache();
 
 // Checks (once per pointer) that a caller-supplied blob carries the header of a

@@ -328,8 +328,12 @@ const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const 
 // matmul/backends/aocl/aocl_kernel.cpp:704-793: a cache of its own keyed like the int8 one; here the key's
 // leading dimension is stored negated, which no s8 entry has).
 const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
-                                 void *widen_slot, void *arena_slot) {
+                                 void *widen_slot, void *arena_slot, const uint8_t **tiles_s4) {
   const int64_t rows = transB ? N : K, cols = transB ? K : N;
+  // one allocation per cached weight: the blob of widened codes (every kernel reads it), then the 4-bit tiles
+  // the decode-shaped kernel streams instead (half the bytes per call)
+  const size_t blob_bytes = (size_t)zmi_round_up(zmi_blob_bytes(K, N), 256);
+  *tiles_s4 = nullptr;
   if (!use_cache) {
     if (!hip_ok(zmi_launch_s4_widen(weight, rows, cols, ldb, (int8_t *)widen_slot, stream()), "s4 widen launch") ||
         !hip_ok(zmi_launch_prepack((const int8_t *)widen_slot, K, N, cols, transB, ZMI_DT_S8, 0, (uint8_t *)arena_slot,
@@ -342,14 +346,16 @@ const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64
   auto it = g_cache.find(key);
   if (it != g_cache.end()) {
     g_lru.splice(g_lru.begin(), g_lru, it->second.lru);
+    *tiles_s4 = it->second.blob + blob_bytes;
     return it->second.blob;
   }
   void *blob = nullptr, *wide = nullptr;
-  if (!hip_ok(hipMalloc(&blob, (size_t)zmi_blob_bytes(K, N)), "hipMalloc(W4A8 weights)")) return nullptr;
+  if (!hip_ok(hipMalloc(&blob, blob_bytes + (size_t)zmi_s4_tiles_bytes(K, N)), "hipMalloc(W4A8 weights)")) return nullptr;
   if (!hip_ok(hipMalloc(&wide, (size_t)K * N), "hipMalloc(s4 widen)")) { (void)hipFree(blob); return nullptr; }
   bool ok = hip_ok(zmi_launch_s4_widen(weight, rows, cols, ldb, (int8_t *)wide, stream()), "s4 widen launch") &&
             hip_ok(zmi_launch_prepack((const int8_t *)wide, K, N, cols, transB, ZMI_DT_S8, 0, (uint8_t *)blob, stream()),
                    "prepack launch") &&
+            hip_ok(zmi_launch_s4_tiles((const uint8_t *)blob, K, N, (uint8_t *)blob + blob_bytes, stream()), "s4 tiles launch") &&
             hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize");   // the widened copy is freed next
   (void)hipFree(wide);
   if (!ok) { (void)hipFree(blob); return nullptr; }
@@ -362,6 +368,7 @@ const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64
     (void)hipFree(g_cache[old].blob);
     g_cache.erase(old);
   }
+  *tiles_s4 = (const uint8_t *)blob + blob_bytes;
   return (const uint8_t *)blob;
 }
 

@@ -79,6 +79,7 @@ struct ZmiFusedQuant {
   int32_t user_dt;
   unsigned int *counter;  // device counter, monotonically increasing across launches
   unsigned int target;    // value the counter reaches when all M rows of this launch are published
+  int32_t per_row;        // per-group kernels only: one scale per row (scales[row]) stands for all its groups
 };
 
 int zmi_smallm_grid(const ZmiProblem &p);
@@ -91,10 +92,15 @@ hipError_t zmi_launch_gemm_smallm(const ZmiProblem &p, const ZmiEpilogue &epi, h
 bool zmi_pergroup_group_size_ok(int64_t gs);
 struct ZmiFusedQuant;
 // fq != null (decode-shaped problems only): the per-group quantization of the M rows is part of the launch
+// tiles_s4 != null (widened s4 weights): decode-shaped problems with K >= 1024 stream the 4-bit tiles instead of the blob
 hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
-                                    hipStream_t stream);
-// true when the launch above takes the decode-shaped kernel (up to 16 rows, K = 512 .. 4096 in whole eighths, G <= 64)
+                                    hipStream_t stream, const uint8_t *tiles_s4 = nullptr);
+// true when the launch above takes the decode-shaped kernel (up to 16 rows, K = 512 .. 4096 in whole eighths)
 bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G);
+// true when it would stream 4-bit tiles if it had them
+bool zmi_pergroup_s4_shape(const ZmiProblem &p, int G);
+// 4-bit tiles of a blob of widened s4 weights (zmi_s4_tiles_bytes(K, N) bytes)
+hipError_t zmi_launch_s4_tiles(const uint8_t *blob, int64_t K, int64_t N, uint8_t *out, hipStream_t stream);
 // per (row, group) dynamic quantization of bf16 / f32 rows: s8 rows (ld ldq), f32 scales {M,G} and an
 // optional copy of the scales in the caller's buffer (f32 or bf16)
 hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
