@@ -111,7 +111,8 @@ typedef struct zmi_batch_params_t {
 
 /* matmul_params (matmul/lowoha_common.hpp:145-227), flattened. */
 typedef struct zmi_matmul_params_t {
-  int32_t dt_src, dt_wei, dt_dst, dt_bias, dt_compute;  /* matmul_data_types */
+  int32_t dt_src, dt_wei, dt_dst, dt_bias, dt_compute;  /* matmul_data_types; dt_wei: s8, or s4 for W4A8 (bf16 src, dynamic_quant,
+                                                          * s8 compute, bf16 dst: lowoha_matmul_utils.cpp:72-176) */
   int32_t n_postops;
   const zmi_post_op_t *postops;
   zmi_quant_t src_scale, wei_scale, dst_scale, src_zp, wei_zp, dst_zp;

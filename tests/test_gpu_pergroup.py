@@ -276,3 +276,103 @@ def test_group_dynamic_quant_per_token_and_per_group(zo, G):
         assert np.array_equal(H.to_host(keep[3 * i + 1])[:M, :K], q[:M])
         assert np.array_equal(H.to_host(keep[3 * i + 2])[:M * G], np.asarray(s).reshape(-1)[:M * G])
         assert np.all(H.to_host(keep[3 * i + 1])[:, K:] == 0)          # padding bytes of dst are left alone
+
+
+def test_grouped_call_with_per_group_ggml_and_s4_experts(zo):
+    """group_matmul_direct with experts the grouped kernels do not take -- per-group scales on static s8 rows, per-group
+    dynamic quantization, GGML Q8_0 packed weights, W4A8 -- runs them on the matmul_direct path (reference:
+    group_matmul/group_matmul_dispatch.cpp:472-515, group_matmul_direct.cpp:1222-1260); followed here by the
+    weighted reduce over the f32 expert outputs.  A fused MoE or gated activation on top is refused."""
+    rng = np.random.default_rng(77)
+    K, N, T = 256, 48, 6
+    G = K // 32
+    E = 3
+    # expert 0: static s8 rows, {T,G} x {G,N} f32 scales
+    a0 = rng.integers(-128, 128, (T, K), dtype=np.int8)
+    w0 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    ss0 = rng.uniform(0.005, 0.03, (T, G)).astype(np.float32)
+    ws0 = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    p0 = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
+    ss0_d, ws0_d = H.to_dev(ss0), H.to_dev(ws0)
+    p0.src_scale = lowoha.QuantParam(ss0_d, capi.DT_F32, (T, G))
+    p0.wei_scale = lowoha.QuantParam(ws0_d, capi.DT_F32, (G, N))
+    # expert 1: bf16 rows quantized per group, f32 out
+    x1 = H.bf16_bits(rng.standard_normal((T, K)).astype(np.float32))
+    w1 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    ws1 = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    ws1_d = H.to_dev(ws1)
+    p1 = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_F32, compute=capi.DT_S8)
+    p1.dynamic_quant = True
+    p1.src_scale = lowoha.QuantParam(None, capi.DT_F32, (T, G))
+    p1.wei_scale = lowoha.QuantParam(ws1_d, capi.DT_F32, (G, N))
+    # expert 2: static s8 rows, GGML Q8_0 packed weights ([N][K/32] blocks of {fp16 d, int8 qs[32]})
+    a2 = rng.integers(-128, 128, (T, K), dtype=np.int8)
+    rows2 = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    d16 = rng.uniform(1e-3, 0.02, (N, G)).astype(np.float16)
+    blk = np.zeros((N, G, 34), dtype=np.uint8)
+    blk[:, :, :2] = d16.view(np.uint16).reshape(N, G, 1).view(np.uint8)
+    blk[:, :, 2:] = rows2.reshape(N, G, 32).view(np.uint8)
+    packed2 = blk.reshape(-1)
+    ss2 = rng.uniform(0.005, 0.03, (T, G)).astype(np.float32)
+    ss2_d = H.to_dev(ss2)
+    p2 = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
+    p2.src_scale = lowoha.QuantParam(ss2_d, capi.DT_F32, (T, G))
+    p2.pack_format_b = 1
+
+    srcs = [H.to_dev(a0), H.to_dev(x1), H.to_dev(a2)]
+    weis = [H.to_dev(w0), H.to_dev(w1), H.to_dev(packed2)]
+    dst = [torch.zeros((T, N), dtype=torch.float32, device=H.DEV) for _ in range(E)]
+    ids = [(t % E, (t + 1) % E) for t in range(T)]
+    rp = [dst[e].data_ptr() + t * N * 4 for t in range(T) for e in ids[t]]
+    tw_h = rng.uniform(0.2, 0.8, (T, 2)).astype(np.float32)
+    out = torch.zeros((T, N), dtype=torch.float32, device=H.DEV)
+    pp = lowoha.MoePostop(T, 2, out, N, H.to_dev(tw_h), rp)
+    args = (["r"] * E, [False] * E, [False, False, True], [T] * E, [N] * E, [K] * E, [1.0] * E,
+            srcs, [K] * E, weis, [N, N, K], [None] * E, [0.0] * E, dst, [N] * E, [True] * E, [p0, p1, p2])
+    st = lowoha.group_matmul_direct(*args, moe_postop=pp)
+    assert st == capi.SUCCESS, lowoha.last_error()
+
+    want = []
+    keep = []
+    st, y, _, _ = zo.matmul_int8(a0, w0, H.host_params(p0, src_scale=ss0, wei_scale=ws0).flat(keep), T, N, K)
+    assert st == capi.SUCCESS
+    want.append(y)
+    st, y, _, _ = zo.matmul_int8(x1, w1, H.host_params(p1, src_scale=None, wei_scale=ws1).flat(keep), T, N, K)
+    assert st == capi.SUCCESS
+    want.append(y)
+    st, y, _, _ = zo.matmul_int8(a2, packed2, H.host_params(p2, src_scale=ss2).flat(keep), T, N, K, transB=True, ldb=K)
+    assert st == capi.SUCCESS
+    want.append(y)
+    for e in range(E):
+        assert np.array_equal(H.to_host(dst[e]), want[e])
+    red = zo.moe_reduce([want[e][t] for t in range(T) for e in ids[t]], tw_h, capi.DT_F32, N)
+    assert np.array_equal(H.to_host(out), red)
+
+    # refused on top of a gated activation
+    st = lowoha.group_matmul_direct(*args, gated_act=capi.ACT_SILU_AND_MUL)
+    assert st == capi.UNIMPLEMENTED
+
+    # two W4A8 experts (bf16 rows, packed s4 weights, bf16 out), ragged row counts
+    Ms = [5, 9]
+    xs, w4s, wss, ps, dsts = [], [], [], [], []
+    for e, m in enumerate(Ms):
+        xs.append(H.bf16_bits(rng.standard_normal((m, K)).astype(np.float32)))
+        codes = rng.integers(0, 256, K * N // 2, dtype=np.uint8)
+        w4s.append(codes)
+        wss.append(rng.uniform(0.01, 0.1, (G, N)).astype(np.float32))
+        pe = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S4, dst=capi.DT_BF16, compute=capi.DT_S8)
+        pe.dynamic_quant = True
+        pe.src_scale = lowoha.QuantParam(None, capi.DT_F32, (m, 1))
+        pe.wei_scale = lowoha.QuantParam(H.to_dev(wss[e]), capi.DT_F32, (G, N))
+        ps.append(pe)
+        dsts.append(torch.zeros((m, N), dtype=torch.bfloat16, device=H.DEV))
+    st = lowoha.group_matmul_direct(["r"] * 2, [False] * 2, [False] * 2, Ms, [N] * 2, [K] * 2, [1.0] * 2,
+                                    [H.to_dev(x) for x in xs], [K] * 2, [H.to_dev(w) for w in w4s], [N] * 2, [None] * 2,
+                                    [0.0] * 2, dsts, [N] * 2, [True] * 2, ps)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for e, m in enumerate(Ms):
+        st, y, _, _ = zo.matmul_int8(xs[e], w4s[e], H.host_params(ps[e], src_scale=None, wei_scale=wss[e]).flat(keep), m, N, K,
+                                     ldb=N)
+        assert st == capi.SUCCESS
+        assert np.array_equal(H.to_host(dsts[e]), y)
+    capi.load().zmi_clear_weight_cache()

@@ -288,6 +288,40 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     return ZMI_SUCCESS;
   }
 
+  // ---- experts the grouped kernels do not take: per-group scales ({M,G} source with {G,N} weight scales), GGML
+  // Q8_0 packed weights and W4A8 (s4 weights).  The reference runs them through the same per-expert sym-quant
+  // GEMM as matmul_direct (group_matmul/group_matmul_dispatch.cpp:472-515, group_matmul_direct.cpp:1222-1260);
+  // here a plain grouped call (no fused MoE, no gated activation) runs such experts one by one on the
+  // matmul_direct path, then the weighted reduce if there is one. ----
+  const bool run_act = gated_act != ZMI_ACT_NONE;
+  bool one_by_one = false;
+  for (size_t i = 0; i < num_ops; ++i) {
+    if (a.M[i] <= 0) continue;
+    const zmi_matmul_params_t &pi = a.params[i];
+    int64_t sn = 1;
+    for (int d = 0; d < pi.src_scale.ndims; ++d) sn *= pi.src_scale.dims[d];
+    const bool has_scale_dims = pi.src_scale.ndims > 0 && (pi.src_scale.buff || pi.dynamic_quant);
+    if (pi.dt_wei == ZMI_DT_S4 || pi.pack_format_b == 1 || (has_scale_dims && sn > a.M[i] && sn % a.M[i] == 0))
+      one_by_one = true;
+  }
+  if (one_by_one) {
+    if (fused_moe || run_act) {
+      set_error("per-group scales, GGML-packed and s4 weights are implemented for plain grouped calls only (no fused_moe / gated_act)");
+      return ZMI_UNIMPLEMENTED;
+    }
+    for (size_t i = 0; i < num_ops; ++i) {
+      if (a.M[i] <= 0) continue;
+      zmi_batch_params_t bp;
+      zmi_batch_params_init(&bp);
+      st = zmi_matmul_direct(a.layout[i], a.transA[i], a.transB[i], a.M[i], a.N[i], a.K[i], a.alpha[i], a.src[i], a.lda[i],
+                             a.weight[i], a.ldb[i], a.bias[i], a.beta[i], a.dst[i], a.ldc[i], a.is_weights_const[i], &bp,
+                             &a.params[i]);
+      if (st != ZMI_SUCCESS) return st;
+    }
+    if (moe_postop) goto postop_only;
+    return ZMI_SUCCESS;
+  }
+
   // ---- per-expert validation through the single-matmul rules ----
   for (size_t i = 0; i < num_ops; ++i) {
     if (a.M[i] <= 0) continue;
@@ -300,7 +334,6 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     if (a.layout[i] != 'r' && a.layout[i] != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
     if (a.params[i].pack_format_b != 0) { set_error("GGML-packed weights are not implemented"); return ZMI_UNIMPLEMENTED; }
   }
-  const bool run_act = gated_act != ZMI_ACT_NONE;
 
   if (!params_uniform(a, num_ops)) {
     // experts disagree on dtypes / post-ops: run them one by one
