@@ -115,9 +115,14 @@ __device__ __forceinline__ void zmi_quant_row(const void *srcv, int8_t *dst, int
 template <bool BF16>
 __global__ __launch_bounds__(QT_THREADS) void zmi_quant_rows_kernel(ZmiQuantMat mat0,
                                                                     const ZmiQuantMat *mats, int n_mat,
-                                                                    int scale_dt) {
+                                                                    int scale_dt, int n_rows) {
   __shared__ float red[QT_THREADS / 64];
-  const int row = blockIdx.x;
+  // Workgroups are dealt round robin to the 8 XCDs, whose L2s are private.  Runs of 32 rows go to one XCD: in
+  // fragment-major output 32 consecutive rows fill whole cache lines between them, 8 bytes per row and line,
+  // and only one L2 can merge them before they go to memory.  (The grid is a multiple of 256.)
+  const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+  const int row = (xcd + 8 * (j / 32)) * 32 + j % 32;
+  if (row >= n_rows) return;
   ZmiQuantMat m = mat0;
   if (mats) {
     // find the matrix that owns this global row (row_start is ascending)
@@ -330,11 +335,11 @@ hipError_t zmi_launch_quant_rows(const void *src, int32_t src_dt, int64_t M, int
     return hipGetLastError();
   }
   if (src_dt == ZMI_DT_BF16)
-    hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, m,
-                       (const ZmiQuantMat *)nullptr, 1, scale_dt);
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)((M + 255) / 256 * 256)), dim3(QT_THREADS), 0, stream, m,
+                       (const ZmiQuantMat *)nullptr, 1, scale_dt, (int)M);
   else
-    hipLaunchKernelGGL(zmi_quant_rows_kernel<false>, dim3((unsigned)M), dim3(QT_THREADS), 0, stream, m,
-                       (const ZmiQuantMat *)nullptr, 1, scale_dt);
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<false>, dim3((unsigned)((M + 255) / 256 * 256)), dim3(QT_THREADS), 0, stream, m,
+                       (const ZmiQuantMat *)nullptr, 1, scale_dt, (int)M);
   return hipGetLastError();
 }
 
@@ -355,11 +360,11 @@ hipError_t zmi_launch_quant_group(const ZmiQuantMat *mats_dev, int n_mat, int64_
     return hipGetLastError();
   }
   if (src_dt == ZMI_DT_BF16)
-    hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)total_rows), dim3(QT_THREADS), 0,
-                       stream, m0, mats_dev, n_mat, scale_dt);
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<true>, dim3((unsigned)((total_rows + 255) / 256 * 256)), dim3(QT_THREADS), 0,
+                       stream, m0, mats_dev, n_mat, scale_dt, (int)total_rows);
   else
-    hipLaunchKernelGGL(zmi_quant_rows_kernel<false>, dim3((unsigned)total_rows), dim3(QT_THREADS), 0,
-                       stream, m0, mats_dev, n_mat, scale_dt);
+    hipLaunchKernelGGL(zmi_quant_rows_kernel<false>, dim3((unsigned)((total_rows + 255) / 256 * 256)), dim3(QT_THREADS), 0,
+                       stream, m0, mats_dev, n_mat, scale_dt, (int)total_rows);
   return hipGetLastError();
 }
 
