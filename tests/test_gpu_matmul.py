@@ -221,3 +221,38 @@ def test_row_groups_s32_accumulators_bit_exact(zo, small_m_kernel, M, K, N):
     assert small_m_kernel in lowoha.last_kernel() or "ring" in lowoha.last_kernel()
     want = (a.astype(np.int64) - 77) @ w.astype(np.int64)
     assert np.array_equal(H.to_host(dst).astype(np.int64), want)
+
+
+@pytest.mark.parametrize("M,K,N,force", [(40, 520, 96, True), (64, 4096, 1000, True), (33, 256, 300, True),
+                                         (48, 256, 10752, False), (64, 128, 8192, False)])
+def test_four_row_groups_per_workgroup_below_65_rows(zo, quant_launch, M, K, N, force, monkeypatch):
+    """33 .. 64 rows on the decode kernel's four-groups-per-workgroup form (weights kept in registers for all row
+    groups): taken by itself when the one-group form would need more than ~1000 workgroups, forced here on the small
+    shapes through ZMI_DECODE_RPW."""
+    if force:
+        monkeypatch.setenv("ZMI_DECODE_RPW", "4")
+    rng = np.random.default_rng(M * 17 + N)
+    x = H.gen_bf16_normal(rng, (M, K))
+    w = H.gen_weights(rng, K, N)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    x_d, w_d, ws_d = H.to_dev(x), H.to_dev(w), H.to_dev(ws)
+    blob = H.prepack(w_d, K, N)
+    scales_d = torch.zeros(M, dtype=torch.float32, device=H.DEV)
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_F32, compute=capi.DT_S8, bias=capi.DT_F32)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(scales_d, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.mem_format_b = "r"
+    p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+    dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, blob, N, H.to_dev(b), 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert "decode_lds_rows" in lowoha.last_kernel()
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    ph.mem_format_b = "n"
+    keep = []
+    st, want, _, scales = zo.matmul_int8(x, w, ph.flat(keep), M, N, K, bias=b, want_scales=True)
+    assert st == capi.SUCCESS
+    assert np.array_equal(H.to_host(scales_d), scales)
+    assert np.array_equal(H.to_host(dst), want)      # no activation: bit-identical f32

@@ -259,7 +259,12 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
   // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at
   // 32 / 64 rows, N = K = 4096, against 13 / 20 us with 64); above that, 64 rows per workgroup
   // keep the weights in registers for four row groups (128 rows: 23 against 27 us)
-  const int rpw = p.M <= 64 ? 1 : 4;
+  // (33 .. 64 rows whose one-group workgroups would not all be resident -- more than ~1000 of them -- also take the
+  // four-group form: 48 / 64 rows at N = 14336: 27.0 / 30.2 against 28.1 / 32.3 us; 64 rows at K = 2048, N = 8192: 17.7
+  // against 20.3 us; ZMI_DECODE_RPW = 1 | 4 overrides the choice above 16 rows)
+  int rpw = p.M <= 64 ? 1 : 4;
+  if (p.M > 32 && (int64_t)n_blk * ((p.M + 15) / 16) > 1000) rpw = 4;
+  if (const char *e = getenv("ZMI_DECODE_RPW")) { const int v = atoi(e); if ((v == 1 || v == 4) && p.M > 16) rpw = v; }
   const int n_rg = (p.M + 16 * rpw - 1) / (16 * rpw);
   // (several workgroups per column block: a multiple of 8, for the renumbering over the XCDs)
   const int grid = n_rg == 1 ? n_blk : (n_blk * n_rg + 7) / 8 * 8;
