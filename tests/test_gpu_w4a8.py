@@ -141,3 +141,30 @@ def test_w4a8_rejections(zo):
     assert call(wdims=(32, N)) == capi.FAILURE             # groups of 2
     assert call(fmt="r") == capi.FAILURE                   # no prepacked form of s4 weights
     capi.load().zmi_clear_weight_cache()
+
+
+def test_w4a8_reference_example_recipe(zo):
+    """The reference's W4A8 example (examples/lowoha_matmul_example.cpp:370-457): M=8 K=128 N=64, groups of 32, bf16
+    ones as activations, every s4 code 1, bf16 weight scales 1 + 0.05 g, bf16 {M,1} source-scale buffer (overwritten
+    by the dynamic quantization).  Every row quantizes to 127 with scale 1/127, every group sum is 32 * 127, so the
+    output is 32 * sum_g bf16(1 + 0.05 g) = 137.5 up to f32 rounding: 137 or 138 in bf16."""
+    M, K, N, G = 8, 128, 64, 4
+    x = np.full((M, K), 0x3F80, dtype=np.uint16)
+    packed = np.full(K * N // 2, 0x11, dtype=np.uint8)
+    ws = H.bf16_bits(np.repeat((1.0 + 0.05 * np.arange(G, dtype=np.float32))[:, None], N, axis=1))
+    sc_d = H.to_dev(H.bf16_bits((0.02 + 0.001 * np.arange(M)).astype(np.float32)))
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S4, dst=capi.DT_BF16, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+    p.src_scale = lowoha.QuantParam(sc_d, capi.DT_BF16, (M, 1))
+    p.wei_scale = lowoha.QuantParam(H.to_dev(ws), capi.DT_BF16, (G, N))
+    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(x), K, H.to_dev(packed), N, None, 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    got = H.to_host(dst)
+    vals = (got.astype(np.uint32) << 16).view(np.float32)
+    assert np.all((vals == 137.0) | (vals == 138.0)), np.unique(vals)
+    # the computed scales replace the caller's: bf16(1 / 127)
+    want_s = H.bf16_bits(np.full(M, np.float32(1.0) / np.float32(127.0), dtype=np.float32))
+    assert np.array_equal(H.to_host(sc_d), want_s)
+    capi.load().zmi_clear_weight_cache()
