@@ -216,7 +216,8 @@ def main():
 
     def run_decode_per_group(m, gs):
         # the decode call with per-group scales: {M,G} source scales computed by the library, {G,N} weight scales,
-        # G = K / gs; two launches (per-group quantization, per-group GEMM); bytes = the per-token call's + the scales
+        # G = K / gs; one launch (the per-group quantization is part of the decode-shaped GEMM launch); bytes = the
+        # per-token call's + the scales
         G = K_DEC // gs
         blobs = [prepack(rand_w(K_DEC, N_DEC), K_DEC, N_DEC) for _ in range(n_sets)]
         ws = torch.rand((G, N_DEC), device=dev, generator=g) * 0.009 + 0.001
