@@ -3,7 +3,7 @@
 // every call is rejected by validation.  Without it, it runs the deterministic
 // recipe of the reference's int8 example (examples/lowoha_matmul_example.cpp:509-535:
 // w = (i % 7) - 3, a = (i + 17 * iter) % 256) through matmul_direct, with plain and
-// with prepacked weights, and compares the s32 result with a host triple loop.
+// with prepacked weights, and compares the s32 result with a host triple loop; then the reference's W4A8 example.
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -107,9 +107,66 @@ static void gpu_example() {
   hipFree(w_d); hipFree(a_d); hipFree(c_d); hipFree(blob);
 }
 
+// The reference's W4A8 example as its caller writes it (examples/lowoha_matmul_example.cpp:370-457): M = 8, K = 128,
+// N = 64, groups of 32, bf16 ones as activations, every s4 code 1, bf16 weight scales 1 + 0.05 g, a bf16 {M,1}
+// source-scale buffer that the dynamic quantization overwrites.  Every row quantizes to 127 with scale 1/127, so the
+// output is 32 * sum_g bf16(1 + 0.05 g) = 137.5 up to f32 rounding: 137 or 138 in bf16 (0x4309 / 0x430a).
+static uint16_t to_bf16(float f) {
+  uint32_t u; std::memcpy(&u, &f, 4);
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+static void gpu_w4a8_example() {
+  const int M = 8, K = 128, N = 64, G = 4;
+  std::vector<uint16_t> src_scale(M), wei_scale(G * N), input(M * K, 0x3F80), output(M * N, 0);
+  for (int m = 0; m < M; ++m) src_scale[m] = to_bf16(0.02f + 0.001f * m);
+  for (int g = 0; g < G; ++g)
+    for (int n = 0; n < N; ++n) wei_scale[g * N + n] = to_bf16(1.0f + 0.05f * g);
+  std::vector<int8_t> weights((K * N + 1) / 2, (int8_t)0x11);
+  void *ss_d, *ws_d, *w_d, *x_d, *y_d;
+  hipMalloc(&ss_d, M * 2); hipMalloc(&ws_d, G * N * 2); hipMalloc(&w_d, weights.size()); hipMalloc(&x_d, M * K * 2); hipMalloc(&y_d, M * N * 2);
+  hipMemcpy(ss_d, src_scale.data(), M * 2, hipMemcpyHostToDevice);
+  hipMemcpy(ws_d, wei_scale.data(), G * N * 2, hipMemcpyHostToDevice);
+  hipMemcpy(w_d, weights.data(), weights.size(), hipMemcpyHostToDevice);
+  hipMemcpy(x_d, input.data(), M * K * 2, hipMemcpyHostToDevice);
+  matmul_params params;
+  params.dtypes.src = data_type_t::bf16;
+  params.dtypes.wei = data_type_t::s4;
+  params.dtypes.dst = data_type_t::bf16;
+  params.dtypes.bias = data_type_t::none;
+  params.dtypes.compute = data_type_t::s8;
+  params.dynamic_quant = true;
+  params.lowoha_algo = zendnnl::ops::matmul_algo_t::aocl_dlp_blocked;
+  params.quant_params.src_scale.buff = ss_d;
+  params.quant_params.src_scale.dt = data_type_t::bf16;
+  params.quant_params.src_scale.dims = {M, 1};
+  params.quant_params.wei_scale.buff = ws_d;
+  params.quant_params.wei_scale.dt = data_type_t::bf16;
+  params.quant_params.wei_scale.dims = {G, N};
+  matmul_batch_params_t batch_params;
+  CHECK(matmul_direct('r', false, false, M, N, K, 1.0f, x_d, K, w_d, N, nullptr, 0.0f, y_d, N, true, batch_params, params) ==
+        status_t::success);
+  hipMemcpy(output.data(), y_d, M * N * 2, hipMemcpyDeviceToHost);
+  hipMemcpy(src_scale.data(), ss_d, M * 2, hipMemcpyDeviceToHost);
+  int bad = 0;
+  for (int i = 0; i < M * N; ++i) if (output[i] != 0x4309 && output[i] != 0x430a) ++bad;
+  CHECK(bad == 0);
+  for (int m = 0; m < M; ++m) CHECK(src_scale[m] == to_bf16(1.0f / 127.0f));
+  // the validator's outcomes for this path (lowoha_matmul_utils.cpp:72-176)
+  params.dtypes.dst = data_type_t::f32;
+  CHECK(matmul_direct('r', false, false, M, N, K, 1.0f, x_d, K, w_d, N, nullptr, 0.0f, y_d, N, true, batch_params, params) ==
+        status_t::failure);
+  params.dtypes.dst = data_type_t::bf16;
+  params.dynamic_quant = false;    // bf16 x s4 without dynamic quantization is weight-only quantization: not this path
+  CHECK(matmul_direct('r', false, false, M, N, K, 1.0f, x_d, K, w_d, N, nullptr, 0.0f, y_d, N, true, batch_params, params) ==
+        status_t::unimplemented);
+  clear_matmul_weight_caches();
+  hipFree(ss_d); hipFree(ws_d); hipFree(w_d); hipFree(x_d); hipFree(y_d);
+}
+
 int main(int argc, char **argv) {
   validate_only();
-  if (!(argc > 1 && std::strcmp(argv[1], "--validate-only") == 0)) gpu_example();
+  if (!(argc > 1 && std::strcmp(argv[1], "--validate-only") == 0)) { gpu_example(); gpu_w4a8_example(); }
   std::printf(fails ? "adapter example: %d check(s) failed\n" : "adapter example: ok\n", fails);
   return fails ? 1 : 0;
 }
