@@ -518,6 +518,13 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
       }
       dn = 1;
     }
+    if (p->src_scale.dt == ZMI_DT_BF16) {
+      /* the computed f32 scales are narrowed into the scale buffer's dtype (write_scale / float_to_bf16 =
+       * bfloat16_t::f32_to_bf16_val, lowoha_operators/reorder/lowoha_reorder_utils.cpp:600-628, :835-856) and the
+       * GEMM reads the narrowed values back; the rows above were quantized with the f32 scales */
+      const int64_t ns = dn == 1 ? M : dn;
+      for (int64_t i = 0; i < ns; ++i) sbuf[i] = zo_bf16_to_f32(zo_f32_to_bf16_rne(sbuf[i]));
+    }
     if (c->scale_out) memcpy(c->scale_out, sbuf, sizeof(float) * (size_t)dn);
     if (w4a8_groups > 1 && dn <= M) {
       /* broadcast_w4a8_src_scale, backends/aocl/aocl_kernel.cpp:167-236: compact per-tensor / per-token

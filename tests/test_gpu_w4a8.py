@@ -168,3 +168,43 @@ def test_w4a8_reference_example_recipe(zo):
     want_s = H.bf16_bits(np.full(M, np.float32(1.0) / np.float32(127.0), dtype=np.float32))
     assert np.array_equal(H.to_host(sc_d), want_s)
     capi.load().zmi_clear_weight_cache()
+
+
+@pytest.mark.parametrize("with_buffer", [True, False])
+@pytest.mark.parametrize("wei,M,K,N,G,sdims", [
+    (capi.DT_S4, 16, 4096, 200, 32, "token"), (capi.DT_S4, 16, 4096, 72, 32, "group"), (capi.DT_S4, 40, 512, 64, 8, "token"),
+    (capi.DT_S4, 9, 256, 48, 4, "group"),
+    (capi.DT_S8, 16, 4096, 320, 1, "token"), (capi.DT_S8, 4, 512, 96, 1, "token"), (capi.DT_S8, 100, 1024, 64, 1, "token"),
+    (capi.DT_S8, 300, 256, 300, 1, "token"), (capi.DT_S8, 16, 4096, 64, 32, "group"), (capi.DT_S8, 33, 512, 40, 8, "group")])
+def test_bf16_source_scale_dtype_is_what_the_gemm_multiplies_by(zo, wei, M, K, N, G, sdims, with_buffer):
+    """src_scale.dt = bf16 (as in the reference's W4A8 example): the computed f32 scales are narrowed into the scale
+    buffer -- the caller's, or the library's own of that dtype -- and the GEMM reads the narrowed values, while the
+    rows are quantized with the f32 scales (lowoha_reorder_utils.cpp:600-628, 835-856; reorder_quantization.cpp:103-117).
+    Covers W4A8 and s8 weights, per-token and per-group scales, the fused decode launches and the separate ones."""
+    rng = np.random.default_rng(M + K + N + G + int(with_buffer))
+    x = H.bf16_bits((rng.standard_normal((M, K)) * 2).astype(np.float32))
+    if wei == capi.DT_S4:
+        w = rng.integers(0, 256, K * N // 2, dtype=np.uint8)
+        ws = rng.uniform(0.01, 0.1, (G, N)).astype(np.float32)
+    else:
+        w = H.gen_weights(rng, K, N)
+        ws = rng.uniform(0.001, 0.01, (G, N)).astype(np.float32)
+    dims = (M, 1) if sdims == "token" else (M, G)
+    n_sc = int(np.prod(dims))
+    sc_d = torch.zeros(n_sc, dtype=torch.bfloat16, device=H.DEV) if with_buffer else None
+    dst_dt = capi.DT_BF16 if wei == capi.DT_S4 else capi.DT_F32
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=wei, dst=dst_dt, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(sc_d, capi.DT_BF16, dims)
+    p.wei_scale = lowoha.QuantParam(H.to_dev(ws), capi.DT_F32, (G, N) if G > 1 else (1, N))
+    dst = torch.zeros((M, N), dtype=torch.bfloat16 if dst_dt == capi.DT_BF16 else torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(x), K, H.to_dev(w), N, None, 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    keep = []
+    st, want, _, scales = zo.matmul_int8(x, w, ph.flat(keep), M, N, K, ldb=N, want_scales=True, n_scales=max(n_sc, M))
+    assert st == capi.SUCCESS
+    if with_buffer:
+        assert np.array_equal(H.to_host(sc_d), H.bf16_bits(scales[:n_sc]))      # (the oracle's are bf16 values held in f32)
+    assert np.array_equal(H.to_host(dst), want), lowoha.last_kernel()
+    capi.load().zmi_clear_weight_cache()

@@ -591,7 +591,8 @@ __global__ __launch_bounds__(256) void zmi_quant_groups_kernel(const void *x, in
   if (s < 1e-10f) s = 1e-10f;
   const float inv = __fdiv_rn(1.0f, s);
   if (lane == 0) {
-    scales[item] = s;
+    // (the GEMM multiplies by the scale as the scale buffer's dtype holds it: see zmi_fused_scale_as_stored)
+    scales[item] = user_dt == ZMI_DT_BF16 ? zmi_bf16_to_f32(zmi_f32_to_bf16_rne(s)) : s;
     if (user_scales) {
       if (user_dt == ZMI_DT_BF16) ((uint16_t *)user_scales)[item] = zmi_f32_to_bf16_rne(s);
       else ((float *)user_scales)[item] = s;

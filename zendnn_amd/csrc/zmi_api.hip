@@ -602,7 +602,8 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = 1;
     } else if (dyn_scale_n == M && M > 1) {
       void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
-      if (!p.src_scale.buff) sdt = ZMI_DT_F32;
+      // (without a caller buffer the scales live in scratch, in the dtype the params name: the reference allocates
+      // its own buffer of that dtype, reorder_quantization.cpp:103-117, and its GEMM reads the narrowed values back)
       if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, frag_kpad, scale_out, sdt, stream()), "quant launch"))
         return ZMI_FAILURE;
       ep.src_scale.buff = scale_out;

@@ -13,6 +13,13 @@
 // would write back and invalidate whole caches in the middle of the weight
 // stream.  Readers on other XCDs miss in their own L2 (invalidated when the
 // kernel started) and fetch the fresh bytes.
+// The scale the GEMM multiplies by is the one the scale buffer holds: with a bf16 scale dtype the reference narrows the
+// computed f32 scale (bfloat16_t::f32_to_bf16_val, lowoha_operators/reorder/lowoha_reorder_utils.cpp:600-628) and its
+// GEMM reads the narrowed value back, while the rows were quantized with the f32 scale.
+static __device__ __forceinline__ float zmi_fused_scale_as_stored(const ZmiFusedQuant &fq, float s) {
+  return fq.user_dt == ZMI_DT_BF16 ? zmi_bf16_to_f32(zmi_f32_to_bf16_rne(s)) : s;
+}
+
 static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int K, float *red) {
   const int t = threadIdx.x, nt = blockDim.x;
   const bool bf16 = fq.x_dt == ZMI_DT_BF16;
@@ -56,7 +63,7 @@ static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int
   if (s < 1e-10f) s = 1e-10f;
   const float inv = __fdiv_rn(1.0f, s);
   if (t == 0) {
-    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(zmi_fused_scale_as_stored(fq, s)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (fq.user_scales) {
       if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[row] = zmi_f32_to_bf16_rne(s);
       else ((float *)fq.user_scales)[row] = s;
@@ -125,7 +132,7 @@ static __device__ void zmi_fused_quant_row_wave(const ZmiFusedQuant &fq, int row
   if (s < 1e-10f) s = 1e-10f;
   const float inv = __fdiv_rn(1.0f, s);
   if (lane == 0) {
-    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store((unsigned int *)&fq.scales[row], __float_as_uint(zmi_fused_scale_as_stored(fq, s)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (fq.user_scales) {
       if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[row] = zmi_f32_to_bf16_rne(s);
       else ((float *)fq.user_scales)[row] = s;
@@ -204,7 +211,7 @@ static __device__ void zmi_fused_quant_row_groups(const ZmiFusedQuant &fq, int r
     if (t * 8 < K) {
       const int g = t * 8 / gs;
       if (t % lpg == 0) {
-        __hip_atomic_store((unsigned int *)&fq.scales[(int64_t)row * G + g], __float_as_uint(s), __ATOMIC_RELAXED,
+        __hip_atomic_store((unsigned int *)&fq.scales[(int64_t)row * G + g], __float_as_uint(zmi_fused_scale_as_stored(fq, s)), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
         if (fq.user_scales) {
           if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[(int64_t)row * G + g] = zmi_f32_to_bf16_rne(s);
@@ -237,7 +244,7 @@ static __device__ void zmi_fused_quant_row_groups(const ZmiFusedQuant &fq, int r
     if (s < 1e-10f) s = 1e-10f;
     const float inv = __fdiv_rn(1.0f, s);
     if (lane == 0) {
-      __hip_atomic_store((unsigned int *)&fq.scales[(int64_t)row * G + g], __float_as_uint(s), __ATOMIC_RELAXED,
+      __hip_atomic_store((unsigned int *)&fq.scales[(int64_t)row * G + g], __float_as_uint(zmi_fused_scale_as_stored(fq, s)), __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
       if (fq.user_scales) {
         if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[(int64_t)row * G + g] = zmi_f32_to_bf16_rne(s);
