@@ -310,3 +310,37 @@ def test_group_of_unrelated_gemms_random_configuration(zo, seed):
         else:
             assert np.array_equal(got, want), f"seed {seed} expert {e}: M={M} K={K} N={N}"
         assert np.all(H.to_host(dsts[e])[:, N:] == 0)
+
+
+@pytest.mark.parametrize("with_buffer", [True, False])
+def test_group_bf16_source_scale_dtype(zo, with_buffer):
+    """Grouped dynamic-quant GEMMs with src_scale.dt = bf16: the scales are narrowed into the caller's buffer or into
+    scratch of that dtype and the GEMM multiplies by the narrowed values (as matmul_direct does)."""
+    rng = np.random.default_rng(91 + int(with_buffer))
+    Ms, K, N = [70, 5, 130], 256, 96
+    E = len(Ms)
+    xs = [H.gen_bf16_normal(rng, (m, K)) for m in Ms]
+    wsrc = [H.gen_weights(rng, K, N) for _ in Ms]
+    wsc = [rng.uniform(0.001, 0.01, N).astype(np.float32) for _ in Ms]
+    sc_d = [torch.zeros(m, dtype=torch.bfloat16, device=H.DEV) if with_buffer else None for m in Ms]
+    wsc_d = [H.to_dev(s) for s in wsc]
+    params = []
+    for e, m in enumerate(Ms):
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_F32, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(sc_d[e], capi.DT_BF16, (m, 1))
+        p.wei_scale = lowoha.QuantParam(wsc_d[e], capi.DT_F32, (1, N))
+        params.append(p)
+    dst = [torch.zeros((m, N), dtype=torch.float32, device=H.DEV) for m in Ms]
+    st = lowoha.group_matmul_direct(["r"] * E, [False] * E, [False] * E, Ms, [N] * E, [K] * E, [1.0] * E,
+                                    [H.to_dev(x) for x in xs], [K] * E, [H.to_dev(w) for w in wsrc], [N] * E, [None] * E,
+                                    [0.0] * E, dst, [N] * E, [True] * E, params)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    keep = []
+    for e, m in enumerate(Ms):
+        ph = H.host_params(params[e], src_scale=None, wei_scale=wsc[e])
+        st, want, _, scales = zo.matmul_int8(xs[e], wsrc[e], ph.flat(keep), m, N, K, want_scales=True)
+        assert st == capi.SUCCESS
+        if with_buffer:
+            assert np.array_equal(H.to_host(sc_d[e]), H.bf16_bits(scales))
+        assert np.array_equal(H.to_host(dst[e]), want)

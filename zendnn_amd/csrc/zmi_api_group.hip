@@ -438,7 +438,8 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
         mats.push_back(m);
         A1[i] = m.dst; lda1[i] = kp; s1[i] = m.scale;
       }
-      s1_dt = (p0.src_scale.buff && p0.src_scale.dt != ZMI_DT_NONE) ? p0.src_scale.dt : ZMI_DT_F32;
+      // (the dtype the params name, whether the scales go to a caller's buffer or to scratch: the GEMM reads them back)
+      s1_dt = p0.src_scale.dt != ZMI_DT_NONE ? p0.src_scale.dt : ZMI_DT_F32;
       if (s1_dt != ZMI_DT_F32 && s1_dt != ZMI_DT_BF16) { set_error("source scale must be f32 or bf16"); return ZMI_FAILURE; }
       r0 = renumber_rows8(mats, p0.dt_src, r0, &rows8);
       const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
