@@ -173,7 +173,8 @@ def test_w4a8_reference_example_recipe(zo):
 @pytest.mark.parametrize("with_buffer", [True, False])
 @pytest.mark.parametrize("wei,M,K,N,G,sdims", [
     (capi.DT_S4, 16, 4096, 200, 32, "token"), (capi.DT_S4, 16, 4096, 72, 32, "group"), (capi.DT_S4, 40, 512, 64, 8, "token"),
-    (capi.DT_S4, 9, 256, 48, 4, "group"),
+    (capi.DT_S4, 9, 256, 48, 4, "group"), (capi.DT_S4, 1, 256, 254, 16, "token"), (capi.DT_S4, 1, 4096, 64, 32, "token"),
+    (capi.DT_S8, 1, 520, 96, 1, "token"), (capi.DT_S8, 1, 8192, 40, 1, "token"),
     (capi.DT_S8, 16, 4096, 320, 1, "token"), (capi.DT_S8, 4, 512, 96, 1, "token"), (capi.DT_S8, 100, 1024, 64, 1, "token"),
     (capi.DT_S8, 300, 256, 300, 1, "token"), (capi.DT_S8, 16, 4096, 64, 32, "group"), (capi.DT_S8, 33, 512, 40, 8, "group")])
 def test_bf16_source_scale_dtype_is_what_the_gemm_multiplies_by(zo, wei, M, K, N, G, sdims, with_buffer):

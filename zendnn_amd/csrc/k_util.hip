@@ -142,3 +142,22 @@ hipError_t zmi_launch_broadcast_scales(const void *src, int32_t dt, int per_tens
                      per_tensor, M, G, out);
   return hipGetLastError();
 }
+
+// ---- f32 scales -> the values a bf16 scale buffer holds ---------------------------------------------
+// The reference narrows computed scales into the buffer's dtype and its GEMM reads them back
+// (lowoha_operators/reorder/lowoha_reorder_utils.cpp:600-628): sc[i] becomes bf16(sc[i]) as f32 for i < n, and the
+// first n_user narrowed values go to the caller's bf16 buffer when there is one.
+__global__ __launch_bounds__(256) void zmi_narrow_scales_kernel(float *sc, int64_t n, uint16_t *user, int64_t n_user) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const uint16_t h = zmi_f32_to_bf16_rne(sc[i]);
+  sc[i] = zmi_bf16_to_f32(h);
+  if (user && i < n_user) user[i] = h;
+}
+
+hipError_t zmi_launch_narrow_scales(float *sc, int64_t n, void *user_bf16, int64_t n_user, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(zmi_narrow_scales_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, sc, n,
+                     (uint16_t *)user_bf16, n_user);
+  return hipGetLastError();
+}

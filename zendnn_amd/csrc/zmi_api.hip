@@ -613,8 +613,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       // one scale for the whole tensor; with M == 1 this is the per-token case too
       if (!hip_ok(zmi_launch_quant_tensor(src, p.dt_src, M, K, lda, q, K16, frag_kpad, sc, amax, stream()), "quant launch"))
         return ZMI_FAILURE;
-      if (p.src_scale.buff) {
-        if (sdt != ZMI_DT_F32) { set_error("per-tensor dynamic scale output must be f32"); return ZMI_UNIMPLEMENTED; }
+      if (sdt == ZMI_DT_BF16) {
+        // a bf16 scale dtype: the GEMM multiplies by the narrowed value, which also goes to the caller's buffer
+        if (!hip_ok(zmi_launch_narrow_scales(sc, M, (void *)p.src_scale.buff, 1, stream()), "scale narrowing launch"))
+          return ZMI_FAILURE;
+      } else if (p.src_scale.buff) {
         if (!hip_ok(hipMemcpyAsync((void *)p.src_scale.buff, sc, sizeof(float), hipMemcpyDeviceToDevice, stream()),
                     "hipMemcpyAsync(scale)"))
           return ZMI_FAILURE;

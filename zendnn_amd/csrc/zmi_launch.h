@@ -158,6 +158,8 @@ hipError_t zmi_launch_s4_widen(const void *packed, int64_t rows, int64_t cols, i
 // one f32 / bf16 scale per tensor or per row -> f32 {M, G}
 hipError_t zmi_launch_broadcast_scales(const void *src, int32_t dt, int per_tensor, int64_t M, int64_t G, float *out,
                                        hipStream_t stream);
+// sc[i] = bf16(sc[i]) for i < n; the first n_user narrowed values also go to a caller's bf16 buffer (may be null)
+hipError_t zmi_launch_narrow_scales(float *sc, int64_t n, void *user_bf16, int64_t n_user, hipStream_t stream);
 // u8 / s8 rows (or their transpose) -> fragment-major s8; u8 values are shifted by -128
 hipError_t zmi_launch_repack_frag(const void *src, int64_t M, int64_t K, int64_t ld_src, int trans, int is_u8,
                                   int8_t *dst, hipStream_t stream);
