@@ -20,7 +20,8 @@ def _scales(rng, M, N, G):
 
 
 # (M, K, N, G): group sizes 64, 128, 256, 32 and 16; one row .. several 64-row blocks; ragged N
-SHAPES = [(1, 128, 32, 2), (5, 256, 33, 4), (16, 4096, 512, 32), (16, 1024, 100, 4), (40, 512, 100, 16),
+SHAPES = [(2, 192, 354, 3), (40, 192, 154, 3), (200, 320, 294, 5),   # K = 64 x odd: K_pad holds one chunk past K
+          (1, 128, 32, 2), (5, 256, 33, 4), (16, 4096, 512, 32), (16, 1024, 100, 4), (40, 512, 100, 16),
           (70, 192, 64, 12), (17, 64, 16, 4), (300, 1024, 260, 8), (130, 2048, 48, 32), (3, 32, 5, 2),
           # up to 16 rows with K = 512 .. 4096 and whole groups per eighth of K: the decode-shaped kernel, every
           # (chunks, groups) per wavefront pair it is built for

@@ -165,7 +165,9 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
 #pragma unroll
       for (int j = 0; j < RB; ++j)
         acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(operand(s, j), b[set][s], acc[j], 0, 0, 0);
-      if (CPG ? (s + 1) % (CPG ? CPG : 1) == 0 : (c + 1) % cpg == 0) fold(c / cpg - gb0);
+      // (K_pad may reach one chunk past K: that chunk's weights are zero and its group does not exist -- no fold,
+      // its scales were never staged)
+      if ((CPG ? (s + 1) % (CPG ? CPG : 1) == 0 : (c + 1) % cpg == 0) && c / cpg < G) fold(c / cpg - gb0);
     } else {
 #pragma unroll
       for (int t = 0; t < SUB; ++t) {
