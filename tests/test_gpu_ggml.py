@@ -26,7 +26,7 @@ def _weights(rng, N, K):
     return rows, d16, _pack(rows, d16)
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 64, 16), (16, 4096, 96), (5, 512, 33), (40, 256, 70), (130, 1024, 48)])
+@pytest.mark.parametrize("M,K,N", [(1, 64, 16), (16, 4096, 96), (5, 512, 33), (40, 256, 70), (130, 1024, 48), (7, 32, 50)])
 @pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_BF16])
 def test_static_s8_rows_with_q8_0_weights(zo, M, K, N, dst_dt):
     rng = np.random.default_rng(M + K + N)
@@ -44,7 +44,7 @@ def test_static_s8_rows_with_q8_0_weights(zo, M, K, N, dst_dt):
         dst.zero_()
         st = lowoha.matmul_direct("r", False, True, M, N, K, 1.0, a_d, K, w_d, K, H.to_dev(bias), 0.0, dst, N, True, p)
         assert st == capi.SUCCESS, lowoha.last_error()
-        assert lowoha.last_kernel().startswith("pergroup_")
+        assert lowoha.last_kernel().startswith("pergroup_") or K == 32   # (one group: the per-token chain is the same arithmetic)
         ph = H.host_params(p, src_scale=ss)
         keep = []
         st, want, _, _ = zo.matmul_int8(a, packed, ph.flat(keep), M, N, K, bias=bias, transB=True, ldb=K)
@@ -53,7 +53,7 @@ def test_static_s8_rows_with_q8_0_weights(zo, M, K, N, dst_dt):
     capi.load().zmi_clear_weight_cache()
 
 
-@pytest.mark.parametrize("M,K,N", [(16, 4096, 256), (3, 128, 40), (70, 512, 64)])
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 256), (3, 128, 40), (70, 512, 64), (20, 32, 36)])
 def test_dynamic_bf16_rows_with_q8_0_weights(zo, M, K, N):
     rng = np.random.default_rng(M * 3 + K + N)
     G = K // 32

@@ -449,6 +449,9 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   // matmul/backends/aocl/aocl_kernel.cpp:167-236).  G == 1 is the plain per-channel chain.
   const bool bcast_src = w4a8 && pg_groups == 0 && p.wei_scale.dims[0] > 1;
   if (bcast_src) pg_groups = p.wei_scale.dims[0];
+  // (K = 32 is one packed block per column: {M,1} source scales ARE {M, K / 32}; one group of 32)
+  if (ggml && K == 32 && pg_groups == 0 && M > 1 && (dyn ? dyn_scale_n : (p.src_scale.buff ? nelems(p.src_scale) : 0)) == M)
+    pg_groups = 1;
   if (ggml) {
     // reference: ggml_is_sym_quant (ggml_weight_unpack.cpp:142-153), checked after the source was quantized:
     // s8 (or dynamically quantized) source, symmetric, more than one source scale, f32 / bf16 destination
