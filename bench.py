@@ -47,6 +47,9 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run")
+    ap.add_argument("--no-calib", action="store_true",
+                    help="skip the measured ceilings (read-only streaming kernel, pure MFMA loop)")
+    ap.add_argument("--calib", action="store_true", help="run the measured ceilings alone and print them")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; the path has no multi-GPU part (--gpus must be 1)",
@@ -82,11 +85,19 @@ def main():
     def rand_w(K, N):
         return torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
 
-    def ev_time(fn, steps, warmup):
+    def ev_time(fn, steps, warmup, ramp_ms=30.0):
         """Average milliseconds per call: warmup untimed calls, then `steps` calls between two
-        events on the library's stream, synchronised on both sides."""
-        for _ in range(warmup):
+        events on the library's stream, synchronised on both sides.  The untimed part lasts at
+        least ramp_ms of wall clock whatever `warmup` says: after the set-up the device sits in a
+        low power state, and a handful of 15 us calls does not bring its clocks up (20 timed steps
+        right after 5 warm-up calls read 25 % slow)."""
+        t_end = time.perf_counter() + ramp_ms * 1e-3
+        n = 0
+        while n < warmup or time.perf_counter() < t_end:
             fn()
+            n += 1
+            if n % 64 == 0:
+                torch.cuda.synchronize()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
@@ -154,6 +165,58 @@ def main():
         del ca, cb_
         torch.cuda.empty_cache()
 
+    def run_calib():
+        """What this device sustains with nothing in the way (hand-written kernels in csrc/k_calib.hip)."""
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        out = {}
+        us = ctypes.c_float()
+        span = ctypes.c_float()
+        nbytes = K_DEC * N_DEC
+        bufs = [torch.randint(-127, 128, (nbytes,), dtype=torch.int8, device=dev, generator=g) for _ in range(8)]
+        arr = (ctypes.c_void_p * 8)(*[b.data_ptr() for b in bufs])
+        best = None
+        for _ in range(3):
+            st = lib.zmi_calib_hbm_read(arr, 8, nbytes, 200, 400, stream, ctypes.byref(us), ctypes.byref(span))
+            assert st == capi.SUCCESS
+            if best is None or us.value < best[0]:
+                best = (us.value, span.value)
+        out["hbm_read_decode_shape"] = {
+            "bytes_per_launch": nbytes, "buffers_rotated": 8, "us_per_launch": round(best[0], 2),
+            "GBps": round(nbytes / best[0] / 1e3, 1), "in_kernel_span_us": round(best[1], 2),
+            "GBps_in_kernel": round(nbytes / best[1] / 1e3, 1),
+            "what": "a kernel that only reads the 58.7 MB of one decode call's weights (448 workgroups x 8 wavefronts x 16 "
+                    "requests of 16 B per lane, all in flight), launched back to back over 8 rotating buffers"}
+        del bufs
+        big = torch.randint(-127, 128, (1 << 30,), dtype=torch.int8, device=dev, generator=g)
+        arr1 = (ctypes.c_void_p * 1)(big.data_ptr())
+        st = lib.zmi_calib_hbm_read(arr1, 1, 1 << 30, 3, 10, stream, ctypes.byref(us), ctypes.byref(span))
+        assert st == capi.SUCCESS
+        out["hbm_read_1GiB"] = {"us_per_launch": round(us.value, 1), "GBps": round((1 << 30) / us.value / 1e3, 1)}
+        del big
+        torch.cuda.empty_cache()
+        ops = torch.randint(-127, 128, (6 * 1024,), dtype=torch.int8, device=dev, generator=g)
+        tops = ctypes.c_float()
+        mhz = ctypes.c_float()
+        for name, vary, per_cu in (("constant_operands_1wg_per_cu", 0, 1), ("varying_operands_1wg_per_cu", 1, 1),
+                                   ("varying_operands_2wg_per_cu", 1, 2)):
+            st = lib.zmi_calib_mfma_i8(ctypes.c_void_p(ops.data_ptr()), vary, per_cu, 6000, stream,
+                                       ctypes.byref(tops), ctypes.byref(mhz))
+            assert st == capi.SUCCESS
+            out["mfma_i8_" + name] = {"TOPS": round(tops.value, 1), "shader_MHz": round(mhz.value, 0),
+                                      "pct_of_nominal": round(100 * tops.value / INT8_PEAK_TOPS, 1)}
+        out["mfma_i8_what"] = ("a loop of nothing but v_mfma_i32_32x32x32_i8, 4 wavefronts per workgroup on every compute "
+                               "unit, ~0.2 ms per launch; 'varying': consecutive instructions get different random int8 operand "
+                               "fragments, as in a GEMM on random data (the multipliers' toggling sets the power, the clock follows)")
+        return out
+
+    calib = None
+    if args.calib or not (args.no_calib or args.only):
+        calib = run_calib()
+        torch.cuda.empty_cache()
+        if args.calib:
+            print(json.dumps({"calibration": calib}))
+            return
+
     M = 16
     n_sets = 8
     keep = None
@@ -204,6 +267,14 @@ def main():
                                  "from the rocprofv3 --pmc runs summarised under profiles/ (null if not measured "
                                  "for this build)"},
         }
+        if calib:
+            ceil = calib["hbm_read_decode_shape"]["GBps"]
+            result["roofline"]["measured_peak"] = {
+                "value": ceil, "unit": "GB/s", "frac_of_measured": round(achieved / ceil, 4),
+                "gemm_only_frac_of_measured": round(gemm_only / ceil, 4),
+                "what": "the read-only kernel of the same launch shape over the same 8 rotating buffers, launch to launch "
+                        "(calibration.hbm_read_decode_shape); the kernel that does nothing but read the bytes"}
+            result["calibration"] = calib
 
     # ---------------------------------------------------------------- other configs
     def run_decode_m(m):
@@ -295,9 +366,13 @@ def main():
         p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
         t = ev_time(lambda: lowoha.matmul_direct("r", False, False, Mp, N, K, 1.0, x, K, blob, N, bias, 0.0, dst, N, True, p), 30, 5)
         ops = 2.0 * Mp * N * K
-        return {"TOPS_whole_call": round(ops / (t * 1e-3) / 1e12, 1),
-                "pct_of_int8_mfma_peak": round(100 * ops / (t * 1e-3) / 1e12 / INT8_PEAK_TOPS, 1),
-                "us_whole_call": round(t * 1e3, 1), "kernel": lowoha.last_kernel()}
+        r = {"TOPS_whole_call": round(ops / (t * 1e-3) / 1e12, 1),
+             "pct_of_int8_mfma_peak": round(100 * ops / (t * 1e-3) / 1e12 / INT8_PEAK_TOPS, 1),
+             "us_whole_call": round(t * 1e3, 1), "kernel": lowoha.last_kernel()}
+        if calib:
+            r["pct_of_measured_mfma_loop"] = round(100 * ops / (t * 1e-3) / 1e12 /
+                                                   calib["mfma_i8_varying_operands_1wg_per_cu"]["TOPS"], 1)
+        return r
 
     def run_config1():
         Mc, K, N = 128, 4096, 4096
@@ -389,30 +464,44 @@ def main():
         from oracle import build as obuild, oracle as zo
         obuild.build(force=False)
         rng = np.random.default_rng(1)
-        Mb = 16
-        A = rng.integers(-127, 128, (Mb, K_DEC), dtype=np.int8)
-        Bt = rng.integers(-127, 128, (N_DEC, K_DEC), dtype=np.int8)   # pre-transposed: the packed form of the CPU path
-        sa = rng.uniform(0.01, 0.03, Mb).astype(np.float32)
-        sb = rng.uniform(0.001, 0.01, N_DEC).astype(np.float32)
-        out = np.zeros((Mb, N_DEC), dtype=np.uint16)
         L = zo.lib()
-        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+        L.zo_omp_threads.restype = ctypes.c_int32
+        cores = int(L.zo_omp_threads())     # threads the port's OpenMP regions really run on
 
-        def cpu_call():
-            L.zo_bench_s8_gemm(A.ctypes.data, Bt.ctypes.data, sa.ctypes.data, sb.ctypes.data, Mb, N_DEC, K_DEC,
-                               capi.PO_SWISH, out.ctypes.data)
-        cpu_call()
-        t0 = time.perf_counter()
-        n = 0
-        while time.perf_counter() - t0 < 10.0:
-            cpu_call()
-            n += 1
-        dt = (time.perf_counter() - t0) / n
-        cb = K_DEC * N_DEC + Mb * K_DEC + Mb * 4 + N_DEC * 4 + Mb * N_DEC * 2
+        def cpu_gemm(Mb, Nb, Kb, po, seconds):
+            A = rng.integers(-127, 128, (Mb, Kb), dtype=np.int8)
+            Bt = rng.integers(-127, 128, (Nb, Kb), dtype=np.int8)   # pre-transposed: the packed form of the CPU path
+            sa = rng.uniform(0.01, 0.03, Mb).astype(np.float32)
+            sb = rng.uniform(0.001, 0.01, Nb).astype(np.float32)
+            out = np.zeros((Mb, Nb), dtype=np.uint16)
+
+            def call():
+                L.zo_bench_s8_gemm(A.ctypes.data, Bt.ctypes.data, sa.ctypes.data, sb.ctypes.data, Mb, Nb, Kb, po,
+                                   out.ctypes.data)
+            call()
+            t0 = time.perf_counter()
+            n = 0
+            while time.perf_counter() - t0 < seconds:
+                call()
+                n += 1
+            return (time.perf_counter() - t0) / n, n
+
+        dt, n = cpu_gemm(16, N_DEC, K_DEC, capi.PO_SWISH, 8.0)
+        cb = K_DEC * N_DEC + 16 * K_DEC + 16 * 4 + N_DEC * 4 + 16 * N_DEC * 2
         result["cpu_baseline"] = {"value": round(cb / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
                                   "sample": f"{n} calls of the same M=16 K=4096 N=14336 s8 x s8 GEMM + scales + SiLU + bf16 "
-                                            f"store through the oracle's OpenMP port (about 10 s); not AOCL-DLP",
+                                            f"store through the oracle's OpenMP port (about 8 s); not AOCL-DLP",
                                   "ms_per_call": round(dt * 1e3, 3)}
+        # the other workloads, each on a bounded sample through the same port
+        dtp, n = cpu_gemm(64, 4096, 4096, capi.PO_GELU_TANH, 5.0)
+        dtm1, n1 = cpu_gemm(32, 28672, 4096, 0, 4.0)
+        dtm2, n2 = cpu_gemm(32, 4096, 14336, 0, 3.0)
+        result["cpu_baseline"]["other_workloads"] = {
+            "prefill_N4096": {"TOPS": round(2.0 * 64 * 4096 * 4096 / dtp / 1e12, 3), "cores": cores,
+                              "sample": f"{n} calls on 64 of the 2048 rows (GEMM + scales + GELU-tanh + bf16 store); rows are independent"},
+            "moe_config4": {"tokens_per_s": round(16 / (dtm1 + dtm2), 1), "cores": cores,
+                            "sample": f"the two GEMMs of one expert on the 32 routed rows of 16 tokens ({n1} + {n2} calls; "
+                                      "4096 -> 28672 and 14336 -> 4096), without activation, re-quantization and reduce"}}
     print(json.dumps(result))
 
 

@@ -318,6 +318,29 @@ typedef struct zmi_moe_device_t {
 } zmi_moe_device_t;
 ZMI_API int32_t zmi_moe_fused_device(const zmi_moe_device_t *d);
 
+/* ---- Measurement aids (no counterpart in the reference; not on the path of any
+ * call above).  They measure what this device sustains with nothing in the way,
+ * the denominators next to the nominal peaks.
+ *
+ * zmi_calib_hbm_read: launches a kernel that only reads `bytes` bytes (a multiple
+ * of 128 KiB) with the decode kernels' launch shape, `warm` untimed and `launches`
+ * timed launches over the n_bufs device buffers in turn (rotate enough of them to
+ * exceed the on-die cache).  us_per_launch: between two events on `stream`;
+ * span_us: first wavefront's start to last wavefront's end inside one launch.
+ *
+ * zmi_calib_mfma_i8: one launch of `iters` x 8 v_mfma_i32_32x32x32_i8 per wavefront,
+ * 4 wavefronts per workgroup, wgs_per_cu workgroups per compute unit.  operands:
+ * 6 KiB of int8 operand fragments in device memory; vary_operands != 0 feeds
+ * consecutive instructions different fragments (what random GEMM data does to the
+ * multipliers).  tops: 1e12 int8 operations per second (2 per multiply-add);
+ * shader_mhz: average shader clock inside the loop. */
+ZMI_API int32_t zmi_calib_hbm_read(void *const *bufs, int32_t n_bufs, uint64_t bytes,
+                           int32_t warm, int32_t launches, void *stream,
+                           float *us_per_launch, float *span_us);
+ZMI_API int32_t zmi_calib_mfma_i8(const void *operands, int32_t vary_operands,
+                          int32_t wgs_per_cu, int32_t iters, void *stream,
+                          float *tops, float *shader_mhz);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,6 +47,7 @@
  * rounded f32 operations.
  */
 #include <math.h>
+#include <omp.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -716,6 +717,17 @@ ZO_EXPORT void zo_moe_reduce(const void *const *row_ptrs, const float *w, int32_
 }
 
 /* ---- timed CPU baseline helper ------------------------------------------------ */
+
+/* Threads an OpenMP parallel region of this library runs on (what the timed helper below uses). */
+ZO_EXPORT int32_t zo_omp_threads(void) {
+  int32_t n = 1;
+  #pragma omp parallel
+  {
+    #pragma omp single
+    n = omp_get_num_threads();
+  }
+  return n;
+}
 
 /* One decode-style call on already-quantized operands, the shape of work the
  * reference's CPU path spends its time on (s8 x s8 -> s32 GEMM over

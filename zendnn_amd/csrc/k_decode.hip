@@ -61,9 +61,7 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
   // publish it and leave; the streaming workgroups follow them in dispatch order.
   if (fq.x && (int)blockIdx.x < M) {
     zmi_fused_quant_row(fq, blockIdx.x, K, reinterpret_cast<float *>(lds));
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
-    __syncthreads();
-    if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
+    zmi_fq_publish(fq, blockIdx.x);
     return;
   }
   // column block and rows: with at most RPW row groups the workgroup index is the column
@@ -86,24 +84,41 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
   // the two 16-column groups h = 0, 1 of the block
   const int wcol[2] = {blk * 32, blk * 32 + 16};
 
-  // ---- epilogue constants of this thread's output element, fetched first ----
-  // element (row tid/32, column tid%32) of every row group
+  // ---- this thread's output element: (row tid/32, column tid%32) of every row group.  With rows that
+  // are given, its epilogue constants are requested BEHIND the weights, as raw words (branch-free, decoded
+  // after the reduction): ahead of them, every dependent wait would hold the weight stream back by a memory
+  // round trip.  With the quantization inside the launch the column constants come first, as they always
+  // did: measured, the streaming workgroups' late start is what lets the quantizing workgroups' own loads
+  // and stores through (M = 16, N = 14336: 14.6 against 15.1 us per call; an idle wait of the same length
+  // in their place: 15.5 .. 16.2 us) ----
   const int e_row = tid / 32;
   const int e_h = (tid % 32) / 16;
   const int e_c = tid % 16;
   const int e_n = wcol[e_h] + e_c;
   const bool e_col = e_n < N;
-  const ZmiColCtx cc0 = zmi_col_ctx(epi, p, colsum, e_col ? e_n : N, N);
-  // (with fused quantization the row scales exist only after the wait below)
-  float rs[RPW];
-  auto load_rs = [&]() {
+  const int n_ok = e_col ? e_n : N - 1;
+  ZmiColRaw craw = {};
+  int32_t zp_word = 0;
+  uint32_t rs_word[RPW];
+  auto load_consts = [&]() {
+    craw = zmi_col_raw(epi, p, colsum, n_ok);
+    zp_word = zmi_zp_raw(p, colsum);
     #pragma unroll
     for (int j = 0; j < RPW; ++j) {
       const int m = r0 + j * 16 + e_row;
-      rs[j] = zmi_row_scale(epi, p, e_col && m < M ? m : 0);
+      rs_word[j] = zmi_row_scale_raw(epi, p, colsum, m < M ? m : M - 1);
     }
   };
-  if (!fq.x) load_rs();
+  ZmiColCtx cc_first = {};
+  float rs_first[RPW];
+  if (fq.x) cc_first = zmi_col_ctx(epi, p, colsum, e_col ? e_n : N, N);
+  auto load_rs_first = [&]() {
+    #pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int m = r0 + j * 16 + e_row;
+      rs_first[j] = zmi_row_scale(epi, p, e_col && m < M ? m : 0);
+    }
+  };
 
   // ---- activation loads: every wavefront stages its own slice of K (at most 8 chunks = 32 granules
   // of 16 bytes per row) of the group's 16 rows, so no wavefront waits for another one: lanes 0..31
@@ -155,8 +170,16 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
   auto load_b = [&](int u) {
     // past the end of the slice: re-read the slice's first chunk (valid memory), result unused
     const int c = c_begin + u < c_end ? c_begin + u : c_begin;
-    b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)c * 2048);
-    b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)c * 2048);
+    if (RPW == 1 && n_rg == 1) {
+      // read by this workgroup only: the streaming hint keeps the weights from pushing the rows out of the caches
+      // (M = 16, N = 14336: 13.0 against 14.2 us); with several workgroups per column block the others
+      // find the weights in L2 and the hint costs (M = 128, N = K = 4096: 13.4 against 12.8 us)
+      b[u][0] = __builtin_nontemporal_load((const v4i *)(bsrc[0] + (int64_t)c * 2048));
+      b[u][1] = __builtin_nontemporal_load((const v4i *)(bsrc[1] + (int64_t)c * 2048));
+    } else {
+      b[u][0] = *(const v4i *)(bsrc[0] + (int64_t)c * 2048);
+      b[u][1] = *(const v4i *)(bsrc[1] + (int64_t)c * 2048);
+    }
   };
 
   if (!fq.x) {
@@ -165,19 +188,22 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
     #pragma unroll
     for (int u = 0; u < 8; ++u) load_b(u);
     if (RPW > 1 && r0 + 16 < M) load_rows(1);
+    load_consts();
   } else {
     #pragma unroll
     for (int u = 0; u < DEC_FQ_FIRST; ++u) load_b(u);
-    if (tid == 0) {
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        const unsigned int v = __hip_atomic_load(fq.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((int)(v - fq.target) >= 0) break;
-        __builtin_amdgcn_s_sleep(1);
-      }
+    // (one waiting wavefront per streaming workgroup; the others learn the outcome through LDS)
+    int *ok_l = reinterpret_cast<int *>(lds);
+    if (wave == 0) {
+      const bool ok = zmi_fq_wait(fq, M);
+      if (lane == 0) *ok_l = ok ? 1 : 0;
     }
     __syncthreads();
+    const bool rows_ok = *ok_l != 0;
+    __syncthreads();                 // (the operand area is written next)
+    if (!rows_ok) return;            // the wait ran out: nothing is computed from unpublished rows
     asm volatile("" ::: "memory");   // the loads below stay below the wait
-    load_rs();
+    load_rs_first();   // (the row scales exist only now)
     load_rows(0);
     #pragma unroll
     for (int u = DEC_FQ_FIRST; u < 8; ++u) load_b(u);
@@ -236,12 +262,129 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
     for (int w = 0; w < DEC_WAVES; ++w) s += red[w * RPW * 512 + off];
     return s;
   };
+  const ZmiColCtx cc0 = fq.x ? cc_first : zmi_col_ctx_raw(epi, p, craw, zp_word, e_n, n_ok, N);
   #pragma unroll
   for (int j = 0; j < RPW; ++j) {
     const int m = r0 + j * 16 + e_row;
     if (m >= M) break;
-    zmi_finish_element(p, epi, cc0, rs[j], fetch(j, e_h), m, e_n);
+    const float rs = fq.x ? rs_first[j] : zmi_row_scale_from_raw(epi, p, rs_word[j], m);
+    zmi_finish_element(p, epi, cc0, rs, fetch(j, e_h), m, e_n);
   }
+}
+
+// ---------------------------------------------------------------------------------------
+// Up to 16 rows that are given as s8 / u8 (the decode step proper): nothing stands in front of the
+// weight stream.  A wavefront's loads return in order and every compute unit works its requests off
+// in order, so whatever is requested ahead of the weights with a dependent wait holds the stream
+// back by a memory round trip.  Here every wavefront requests
+//   1. the first two chunks of its weights (memory has work while the address unit, which takes 64
+//      bytes per cycle whatever they are, works the row requests off),
+//   2. the rows of its own slice of K by global->LDS loads (no registers, nothing waits for them),
+//   3. the rest of its 16 KiB of weights, with the streaming hint (each byte is read once; without
+//      the hint the weights push the rows out of the caches: 13.3 against 12.6 us at M = 16, N = 14336),
+//   4. this thread's epilogue constants as raw words (branch-free, decoded after the reduction).
+// There is no barrier in front of the MFMAs: a wavefront reads back only the rows it requested.
+// Rows -> LDS: one global->LDS request per chunk of 64 k.  Lane l lands at byte 16 l of the
+// chunk's 1 KiB; it fetches row l / 4, and four consecutive lanes fetch the row's 64 bytes of the
+// chunk (one contiguous run per row) in the order k group (l % 4) ^ (row / 4 % 4): with that twist
+// the MFMA's lanes (row l % 16, k group l / 16) read the 1 KiB back without bank conflicts.  Lanes
+// of rows past M request nothing (their results are never stored, and fewer rows are fewer bytes
+// through L2: 11.9 / 12.2 / 12.6 us at 1 / 8 / 16 rows); bytes past the readable end of a row meet
+// zero weights and are fetched from the row's last 16 bytes.
+// (Measured and dropped: the rows by helper wavefronts -- their requests end up behind the weights of
+// the whole compute unit; at most 2 .. 6 chunks of weights in flight per wavefront; neighbouring
+// workgroups starting at different slices of K; rows and weights requested alternately; the
+// quantization of bf16 rows inside this kernel behind helper wavefronts that wait for the quantizing
+// workgroups -- 15.8 us against 14.6 us for the row-group kernel's form.)
+__device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+#define D16_W_FIRST 2    // chunks of weights requested ahead of the rows
+
+__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int M = p.M, N = p.N, K = p.K;
+  const int K_pad = (int)zmi_blob_kpad(K);
+  const int nchunks = K_pad / 64;
+  const int blk = (int)blockIdx.x;
+
+  // one chunk of rows -> LDS
+  const int G = ((K + 15) & ~15) / 16;      // readable 16-byte granules per row
+  const int a_r = lane / 4;
+  const uint32_t a_row_off = (uint32_t)a_r * (uint32_t)p.lda;
+  const int a_kg = (lane % 4) ^ ((a_r >> 2) & 3);
+  auto stage_chunk = [&](int c) {
+    const int gran = c * 4 + a_kg;
+    const uint32_t voff = a_row_off + (uint32_t)(gran < G ? gran : G - 1) * 16u;
+    if (a_r < M)
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(c * 1024), "v"(voff), "s"(p.A) : "memory", "m0");
+  };
+
+  const int c_begin = wave * nchunks / DEC_WAVES;
+  const int c_end = (wave + 1) * nchunks / DEC_WAVES;
+  const int c16 = lane % 16, g = lane / 16;
+  const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
+  const uint8_t *bsrc[2];
+  #pragma unroll
+  for (int h = 0; h < 2; ++h)
+    bsrc[h] = tiles + (int64_t)blk * zmi_blob_nb_stride(K) + (g / 2) * 1024 + ((g % 2) * 32 + h * 16 + c16) * 16;
+  v4i b[8][2];
+  auto load_b = [&](int u) {
+    // past the end of the slice: re-read the slice's first chunk (valid memory), result unused
+    const int c = c_begin + u < c_end ? c_begin + u : c_begin;
+    b[u][0] = __builtin_nontemporal_load((const v4i *)(bsrc[0] + (int64_t)c * 2048));
+    b[u][1] = __builtin_nontemporal_load((const v4i *)(bsrc[1] + (int64_t)c * 2048));
+  };
+  #pragma unroll
+  for (int u = 0; u < D16_W_FIRST; ++u) load_b(u);
+  #pragma unroll
+  for (int u = 0; u < 8; ++u)
+    if (c_begin + u < c_end) stage_chunk(c_begin + u);
+  #pragma unroll
+  for (int u = D16_W_FIRST; u < 8; ++u) load_b(u);
+  // this thread's output element (row tid / 32, column tid % 32) and its constants, as raw words
+  const int e_row = tid / 32, e_col = tid % 32;
+  const int e_n = blk * 32 + e_col;
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+  const int n_ok = e_n < N ? e_n : N - 1, m_ok = e_row < M ? e_row : M - 1;
+  const ZmiColRaw craw = zmi_col_raw(epi, p, colsum, n_ok);
+  const int32_t zp_word = zmi_zp_raw(p, colsum);
+  const uint32_t rs_word = zmi_row_scale_raw(epi, p, colsum, m_ok);
+  // requests complete in order: once the rows are in LDS, at most the weight requests that followed them
+  // and the 5 constant words are outstanding
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (8 - D16_W_FIRST) + 5) : "memory");
+  const uint32_t xm = p.a_is_u8 ? 0x80808080u : 0u;
+
+  v4i acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  #pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const bool live = c_begin + u < c_end;
+    const int c = live ? c_begin + u : c_begin;
+    v4i a = *(const v4i *)(lds + c * 1024 + (c16 * 4 + (g ^ ((c16 >> 2) & 3))) * 16);
+    a[0] ^= xm; a[1] ^= xm; a[2] ^= xm; a[3] ^= xm;   // u8 rows enter the MFMA as (a - 128)
+    if (!live) a = (v4i){0, 0, 0, 0};   // whatever b holds then adds nothing
+    acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[1], 0, 0, 0);
+  }
+
+  // ---- cross-wavefront reduction through LDS (reuses the operand area) ----
+  zmi_lds_barrier();
+  int32_t *red = (int32_t *)lds;
+  #pragma unroll
+  for (int h = 0; h < 2; ++h)
+    #pragma unroll
+    for (int q = 0; q < 4; ++q) red[wave * 512 + (h * 4 + q) * 64 + lane] = acc[h][q];
+  zmi_lds_barrier();
+  if (e_n >= N || e_row >= M) return;
+
+  // acc[h][q] of lane l is row (l/16)*4 + q, column h*16 + l%16
+  const int off = ((e_col / 16) * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_col % 16;
+  int32_t s = 0;
+  #pragma unroll
+  for (int w = 0; w < DEC_WAVES; ++w) s += red[w * 512 + off];
+  const ZmiColCtx cc0 = zmi_col_ctx_raw(epi, p, craw, zp_word, e_n, n_ok, N);
+  zmi_finish_element(p, epi, cc0, zmi_row_scale_from_raw(epi, p, rs_word, m_ok), s, e_row, e_n);
 }
 
 int zmi_decode_grid(const ZmiProblem &p) { return (int)(zmi_blob_npad(p.N) / 32); }
@@ -250,12 +393,27 @@ bool zmi_decode_kernel_fits(const ZmiProblem &p) {
   return p.M > 0 && p.M <= 128 && zmi_blob_kpad(p.K) <= 4096;
 }
 
+// Rows given as s8 / u8, at most 16 of them: the kernel without anything in front of the weight stream.
+// (ZMI_DECODE_ROWGROUP_KERNEL: the tests reach the row-group kernel with few rows through it.)
+bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant) {
+  return !fused_quant && p.M <= 16 && (int64_t)p.lda * 16 < ((int64_t)1 << 31) && !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
+}
+
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
                                   hipStream_t stream) {
   if (!zmi_decode_kernel_fits(p)) return hipErrorInvalidValue;
   if (epi.gated_act != 0) return hipErrorInvalidValue;   // gated GEMMs are grouped launches: the large-M kernel
   const int n_blk = zmi_decode_grid(p);
   if (n_blk <= 0) return hipSuccess;
+  ZmiFusedQuant none = {};
+  if (zmi_decode_16row_kernel(p, fq != nullptr)) {
+    const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel, 4096 * 16);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(zmi_gemm_decode16_kernel, dim3(n_blk), dim3(DEC_THREADS), op > DEC_RED_BYTES ? op : DEC_RED_BYTES, stream,
+                       p, epi);
+    return hipGetLastError();
+  }
   // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at
   // 32 / 64 rows, N = K = 4096, against 13 / 20 us with 64); above that, 64 rows per workgroup
   // keep the weights in registers for four row groups (128 rows: 23 against 27 us)
@@ -272,15 +430,10 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
   const size_t a_bytes = (size_t)zmi_blob_kpad(p.K) * 16;
   const size_t r_bytes = (size_t)DEC_RED_BYTES * rpw;
   const size_t smem = a_bytes > r_bytes ? a_bytes : r_bytes;
-  static bool attr_done = false;
-  if (!attr_done) {
-    for (const void *f : {(const void *)zmi_gemm_decode_kernel<1>, (const void *)zmi_gemm_decode_kernel<4>}) {
-      hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * 16);
-      if (e != hipSuccess) return e;
-    }
-    attr_done = true;
+  for (const void *f : {(const void *)zmi_gemm_decode_kernel<1>, (const void *)zmi_gemm_decode_kernel<4>}) {
+    hipError_t e = zmi_func_smem_once(f, 4096 * 16);
+    if (e != hipSuccess) return e;
   }
-  ZmiFusedQuant none = {};
   const dim3 g3(grid + (fq ? p.M : 0)), b3(DEC_THREADS);
   if (rpw == 1) hipLaunchKernelGGL(zmi_gemm_decode_kernel<1>, g3, b3, smem, stream, p, epi, fq ? *fq : none, n_blk);
   else hipLaunchKernelGGL(zmi_gemm_decode_kernel<4>, g3, b3, smem, stream, p, epi, fq ? *fq : none, n_blk);

@@ -52,12 +52,9 @@ hipError_t zmi_launch_gated_act(const ZmiActMat *mats_dev, const ZmiActMat *mat0
   if (total_rows <= 0) return hipSuccess;
   const size_t smem = (size_t)(max_N / 2) * sizeof(float);
   if (smem > 160 * 1024) return hipErrorInvalidValue;
-  static size_t attr = 0;
-  if (smem > attr) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gated_act_kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  {
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gated_act_kernel, (int)smem);
     if (e != hipSuccess) return e;
-    attr = smem;
   }
   ZmiActMat m0 = {};
   if (mat0) m0 = *mat0;
@@ -302,12 +299,9 @@ hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E,
   const int n = T * topk;
   const int G = hist_scratch ? zmi_moe_route_groups(n, E) : 1;
   const size_t smem = ((size_t)RT_WAVES * E + E + 1 + (G > 1 ? (size_t)G * RT_WAVES * E : 0)) * sizeof(int32_t);
-  static size_t attr = 0;
-  if (smem > attr) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_moe_route_kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  {
+    hipError_t e = zmi_func_smem_once((const void *)zmi_moe_route_kernel, (int)smem);
     if (e != hipSuccess) return e;
-    attr = smem;
   }
   const int al = align < 1 ? 1 : align;
   if (G > 1)

@@ -276,9 +276,7 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   if (fq.x && (int)blockIdx.x < M) {
     if (fq.per_row) zmi_fused_quant_row(fq, blockIdx.x, K, reinterpret_cast<float *>(lds));
     else zmi_fused_quant_row_groups(fq, blockIdx.x, K, G);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
-    __syncthreads();
-    if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
+    zmi_fq_publish(fq, blockIdx.x);
     return;
   }
   const int blk = fq.x ? (int)blockIdx.x - M : (int)blockIdx.x;
@@ -348,14 +346,16 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   };
   if (fq.x) {
     // the quantized rows and their scales exist once the counter says so
-    if (tid == 0) {
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        const unsigned int v = __hip_atomic_load(fq.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((int)(v - fq.target) >= 0) break;
-        __builtin_amdgcn_s_sleep(1);
-      }
+    // (one waiting wavefront per streaming workgroup; the others learn the outcome through LDS)
+    int *ok_l = reinterpret_cast<int *>(lds);
+    if (wave == 0) {
+      const bool ok = zmi_fq_wait(fq, M);
+      if (lane == 0) *ok_l = ok ? 1 : 0;
     }
     __syncthreads();
+    const bool rows_ok = *ok_l != 0;
+    __syncthreads();                 // (the operand area is written next)
+    if (!rows_ok) return;            // the wait ran out: nothing is computed from unpublished rows
     asm volatile("" ::: "memory");   // the loads below stay below the wait
     load_rows();
     load_ss();
@@ -449,12 +449,9 @@ static hipError_t pgd_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const 
   constexpr int G = PGD_WAVES * GPW, NCH = PGD_WAVES * CPW, RT = G <= 32 ? G : 16;
   constexpr size_t main_bytes = (size_t)NCH * 1024 > (size_t)RT * 2048 ? (size_t)NCH * 1024 : (size_t)RT * 2048;
   constexpr size_t smem = main_bytes + (size_t)G * 32 * 4 + (size_t)16 * G * 4;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_decode_pergroup_kernel<CPW, GPW, S4>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  {
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode_pergroup_kernel<CPW, GPW, S4>, (int)smem);
     if (e != hipSuccess) return e;
-    attr_done = true;
   }
   ZmiFusedQuant none = {};
   const dim3 grid((unsigned)(zmi_blob_npad(p.N) / 32) + (fq ? p.M : 0)), block(PGD_THREADS);

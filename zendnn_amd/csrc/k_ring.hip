@@ -47,7 +47,7 @@ __device__ __forceinline__ void zmi_dma_pair(const void *base, uint32_t voff, ui
   // two consecutive 1 KiB fragments: LDS address = m0 + offset + lane * 16
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024"
                ::"s"(lds), "v"(voff), "s"(base)
-               : "memory");
+               : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void zmi_wait_vm() {
@@ -675,12 +675,9 @@ static hipError_t ring_launch_cfg(const ZmiProblem &p0, const ZmiProblem *probs,
                                   const int *tile_tab, int top, const ZmiRingSplit &split, const ZmiEpilogue &epi,
                                   hipStream_t stream) {
   const size_t smem = RingCfg<BM, DEEP>::SMEM;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_ring_kernel<BM, DEEP>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  {
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_ring_kernel<BM, DEEP>, (int)smem);
     if (e != hipSuccess) return e;
-    attr_done = true;
   }
   const int grid = (n_items + 7) / 8 * 8;   // a multiple of 8 so the XCD renumbering applies
   hipLaunchKernelGGL((zmi_gemm_ring_kernel<BM, DEEP>), dim3(grid), dim3(R_THREADS), smem, stream, p0, probs, n_prob,

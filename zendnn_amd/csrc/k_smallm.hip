@@ -86,9 +86,7 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p, Zmi
     float *fred = reinterpret_cast<float *>(red);
     for (int row = blockIdx.x; row < M; row += gridDim.x) {
       zmi_fused_quant_row(fq, row, K, fred);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's write-through stores have landed ...
-      __syncthreads();
-      if (tid == 0) atomicAdd(fq.counter, 1u);           // ... before the row is published
+      zmi_fq_publish(fq, row);
     }
   }
   // The first group of weight loads goes out before anything else.  With fused
@@ -96,16 +94,16 @@ __global__ __launch_bounds__(1024) void zmi_gemm_smallm_kernel(ZmiProblem p, Zmi
   // own weight loads would only return after them) and streams afterwards.
   if (!fq.x || wave != 0) load_b(c_begin);
   if (fq.x) {
-    if (tid == 0) {
-      // bounded wait: producers are the lowest-numbered workgroups and wait for nothing
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        const unsigned int v = __hip_atomic_load(fq.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((int)(v - fq.target) >= 0) break;
-        __builtin_amdgcn_s_sleep(1);
-      }
+    // (one waiting wavefront per workgroup; the others learn the outcome through LDS)
+    if (wave == 0) {
+      const bool ok = zmi_fq_wait(fq, M);
+      if (lane == 0) red[0] = ok ? 1 : 0;
+      load_b(c_begin);
     }
-    if (wave == 0) load_b(c_begin);
     __syncthreads();
+    const bool rows_ok = red[0] != 0;
+    __syncthreads();                 // (the partial tiles are written there later)
+    if (!rows_ok) return;            // the wait ran out: nothing is computed from unpublished rows
     asm volatile("" ::: "memory");   // the row loads below stay below the wait
   }
 
@@ -172,12 +170,9 @@ static hipError_t launch_small(const ZmiProblem &p, int grid, int W, const ZmiEp
                                hipStream_t stream) {
   size_t smem = (size_t)W * MB * 2 * 4 * 64 * sizeof(int32_t);
   if (smem < 256) smem = 256;
-  static size_t attr_smem = 0;
-  if (smem > attr_smem) {
-    hipError_t e = hipFuncSetAttribute((const void *)zmi_gemm_smallm_kernel<MB, UNROLL>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  {
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_smallm_kernel<MB, UNROLL>, (int)smem);
     if (e != hipSuccess) return e;
-    attr_smem = smem;
   }
   hipLaunchKernelGGL((zmi_gemm_smallm_kernel<MB, UNROLL>), dim3(grid), dim3(W * 64), smem, stream, p, epi, fq);
   return hipGetLastError();

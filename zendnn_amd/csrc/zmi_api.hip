@@ -278,7 +278,7 @@ ZmiRingPlan plan_ring_gemm(int M, int N, int K) {
 
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
   if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
-    set_kernel_name("decode_lds_rows_mfma16x16x64");
+    set_kernel_name(zmi_decode_16row_kernel(prob, false) ? "decode16_dma_rows_mfma16x16x64" : "decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
   } else if (!use_ring_kernel(prob.M, prob.N, prob.K)) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
@@ -380,6 +380,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                           const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
                           const zmi_batch_params_t *batch_params, const zmi_matmul_params_t *params) {
   clear_error();
+  if (async_failure_pending()) return ZMI_FAILURE;
   if (!params) { set_error("null params"); return ZMI_FAILURE; }
   const zmi_matmul_params_t &p = *params;
   const int Batch_A = batch_params ? batch_params->Batch_A : 1;
@@ -482,6 +483,11 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
     }
   }
   if (!ensure_device()) return ZMI_FAILURE;
+  if (dyn && p.src_scale.buff && !is_device_pointer(p.src_scale.buff)) {
+    // with dynamic_quant the scale buffer is an OUTPUT that the kernels write
+    set_error("dynamic_quant: src_scale.buff receives the computed scales and must be device memory (or null)");
+    return ZMI_FAILURE;
+  }
 
   // ---- scratch plan ----
   const bool use_cache = !ggml && p.mem_format_b != 'r' && is_weights_const &&
@@ -562,12 +568,10 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       // (matmul/quantization/reorder_quantization.cpp:43-280 with {M,G} scale dims)
       if (zmi_pergroup_decode_shape(prob, (int)pg_groups) && !std::getenv("ZMI_NO_FUSED_QUANT")) {
         // decode shapes: the quantization is part of the GEMM launch (its first M workgroups)
-        unsigned int *ctr = fused_counter();
-        if (!ctr) return ZMI_FAILURE;
+        if (!fused_handoff(&fused)) return ZMI_FAILURE;
         fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
         fused.q = q; fused.ldq = K16; fused.scales = sc;
         fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
-        fused.counter = ctr; fused.target = fused_next_target(M);
         use_fused = true;
       } else if (!hip_ok(zmi_launch_quant_groups(src, p.dt_src, M, K, lda, pg_groups, q, K16, sc, (void *)p.src_scale.buff,
                                                  sdt, stream()), "per-group quant launch")) {
@@ -580,12 +584,10 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                !std::getenv("ZMI_NO_FUSED_QUANT")) {
       // W4A8 decode shapes with one scale per row: the per-token quantization is part of the per-group GEMM
       // launch, whose workgroups read the row's scale for every group (no broadcast copy)
-      unsigned int *ctr = fused_counter();
-      if (!ctr) return ZMI_FAILURE;
+      if (!fused_handoff(&fused)) return ZMI_FAILURE;
       fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
       fused.q = q; fused.ldq = K16; fused.scales = sc;
       fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
-      fused.counter = ctr; fused.target = fused_next_target(M);
       fused.per_row = 1;
       use_fused = true;
       ep.src_scale.buff = sc;
@@ -593,12 +595,10 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
     } else if (per_token && !bcast_src && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
         !std::getenv("ZMI_NO_FUSED_QUANT")) {
-      unsigned int *ctr = fused_counter();
-      if (!ctr) return ZMI_FAILURE;
+      if (!fused_handoff(&fused)) return ZMI_FAILURE;
       fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
       fused.q = q; fused.ldq = K16; fused.scales = sc;
       fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
-      fused.counter = ctr; fused.target = fused_next_target(M);
       use_fused = true;
       ep.src_scale.buff = sc;
       ep.src_scale.dt = ZMI_DT_F32;

@@ -1,8 +1,8 @@
 // Per-token quantization of one source row by a whole workgroup, used by the
 // small-M kernels that fuse the quantization into the GEMM launch: the
-// workgroups with the lowest indices quantize one row each, publish it with a
-// device-scope counter, and every workgroup waits for the counter before it
-// reads the s8 rows (same arithmetic as k_quant.hip).
+// workgroups with the lowest indices quantize one row each and publish it through
+// the row's device-scope flag, and every workgroup waits for the flags of all rows
+// before it reads the s8 rows (same arithmetic as k_quant.hip).
 #pragma once
 #include "zmi_device.h"
 #include "zmi_launch.h"
@@ -18,6 +18,53 @@
 // GEMM reads the narrowed value back, while the rows were quantized with the f32 scale.
 static __device__ __forceinline__ float zmi_fused_scale_as_stored(const ZmiFusedQuant &fq, float s) {
   return fq.user_dt == ZMI_DT_BF16 ? zmi_bf16_to_f32(zmi_f32_to_bf16_rne(s)) : s;
+}
+
+// ---- hand-off --------------------------------------------------------------------------
+// Producer side, called by every thread of a workgroup that has just quantized row `row`: the
+// row's flag takes the launch's epoch once all the workgroup's write-through stores have landed.
+static __device__ __forceinline__ void zmi_fq_publish(const ZmiFusedQuant &fq, int row) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(&fq.flags[row], fq.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Consumer side, called by whole wavefronts (every lane): polls the flags of rows 0 .. rows-1
+// (lane l looks at rows l and l + 64; rows <= 128) until all carry the launch's epoch or the time
+// limit passes.  Returns true when the rows are there.  When the limit ran out the error word is
+// set and the caller must not touch the rows: the host reports the failure on the thread's next call.
+static __device__ __forceinline__ bool zmi_fq_wait(const ZmiFusedQuant &fq, int rows) {
+  const int lane = threadIdx.x % 64;
+  const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+  const unsigned int *f0 = &fq.flags[lane < rows ? lane : 0];
+  const unsigned int *f1 = &fq.flags[lane + 64 < rows ? lane + 64 : 0];
+  const bool two = rows > 64;   // (uniform)
+  bool ok = false;
+  // A look at the flags is a trip to memory behind everything the compute unit has already asked for (microseconds
+  // under load), so several looks are kept in flight, a fraction of a microsecond apart, and examined oldest first.
+  constexpr int NP = 4;
+  unsigned int v0[NP], v1[NP];
+  if (fq.wait_ticks != 0) {
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      v0[j] = __hip_atomic_load(f0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v1[j] = two ? __hip_atomic_load(f1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : fq.epoch;
+      __builtin_amdgcn_s_sleep(4);
+    }
+    for (;;) {
+      bool done = false;
+#pragma unroll
+      for (int j = 0; j < NP; ++j) {
+        if (__all(v0[j] == fq.epoch && v1[j] == fq.epoch)) { ok = true; done = true; break; }
+        if (__builtin_amdgcn_s_memrealtime() - t0 > (uint64_t)fq.wait_ticks) { done = true; break; }
+        v0[j] = __hip_atomic_load(f0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v1[j] = two ? __hip_atomic_load(f1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : fq.epoch;
+      }
+      if (done) break;
+    }
+  }
+  if (!ok && lane == 0) __hip_atomic_store(fq.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  return ok;
 }
 
 static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int K, float *red) {

@@ -48,17 +48,22 @@ void *upload(const void *host, size_t bytes);
 // Ends a call's uploads: the slots it used stay reserved until the stream gets here.
 void upload_fence();
 
-// ---- fused-quantization counter ------------------------------------------------------
-// Device counter the fused decode kernel publishes quantized rows through, owned by
-// the calling thread.  next_target(rows) returns the value the counter will have
-// reached when `rows` more rows are published (launches run in stream order).
-unsigned int *fused_counter();
-unsigned int fused_next_target(int rows);
+// ---- fused-quantization hand-off ------------------------------------------------------
+// Fills the hand-off fields of a launch that quantizes its own rows (ZmiFusedQuant::sync, error,
+// wait_ticks) with the calling thread's words, allocating them on first use.
+bool fused_handoff(ZmiFusedQuant *fq);
+// True (with the error text set) when a launch of this thread gave up waiting for its quantized rows
+// since the last check; entry points call it first and return failure.
+bool async_failure_pending();
+// Marks that the calling thread has queued work on its current stream (see zmi_set_stream).
+void note_enqueue();
 
 // ---- one-element parameters ------------------------------------------------------
 // A scale / zero-point of one element may live in host or device memory.
 // Host: *value receives it and *dev_ptr is null.  Device: *dev_ptr receives
 // the pointer and the kernel reads it.
+// True for device (or managed) memory, false for ordinary host memory.
+bool is_device_pointer(const void *p);
 bool scalar_param_f32(const void *buff, int32_t dt, float *value, const void **dev_ptr);
 bool scalar_param_s32(const void *buff, int32_t dt, int32_t *value, const int32_t **dev_ptr);
 

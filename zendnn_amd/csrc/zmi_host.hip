@@ -1,13 +1,14 @@
 // Host-side services behind the C ABI (see zmi_host.h).
 #include "zmi_host.h"
 
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <list>
 #include <map>
 #include <mutex>
 #include <tuple>
-#include <unordered_set>
+#include <set>
 #include <vector>
 
 namespace zmi {
@@ -27,8 +28,14 @@ struct ThreadCtx {
   bool ev_live[kSlots] = {};   // an event is recorded and the slot is busy until it fires
   bool used[kSlots] = {};      // written during the current call, not fenced yet
   int next = 0;
-  unsigned int *fq_counter = nullptr;
-  unsigned int fq_total = 0;
+  // hand-off words of the launches that quantize their own rows (ZmiFusedQuant::sync / error)
+  unsigned int *fq_flags = nullptr;      // device: one flag per row, holding the epoch of the launch that published it
+  unsigned int fq_epoch = 0;             // name of this thread's latest launch of that kind
+  unsigned int *fq_err_host = nullptr;   // pinned host word the kernels set when a wait ran out
+  unsigned int *fq_err_dev = nullptr;    // the same word as the device addresses it
+  // stream hand-over (zmi_set_stream): work of this thread may still be queued on `stream`
+  bool enqueued = false;
+  hipEvent_t handover = nullptr;
 };
 thread_local ThreadCtx tctx;
 
@@ -49,7 +56,7 @@ struct CacheVal {
 };
 std::map<CacheKey, CacheVal> g_cache;
 std::list<CacheKey> g_lru;
-std::unordered_set<const void *> g_checked_blobs;
+std::set<std::tuple<const void *, int64_t, int64_t>> g_checked_blobs;   // (blob, K, N) whose header was read
 
 size_t cache_capacity() {
   // same variable the reference reads for its weight caches
@@ -75,8 +82,11 @@ bool hip_ok(hipError_t e, const char *what) {
 }
 
 bool ensure_device() {
+  tctx.enqueued = true;   // every entry point passes here before it queues work
+  static std::atomic<bool> ready{false};
+  if (ready.load(std::memory_order_acquire)) return true;
   std::lock_guard<std::mutex> lk(g_mu);
-  if (g_device_ready) return true;
+  if (g_device_ready) { ready.store(true, std::memory_order_release); return true; }
   int n = 0;
   hipError_t e = hipGetDeviceCount(&n);
   if (e != hipSuccess || n <= 0) {
@@ -85,8 +95,11 @@ bool ensure_device() {
     return false;
   }
   g_device_ready = true;
+  ready.store(true, std::memory_order_release);
   return true;
 }
+
+void note_enqueue() { tctx.enqueued = true; }
 
 // ---- arena ---------------------------------------------------------------------
 bool Arena::begin(size_t total) {
@@ -186,25 +199,46 @@ void upload_fence() {
   }
 }
 
-unsigned int *fused_counter() {
+bool fused_handoff(ZmiFusedQuant *fq) {
   ThreadCtx &c = tctx;
-  if (!c.fq_counter) {
-    void *p = nullptr;
-    if (!hip_ok(hipMalloc(&p, 256), "hipMalloc(counter)")) return nullptr;
-    if (!hip_ok(hipMemset(p, 0, 256), "hipMemset(counter)")) return nullptr;
-    c.fq_counter = (unsigned int *)p;
-    c.fq_total = 0;
+  if (!c.fq_flags) {
+    void *d = nullptr, *h = nullptr, *hd = nullptr;
+    if (!hip_ok(hipMalloc(&d, 512), "hipMalloc(hand-off words)")) return false;
+    if (!hip_ok(hipMemset(d, 0, 512), "hipMemset(hand-off words)")) return false;
+    if (!hip_ok(hipHostMalloc(&h, 64, hipHostMallocMapped), "hipHostMalloc(error word)")) return false;
+    std::memset(h, 0, 64);
+    if (!hip_ok(hipHostGetDevicePointer(&hd, h, 0), "hipHostGetDevicePointer(error word)")) return false;
+    c.fq_flags = (unsigned int *)d;
+    c.fq_err_host = (unsigned int *)h;
+    c.fq_err_dev = (unsigned int *)hd;
   }
-  return c.fq_counter;
+  fq->flags = c.fq_flags;
+  if (++c.fq_epoch == 0) c.fq_epoch = 1;   // (0 is what the flags hold before the first launch)
+  fq->epoch = c.fq_epoch;
+  fq->error = c.fq_err_dev;
+  // 100 ms unless ZMI_FUSED_WAIT_US says otherwise (0: every wait gives up at once; the tests of the
+  // failure path use it)
+  uint64_t us = 100000;
+  if (const char *e = std::getenv("ZMI_FUSED_WAIT_US")) us = (uint64_t)std::strtoull(e, nullptr, 10);
+  const uint64_t ticks = us * 100;
+  fq->wait_ticks = ticks > 0xffffffffull ? 0xffffffffu : (uint32_t)ticks;
+  return true;
 }
 
-unsigned int fused_next_target(int rows) {
-  tctx.fq_total += (unsigned int)rows;
-  return tctx.fq_total;
+bool async_failure_pending() {
+  ThreadCtx &c = tctx;
+  if (!c.fq_err_host || *(volatile unsigned int *)c.fq_err_host == 0) return false;
+  // a launch of this thread gave up waiting for its quantized rows and stored nothing
+  (void)hipStreamSynchronize(c.stream);
+  *(volatile unsigned int *)c.fq_err_host = 0;
+  (void)hipGetLastError();
+  set_error("an earlier call on this thread did not get its quantized rows in time and wrote no output "
+            "(fused per-token quantization hand-off timed out)");
+  return true;
 }
 
 // ---- one-element parameters ------------------------------------------------------
-static bool is_device_pointer(const void *p) {
+bool is_device_pointer(const void *p) {
   hipPointerAttribute_t attr;
   hipError_t e = hipPointerGetAttributes(&attr, p);
   if (e != hipSuccess) {
@@ -270,8 +304,11 @@ const uint8_t *packed_weights(const void *weight, int64_t K, int64_t N, int64_t 
   }
   void *blob = nullptr;
   if (!hip_ok(hipMalloc(&blob, (size_t)zmi_blob_bytes(K, N)), "hipMalloc(packed weights)")) return nullptr;
+  // the entry becomes visible to every thread (each on its own stream) as soon as it is inserted: the blob
+  // must be complete by then
   if (!hip_ok(zmi_launch_prepack((const int8_t *)weight, K, N, ldb, transB, src_dtype, 0, (uint8_t *)blob,
-                                 stream()), "prepack launch")) {
+                                 stream()), "prepack launch") ||
+      !hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize(prepack)")) {
     (void)hipFree(blob);
     return nullptr;
   }
@@ -384,7 +421,7 @@ void clear_weight_cache() {
 bool blob_matches(const void *blob, int64_t K, int64_t N) {
   {
     std::lock_guard<std::mutex> lk(g_mu);
-    if (g_checked_blobs.count(blob)) return true;
+    if (g_checked_blobs.count(std::make_tuple(blob, K, N))) return true;
   }
   ZmiBlobHeader h;
   if (!hip_ok(hipMemcpyAsync(&h, blob, sizeof(h), hipMemcpyDeviceToHost, stream()), "hipMemcpy(blob header)"))
@@ -395,7 +432,7 @@ bool blob_matches(const void *blob, int64_t K, int64_t N) {
     return false;
   }
   std::lock_guard<std::mutex> lk(g_mu);
-  g_checked_blobs.insert(blob);
+  g_checked_blobs.insert(std::make_tuple(blob, K, N));
   return true;
 }
 
@@ -430,7 +467,27 @@ int32_t zmi_init(int32_t device) {
   return ZMI_SUCCESS;
 }
 
-void zmi_set_stream(void *hip_stream) { zmi::tctx.stream = (hipStream_t)hip_stream; }
+void zmi_set_stream(void *hip_stream) {
+  // The thread's scratch arena, upload ring and hand-off words are ordered by the stream its calls
+  // run on: work queued on the old stream has to finish before calls on the new one reuse them.
+  auto &c = zmi::tctx;
+  hipStream_t next = (hipStream_t)hip_stream;
+  if (next != c.stream && c.enqueued) {
+    bool chained = false;
+    if (!c.handover && hipEventCreateWithFlags(&c.handover, hipEventDisableTiming) != hipSuccess) c.handover = nullptr;
+    if (c.handover && hipEventRecord(c.handover, c.stream) == hipSuccess &&
+        hipStreamWaitEvent(next, c.handover, 0) == hipSuccess)
+      chained = true;
+    if (!chained) {
+      // (e.g. the old stream no longer exists: whatever ran on it has then finished or is lost)
+      (void)hipGetLastError();
+      (void)hipDeviceSynchronize();
+      (void)hipGetLastError();
+    }
+    c.enqueued = false;
+  }
+  c.stream = next;
+}
 void *zmi_get_stream(void) { return (void *)zmi::tctx.stream; }
 const char *zmi_last_error(void) { return zmi::tctx.error.c_str(); }
 const char *zmi_last_kernel(void) { return zmi::tctx.kernel; }

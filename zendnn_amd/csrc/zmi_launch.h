@@ -3,7 +3,27 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "zmi_device.h"
+
+// Raises a kernel's limit of dynamic LDS to `bytes` the first time it is needed on the current
+// device (the attribute belongs to the device's copy of the kernel); callable from any thread.
+inline hipError_t zmi_func_smem_once(const void *func, int bytes) {
+  static std::mutex mu;
+  static std::map<std::pair<int, const void *>, int> done;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lk(mu);
+  int &have = done[std::make_pair(dev, func)];
+  if (have >= bytes) return hipSuccess;
+  e = hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) have = bytes;
+  return e;
+}
 
 // One matrix of a (possibly grouped) per-token quantization launch; row_start is
 // the index of its first row in the launch's global row numbering.
@@ -77,8 +97,14 @@ struct ZmiFusedQuant {
   float *scales;          // f32 scale per row out (== ZmiProblem::src_scale_ptr)
   void *user_scales;      // optional copy in user_dt
   int32_t user_dt;
-  unsigned int *counter;  // device counter, monotonically increasing across launches
-  unsigned int target;    // value the counter reaches when all M rows of this launch are published
+  // Hand-off between the quantizing and the streaming workgroups of one launch: one device word per row,
+  // set to the launch's `epoch` once the row and its scale are in memory.  The epoch only names the launch
+  // (a fresh value per launch from the calling thread); nothing is counted, so a launch that fails or never
+  // runs leaves nothing behind that a later launch could trip over.
+  unsigned int *flags;    // [>= M]
+  unsigned int epoch;
+  unsigned int *error;    // host-visible word, set to 1 by a wavefront whose wait ran out
+  uint32_t wait_ticks;    // limit of the wait in ticks of the 100 MHz real-time counter; 0: give up at once
   int32_t per_row;        // per-group kernels only: one scale per row (scales[row]) stands for all its groups
 };
 
@@ -112,6 +138,8 @@ bool zmi_decode_kernel_fits(const ZmiProblem &p);
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
                                   hipStream_t stream);
 int zmi_decode_grid(const ZmiProblem &p);
+// true when the launch above takes the 16-row kernel (rows fetched by global->LDS loads behind the first weights)
+bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant);
 
 // k_moe.hip
 struct ZmiActMat {
