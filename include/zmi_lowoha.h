@@ -262,6 +262,29 @@ ZMI_API int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src,
                                 void *const *scale,
                                 const zmi_group_dq_params_t *params);
 
+/* zmi_matmul_direct_noalloc: zmi_matmul_direct for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid it).  It has no counterpart in the reference.  Same arguments,
+ * arithmetic and kernels as zmi_matmul_direct, for the decode-shaped call whose
+ * source rows are quantized at run time: bf16 / f32 source with dynamic_quant and
+ * s8 compute, source scale dims {1} or {M,1} (buff null or a device buffer that
+ * receives the scales), prepacked weights (mem_format_b 'r'), no transposes,
+ * M <= 128 and K <= 4096; anything else returns unimplemented / failure.  The
+ * quantized rows and their scales live in a fixed 514 KiB array inside the
+ * library's device image (one copy per GPU, held until the process ends) instead
+ * of the calling thread's scratch arena; the call makes no hipMalloc / hipFree.
+ * All calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered by the stream.
+ * The first call with a given blob reads the blob's header back once. */
+ZMI_API int32_t zmi_matmul_direct_noalloc(char layout, int32_t transA, int32_t transB,
+                          int32_t M, int32_t N, int32_t K, float alpha,
+                          const void *src, int32_t lda,
+                          const void *weight, int32_t ldb,
+                          const void *bias, float beta,
+                          void *dst, int32_t ldc, int32_t is_weights_const,
+                          const zmi_batch_params_t *batch_params,
+                          const zmi_matmul_params_t *params);
+
 /* ---- Library services with no counterpart in the reference ------------ */
 
 /* Selects the GPU (hipSetDevice) and creates the per-device state.  Optional:

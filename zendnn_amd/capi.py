@@ -143,6 +143,11 @@ SIGNATURES = {
                                       C.c_int32, C.c_void_p, C.c_float, C.c_void_p, C.c_int32,
                                       C.c_int32, C.POINTER(BatchParamsT),
                                       C.POINTER(MatmulParamsT)]),
+    "zmi_matmul_direct_noalloc": (C.c_int32, [C.c_char, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                              C.c_int32, C.c_float, C.c_void_p, C.c_int32, C.c_void_p,
+                                              C.c_int32, C.c_void_p, C.c_float, C.c_void_p, C.c_int32,
+                                              C.c_int32, C.POINTER(BatchParamsT),
+                                              C.POINTER(MatmulParamsT)]),
     "zmi_group_matmul_direct": (C.c_int32, [C.POINTER(GroupArgsT), C.POINTER(MoePostopT),
                                             C.c_int32, C.POINTER(FusedMoeT)]),
     "zmi_reorder_params_init": (None, [C.POINTER(ReorderParamsT)]),

@@ -88,6 +88,9 @@ void clear_weight_cache();
 // blob packed for this K and N.
 bool blob_matches(const void *blob, int64_t K, int64_t N);
 
+// Looks up the current device's copy of zmi_matmul_direct_noalloc's scratch array (zmi_api_noalloc.hip).
+bool noalloc_setup();
+
 int64_t nelems(const zmi_quant_t &q);
 bool diagnostics_enabled();
 int weight_cache_env();

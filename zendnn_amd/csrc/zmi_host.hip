@@ -464,6 +464,7 @@ int32_t zmi_init(int32_t device) {
   zmi::clear_error();
   if (!zmi::ensure_device()) return ZMI_FAILURE;
   if (!zmi::hip_ok(hipSetDevice(device), "hipSetDevice")) return ZMI_FAILURE;
+  if (!zmi::noalloc_setup()) return ZMI_FAILURE;   // the device's address of zmi_matmul_direct_noalloc's scratch array
   return ZMI_SUCCESS;
 }
 

@@ -111,14 +111,16 @@ def last_kernel():
 
 
 def matmul_direct(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc,
-                  is_weights_const, params, batch_a=1, batch_b=1):
+                  is_weights_const, params, batch_a=1, batch_b=1, noalloc=False):
+    """noalloc=True: the entry point that allocates no device memory (zmi_matmul_direct_noalloc)."""
     lib = capi.load()
     keep = []
     p = params.flat(keep)
     b = capi.BatchParamsT()
     lib.zmi_batch_params_init(C.byref(b))
     b.Batch_A, b.Batch_B = batch_a, batch_b
-    return lib.zmi_matmul_direct(layout.encode(), int(transA), int(transB), M, N, K, alpha, _ptr(src), lda,
+    fn = lib.zmi_matmul_direct_noalloc if noalloc else lib.zmi_matmul_direct
+    return fn(layout.encode(), int(transA), int(transB), M, N, K, alpha, _ptr(src), lda,
                                  _ptr(weight), ldb, _ptr(bias), beta, _ptr(dst), ldc, int(is_weights_const),
                                  C.byref(b), C.byref(p))
 
