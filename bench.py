@@ -42,7 +42,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
     ap.add_argument("--only", default=None,
                     choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "decode_M16_w4a8_group128", "decode_M16_w4a8_group128_per_token_rows", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
-                             "moe_config4", "moe_config5"],
+                             "moe_decode_T16", "moe_config4", "moe_config5"],
                     help="run one of the other configs alone and print its entry (for profiler runs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, the known-size kernel that scales the "
@@ -443,6 +443,8 @@ def main():
         "prefill_N4096": lambda: run_prefill(4096),
         "prefill_N14336": lambda: run_prefill(14336),
         "config1_u8s8_M128": run_config1,
+        # a decode step of configuration 4's block: 16 tokens, every expert has a handful of rows (decode-shaped grouped kernel)
+        "moe_decode_T16": lambda: run_moe(16, 4096, 14336, 8, 2, False),
         "moe_config4": lambda: run_moe(512, 4096, 14336, 8, 2, False),
         "moe_config5": lambda: run_moe(4096, 2048, 1408, 64, 6, True),
     }

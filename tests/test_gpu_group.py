@@ -344,3 +344,121 @@ def test_group_bf16_source_scale_dtype(zo, with_buffer):
         if with_buffer:
             assert np.array_equal(H.to_host(sc_d[e]), H.bf16_bits(scales))
         assert np.array_equal(H.to_host(dst[e]), want)
+
+
+# ------------------------------------------------------------------ experts with 1 .. 16 rows
+@pytest.mark.parametrize("T,Hd,I,E,topk", [(1, 1024, 512, 8, 2), (4, 1024, 512, 8, 2), (16, 1024, 512, 8, 2),
+                                           (16, 4096, 14336, 8, 2),        # a decode step of configuration 4's block
+                                           (40, 2048, 1408, 64, 6)])       # configuration 5's shapes, every expert small
+def test_decode_shaped_grouped_kernel(zo, T, Hd, I, E, topk, monkeypatch):
+    """Experts with at most 16 rows run on the decode-shaped grouped kernel (weights streamed once, gate * SiLU x up in
+    its epilogue): every token against the oracle, and bit-identical to the same block with those experts on the
+    MFMA-bound kernel, through group_matmul_direct with fused_moe and through the device-routed form."""
+    c = MH.make_case(0x5EED0D00 + T + E, T, Hd, I, E, topk, skew=False)
+    assert max(c.M) <= 16 or T == 40
+    monkeypatch.setenv("ZMI_GROUP_DECODE", "1")     # (the split also where large experts outnumber the small ones)
+    d = MH.DeviceMoe(c, packed=True)
+    st = d.call_fused()
+    assert st == capi.SUCCESS, lowoha.last_error()
+    got = H.to_host(d.out).copy()
+    want = MH.oracle_moe(zo, c, list(range(T)))
+    check_moe_out(got, want)
+    w13b = [H.prepack(w, c.H, 2 * c.I) for w in d.w13]
+    w2b = [H.prepack(w, c.I, c.H) for w in d.w2]
+    out2 = torch.zeros((c.T, c.H), dtype=torch.bfloat16, device=H.DEV)
+    st = lowoha.moe_fused_device(d.x, H.to_dev(c.ids), d.topk_w, w13b, w2b, d.s13, d.s2, c.I, capi.ACT_SILU_AND_MUL, out2)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert np.array_equal(H.to_host(out2), got)
+    # the same experts on the MFMA-bound kernel
+    monkeypatch.delenv("ZMI_GROUP_DECODE")
+    monkeypatch.setenv("ZMI_NO_GROUP_DECODE", "1")
+    d.out.zero_()
+    st = d.call_fused()
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert np.array_equal(H.to_host(d.out), got)
+
+
+@pytest.mark.parametrize("Ms", [[3, 0, 16, 40, 1, 130], [16, 16], [1, 200]])
+@pytest.mark.parametrize("dst_dt", [capi.DT_BF16, capi.DT_F32])
+def test_decode_shaped_grouped_kernel_mixed_with_large_experts(zo, Ms, dst_dt, monkeypatch):
+    """A grouped gated call (no fused_moe) whose experts fall on both kernels: each expert against the oracle's single
+    GEMM + activation, and the small ones bit-identical to their MFMA-bound results."""
+    rng = np.random.default_rng(sum(Ms) + dst_dt)
+    K, I = 512, 96
+    E = len(Ms)
+    xs = [H.gen_bf16_normal(rng, (max(m, 1), K)) for m in Ms]
+    ws = [H.gen_weights(rng, K, 2 * I) for _ in Ms]
+    sc = [rng.uniform(0.001, 0.01, 2 * I).astype(np.float32) for _ in Ms]
+    sc_d = [H.to_dev(s) for s in sc]
+    tdt = torch.bfloat16 if dst_dt == capi.DT_BF16 else torch.float32
+    outs = []
+    for forced in (False, True):
+        if forced:
+            monkeypatch.delenv("ZMI_GROUP_DECODE")
+            monkeypatch.setenv("ZMI_NO_GROUP_DECODE", "1")
+        else:
+            monkeypatch.setenv("ZMI_GROUP_DECODE", "1")
+        dst = [torch.zeros((max(m, 1), 2 * I), dtype=tdt, device=H.DEV) for m in Ms]
+        params = [MH.dyn_params(m, 2 * I, sc_d[e], dst_dt=dst_dt) for e, m in enumerate(Ms)]
+        st = lowoha.group_matmul_direct(["r"] * E, [False] * E, [False] * E, Ms, [2 * I] * E, [K] * E, [1.0] * E,
+                                        [H.to_dev(x) for x in xs], [K] * E, [H.to_dev(w) for w in ws], [2 * I] * E,
+                                        [None] * E, [0.0] * E, dst, [2 * I] * E, [True] * E, params,
+                                        gated_act=capi.ACT_SILU_AND_MUL)
+        assert st == capi.SUCCESS, lowoha.last_error()
+        outs.append([H.to_host(t) for t in dst])
+    for e, m in enumerate(Ms):
+        if m == 0:
+            continue
+        assert np.array_equal(outs[0][e][:m, :I], outs[1][e][:m, :I]), f"expert {e} ({m} rows)"
+        keep = []
+        p1 = MH.dyn_params(m, 2 * I, sc[e].ctypes.data, dst_dt=dst_dt).flat(keep)
+        _, y1, _, _ = zo.matmul_int8(xs[e][:m], ws[e], p1, m, 2 * I, K)
+        zo.gated_act(capi.ACT_SILU_AND_MUL, y1, dst_dt)
+        if dst_dt == capi.DT_BF16:
+            H.check_bf16(outs[0][e][:m, :I], y1[:, :I], max_frac=5e-3)
+        else:
+            H.check_f32(outs[0][e][:m, :I], y1[:, :I])
+
+
+# ------------------------------------------------------------------ gelu_and_mul
+@pytest.mark.parametrize("T,Hd,I,E,topk", [(64, 256, 128, 4, 2), (9, 512, 96, 8, 2)])
+def test_fused_moe_gelu_and_mul(zo, T, Hd, I, E, topk):
+    """gated_act = gelu_and_mul (erf form, group_matmul_moe_act.cpp:119-154) in the fused block, both kernels' epilogues."""
+    c = MH.make_case(0x5EED0E00 + T, T, Hd, I, E, topk)
+    d = MH.DeviceMoe(c)
+    st = d.call_fused(act=capi.ACT_GELU_AND_MUL)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    need = {}
+    rows = []
+    for t in range(T):
+        for k in range(topk):
+            e, j = c.slot[t, k]
+            need.setdefault(int(e), []).append((t, k))
+    y2_of = {}
+    for e, lst in need.items():
+        xr = np.ascontiguousarray(c.x[[t for t, _ in lst]])
+        _, y2 = MH.oracle_expert(zo, c, e, xr, act=capi.ACT_GELU_AND_MUL)
+        for i, (t, k) in enumerate(lst):
+            y2_of[(t, k)] = y2[i]
+    rows = [np.ascontiguousarray(y2_of[(t, k)]) for t in range(T) for k in range(topk)]
+    want = zo.moe_reduce(rows, np.ascontiguousarray(c.w), capi.DT_BF16, c.H)
+    check_moe_out(H.to_host(d.out), want)
+
+
+def test_group_gated_gelu_and_mul_unfused_block(zo):
+    """gelu_and_mul on independent grouped GEMMs (no Op2): activation output against the oracle."""
+    c = MH.make_case(0x5EED0E10, 70, 256, 64, 4, 2)
+    d = MH.DeviceMoe(c)
+    E = c.E
+    dst = [torch.zeros((max(c.M[e], 1), 2 * c.I), dtype=torch.bfloat16, device=H.DEV) for e in range(E)]
+    params = [MH.dyn_params(c.M[e], 2 * c.I, d.s13[e]) for e in range(E)]
+    st = lowoha.group_matmul_direct(
+        ["r"] * E, [False] * E, [False] * E, c.M, [2 * c.I] * E, [c.H] * E, [1.0] * E,
+        d.src, [c.H] * E, d.w13, [2 * c.I] * E, [None] * E, [0.0] * E,
+        dst, [2 * c.I] * E, [True] * E, params, gated_act=capi.ACT_GELU_AND_MUL)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for e in range(E):
+        if c.M[e] == 0:
+            continue
+        a, _ = MH.oracle_expert(zo, c, e, np.ascontiguousarray(c.x[c.rows_of[e]]), act=capi.ACT_GELU_AND_MUL)
+        H.check_bf16(H.to_host(dst[e])[:, :c.I], a, max_frac=5e-3)

@@ -6,6 +6,7 @@
 
 #include "zmi_api.h"
 #include "zmi_host.h"
+#include "zmi_ring_table.h"
 
 using namespace zmi;
 
@@ -242,19 +243,37 @@ int group_top(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated) {
   return zmi_ring_pick_top_group(rows, n_prob, K, N, gated);
 }
 
-// Every expert's activations are fragment-major; one launch per tile height.
+// Every expert's activations are fragment-major.  Experts with more than 16 rows: one launch of the MFMA-bound
+// kernel; experts with 1 .. 16 rows: one launch of the decode-shaped grouped kernel (weight streaming, gated
+// activation in its epilogue), reference: the ALGO-3 decode tile, group_matmul/group_matmul_dispatch.cpp:779.
 int32_t launch_stage(const Stage &st, const char *what) {
   if (st.probs.empty()) return ZMI_SUCCESS;
   const ZmiProblem *dev = (const ZmiProblem *)upload(st.probs.data(), st.probs.size() * sizeof(ZmiProblem));
   if (!dev) return ZMI_FAILURE;
   const int n = (int)st.probs.size();
+  const bool gated = st.epi.gated_act != 0;
   int64_t rows = 0;
-  int cols = 0, kmax = 0;
-  for (const ZmiProblem &q : st.probs) { rows += q.M; cols = std::max(cols, (int)q.N); kmax = std::max(kmax, (int)q.K); }
-  const int top = group_top(rows, n, kmax, cols, st.epi.gated_act != 0);
-  int *tab = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)n));
-  if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
-  if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) return ZMI_FAILURE;
+  int cols = 0, kmax = 0, small = 0, large = 0;
+  bool small_ok = true;
+  for (const ZmiProblem &q : st.probs) {
+    rows += q.M; cols = std::max(cols, (int)q.N); kmax = std::max(kmax, (int)q.K);
+    if (q.M > 0 && q.M <= 16) { ++small; small_ok = small_ok && zmi_group_decode_takes(st.epi, q.N); }
+    else if (q.M > 16) ++large;
+  }
+  // The decode-shaped kernel runs as a launch of its own, behind the MFMA-bound one: worth it when the small experts
+  // are most of the weight traffic (a decode step: 0.26 against 0.32 ms for 8 experts x 2 .. 6 rows of configuration
+  // 4's block); a few small experts among large ones stream under the large ones' MFMA work inside the one launch
+  // instead (configuration 5: 0.45 against 0.49 ms).  ZMI_GROUP_DECODE=1 forces the split (tests).
+  const bool force_split = getenv("ZMI_GROUP_DECODE") != nullptr;
+  const bool split = small > 0 && small_ok && (small >= large || force_split);
+  int top = group_top(rows, n, kmax, cols, gated);
+  if (split) top |= ZMI_RING_SKIP_SMALL;
+  if (large > 0 || !split) {
+    int *tab = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)n));
+    if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
+    if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) return ZMI_FAILURE;
+  }
+  if (split && !hip_ok(zmi_launch_gemm_group_decode(dev, n, gated ? cols / 2 : cols, st.epi, stream()), what)) return ZMI_FAILURE;
   return ZMI_SUCCESS;
 }
 
@@ -696,7 +715,20 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   }
   // row counts live on the device: the grids are sized for the worst case, and the kernel that builds
   // the per-expert problem tables fills the tile tables of both grouped launches as well
-  const int top1 = group_top(R, E, H, 2 * I, true), top2 = group_top(R, E, I, H, false);
+  int top1 = group_top(R, E, H, 2 * I, true), top2 = group_top(R, E, I, H, false);
+  // (the row counts are not known here: experts with 1 .. 16 rows, if there are any, are the decode-shaped grouped
+  // kernel's, whose workgroups leave at once for every other expert; the MFMA-bound kernel's tile table skips them)
+  ZmiEpilogue probe;
+  std::memset(&probe, 0, sizeof(probe));
+  probe.fast_kind = ZMI_EK_NONE;
+  // (worth a launch of its own only when small experts are most of the work: see launch_stage; the row counts live
+  // on the device, so the average decides)
+  const bool decode_step = R <= 16 * (int64_t)E || getenv("ZMI_GROUP_DECODE") != nullptr;
+  const bool small2 = decode_step && zmi_group_decode_takes(probe, H);
+  probe.gated_act = d->gated_act;
+  const bool small1 = decode_step && zmi_group_decode_takes(probe, 2 * I);
+  if (small1) top1 |= ZMI_RING_SKIP_SMALL;
+  if (small2) top2 |= ZMI_RING_SKIP_SMALL;
   if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, top1, top2, tile_tab1, tile_tab2, s), "problem table launch")) return ZMI_FAILURE;
 
   ZmiEpilogue e1;
@@ -707,9 +739,11 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
   if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, true, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+  if (small1 && !hip_ok(zmi_launch_gemm_group_decode(op1, E, I, e1, s), "Op1 decode-shaped GEMM launch")) return ZMI_FAILURE;
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
+  if (small2 && !hip_ok(zmi_launch_gemm_group_decode(op2, E, H, e2, s), "Op2 decode-shaped GEMM launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;
   upload_fence();
   set_kernel_name("moe_fused_device");

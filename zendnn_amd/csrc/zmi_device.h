@@ -532,4 +532,67 @@ __device__ __forceinline__ void zmi_finish_element(const ZmiProblem &p, const Zm
     else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, c, rs, m, n, p.dst, p.ldc));
   }
 }
+// ---- one element finished with the arithmetic of the MFMA-bound kernel's epilogue (k_ring.hip) ----
+// The kernels that take part of a grouped launch beside it end here, so that a result does not depend on which
+// kernel computed it: bf16 destinations with a straight-line epilogue use the separately rounded scale chain with
+// absent scales as 1 and an absent bias as -0, the hardware exponential / reciprocal forms of the activations and the
+// hardware bf16 conversion under the flush-denormals mode; f32 destinations the conditional chain of zmi_fast_value;
+// everything else the interpreter.
+__device__ __forceinline__ float zmi_ring_chain(int32_t acc, const ZmiColCtx &c, float rs, bool has_bias) {
+  return __fadd_rn(__fmul_rn(__fmul_rn((float)(acc + c.comp), rs), c.wscale), has_bias ? c.bias : -0.0f);
+}
+
+__device__ __forceinline__ void zmi_finish_element_ring(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &c,
+                                                        float rs, int32_t s, int m, int n) {
+  const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+  const bool has_bias = p.bias != nullptr;
+  const int64_t o = (int64_t)m * p.ldc + n;
+  if (epi.fast_kind != ZMI_EK_GENERIC && epi.dst_dt == ZMI_DT_BF16) {
+    zmi_set_f32_flush();
+    float y = zmi_ring_chain(s, c, rs, has_bias);
+    switch (epi.fast_kind) {
+    case ZMI_EK_SWISH: y = zmi_act_bf16<ZMI_EK_SWISH>(y); break;
+    case ZMI_EK_GELU_TANH: y = zmi_act_bf16<ZMI_EK_GELU_TANH>(y); break;
+    case ZMI_EK_RELU: y = zmi_act_bf16<ZMI_EK_RELU>(y); break;
+    default: break;
+    }
+    zmi_global<uint16_t>(p.dst)[o] = (uint16_t)zmi_pack_bf16(y, 0.0f);
+    return;
+  }
+  if (epi.fast_kind != ZMI_EK_GENERIC && epi.dst_dt == ZMI_DT_F32) {
+    float y;
+    switch (epi.fast_kind) {
+    case ZMI_EK_SWISH: y = zmi_fast_value<ZMI_EK_SWISH>(s, c, rs, has_rs, has_ws, has_bias); break;
+    case ZMI_EK_GELU_TANH: y = zmi_fast_value<ZMI_EK_GELU_TANH>(s, c, rs, has_rs, has_ws, has_bias); break;
+    case ZMI_EK_RELU: y = zmi_fast_value<ZMI_EK_RELU>(s, c, rs, has_rs, has_ws, has_bias); break;
+    default: y = zmi_fast_value<ZMI_EK_NONE>(s, c, rs, has_rs, has_ws, has_bias); break;
+    }
+    zmi_global<float>(p.dst)[o] = y;
+    return;
+  }
+  if (zmi_epilogue_is_raw_s32(epi, p.bias)) ((int32_t *)p.dst)[o] = s + c.comp;
+  else zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_value(epi, s, c, rs, m, n, p.dst, p.ldc));
+}
+
+// Gated pair (gate column n, up column n + N/2) -> output column n; straight-line epilogues only (no element-wise
+// post-op in front of the activation), bf16 or f32 destination.
+__device__ __forceinline__ void zmi_finish_gated_ring(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &cg,
+                                                      const ZmiColCtx &cu, float rs, int32_t sg, int32_t su, int m, int n) {
+  const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
+  const bool has_bias = p.bias != nullptr;
+  const int64_t o = (int64_t)m * p.ldc + n;
+  if (epi.dst_dt == ZMI_DT_BF16) {
+    zmi_set_f32_flush();
+    const float y0 = zmi_ring_chain(sg, cg, rs, has_bias), y1 = zmi_ring_chain(su, cu, rs, has_bias);
+    // gate and up are rounded to bf16 first, as when the activation reads a stored GEMM result
+    const uint32_t gu = zmi_pack_bf16(y0, y1);
+    const float g = __uint_as_float(gu << 16), u = __uint_as_float(gu & 0xffff0000u);
+    const float z = epi.gated_act == ZMI_ACT_SILU_AND_MUL ? zmi_act_bf16<ZMI_EK_SWISH>(g) * u : zmi_gated(epi.gated_act, g, u);
+    zmi_global<uint16_t>(p.dst)[o] = (uint16_t)zmi_pack_bf16(z, 0.0f);
+  } else {
+    const float y0 = zmi_fast_value<ZMI_EK_NONE>(sg, cg, rs, has_rs, has_ws, has_bias);
+    const float y1 = zmi_fast_value<ZMI_EK_NONE>(su, cu, rs, has_rs, has_ws, has_bias);
+    zmi_global<float>(p.dst)[o] = zmi_gated(epi.gated_act, y0, y1);
+  }
+}
 #endif  // __HIPCC__

@@ -87,6 +87,12 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
                                       const ZmiEpilogue &epi, hipStream_t stream);
 
+// k_group_decode.hip: the problems of a grouped launch that have 1 .. 16 rows (rows in fragment order), gated or not;
+// one workgroup per (problem, 32 output columns), max_out_cols = the widest problem's output columns
+bool zmi_group_decode_takes(const ZmiEpilogue &epi, int N);
+hipError_t zmi_launch_gemm_group_decode(const ZmiProblem *probs_dev, int n_prob, int max_out_cols, const ZmiEpilogue &epi,
+                                        hipStream_t stream);
+
 // k_smallm.hip
 struct ZmiFusedQuant {
   const void *x;          // bf16 / f32 rows, null: no fused quantization

@@ -10,9 +10,12 @@
 // filled block, so that the weights of a problem are streamed by one launch only
 // (the choice when the launch is bound by weight traffic, not by MFMA work).
 #define ZMI_RING_PAD 0x10000
+// Problems with at most 16 rows get no tiles: the decode-shaped grouped kernel (k_group_decode.hip) takes them.
+#define ZMI_RING_SKIP_SMALL 0x20000
 template <int BM>
 __device__ __host__ __forceinline__ void zmi_ring_rows(int M, int top_flags, int &full, bool &has_rem) {
   const int top = top_flags & 0xffff;
+  if ((top_flags & ZMI_RING_SKIP_SMALL) && M <= 16) { full = 0; has_rem = false; return; }
   full = BM == top ? M / top : 0;
   const int r = M % top;
   if (top_flags & ZMI_RING_PAD) has_rem = BM == top && r > 0;
