@@ -315,6 +315,13 @@ ZO_EXPORT float zo_eltwise(int32_t po, float x, float alpha, float beta) {
   case ZMI_PO_SWISH: return zo_swish(x, 1.0f);
   case ZMI_PO_TANH: return tanhf(x);
   case ZMI_PO_CLIP: { x = x > alpha ? x : alpha; return x > beta ? beta : x; }
+  /* elu_fwd .. log_fwd, operators/matmul/matmul_ref_kernel.cpp:694-751 (elu subtracts the double constant 1.0) */
+  case ZMI_PO_ELU: return x > 0 ? x : (float)(alpha * (expf(x) - 1.0));
+  case ZMI_PO_SQUARE: return x * x;
+  case ZMI_PO_ABS: return x > 0 ? x : -x;
+  case ZMI_PO_SQRT: return sqrtf(x);
+  case ZMI_PO_EXP: return expf(x);
+  case ZMI_PO_LOG: return logf(x);
   default: return x;
   }
 }

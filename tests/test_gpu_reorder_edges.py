@@ -181,6 +181,56 @@ def test_every_eltwise_post_op_f32(zo, po, M):
     H.check_f32(got, want, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("po", [capi.PO_ELU, capi.PO_SQUARE, capi.PO_ABS, capi.PO_SQRT, capi.PO_EXP, capi.PO_LOG])
+@pytest.mark.parametrize("M,dst_dt", [(7, capi.DT_F32), (24, capi.DT_BF16), (200, capi.DT_F32), (200, capi.DT_BF16)])
+def test_remaining_eltwise_post_ops(zo, po, M, dst_dt):
+    """elu (alpha from the post-op) / square / abs / sqrt / exp / log through the interpreter of every kernel that can
+    take the call: f32 within 1e-5 relative, bf16 within one ulp.  sqrt and log see a chain whose result is positive
+    (ReLU + a bias in front of them keeps them off the reference's NaN / -inf cases, which are compared too: NaN == NaN)."""
+    rng = np.random.default_rng(po * 100 + M)
+    K, N = 256, 96
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    ss = np.array([0.01], dtype=np.float32)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.uniform(0.5, 1.5, N).astype(np.float32)
+    ws_d, b_d = H.to_dev(ws), H.to_dev(b)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=dst_dt, bias=capi.DT_F32)
+    p.src_scale = lowoha.QuantParam(ss.ctypes.data, capi.DT_F32, (1,))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    chain = [lowoha.PostOp(po, alpha=1.7)]
+    if po in (capi.PO_SQRT, capi.PO_LOG):
+        add = np.full((1, N), 0.25, dtype=np.float32)
+        add_d = H.to_dev(add)
+        chain = [lowoha.PostOp(capi.PO_RELU), lowoha.PostOp(capi.PO_BINARY_ADD, add_d, capi.DT_F32, (1, N)), lowoha.PostOp(po)]
+    p.postop_ = chain
+    dst = torch.zeros((M, N), dtype=torch.float32 if dst_dt == capi.DT_F32 else torch.bfloat16, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(a), K, H.to_dev(w), N, b_d, 0.0, dst, N, True, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    ph = H.host_params(p, src_scale=ss, wei_scale=ws)
+    if po in (capi.PO_SQRT, capi.PO_LOG):
+        ph.postop_ = [lowoha.PostOp(capi.PO_RELU), lowoha.PostOp(capi.PO_BINARY_ADD, add.ctypes.data, capi.DT_F32, (1, N)),
+                      lowoha.PostOp(po)]
+    keep = []
+    st, want, _, _ = zo.matmul_int8(a, w, ph.flat(keep), M, N, K, bias=b)
+    assert st == capi.SUCCESS
+    if dst_dt == capi.DT_F32:
+        H.check_f32(H.to_host(dst), want, rtol=1e-5, atol=1e-6)
+    else:
+        H.check_bf16(H.to_host(dst), want, max_frac=5e-3)
+
+
+def test_softmax_post_op_is_refused():
+    rng = np.random.default_rng(1)
+    M, K, N = 8, 64, 32
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
+    p.postop_ = [lowoha.PostOp(capi.PO_SOFTMAX)]
+    dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(rng.integers(-128, 128, (M, K), dtype=np.int8)), K,
+                              H.to_dev(H.gen_weights(rng, K, N)), N, None, 0.0, dst, N, True, p)
+    assert st == capi.UNIMPLEMENTED
+
+
 def test_binary_post_ops_chain_and_dst_quant(zo):
     rng = np.random.default_rng(99)
     M, K, N = 40, 128, 80

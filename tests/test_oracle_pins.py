@@ -566,6 +566,34 @@ def test_eltwise_against_libm_double(zo):
     assert np.array_equal(lr, np.where(xs > 0, xs, np.float32(0.01) * xs))
 
 
+def test_remaining_eltwise_types_closed_forms_and_libm(zo):
+    """elu / square / abs / sqrt / exp / log (matmul_ref_kernel.cpp:694-751): exact where the mathematics fixes
+    the float (squares and roots of small integers, |x|, elu above zero, exp(0), log(1)), libm in double elsewhere."""
+    ints = np.arange(-20, 21, dtype=np.float32)
+    assert np.array_equal(zo.eltwise(capi.PO_SQUARE, ints), ints * ints)
+    assert np.array_equal(zo.eltwise(capi.PO_ABS, ints), np.abs(ints))
+    assert np.signbit(zo.eltwise(capi.PO_ABS, np.array([-0.0], dtype=np.float32)))[0] == False   # noqa: E712  (-(-0) = +0)
+    sq = np.arange(0, 40, dtype=np.float32)
+    assert np.array_equal(zo.eltwise(capi.PO_SQRT, sq * sq), sq)
+    assert np.isnan(zo.eltwise(capi.PO_SQRT, np.array([-1.0], dtype=np.float32)))[0]
+    assert zo.eltwise(capi.PO_EXP, np.array([0.0], dtype=np.float32))[0] == 1.0
+    assert zo.eltwise(capi.PO_LOG, np.array([1.0], dtype=np.float32))[0] == 0.0
+    pos = np.linspace(0.001, 9, 200).astype(np.float32)
+    assert np.array_equal(zo.eltwise(capi.PO_ELU, pos, 1.7), pos)                  # identity above zero
+    xs = np.linspace(-15, 15, 2001).astype(np.float32)
+    ex = zo.eltwise(capi.PO_EXP, xs)
+    el = zo.eltwise(capi.PO_ELU, xs, 1.7)
+    lg = zo.eltwise(capi.PO_LOG, np.abs(xs) + np.float32(1e-3))
+    for i, x in enumerate(xs.astype(np.float64)):
+        assert abs(float(ex[i]) - math.exp(x)) <= 2 * float(np.spacing(np.float32(math.exp(x))))
+        if x <= 0:
+            # alpha * (float(e^x) - 1) in double: the float rounding of e^x is the only error before the final rounding
+            want = 1.7 * (math.exp(x) - 1.0)
+            assert abs(float(el[i]) - want) <= 1.7 * 6e-8 + abs(want) * 1.2e-7
+        v = float(np.abs(xs[i]) + np.float32(1e-3))
+        assert abs(float(lg[i]) - math.log(v)) <= 2 * float(np.spacing(np.float32(abs(math.log(v))))) + 1e-45
+
+
 # ---------------------------------------------------- gated act / reduce
 def test_gated_act_brute_force(zo):
     rng = np.random.default_rng(13)

@@ -208,6 +208,11 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
     case ZMI_PO_RELU: case ZMI_PO_LEAKY_RELU: case ZMI_PO_GELU_TANH: case ZMI_PO_GELU_ERF:
     case ZMI_PO_SIGMOID: case ZMI_PO_SWISH: case ZMI_PO_TANH:
       break;
+    // The reference's AOCL wiring drops these types without a word (backends/aocl/aocl_postop.cpp:476-479, the
+    // fault its validator already refuses mish for); here they compute what the reference's own kernel defines
+    // (operators/matmul/matmul_ref_kernel.cpp:694-751; elu's alpha is the post-op's alpha).
+    case ZMI_PO_ELU: case ZMI_PO_SQUARE: case ZMI_PO_ABS: case ZMI_PO_SQRT: case ZMI_PO_EXP: case ZMI_PO_LOG:
+      break;
     case ZMI_PO_CLIP:
       if (d.alpha > d.beta) { float t = d.alpha; d.alpha = d.beta; d.beta = t; }
       break;
@@ -223,8 +228,7 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
       break;
     }
     default:
-      // the reference's AOCL wiring skips the remaining types silently
-      // (backends/aocl/aocl_postop.cpp:476-479); refusing is the safer reading
+      // (softmax and pooling are not element-wise)
       set_error("post-op type not implemented on the int8 path");
       return ZMI_UNIMPLEMENTED;
     }

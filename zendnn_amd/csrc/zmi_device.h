@@ -246,6 +246,13 @@ __device__ __forceinline__ float zmi_eltwise(int type, float x, float alpha, flo
   case ZMI_PO_SWISH: return x * zmi_sigmoid(x);
   case ZMI_PO_TANH: return tanhf(x);
   case ZMI_PO_CLIP: { x = x > alpha ? x : alpha; return x > beta ? beta : x; }
+  // (the remaining element-wise types of the reference's kernel, matmul_ref_kernel.cpp:694-751)
+  case ZMI_PO_ELU: return x > 0.0f ? x : alpha * (zmi_expf(x) - 1.0f);
+  case ZMI_PO_SQUARE: return x * x;
+  case ZMI_PO_ABS: return x > 0.0f ? x : -x;
+  case ZMI_PO_SQRT: return __fsqrt_rn(x);
+  case ZMI_PO_EXP: return zmi_expf(x);
+  case ZMI_PO_LOG: return logf(x);
   default: return x;
   }
 }
