@@ -321,6 +321,21 @@ ZMI_API int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk,
                       int32_t E, int32_t *counts, int32_t *offsets,
                       int32_t *slot_of);
 
+/* zmi_moe_router_topk: the step in front of zmi_moe_route -- router logits
+ * [T, E] (f32 or bf16, device, row stride ldl elements) -> topk_ids [T, topk]
+ * (s32) and topk_weights [T, topk] (f32), both device.  The reference has no
+ * counterpart (routing is the framework's, same document); its MoE post-op
+ * consumes exactly these two arrays (group_matmul_moe_postop.cpp:103-129).
+ *   ids:     the topk largest logits of the token in descending order, equal
+ *            logits in ascending expert order (the head of a stable descending
+ *            sort); -0 == +0, NaN sorts last;
+ *   weights: softmax over all E logits in f32, of the selected experts; with
+ *            renormalize != 0 divided by the sum of the topk selected weights.
+ * Limits: E <= 512, topk <= min(E, 64). */
+ZMI_API int32_t zmi_moe_router_topk(const void *logits, int32_t logits_dt, int64_t ldl,
+                            int32_t T, int32_t E, int32_t topk, int32_t renormalize,
+                            int32_t *topk_ids, float *topk_weights);
+
 /* zmi_moe_fused_device: whole MoE block with routing kept on the device.
  * x [T,H] bf16 -> per-token s8 quantization -> expert-sorted scatter ->
  * Op1 (gate|up, s8 blob) -> act(gate)*up -> bf16 -> per-token s8 ->

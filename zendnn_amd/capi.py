@@ -168,6 +168,8 @@ SIGNATURES = {
     "zmi_version": (C.c_char_p, []),
     "zmi_moe_route": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                   C.c_void_p, C.c_void_p]),
+    "zmi_moe_router_topk": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                        C.c_void_p, C.c_void_p]),
     "zmi_moe_fused_device": (C.c_int32, [C.POINTER(MoeDeviceT)]),
     "zmi_calib_hbm_read": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.c_uint64, C.c_int32, C.c_int32,
                                        C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),

@@ -218,8 +218,9 @@ __device__ __forceinline__ float zmi_expf(float x) {
   float t = x * l2e_hi;
   float r = __builtin_fmaf(x, l2e_hi, -t) + x * l2e_lo;   // rounding error of t plus the low part
   float e = __builtin_amdgcn_exp2f(t);
-  // an overflowed e must stay +inf (inf * negative correction + inf would be NaN)
-  return e == __builtin_inff() ? e : __builtin_fmaf(e, r * 0.693147182464599609375f, e);
+  // an overflowed e must stay +inf (inf * negative correction + inf would be NaN), and exp(-inf) is 0
+  // (there t = -inf makes the correction term NaN)
+  return (e == __builtin_inff() || e == 0.0f) ? e : __builtin_fmaf(e, r * 0.693147182464599609375f, e);
 }
 
 __device__ __forceinline__ float zmi_sigmoid(float x) {

@@ -163,6 +163,8 @@ hipError_t zmi_launch_moe_combine(const void *const *row_ptrs_dev, const void *r
 // align: every expert's first slot is rounded up to a multiple of it (1: dense numbering).
 // src_of (optional, n_slots entries): the flat (token, k) index that fills each slot, -1 for idle slots.
 size_t zmi_moe_route_scratch_ints(int64_t n, int E);
+hipError_t zmi_launch_moe_router_topk(const void *logits, int logits_dt, int64_t ldl, int T, int E, int topk,
+                                      int renormalize, int32_t *topk_ids, float *topk_weights, hipStream_t stream);
 hipError_t zmi_launch_moe_route(const int32_t *topk_ids, int T, int topk, int E, int align, int32_t *counts,
                                 int32_t *offsets, int32_t *slot_of, int32_t *src_of, int n_slots,
                                 int32_t *hist_scratch, hipStream_t stream);
