@@ -42,10 +42,10 @@ def make_case(seed, T, Hd, I, E, topk, skew=False):
     return c
 
 
-def dyn_params(M, N, ws_buf, dst_dt=capi.DT_BF16, packed=False):
+def dyn_params(M, N, ws_buf, dst_dt=capi.DT_BF16, packed=False, scale_dt=capi.DT_F32):
     p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=dst_dt, compute=capi.DT_S8)
     p.dynamic_quant = True
-    p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (M, 1))
+    p.src_scale = lowoha.QuantParam(None, scale_dt, (M, 1))
     p.wei_scale = lowoha.QuantParam(ws_buf, capi.DT_F32, (1, N))
     if packed:
         p.mem_format_b = "r"
@@ -53,24 +53,25 @@ def dyn_params(M, N, ws_buf, dst_dt=capi.DT_BF16, packed=False):
     return p
 
 
-def oracle_expert(zo, c, e, x_rows, act=capi.ACT_SILU_AND_MUL):
+def oracle_expert(zo, c, e, x_rows, act=capi.ACT_SILU_AND_MUL, scale_dt=capi.DT_F32):
     """Reference composition for the rows of one expert: dynamic-quant Op1 -> bf16 ->
     gated activation -> bf16 -> dynamic-quant Op2 -> bf16
-    (group_matmul_fused_moe.cpp:906-1078, the two-pass form)."""
+    (group_matmul_fused_moe.cpp:906-1078, the two-pass form).  The down projection's source
+    scales take Op1's scale dtype (group_matmul_fused_moe.cpp:816-820)."""
     M = x_rows.shape[0]
     keep = []
-    p1 = dyn_params(M, 2 * c.I, c.s13[e].ctypes.data).flat(keep)
+    p1 = dyn_params(M, 2 * c.I, c.s13[e].ctypes.data, scale_dt=scale_dt).flat(keep)
     st, y1, _, _ = zo.matmul_int8(x_rows, c.w13[e], p1, M, 2 * c.I, c.H)
     assert st == capi.SUCCESS
     zo.gated_act(act, y1, capi.DT_BF16)
     a = np.ascontiguousarray(y1[:, :c.I])
-    p2 = dyn_params(M, c.H, c.s2[e].ctypes.data).flat(keep)
+    p2 = dyn_params(M, c.H, c.s2[e].ctypes.data, scale_dt=scale_dt).flat(keep)
     st, y2, _, _ = zo.matmul_int8(a, c.w2[e], p2, M, c.H, c.I)
     assert st == capi.SUCCESS
     return a, y2
 
 
-def oracle_moe(zo, c, tokens):
+def oracle_moe(zo, c, tokens, scale_dt=capi.DT_F32):
     """Final output rows for the given token indices."""
     need = {}
     for t in tokens:
@@ -80,7 +81,7 @@ def oracle_moe(zo, c, tokens):
     y2_of = {}
     for e, lst in need.items():
         xr = np.ascontiguousarray(c.x[[t for t, _ in lst]])
-        _, y2 = oracle_expert(zo, c, e, xr)
+        _, y2 = oracle_expert(zo, c, e, xr, scale_dt=scale_dt)
         for i, (t, k) in enumerate(lst):
             y2_of[(t, k)] = y2[i]
     rows = [np.ascontiguousarray(y2_of[(int(t), k)]) for t in tokens for k in range(c.topk)]
@@ -124,10 +125,10 @@ class DeviceMoe:
                 out.append(self.dst_down[e].data_ptr() + int(j) * c.H * 2)
         return out
 
-    def call_fused(self, with_postop=True, act=capi.ACT_SILU_AND_MUL):
+    def call_fused(self, with_postop=True, act=capi.ACT_SILU_AND_MUL, scale_dt=capi.DT_F32):
         c = self.c
         E = c.E
-        params = [dyn_params(max(c.M[e], 0), 2 * c.I, self.s13[e], packed=self.packed) for e in range(E)]
+        params = [dyn_params(max(c.M[e], 0), 2 * c.I, self.s13[e], packed=self.packed, scale_dt=scale_dt) for e in range(E)]
         fm = lowoha.FusedMoe(
             down_weight=self.w2, N_down=[c.H] * E, ldb_down=[c.H] * E,
             down_scale=[lowoha.QuantParam(self.s2[e], capi.DT_F32, (1, c.H)) for e in range(E)],

@@ -462,3 +462,112 @@ def test_group_gated_gelu_and_mul_unfused_block(zo):
             continue
         a, _ = MH.oracle_expert(zo, c, e, np.ascontiguousarray(c.x[c.rows_of[e]]), act=capi.ACT_GELU_AND_MUL)
         H.check_bf16(H.to_host(dst[e])[:, :c.I], a, max_frac=5e-3)
+
+
+# ------------------------------------------------------------------ the fused block, stage by stage
+STAGED = [(96, 512, 320, 8, 2, False), (300, 256, 96, 16, 6, True), (64, 1024, 1408, 4, 2, False)]
+
+
+@pytest.mark.parametrize("T,Hd,I,E,topk,skew", STAGED)
+@pytest.mark.parametrize("act", [capi.ACT_SILU_AND_MUL, capi.ACT_GELU_AND_MUL])
+def test_staged_op1_and_activation_within_one_ulp(zo, T, Hd, I, E, topk, skew, act):
+    """Stage 1 of the fused block alone (dynamic quantization, gate | up GEMM, gated activation, bf16): every
+    element within one bf16 ulp of the oracle, differing at all only next to a rounding tie (device exp /
+    reciprocal against libm)."""
+    c = MH.make_case(0x5EED0A00 + T, T, Hd, I, E, topk, skew)
+    d = MH.DeviceMoe(c)
+    dst = [torch.zeros((max(c.M[e], 1), 2 * c.I), dtype=torch.bfloat16, device=H.DEV) for e in range(E)]
+    params = [MH.dyn_params(c.M[e], 2 * c.I, d.s13[e]) for e in range(E)]
+    st = lowoha.group_matmul_direct(
+        ["r"] * E, [False] * E, [False] * E, c.M, [2 * c.I] * E, [c.H] * E, [1.0] * E,
+        d.src, [c.H] * E, d.w13, [2 * c.I] * E, [None] * E, [0.0] * E,
+        dst, [2 * c.I] * E, [True] * E, params, gated_act=act)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for e in range(E):
+        if c.M[e] == 0:
+            continue
+        a, _ = MH.oracle_expert(zo, c, e, np.ascontiguousarray(c.x[c.rows_of[e]]), act=act)
+        H.check_bf16(H.to_host(dst[e])[:, :c.I], a, max_frac=5e-3, atol=1e-6 if act == capi.ACT_GELU_AND_MUL else 0.0)
+
+
+@pytest.mark.parametrize("T,Hd,I,E,topk,skew", STAGED)
+@pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_BF16])
+def test_staged_op2_on_the_oracles_intermediate_is_bit_identical(zo, T, Hd, I, E, topk, skew, dst_dt):
+    """Stage 2 alone: the down projection (dynamic re-quantization of the activated bf16 rows, GEMM, scales) fed
+    with the ORACLE's activated intermediate.  Nothing in this stage depends on exp or a reciprocal, so the result
+    is the oracle's bit for bit, f32 and bf16: the two-ulp allowance of the end-to-end comparison exists only for
+    what a one-ulp difference of stage 1 propagates through the re-quantization."""
+    c = MH.make_case(0x5EED0B00 + T, T, Hd, I, E, topk, skew)
+    acts, wants = [], []
+    keep = []
+    for e in range(E):
+        if c.M[e] == 0:
+            acts.append(None)
+            wants.append(None)
+            continue
+        a, _ = MH.oracle_expert(zo, c, e, np.ascontiguousarray(c.x[c.rows_of[e]]))
+        p2 = MH.dyn_params(c.M[e], c.H, c.s2[e].ctypes.data, dst_dt=dst_dt).flat(keep)
+        st, y2, _, _ = zo.matmul_int8(a, c.w2[e], p2, c.M[e], c.H, c.I)
+        assert st == capi.SUCCESS
+        acts.append(a)
+        wants.append(y2)
+    tdt = torch.float32 if dst_dt == capi.DT_F32 else torch.bfloat16
+    src = [H.to_dev(a) for a in acts]
+    dst = [torch.zeros((max(c.M[e], 1), c.H), dtype=tdt, device=H.DEV) for e in range(E)]
+    s2 = [H.to_dev(s) for s in c.s2]
+    params = [MH.dyn_params(c.M[e], c.H, s2[e], dst_dt=dst_dt) for e in range(E)]
+    st = lowoha.group_matmul_direct(
+        ["r"] * E, [False] * E, [False] * E, c.M, [c.H] * E, [c.I] * E, [1.0] * E,
+        src, [c.I] * E, [H.to_dev(w) for w in c.w2], [c.H] * E, [None] * E, [0.0] * E,
+        dst, [c.H] * E, [True] * E, params)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for e in range(E):
+        if c.M[e] == 0:
+            continue
+        got = H.to_host(dst[e])
+        assert np.array_equal(got[:c.M[e]], wants[e]), f"expert {e}"
+
+
+@pytest.mark.parametrize("T,Hd,I,E,topk", [(96, 512, 320, 8, 2), (16, 1024, 512, 8, 2)])
+def test_fused_moe_bf16_source_scale_dtype(zo, T, Hd, I, E, topk):
+    """src_scale.dt = bf16 on the fused block: Op1's per-token scales AND the down projection's are narrowed to
+    bf16 and the GEMMs multiply by the narrowed values (group_matmul_fused_moe.cpp:816-820)."""
+    c = MH.make_case(0x5EED0C00 + T, T, Hd, I, E, topk)
+    d = MH.DeviceMoe(c)
+    st = d.call_fused(scale_dt=capi.DT_BF16)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    want = MH.oracle_moe(zo, c, list(range(T)), scale_dt=capi.DT_BF16)
+    check_moe_out(H.to_host(d.out), want)
+    # and the result is not the f32-scale one (the narrowing is really applied in both stages)
+    want_f32 = MH.oracle_moe(zo, c, list(range(T)))
+    assert (H.bf16_ulp_diff(want, want_f32) > 2).mean() > 0.05
+
+
+def test_group_experts_with_different_scale_dtypes_run_one_by_one(zo):
+    """Experts whose scale dtypes differ cannot share one epilogue descriptor: each is computed with its own."""
+    rng = np.random.default_rng(77)
+    Ms, K, N = [20, 33], 128, 64
+    xs = [H.gen_bf16_normal(rng, (m, K)) for m in Ms]
+    ws = [H.gen_weights(rng, K, N) for _ in Ms]
+    wsc = [rng.uniform(0.001, 0.01, N).astype(np.float32) for _ in Ms]
+    wsc_bits = H.bf16_bits(wsc[1])
+    wsc_d = [H.to_dev(wsc[0]), H.to_dev(wsc_bits)]
+    params = []
+    for e, m in enumerate(Ms):
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_F32, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32 if e == 0 else capi.DT_BF16, (m, 1))
+        p.wei_scale = lowoha.QuantParam(wsc_d[e], capi.DT_F32 if e == 0 else capi.DT_BF16, (1, N))
+        params.append(p)
+    dst = [torch.zeros((m, N), dtype=torch.float32, device=H.DEV) for m in Ms]
+    st = lowoha.group_matmul_direct(["r"] * 2, [False] * 2, [False] * 2, Ms, [N] * 2, [K] * 2, [1.0] * 2,
+                                    [H.to_dev(x) for x in xs], [K] * 2, [H.to_dev(w) for w in ws], [N] * 2, [None] * 2,
+                                    [0.0] * 2, dst, [N] * 2, [True] * 2, params)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    keep = []
+    host_scales = [wsc[0], wsc_bits]
+    for e, m in enumerate(Ms):
+        ph = H.host_params(params[e], src_scale=None, wei_scale=host_scales[e])
+        st, want, _, _ = zo.matmul_int8(xs[e], ws[e], ph.flat(keep), m, N, K)
+        assert st == capi.SUCCESS
+        assert np.array_equal(H.to_host(dst[e]), want), f"expert {e}"

@@ -98,9 +98,16 @@ def test_quant_invariants_random(zo):
     xf = zo.bf16_to_f32(x)
     assert np.all(np.abs(q.astype(np.int32)).max(axis=1) == 127)
     assert np.array_equal(s, (np.abs(xf).max(axis=1) / np.float32(127.0)).astype(np.float32))
-    # independent evaluation of the rounding in float64 (v/s is far from a tie here or exactly on it)
-    want = np.rint((xf / s[:, None]).astype(np.float32)).astype(np.int8)
-    assert np.array_equal(q, want)
+    # what "quantized" means, in float64 and without the oracle's rounding routine: q is an integer nearest
+    # to x / s (the f32 quotient the oracle rounds is within 2^-24 relative of the exact one, i.e. 127 * 2^-24
+    # absolute), it keeps the sign and the order of x within a row, and x -> q * s loses at most half a step
+    r = xf.astype(np.float64) / s.astype(np.float64)[:, None]
+    assert np.all(np.abs(q.astype(np.float64) - r) <= 0.5 + 127.0 * 2.0 ** -24)
+    assert np.all((q.astype(np.int32) * np.sign(xf).astype(np.int32)) >= 0)
+    order = np.argsort(xf, axis=1, kind="stable")
+    assert np.all(np.diff(np.take_along_axis(q.astype(np.int32), order, axis=1), axis=1) >= 0)
+    assert np.all(np.abs(xf.astype(np.float64) - q.astype(np.float64) * s.astype(np.float64)[:, None])
+                  <= 0.5 * s.astype(np.float64)[:, None] * (1.0 + 1e-5))
 
 
 # ------------------------------------------------------------ s32 GEMM

@@ -20,7 +20,7 @@ int32_t validate_matmul(const void *src, const void *weight, const void *dst, in
   if (Batch_A <= 0 || Batch_B <= 0) { set_error("batch sizes must be positive"); return ZMI_FAILURE; }
   const bool is_int8 = p.dt_wei == ZMI_DT_S8;
   if ((p.src_scale.buff || p.dst_scale.buff || p.src_zp.buff || p.dst_zp.buff) && !is_int8) {
-    set_error("source / destination quantization params need s8 weights");
+    set_error("src / dst scales and zero-points are given but the weights are not s8");
     return ZMI_FAILURE;
   }
   if (p.src_scale.buff) {
@@ -32,23 +32,23 @@ int32_t validate_matmul(const void *src, const void *weight, const void *dst, in
       const bool per_token = n == M;
       const bool per_group = n > M && n % M == 0 && K % (n / M) == 0;
       if (!(src_ok && sym && dst_ok && (per_token || per_group))) {
-        set_error("per-token / per-group source scale needs s8/bf16/f32 src, no source zero-point and f32/bf16 dst");
+        set_error("source scales per row or per K-group: the source must be s8 / bf16 / f32 without a zero-point and the destination f32 / bf16");
         return ZMI_FAILURE;
       }
       const int64_t wn = p.wei_scale.buff ? nelems(p.wei_scale) : 0;
       if (per_token && p.pack_format_b != 1 && wn != N) {
-        set_error("per-token source scale requires a per-channel weight scale of N elements");
+        set_error("a source scale per row goes with a weight scale per column (N elements)");
         return ZMI_FAILURE;
       }
       // (GGML-packed weights carry their per-group scales inside the packed buffer: lowoha_matmul_utils.cpp:276-283)
       if (per_group && p.pack_format_b != 1 && wn != (n / M) * N) {
-        set_error("per-group source scale requires a per-group weight scale");
+        set_error("a source scale per K-group goes with a weight scale of groups x N elements");
         return ZMI_FAILURE;
       }
     }
   }
   auto per_tensor = [](const zmi_quant_t &q, const char *name) {
-    if (q.buff && nelems(q) != 1) { set_error(std::string(name) + " supports only per-tensor"); return false; }
+    if (q.buff && nelems(q) != 1) { set_error(std::string(name) + " must hold exactly one element (one value for the tensor)"); return false; }
     return true;
   };
   if (!per_tensor(p.src_zp, "source zero-point") || !per_tensor(p.dst_scale, "destination scale") ||
@@ -162,7 +162,7 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
       e.wei_scale_mode = 3;
     } else if (e.n_groups > 0) {
       // lowoha_matmul_utils.cpp:292-301
-      set_error("per-group source scale requires a per-group weight scale of G * N elements");
+      set_error("source scales per K-group: the weight scale must hold groups x N elements");
       return ZMI_FAILURE;
     } else {
       set_error("per-group weight scales need a per-group source scale ({M,G} with the same G)");
@@ -326,28 +326,28 @@ bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
 // validate_w4a8_inputs, matmul/lowoha_matmul_utils.cpp:72-176, in its order.  Other uses of s4 weights
 // (weight-only quantization with bf16 compute) are not part of this library.
 int32_t validate_w4a8(const zmi_matmul_params_t &p, int M, int N, int K) {
-  if (p.dt_src == ZMI_DT_S8) { set_error("W4A8 requires a bf16 source with dynamic_quant (a pre-quantized s8 source is not supported)"); return ZMI_FAILURE; }
-  if (p.dynamic_quant && (p.dt_src == ZMI_DT_F32 || p.dt_dst == ZMI_DT_F32)) { set_error("W4A8 supports bf16 source and bf16 output only"); return ZMI_FAILURE; }
-  if (p.dt_src == ZMI_DT_U8 && (p.src_scale.buff || p.dynamic_quant)) { set_error("s4 weights do not support a u8 source"); return ZMI_FAILURE; }
+  if (p.dt_src == ZMI_DT_S8) { set_error("s4 weights with an s8 source: the 4-bit path quantizes a bf16 source itself (set dynamic_quant)"); return ZMI_FAILURE; }
+  if (p.dynamic_quant && (p.dt_src == ZMI_DT_F32 || p.dt_dst == ZMI_DT_F32)) { set_error("s4 weights with dynamic_quant: source and destination must both be bf16 (f32 given)"); return ZMI_FAILURE; }
+  if (p.dt_src == ZMI_DT_U8 && (p.src_scale.buff || p.dynamic_quant)) { set_error("s4 weights with a u8 source: the 4-bit path is symmetric and starts from bf16"); return ZMI_FAILURE; }
   const bool entry = p.dynamic_quant && p.dt_src == ZMI_DT_BF16;
-  if (entry && p.dt_compute != ZMI_DT_S8) { set_error("W4A8 dynamic quantization requires s8 compute"); return ZMI_FAILURE; }
+  if (entry && p.dt_compute != ZMI_DT_S8) { set_error("s4 weights with dynamic_quant: dt_compute must be s8"); return ZMI_FAILURE; }
   if (!entry) { set_error("s4 weights: only W4A8 (bf16 source, dynamic_quant, s8 compute) is implemented, not weight-only quantization"); return ZMI_UNIMPLEMENTED; }
-  if (p.dt_dst != ZMI_DT_BF16) { set_error("W4A8 dynamic quantization requires bf16 output"); return ZMI_FAILURE; }
-  if (p.wei_zp.buff || p.src_zp.buff) { set_error("W4A8 supports symmetric quantization only"); return ZMI_FAILURE; }
+  if (p.dt_dst != ZMI_DT_BF16) { set_error("s4 weights with dynamic_quant: dt_dst must be bf16"); return ZMI_FAILURE; }
+  if (p.wei_zp.buff || p.src_zp.buff) { set_error("s4 weights with dynamic_quant: zero-points are not taken (weights and source are symmetric)"); return ZMI_FAILURE; }
   const zmi_quant_t &ws = p.wei_scale;
-  if (!ws.buff) { set_error("W4A8 requires a weight scale"); return ZMI_FAILURE; }
-  if (ws.dt != ZMI_DT_F32 && ws.dt != ZMI_DT_BF16) { set_error("W4A8 weight scale supports only f32 or bf16"); return ZMI_FAILURE; }
-  if (ws.ndims != 2) { set_error("W4A8 requires weight scale dims {G,N}"); return ZMI_FAILURE; }
+  if (!ws.buff) { set_error("s4 weights with dynamic_quant: wei_scale.buff is missing"); return ZMI_FAILURE; }
+  if (ws.dt != ZMI_DT_F32 && ws.dt != ZMI_DT_BF16) { set_error("s4 weights with dynamic_quant: wei_scale.dt must be f32 or bf16"); return ZMI_FAILURE; }
+  if (ws.ndims != 2) { set_error("s4 weights with dynamic_quant: wei_scale must be two-dimensional, {groups, N}"); return ZMI_FAILURE; }
   const int64_t G = ws.dims[0];
-  if (G <= 0 || ws.dims[1] != N) { set_error("W4A8 requires weight scale dims {G,N}"); return ZMI_FAILURE; }
-  if (K % G != 0) { set_error("W4A8 requires K divisible by the weight group count"); return ZMI_FAILURE; }
-  if ((K / G) % 4 != 0) { set_error("W4A8 requires K/G to be a multiple of 4"); return ZMI_FAILURE; }
+  if (G <= 0 || ws.dims[1] != N) { set_error("s4 weights with dynamic_quant: wei_scale dims must be {groups >= 1, N}"); return ZMI_FAILURE; }
+  if (K % G != 0) { set_error("s4 weights with dynamic_quant: the weight scale groups do not divide K"); return ZMI_FAILURE; }
+  if ((K / G) % 4 != 0) { set_error("s4 weights with dynamic_quant: a scale group must span a multiple of 4 values of K"); return ZMI_FAILURE; }
   const zmi_quant_t &ss = p.src_scale;
-  if (ss.dt != ZMI_DT_F32 && ss.dt != ZMI_DT_BF16) { set_error("W4A8 source scale supports only f32 or bf16"); return ZMI_FAILURE; }
-  if (ss.ndims != 2) { set_error("W4A8 requires source scale dims {1,1}, {M,1}, or {M,G}"); return ZMI_FAILURE; }
+  if (ss.dt != ZMI_DT_F32 && ss.dt != ZMI_DT_BF16) { set_error("s4 weights with dynamic_quant: src_scale.dt must be f32 or bf16"); return ZMI_FAILURE; }
+  if (ss.ndims != 2) { set_error("s4 weights with dynamic_quant: src_scale must be two-dimensional"); return ZMI_FAILURE; }
   const int64_t r = ss.dims[0], c = ss.dims[1];
   if (!((r == 1 && c == 1) || (r == M && c == 1) || (r == M && c == G))) {
-    set_error("W4A8 requires source scale dims {1,1}, {M,1}, or {M,G}");
+    set_error("s4 weights with dynamic_quant: src_scale dims must be {1,1} (tensor), {M,1} (row) or {M,groups}");
     return ZMI_FAILURE;
   }
   return ZMI_SUCCESS;
@@ -379,16 +379,12 @@ void zmi_reorder_params_init(zmi_reorder_params_t *p) {
   p->prepack.algo = ZMI_ALGO_NONE;
 }
 
-int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M, int32_t N, int32_t K,
-                          float alpha, const void *src, int32_t lda, const void *weight, int32_t ldb,
-                          const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
-                          const zmi_batch_params_t *batch_params, const zmi_matmul_params_t *params) {
-  clear_error();
-  if (async_failure_pending()) return ZMI_FAILURE;
-  if (!params) { set_error("null params"); return ZMI_FAILURE; }
-  const zmi_matmul_params_t &p = *params;
-  const int Batch_A = batch_params ? batch_params->Batch_A : 1;
-  const int Batch_B = batch_params ? batch_params->Batch_B : 1;
+// One matrix product (Batch_A == Batch_B == 1): everything matmul_direct does for one (src, weight, dst).
+static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_t M, int32_t N, int32_t K,
+                             float alpha, const void *src, int32_t lda, const void *weight, int32_t ldb,
+                             const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
+                             const zmi_matmul_params_t &p) {
+  const int Batch_A = 1, Batch_B = 1;
   const bool w4a8 = p.dt_wei == ZMI_DT_S4;
   if (w4a8) {
     // (the shape rules of this path keep the kernels inside their buffers: checked whatever the diagnostics switch says)
@@ -406,7 +402,6 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   // ---- what this library implements of matmul_direct: the int8 path ----
   if (p.dt_wei != ZMI_DT_S8 && !w4a8) { set_error("only s8 and (W4A8) s4 weights are implemented"); return ZMI_UNIMPLEMENTED; }
   if (layout != 'r' && layout != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
-  if (Batch_A != 1 || Batch_B != 1) { set_error("batched matmul is not implemented"); return ZMI_UNIMPLEMENTED; }
   const bool ggml = p.pack_format_b == 1;
   if (p.pack_format_b != 0 && !ggml) { set_error("unknown pack_format_b"); return ZMI_FAILURE; }
   if (ggml) {
@@ -682,6 +677,93 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
   }
   upload_fence();
   return st;
+}
+
+// bytes of one element (s4 weights never reach the batched form)
+static size_t dt_bytes(int32_t dt) {
+  switch (dt) {
+  case ZMI_DT_F32: case ZMI_DT_S32: return 4;
+  case ZMI_DT_BF16: case ZMI_DT_F16: case ZMI_DT_S16: return 2;
+  case ZMI_DT_S64: return 8;
+  default: return 1;
+  }
+}
+
+// matmul_direct: one product, or the batched form.  Reference for the batched form: bmm_execute,
+// matmul/partitioning/bmm/looper/bmm_looper.cpp:192-223 (strides: the caller's in elements, or derived from the
+// dimensions when (size_t)-1) and :326-340 (batch b reads src batch b % Batch_A, weight batch b % Batch_B --
+// index 0 when that side has one batch -- and writes dst batch b); every batch runs with the same parameters
+// except binary post-op operands with a leading batch dimension > 1, which advance by dims[1] * dims[2]
+// elements per batch (apply_bmm_postop_offsets, matmul/lowoha_matmul_utils.cpp:36-70).  Here the batches are
+// launches on the one stream, in order.
+int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M, int32_t N, int32_t K,
+                          float alpha, const void *src, int32_t lda, const void *weight, int32_t ldb,
+                          const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
+                          const zmi_batch_params_t *batch_params, const zmi_matmul_params_t *params) {
+  clear_error();
+  if (async_failure_pending()) return ZMI_FAILURE;
+  if (!params) { set_error("null params"); return ZMI_FAILURE; }
+  const zmi_matmul_params_t &p = *params;
+  const int Batch_A = batch_params ? batch_params->Batch_A : 1;
+  const int Batch_B = batch_params ? batch_params->Batch_B : 1;
+  if (Batch_A == 1 && Batch_B == 1) {
+    // (3-D binary operands of one batch read like 2-D ones)
+    bool has_3d = false;
+    for (int i = 0; i < p.n_postops; ++i) has_3d = has_3d || p.postops[i].ndims == 3;
+    if (!has_3d)
+      return matmul_single(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc, is_weights_const, p);
+  }
+  if (diagnostics_enabled() && p.dt_wei != ZMI_DT_S4) {
+    int32_t st = validate_matmul(src, weight, dst, M, N, K, Batch_A, Batch_B, p, is_weights_const != 0);
+    if (st != ZMI_SUCCESS) return st;
+  } else if (!src || !weight || !dst || M <= 0 || N <= 0 || K <= 0 || Batch_A <= 0 || Batch_B <= 0) {
+    set_error("null pointer or non-positive dimension");
+    return ZMI_FAILURE;
+  }
+  const int batch_count = Batch_A > Batch_B ? Batch_A : Batch_B;
+  if (batch_count > 1) {
+    if (p.dt_wei != ZMI_DT_S8) { set_error("batched matmul: only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+    if (p.dynamic_quant) {
+      // (the reference quantizes the {Batch_A, M, K} source as one 3-D tensor in front of the batches,
+      // matmul/quantization/reorder_quantization.cpp:126-137)
+      set_error("batched matmul with dynamic_quant is not implemented");
+      return ZMI_UNIMPLEMENTED;
+    }
+    if (p.pack_format_b != 0) { set_error("GGML packed weights do not take a weight batch"); return ZMI_FAILURE; }
+    if (p.mem_format_b == 'r' && Batch_B > 1 && batch_params->batch_stride_wei == (uint64_t)-1) {
+      set_error("batched prepacked weights need batch_stride_wei (bytes from one packed buffer to the next)");
+      return ZMI_FAILURE;
+    }
+  }
+  const uint64_t none = (uint64_t)-1;
+  const uint64_t s_src = batch_params && batch_params->batch_stride_src != none ? batch_params->batch_stride_src
+                                                                                : (uint64_t)(transA ? K : M) * (uint64_t)lda;
+  const uint64_t s_wei = batch_params && batch_params->batch_stride_wei != none ? batch_params->batch_stride_wei
+                                                                                : (uint64_t)(transB ? N : K) * (uint64_t)ldb;
+  const uint64_t s_dst = batch_params && batch_params->batch_stride_dst != none ? batch_params->batch_stride_dst
+                                                                                : (uint64_t)M * (uint64_t)ldc;
+  const size_t src_b = s_src * dt_bytes(p.dt_src), wei_b = s_wei * dt_bytes(p.dt_wei), dst_b = s_dst * dt_bytes(p.dt_dst);
+  for (int b = 0; b < batch_count; ++b) {
+    zmi_matmul_params_t bp = p;
+    std::vector<zmi_post_op_t> pos(p.postops, p.postops + (p.postops ? p.n_postops : 0));
+    bp.postops = pos.data();
+    for (size_t i = 0; i < pos.size(); ++i) {
+      zmi_post_op_t &po = pos[i];
+      if ((po.po_type != ZMI_PO_BINARY_ADD && po.po_type != ZMI_PO_BINARY_MUL) || !po.buff || po.ndims != 3) continue;
+      const int32_t odt = po.dtype == ZMI_DT_NONE ? ZMI_DT_F32 : po.dtype;
+      if (po.dims[0] > 1) {
+        if (po.dims[0] < batch_count) { set_error("binary post-op operand has fewer batches than the product"); return ZMI_FAILURE; }
+        po.buff = (uint8_t *)po.buff + (size_t)b * (size_t)(po.dims[1] * po.dims[2]) * dt_bytes(odt);
+      }
+      po.ndims = 2; po.dims[0] = po.dims[1]; po.dims[1] = po.dims[2]; po.dims[2] = 0;
+    }
+    const uint8_t *a = (const uint8_t *)src + (size_t)(Batch_A == 1 ? 0 : b % Batch_A) * src_b;
+    const uint8_t *w = (const uint8_t *)weight + (size_t)(Batch_B == 1 ? 0 : b % Batch_B) * wei_b;
+    uint8_t *c = (uint8_t *)dst + (size_t)b * dst_b;
+    int32_t st = matmul_single(layout, transA, transB, M, N, K, alpha, a, lda, w, ldb, bias, beta, c, ldc, is_weights_const, bp);
+    if (st != ZMI_SUCCESS) return st;
+  }
+  return ZMI_SUCCESS;
 }
 
 // ---- prepack ---------------------------------------------------------------------------------

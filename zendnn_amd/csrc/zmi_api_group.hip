@@ -35,12 +35,12 @@ bool all_null(void *const *v, int n, size_t num_ops) {
 int32_t validate_group(const zmi_group_args_t &a, const zmi_moe_postop_t *postop, int gated_act,
                        const zmi_fused_moe_t *fm, size_t *num_ops_out, bool *op1_internal_out,
                        bool *op2_internal_out) {
-  if (a.n_M <= 0 || a.n_params <= 0 || a.n_src <= 0) { set_error("group_matmul_direct: required input vector is empty"); return ZMI_FAILURE; }
+  if (a.n_M <= 0 || a.n_params <= 0 || a.n_src <= 0) { set_error("group call: M, params and src must each hold at least one entry"); return ZMI_FAILURE; }
   const bool opt_in = a.params[0].active_matmul > 0;
   if (opt_in) {
     const uint32_t am = a.params[0].active_matmul, tm = a.params[0].total_matmul;
-    if (am > (uint32_t)a.n_M) { set_error("active_matmul exceeds M.size()"); return ZMI_FAILURE; }
-    if (tm > 0 && tm < am) { set_error("total_matmul must be >= active_matmul"); return ZMI_FAILURE; }
+    if (am > (uint32_t)a.n_M) { set_error("group call: params[0].active_matmul counts more experts than M has entries"); return ZMI_FAILURE; }
+    if (tm > 0 && tm < am) { set_error("group call: params[0].total_matmul is smaller than active_matmul"); return ZMI_FAILURE; }
   }
   const size_t num_ops = opt_in ? (size_t)a.params[0].active_matmul : (size_t)a.n_M;
   *num_ops_out = num_ops;
@@ -53,12 +53,12 @@ int32_t validate_group(const zmi_group_args_t &a, const zmi_moe_postop_t *postop
     if (a.n_dst == 0 || all_null(a.dst, a.n_dst, num_ops)) op1_internal = true;
     else {
       for (size_t i = 0; i < std::min((size_t)a.n_dst, num_ops); ++i)
-        if (!a.dst[i] && i < (size_t)a.n_M && a.M[i] > 0) { set_error("fused_moe dst has a mixed null / non-null state"); return ZMI_FAILURE; }
+        if (!a.dst[i] && i < (size_t)a.n_M && a.M[i] > 0) { set_error("fused_moe: dst entries of active experts must be all null (library scratch) or all set"); return ZMI_FAILURE; }
     }
     if (fm->n_dst_down == 0 || all_null(fm->dst_down, fm->n_dst_down, num_ops)) op2_internal = true;
     else {
       for (size_t i = 0; i < std::min((size_t)fm->n_dst_down, num_ops); ++i)
-        if (!fm->dst_down[i] && i < (size_t)a.n_M && a.M[i] > 0) { set_error("fused_moe dst_down has a mixed null / non-null state"); return ZMI_FAILURE; }
+        if (!fm->dst_down[i] && i < (size_t)a.n_M && a.M[i] > 0) { set_error("fused_moe: dst_down entries of active experts must be all null (library scratch) or all set"); return ZMI_FAILURE; }
     }
   }
   *op1_internal_out = op1_internal;
@@ -68,57 +68,57 @@ int32_t validate_group(const zmi_group_args_t &a, const zmi_moe_postop_t *postop
       sc.bad(a.n_layout) || sc.bad(a.n_transA) || sc.bad(a.n_transB) || sc.bad(a.n_alpha) || sc.bad(a.n_beta) ||
       sc.bad(a.n_bias) || sc.bad(a.n_is_weights_const) || sc.bad(a.n_params) ||
       (!op1_internal && (sc.bad(a.n_dst) || sc.bad(a.n_ldc)))) {
-    set_error("group_matmul_direct: vector size mismatch");
+    set_error("group call: a per-expert array is shorter than the number of experts");
     return ZMI_FAILURE;
   }
   if (opt_in && a.params[0].total_matmul > a.params[0].active_matmul) {
     const size_t tm = a.params[0].total_matmul;
     if ((size_t)a.n_weight < tm || (size_t)a.n_K < tm || (size_t)a.n_N < tm || (size_t)a.n_ldb < tm ||
         (size_t)a.n_transB < tm || (size_t)a.n_is_weights_const < tm) {
-      set_error("weight-side vectors must be sized to total_matmul");
+      set_error("group call: weight-side arrays must cover all total_matmul experts");
       return ZMI_FAILURE;
     }
   }
   if (op1_internal) {
-    if (a.n_dst != 0 && sc.bad(a.n_dst)) { set_error("dst must be empty or sized to num_ops"); return ZMI_FAILURE; }
-    if (a.n_ldc != 0 && sc.bad(a.n_ldc)) { set_error("ldc must be empty or sized to num_ops"); return ZMI_FAILURE; }
+    if (a.n_dst != 0 && sc.bad(a.n_dst)) { set_error("fused_moe with library-held Op1 output: dst has entries but not one per expert"); return ZMI_FAILURE; }
+    if (a.n_ldc != 0 && sc.bad(a.n_ldc)) { set_error("fused_moe with library-held Op1 output: ldc has entries but not one per expert"); return ZMI_FAILURE; }
   }
-  if (op2_internal && fm->n_ldc_down != 0 && sc.bad(fm->n_ldc_down)) { set_error("ldc_down must be empty or sized to num_ops"); return ZMI_FAILURE; }
-  if (a.n_src != 1 && sc.bad(a.n_src)) { set_error("src.size() must be 1 or num_ops"); return ZMI_FAILURE; }
+  if (op2_internal && fm->n_ldc_down != 0 && sc.bad(fm->n_ldc_down)) { set_error("fused_moe with library-held Op2 output: ldc_down has entries but not one per expert"); return ZMI_FAILURE; }
+  if (a.n_src != 1 && sc.bad(a.n_src)) { set_error("group call: src holds neither one entry (chain) nor one per expert"); return ZMI_FAILURE; }
   const bool run_act = gated_act != ZMI_ACT_NONE;
   if (a.n_src == 1) {
-    if (postop) { set_error("moe_postop is only supported in parallel mode"); return ZMI_FAILURE; }
-    if (run_act) { set_error("gated_act is only supported in parallel mode"); return ZMI_FAILURE; }
-    if (fm) { set_error("fused_moe is only supported in parallel mode"); return ZMI_FAILURE; }
+    if (postop) { set_error("moe_postop needs one src per expert (not the one-src chain form)"); return ZMI_FAILURE; }
+    if (run_act) { set_error("gated_act needs one src per expert (not the one-src chain form)"); return ZMI_FAILURE; }
+    if (fm) { set_error("fused_moe needs one src per expert (not the one-src chain form)"); return ZMI_FAILURE; }
   }
-  if (fm && fm->n_down_weight == 0) { set_error("fused_moe is non-null but down_weight is empty"); return ZMI_FAILURE; }
+  if (fm && fm->n_down_weight == 0) { set_error("fused_moe given without down_weight entries (pass no fused_moe to switch it off)"); return ZMI_FAILURE; }
   if (a.n_src == 1) {
     // sequential chain
-    if (!a.src[0]) { set_error("group_matmul sequential: null src"); return ZMI_FAILURE; }
+    if (!a.src[0]) { set_error("chain form: src[0] is null"); return ZMI_FAILURE; }
     for (size_t i = 0; i < num_ops; ++i) {
-      if (!a.weight[i] || !a.dst[i]) { set_error("group_matmul sequential: null pointer"); return ZMI_FAILURE; }
-      if (a.M[i] <= 0 || a.N[i] <= 0 || a.K[i] <= 0) { set_error("group_matmul sequential: invalid dimensions"); return ZMI_FAILURE; }
+      if (!a.weight[i] || !a.dst[i]) { set_error("chain form: a layer has a null weight or dst"); return ZMI_FAILURE; }
+      if (a.M[i] <= 0 || a.N[i] <= 0 || a.K[i] <= 0) { set_error("chain form: M, N, K of every layer must be positive"); return ZMI_FAILURE; }
     }
     for (size_t i = 1; i < num_ops; ++i) {
-      if (a.M[i] != a.M[0]) { set_error("group_matmul sequential: M must be constant across layers"); return ZMI_FAILURE; }
-      if (a.K[i] != a.N[i - 1]) { set_error("group_matmul sequential: K[i] != N[i-1]"); return ZMI_FAILURE; }
+      if (a.M[i] != a.M[0]) { set_error("chain form: every layer must have the first layer's M"); return ZMI_FAILURE; }
+      if (a.K[i] != a.N[i - 1]) { set_error("chain form: a layer's K must equal the previous layer's N"); return ZMI_FAILURE; }
     }
     return ZMI_SUCCESS;
   }
   for (size_t i = 0; i < num_ops; ++i) {
-    if (a.M[i] < 0 || a.N[i] <= 0 || a.K[i] <= 0) { set_error("group_matmul parallel: invalid dimensions"); return ZMI_FAILURE; }
+    if (a.M[i] < 0 || a.N[i] <= 0 || a.K[i] <= 0) { set_error("group call: N and K must be positive and M non-negative for every expert"); return ZMI_FAILURE; }
     if (a.M[i] > 0) {
-      if (!a.src[i] || !a.weight[i]) { set_error("group_matmul parallel: null src / weight at an active expert"); return ZMI_FAILURE; }
-      if (!op1_internal && !a.dst[i]) { set_error("group_matmul parallel: null dst at an active expert"); return ZMI_FAILURE; }
+      if (!a.src[i] || !a.weight[i]) { set_error("group call: an expert with rows has a null src or weight"); return ZMI_FAILURE; }
+      if (!op1_internal && !a.dst[i]) { set_error("group call: an expert with rows has a null dst"); return ZMI_FAILURE; }
     }
   }
   if (run_act) {
     const int dt = a.params[0].dt_dst;
-    if (dt != ZMI_DT_F32 && dt != ZMI_DT_BF16 && dt != ZMI_DT_F16) { set_error("gated_act requires f32, bf16 or f16 dst"); return ZMI_FAILURE; }
+    if (dt != ZMI_DT_F32 && dt != ZMI_DT_BF16 && dt != ZMI_DT_F16) { set_error("gated_act: dt_dst must be f32, bf16 or f16"); return ZMI_FAILURE; }
     for (size_t i = 1; i < num_ops; ++i)
-      if (a.params[i].dt_dst != dt) { set_error("gated_act requires uniform dst dtype"); return ZMI_FAILURE; }
+      if (a.params[i].dt_dst != dt) { set_error("gated_act: all experts must share one dt_dst"); return ZMI_FAILURE; }
     for (size_t i = 0; i < num_ops; ++i)
-      if (a.N[i] % 2 != 0) { set_error("gated_act requires even N"); return ZMI_FAILURE; }
+      if (a.N[i] % 2 != 0) { set_error("gated_act: N holds gate and up halves and must be even"); return ZMI_FAILURE; }
     if (!op1_internal && !fm) {
       bool tight = false, wide = false;
       for (size_t i = 0; i < num_ops; ++i) {
@@ -130,42 +130,42 @@ int32_t validate_group(const zmi_group_args_t &a, const zmi_moe_postop_t *postop
   }
   if (run_act || fm) {
     for (size_t i = 0; i < num_ops; ++i)
-      if (a.layout[i] != 'r' && a.layout[i] != 'R') { set_error("gated_act / fused_moe require row-major layout"); return ZMI_FAILURE; }
+      if (a.layout[i] != 'r' && a.layout[i] != 'R') { set_error("gated_act / fused_moe: layout must be 'r' for every expert"); return ZMI_FAILURE; }
   }
   if (fm) {
     if (sc.bad(fm->n_down_weight) || sc.bad(fm->n_N_down) || sc.bad(fm->n_ldb_down) || sc.bad(fm->n_bias_down) ||
         (!op2_internal && (sc.bad(fm->n_dst_down) || sc.bad(fm->n_ldc_down)))) {
-      set_error("fused_moe vector size mismatch");
+      set_error("fused_moe: a per-expert array is shorter than the number of experts");
       return ZMI_FAILURE;
     }
-    if (fm->n_down_scale != 0 && (size_t)fm->n_down_scale < num_ops) { set_error("fused_moe down_scale is shorter than num_ops"); return ZMI_FAILURE; }
-    if (fm->n_down_zp != 0 && (size_t)fm->n_down_zp < num_ops) { set_error("fused_moe down_zp is shorter than num_ops"); return ZMI_FAILURE; }
+    if (fm->n_down_scale != 0 && (size_t)fm->n_down_scale < num_ops) { set_error("fused_moe: down_scale has entries but fewer than one per expert"); return ZMI_FAILURE; }
+    if (fm->n_down_zp != 0 && (size_t)fm->n_down_zp < num_ops) { set_error("fused_moe: down_zp has entries but fewer than one per expert"); return ZMI_FAILURE; }
     for (size_t i = 0; i < num_ops; ++i) {
-      if (a.N[i] % 2 != 0) { set_error("fused_moe requires even N"); return ZMI_FAILURE; }
+      if (a.N[i] % 2 != 0) { set_error("fused_moe: N holds gate and up halves and must be even"); return ZMI_FAILURE; }
       if (a.M[i] > 0) {
-        if (!fm->down_weight[i]) { set_error("fused_moe down_weight is null at an active expert"); return ZMI_FAILURE; }
-        if (!op2_internal && !fm->dst_down[i]) { set_error("fused_moe dst_down is null at an active expert"); return ZMI_FAILURE; }
+        if (!fm->down_weight[i]) { set_error("fused_moe: an expert with rows has a null down_weight"); return ZMI_FAILURE; }
+        if (!op2_internal && !fm->dst_down[i]) { set_error("fused_moe: an expert with rows has a null dst_down"); return ZMI_FAILURE; }
       }
-      if (fm->N_down[i] <= 0) { set_error("fused_moe N_down must be positive"); return ZMI_FAILURE; }
+      if (fm->N_down[i] <= 0) { set_error("fused_moe: N_down <= 0"); return ZMI_FAILURE; }
       const int kd = op2_k_for_act(a.N[i], gated_act);
       const int min_ldb = a.transB[i] ? kd : fm->N_down[i];
-      if (fm->ldb_down[i] < min_ldb) { set_error("fused_moe ldb_down too small"); return ZMI_FAILURE; }
+      if (fm->ldb_down[i] < min_ldb) { set_error("fused_moe: ldb_down is smaller than a row of down_weight"); return ZMI_FAILURE; }
       if (!op2_internal) {
-        if (fm->ldc_down[i] < fm->N_down[i]) { set_error("fused_moe ldc_down < N_down"); return ZMI_FAILURE; }
+        if (fm->ldc_down[i] < fm->N_down[i]) { set_error("fused_moe: ldc_down is smaller than N_down"); return ZMI_FAILURE; }
       } else {
-        if (a.M[i] > 0 && a.lda[i] < fm->N_down[i]) { set_error("fused_moe internal-alloc requires lda >= N_down"); return ZMI_FAILURE; }
-        if (a.M[i] > 0 && a.params[i].dt_src != a.params[i].dt_dst) { set_error("fused_moe internal-alloc requires matching src / dst dtypes"); return ZMI_FAILURE; }
+        if (a.M[i] > 0 && a.lda[i] < fm->N_down[i]) { set_error("fused_moe with library-held Op2 output: the result goes back into src, whose lda must hold N_down"); return ZMI_FAILURE; }
+        if (a.M[i] > 0 && a.params[i].dt_src != a.params[i].dt_dst) { set_error("fused_moe with library-held Op2 output: the result goes back into src, so dt_src must equal dt_dst"); return ZMI_FAILURE; }
       }
-      if (fm->bias_down[i] && fm->bias_dt_down == ZMI_DT_NONE) { set_error("fused_moe bias_down is set but bias_dt_down is none"); return ZMI_FAILURE; }
+      if (fm->bias_down[i] && fm->bias_dt_down == ZMI_DT_NONE) { set_error("fused_moe: bias_down given without bias_dt_down"); return ZMI_FAILURE; }
     }
     if (postop)
       for (size_t i = 1; i < num_ops; ++i)
-        if (fm->N_down[i] != fm->N_down[0]) { set_error("fused_moe + moe_postop requires uniform N_down"); return ZMI_FAILURE; }
+        if (fm->N_down[i] != fm->N_down[0]) { set_error("fused_moe with moe_postop: all experts must share one N_down"); return ZMI_FAILURE; }
   }
   if (postop) {
     for (size_t i = 1; i < num_ops; ++i) {
-      if (a.N[i] != a.N[0]) { set_error("moe_postop requires identical N across experts"); return ZMI_FAILURE; }
-      if (a.params[i].dt_dst != a.params[0].dt_dst) { set_error("moe_postop requires identical dst dtype"); return ZMI_FAILURE; }
+      if (a.N[i] != a.N[0]) { set_error("moe_postop: all experts must share one N"); return ZMI_FAILURE; }
+      if (a.params[i].dt_dst != a.params[0].dt_dst) { set_error("moe_postop: all experts must share one dt_dst"); return ZMI_FAILURE; }
     }
     // validate_group_matmul_moe_postop (group_matmul/group_matmul_moe_postop.cpp)
     const int D = fm ? fm->N_down[0] : a.N[0];
@@ -210,6 +210,8 @@ bool params_uniform(const zmi_group_args_t &a, size_t num_ops) {
       if (x.po_type == ZMI_PO_BINARY_ADD || x.po_type == ZMI_PO_BINARY_MUL) return false;
     }
     if ((p.src_zp.buff != nullptr) != (p0.src_zp.buff != nullptr)) return false;
+    // (the shared epilogue reads every expert's scales in one dtype)
+    if (p.wei_scale.dt != p0.wei_scale.dt || p.src_scale.dt != p0.src_scale.dt) return false;
     if (p.dst_scale.buff || p.dst_zp.buff || p.wei_zp.buff) return false;
     if ((p.wei_scale.buff != nullptr) != (p0.wei_scale.buff != nullptr)) return false;
     if (p.wei_scale.buff && ((nelems(p.wei_scale) == 1) != (nelems(p0.wei_scale) == 1))) return false;
@@ -577,7 +579,9 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       r0 = renumber_rows8(mats, p0.dt_dst, r0, &rows8);
       const ZmiQuantMat *dev = (const ZmiQuantMat *)upload(mats.data(), mats.size() * sizeof(ZmiQuantMat));
       if (!dev) return ZMI_FAILURE;
-      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_dst, ZMI_DT_F32, rows8, stream()), "grouped quant launch (Op2)")) return ZMI_FAILURE;
+      // the down projection's source scales take Op1's scale dtype (group_matmul_fused_moe.cpp:816-820): with bf16
+      // the scale is narrowed and the GEMM multiplies by the narrowed value
+      if (!hip_ok(zmi_launch_quant_group(dev, (int)mats.size(), r0, p0.dt_dst, s1_dt, rows8, stream()), "grouped quant launch (Op2)")) return ZMI_FAILURE;
 
       Stage op2;
       bool have2 = false;
@@ -597,7 +601,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
         zmi_matmul_params_t ep;
         zmi_matmul_params_init(&ep);
         ep.dt_src = ZMI_DT_S8; ep.dt_wei = ZMI_DT_S8; ep.dt_dst = p0.dt_dst; ep.dt_bias = fm.bias_dt_down;
-        ep.src_scale.buff = s2[i]; ep.src_scale.dt = ZMI_DT_F32; ep.src_scale.ndims = 2;
+        ep.src_scale.buff = s2[i]; ep.src_scale.dt = s1_dt; ep.src_scale.ndims = 2;
         ep.src_scale.dims[0] = a.M[i]; ep.src_scale.dims[1] = 1;
         if (fm.n_down_scale) ep.wei_scale = fm.down_scale[i];
         if (fm.n_down_zp && fm.down_zp[i].buff) { set_error("down_zp is not implemented (symmetric weights only)"); return ZMI_UNIMPLEMENTED; }
@@ -644,6 +648,19 @@ int32_t zmi_moe_route(const int32_t *topk_ids, int32_t T, int32_t topk, int32_t 
   int32_t *hist = hist_ints ? (int32_t *)arena().alloc(hist_ints * sizeof(int32_t)) : nullptr;
   if (!hip_ok(zmi_launch_moe_route(topk_ids, T, topk, E, 1, counts, offsets, slot_of, nullptr, 0, hist, stream()), "moe route launch")) return ZMI_FAILURE;
   set_kernel_name("moe_route");
+  return ZMI_SUCCESS;
+}
+
+int32_t zmi_moe_router_topk(const void *logits, int32_t logits_dt, int64_t ldl, int32_t T, int32_t E, int32_t topk,
+                            int32_t renormalize, int32_t *topk_ids, float *topk_weights) {
+  clear_error();
+  if (!logits || !topk_ids || !topk_weights || T <= 0 || E <= 0 || topk <= 0 || ldl < E) { set_error("moe_router_topk: bad arguments"); return ZMI_FAILURE; }
+  if (topk > E) { set_error("moe_router_topk: topk exceeds the number of experts"); return ZMI_FAILURE; }
+  if (logits_dt != ZMI_DT_F32 && logits_dt != ZMI_DT_BF16) { set_error("moe_router_topk: logits must be f32 or bf16"); return ZMI_FAILURE; }
+  if (E > 512 || topk > 64) { set_error("moe_router_topk: at most 512 experts and topk <= 64"); return ZMI_UNIMPLEMENTED; }
+  if (!ensure_device()) return ZMI_FAILURE;
+  if (!hip_ok(zmi_launch_moe_router_topk(logits, logits_dt, ldl, T, E, topk, renormalize, topk_ids, topk_weights, stream()), "moe router launch")) return ZMI_FAILURE;
+  set_kernel_name("moe_router_topk");
   return ZMI_SUCCESS;
 }
 

@@ -111,14 +111,20 @@ def last_kernel():
 
 
 def matmul_direct(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc,
-                  is_weights_const, params, batch_a=1, batch_b=1, noalloc=False):
-    """noalloc=True: the entry point that allocates no device memory (zmi_matmul_direct_noalloc)."""
+                  is_weights_const, params, batch_a=1, batch_b=1, noalloc=False, batch_strides=None):
+    """noalloc=True: the entry point that allocates no device memory (zmi_matmul_direct_noalloc).
+    batch_strides: (src, wei, dst) strides in elements, None entries (or no tuple) derive them from the
+    dimensions like matmul_batch_params_t's default of (size_t)-1."""
     lib = capi.load()
     keep = []
     p = params.flat(keep)
     b = capi.BatchParamsT()
     lib.zmi_batch_params_init(C.byref(b))
     b.Batch_A, b.Batch_B = batch_a, batch_b
+    if batch_strides is not None:
+        for name, v in zip(("batch_stride_src", "batch_stride_wei", "batch_stride_dst"), batch_strides):
+            if v is not None:
+                setattr(b, name, int(v))
     fn = lib.zmi_matmul_direct_noalloc if noalloc else lib.zmi_matmul_direct
     return fn(layout.encode(), int(transA), int(transB), M, N, K, alpha, _ptr(src), lda,
                                  _ptr(weight), ldb, _ptr(bias), beta, _ptr(dst), ldc, int(is_weights_const),
@@ -332,6 +338,18 @@ def moe_route(topk_ids, E):
     st = capi.load().zmi_moe_route(topk_ids.data_ptr(), T, topk, E, counts.data_ptr(), offsets.data_ptr(),
                                    slot_of.data_ptr())
     return st, counts, offsets, slot_of
+
+
+def moe_router_topk(logits, topk, renormalize=False):
+    """logits: f32 / bf16 tensor [T, E] on the GPU -> (status, topk_ids int32 [T, topk], topk_weights f32 [T, topk])."""
+    import torch
+    T, E = logits.shape
+    ids = torch.empty(T, topk, dtype=torch.int32, device=logits.device)
+    w = torch.empty(T, topk, dtype=torch.float32, device=logits.device)
+    dt = {torch.float32: capi.DT_F32, torch.bfloat16: capi.DT_BF16}[logits.dtype]
+    st = capi.load().zmi_moe_router_topk(logits.data_ptr(), dt, logits.stride(0), T, E, topk, int(bool(renormalize)),
+                                         ids.data_ptr(), w.data_ptr())
+    return st, ids, w
 
 
 def moe_fused_device(x, topk_ids, topk_weights, w13_blobs, w2_blobs, w13_scales, w2_scales, I, gated_act, out):
