@@ -283,7 +283,7 @@ def test_grouped_call_with_per_group_ggml_and_s4_experts(zo):
     """group_matmul_direct with experts the grouped kernels do not take -- per-group scales on static s8 rows, per-group
     dynamic quantization, GGML Q8_0 packed weights, W4A8 -- runs them on the matmul_direct path (reference:
     group_matmul/group_matmul_dispatch.cpp:472-515, group_matmul_direct.cpp:1222-1260); followed here by the
-    weighted reduce over the f32 expert outputs.  A fused MoE or gated activation on top is refused."""
+    weighted reduce over the f32 expert outputs, and by a gated activation over them."""
     rng = np.random.default_rng(77)
     K, N, T = 256, 48, 6
     G = K // 32
@@ -349,9 +349,12 @@ def test_grouped_call_with_per_group_ggml_and_s4_experts(zo):
     red = zo.moe_reduce([want[e][t] for t in range(T) for e in ids[t]], tw_h, capi.DT_F32, N)
     assert np.array_equal(H.to_host(out), red)
 
-    # refused on top of a gated activation
+    # a gated activation on top: the stand-alone activation pass over the experts' (wide, f32) outputs
     st = lowoha.group_matmul_direct(*args, gated_act=capi.ACT_SILU_AND_MUL)
-    assert st == capi.UNIMPLEMENTED
+    assert st == capi.SUCCESS, lowoha.last_error()
+    for e in range(E):
+        act = zo.gated_act(capi.ACT_SILU_AND_MUL, want[e].copy(), capi.DT_F32)
+        H.check_f32(H.to_host(dst[e])[:, :N // 2], act[:, :N // 2], rtol=2e-6, atol=1e-7)
 
     # two W4A8 experts (bf16 rows, packed s4 weights, bf16 out), ragged row counts
     Ms = [5, 9]

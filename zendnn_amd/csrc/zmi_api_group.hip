@@ -326,9 +326,20 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       one_by_one = true;
   }
   if (one_by_one) {
-    if (fused_moe || run_act) {
-      set_error("per-group scales, GGML-packed and s4 weights are implemented for plain grouped calls only (no fused_moe / gated_act)");
+    // A gated activation and the fused block on such experts are the two-pass composition of the reference
+    // (run_fused_moe_legacy_two_pass, group_matmul/group_matmul_fused_moe.cpp:906-1078; per-group scales never take
+    // its vertically fused form, same file :705-711): Op1 per expert into the caller's wide dst, the activation
+    // over all experts in place, Op2 per expert with the parameters setup_op2_dispatch_scratch derives (:761-880).
+    if ((fused_moe || run_act) && (op1_internal || op2_internal)) {
+      set_error("per-group / GGML-packed / s4 experts: fused_moe needs the caller's dst and dst_down (library-held intermediates are not implemented)");
       return ZMI_UNIMPLEMENTED;
+    }
+    if (run_act) {
+      for (size_t i = 0; i < num_ops; ++i)
+        if (a.M[i] > 0 && a.ldc[i] < a.N[i]) {
+          set_error("per-group / GGML-packed / s4 experts: gated_act needs a dst that holds all N columns (ldc >= N)");
+          return ZMI_UNIMPLEMENTED;
+        }
     }
     for (size_t i = 0; i < num_ops; ++i) {
       if (a.M[i] <= 0) continue;
@@ -338,6 +349,72 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
                              a.weight[i], a.ldb[i], a.bias[i], a.beta[i], a.dst[i], a.ldc[i], a.is_weights_const[i], &bp,
                              &a.params[i]);
       if (st != ZMI_SUCCESS) return st;
+    }
+    if (run_act) {
+      // reference: group_matmul_moe_act_execute, group_matmul/group_matmul_moe_act.cpp
+      if (!ensure_device()) return ZMI_FAILURE;
+      std::vector<ZmiActMat> mats;
+      int64_t r0 = 0;
+      int maxN = 0;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        ZmiActMat m;
+        m.buf = a.dst[i]; m.ld = a.ldc[i]; m.M = a.M[i]; m.N = a.N[i]; m.row_start = (int32_t)r0;
+        r0 += a.M[i];
+        maxN = std::max(maxN, a.N[i]);
+        mats.push_back(m);
+      }
+      if (!mats.empty()) {
+        const ZmiActMat *dev = (const ZmiActMat *)upload(mats.data(), mats.size() * sizeof(ZmiActMat));
+        if (!dev) return ZMI_FAILURE;
+        if (!hip_ok(zmi_launch_gated_act(dev, nullptr, (int)mats.size(), r0, maxN, gated_act, a.params[0].dt_dst, stream()), "gated act launch")) return ZMI_FAILURE;
+        upload_fence();
+      }
+    }
+    if (fused_moe) {
+      const zmi_fused_moe_t &fm = *fused_moe;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 0) continue;
+        const zmi_matmul_params_t &p1 = a.params[i];
+        const int kd = op2_k_for_act(a.N[i], gated_act);
+        zmi_matmul_params_t p2;
+        zmi_matmul_params_init(&p2);
+        p2.dt_src = p1.dt_dst; p2.dt_wei = p1.dt_wei; p2.dt_dst = p1.dt_dst; p2.dt_bias = fm.bias_dt_down;
+        p2.dynamic_quant = p1.dynamic_quant; p2.dt_compute = p1.dt_compute;
+        p2.weight_cache_type = p1.weight_cache_type;
+        const bool ggml = p1.pack_format_b == 1;
+        if (ggml) p2.pack_format_b = 1;   // (both projections of a GGML expert are packed; the scales are inside the blocks)
+        else if (fm.n_down_scale) p2.wei_scale = fm.down_scale[i];
+        if (fm.n_down_zp) p2.wei_zp = fm.down_zp[i];
+        if (p2.dynamic_quant) {
+          const bool op1_per_group = p1.src_scale.ndims == 2 && p1.src_scale.dims[1] > 1;
+          p2.src_scale.buff = nullptr;
+          p2.src_scale.dt = p1.src_scale.dt;
+          p2.src_scale.ndims = p1.src_scale.ndims;
+          for (int d = 0; d < p1.src_scale.ndims; ++d) p2.src_scale.dims[d] = p1.src_scale.dims[d];
+          if (op1_per_group) {
+            // Op1's group count does not carry over (K differs): Op2's comes from the down projection's weight scale
+            int64_t g2 = 1;
+            if (ggml) g2 = kd / 32;
+            else if (fm.n_down_scale) {
+              const zmi_quant_t &ds = fm.down_scale[i];
+              if (ds.ndims == 2 && ds.dims[0] > 1) g2 = ds.dims[0];
+              else if (ds.ndims == 3 && ds.dims[1] > 1) g2 = ds.dims[1];
+            }
+            p2.src_scale.ndims = 2; p2.src_scale.dims[0] = p1.src_scale.dims[0]; p2.src_scale.dims[1] = g2;
+          }
+          if (p1.src_zp.dt != ZMI_DT_NONE && p1.src_zp.ndims == 2 && p1.src_zp.dims[1] > 1) {
+            set_error("fused_moe: per-group source zero-points are not supported on the down projection");
+            return ZMI_FAILURE;
+          }
+        }
+        zmi_batch_params_t bp;
+        zmi_batch_params_init(&bp);
+        st = zmi_matmul_direct(a.layout[i], 0, a.transB[i], a.M[i], fm.N_down[i], kd, 1.0f, a.dst[i], a.ldc[i],
+                               fm.down_weight[i], fm.ldb_down[i], fm.bias_down[i], 0.0f, fm.dst_down[i], fm.ldc_down[i],
+                               a.is_weights_const[i], &bp, &p2);
+        if (st != ZMI_SUCCESS) return st;
+      }
     }
     if (moe_postop) goto postop_only;
     return ZMI_SUCCESS;
