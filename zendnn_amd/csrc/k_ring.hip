@@ -661,6 +661,11 @@ __global__ __launch_bounds__(64) void zmi_ring_count_kernel(const ZmiProblem *pr
   zmi_ring_fill_table(probs, n_prob, top, gated, tab, threadIdx.x);
 }
 
+hipError_t zmi_launch_ring_table(const ZmiProblem *probs_dev, int n_prob, int top, bool gated, int *tab_dev, hipStream_t stream) {
+  hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0, tab_dev);
+  return hipGetLastError();
+}
+
 static int ring_cu_count() {
   static const int n_cu = [] {
     int dev = 0, n = 256;
@@ -694,7 +699,8 @@ static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int
   // at most one workgroup per CU anyway: let it have the whole LDS for its ring
   const int n_cu = ring_cu_count();
   (void)exact;   // a bound that fits one workgroup per CU is as good as the exact count
-  if (BM != 256 && n_items <= n_cu)
+  static const bool force_deep = getenv("ZMI_RING_DEEP") != nullptr;   // EXPERIMENT
+  if (BM != 256 && (n_items <= n_cu || force_deep))
     return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
   return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
 }

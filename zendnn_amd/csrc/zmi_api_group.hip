@@ -238,11 +238,26 @@ int64_t renumber_rows8(std::vector<ZmiQuantMat> &mats, int32_t src_dt, int64_t t
 struct Stage {
   std::vector<ZmiProblem> probs;
   ZmiEpilogue epi;
+  mutable bool streamed = false;   // set by launch_stage: the weight-traffic-bound kernel took the large experts
 };
 
 int group_top(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated) {
   if (const char *env = std::getenv("ZMI_GROUP_TOP")) { int v = std::atoi(env); if (v > 0) return v; }
   return zmi_ring_pick_top_group(rows, n_prob, K, N, gated);
+}
+
+// Tile height (with ZMI_RING_PAD) when the weight-traffic-bound kernel should take a grouped launch whose largest
+// expert has max_rows rows (for a launch whose row counts live on the device: a class derived from the average),
+// 0 when the MFMA-bound kernel keeps it.  Up to 256 rows an expert is one row block: its weights pass once, and
+// the MFMA work of 256 rows takes about as long as its weights need to arrive.  A launch with fewer tiles than two
+// per compute unit stays with the MFMA-bound kernel, whose deep-ring build does better on a half-empty chip
+// (8 experts x 14336 -> 4096: 136 against 157 us).
+int group_stream_top(int max_rows, const ZmiEpilogue &epi, int N, int64_t tiles) {
+  int top = 0;
+  if (max_rows > 16 && max_rows <= 256 && tiles >= 512) top = (max_rows <= 128 ? 128 : 256) | ZMI_RING_PAD;
+  if (const char *env = std::getenv("ZMI_GROUP_STREAM_TOP")) top = std::atoi(env);   // (0 switches the kernel off)
+  if (!top || !zmi_group_stream_takes(epi, N, top)) return 0;
+  return top;
 }
 
 // Every expert's activations are fragment-major.  Experts with more than 16 rows: one launch of the MFMA-bound
@@ -255,10 +270,10 @@ int32_t launch_stage(const Stage &st, const char *what) {
   const int n = (int)st.probs.size();
   const bool gated = st.epi.gated_act != 0;
   int64_t rows = 0;
-  int cols = 0, kmax = 0, small = 0, large = 0;
+  int cols = 0, kmax = 0, small = 0, large = 0, max_rows = 0;
   bool small_ok = true;
   for (const ZmiProblem &q : st.probs) {
-    rows += q.M; cols = std::max(cols, (int)q.N); kmax = std::max(kmax, (int)q.K);
+    rows += q.M; cols = std::max(cols, (int)q.N); kmax = std::max(kmax, (int)q.K); max_rows = std::max(max_rows, (int)q.M);
     if (q.M > 0 && q.M <= 16) { ++small; small_ok = small_ok && zmi_group_decode_takes(st.epi, q.N); }
     else if (q.M > 16) ++large;
   }
@@ -269,11 +284,23 @@ int32_t launch_stage(const Stage &st, const char *what) {
   const bool force_split = getenv("ZMI_GROUP_DECODE") != nullptr;
   const bool split = small > 0 && small_ok && (small >= large || force_split);
   int top = group_top(rows, n, kmax, cols, gated);
+  // experts of at most 256 rows are a stream of their weights: the kernel built for that takes the launch
+  int64_t tiles128 = 0;
+  for (const ZmiProblem &q : st.probs)
+    if (q.M > 16) tiles128 += zmi_ring_items<128>(q.M, q.N, 128 | ZMI_RING_PAD, gated);
+  const int stream_top = group_stream_top(max_rows, st.epi, cols, max_rows <= 128 ? tiles128 : 2 * tiles128);
+  if (stream_top) top = stream_top;
   if (split) top |= ZMI_RING_SKIP_SMALL;
   if (large > 0 || !split) {
     int *tab = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)n));
     if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
-    if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) return ZMI_FAILURE;
+    st.streamed = stream_top != 0;
+    if (stream_top) {
+      if (!hip_ok(zmi_launch_ring_table(dev, n, top, gated, tab, stream()), what)) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_gemm_stream_group(st.probs.data(), dev, n, top, 0, 0, tab, st.epi, stream()), what)) return ZMI_FAILURE;
+    } else if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) {
+      return ZMI_FAILURE;
+    }
   }
   if (split && !hip_ok(zmi_launch_gemm_group_decode(dev, n, gated ? cols / 2 : cols, st.epi, stream()), what)) return ZMI_FAILURE;
   return ZMI_SUCCESS;
@@ -609,7 +636,8 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     op1.epi.gated_act = fuse_act ? gated_act : ZMI_ACT_NONE;
     st = launch_stage(op1, "Op1 GEMM launch");
     if (st != ZMI_SUCCESS) return st;
-    set_kernel_name(fuse_act ? "group: ring_mfma32x32x32 (gated epilogue)" : "group: ring_mfma32x32x32");
+    set_kernel_name(op1.streamed ? (fuse_act ? "group: stream_mfma32x32x32 (gated epilogue)" : "group: stream_mfma32x32x32")
+                                 : (fuse_act ? "group: ring_mfma32x32x32 (gated epilogue)" : "group: ring_mfma32x32x32"));
 
     if (run_act && !fuse_act) {
       // reference: group_matmul_moe_act_execute, group_matmul/group_matmul_moe_act.cpp
@@ -821,6 +849,16 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   const bool small2 = decode_step && zmi_group_decode_takes(probe, H);
   probe.gated_act = d->gated_act;
   const bool small1 = decode_step && zmi_group_decode_takes(probe, 2 * I);
+  const int avg_rows = (int)((R + E - 1) / E);
+  ZmiEpilogue probe1 = probe;
+  probe.gated_act = 0;
+  // (an average of up to 96 rows: taken to be at most 128 everywhere; up to 224: at most 256)
+  const int row_class = avg_rows <= 96 ? 128 : (avg_rows <= 224 ? 256 : 0);
+  const int64_t blocks = R / 128 + E;
+  const int stream1 = group_stream_top(row_class, probe1, 2 * I, blocks * ((I + 127) / 128));
+  const int stream2 = group_stream_top(row_class, probe, H, blocks * ((H + 255) / 256));
+  if (stream1) top1 = stream1;
+  if (stream2) top2 = stream2;
   if (small1) top1 |= ZMI_RING_SKIP_SMALL;
   if (small2) top2 |= ZMI_RING_SKIP_SMALL;
   if (!hip_ok(zmi_launch_moe_build_problems(tb, E, H, I, counts, offsets, A1, s1, act, A2, s2, Y, op1, op2, top1, top2, tile_tab1, tile_tab2, s), "problem table launch")) return ZMI_FAILURE;
@@ -832,11 +870,19 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   e1.bias_dt = ZMI_DT_F32; e1.alpha = 1.0f; e1.beta = 0.0f; e1.dst_dt = ZMI_DT_BF16; e1.fast_kind = ZMI_EK_NONE;
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
-  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, true, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+  if (stream1) {
+    if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+  } else if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, true, e1, s), "Op1 GEMM launch")) {
+    return ZMI_FAILURE;
+  }
   if (small1 && !hip_ok(zmi_launch_gemm_group_decode(op1, E, I, e1, s), "Op1 decode-shaped GEMM launch")) return ZMI_FAILURE;
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
-  if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
+  if (stream2) {
+    if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op2, E, top2, R, H, tile_tab2, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
+  } else if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s), "Op2 GEMM launch")) {
+    return ZMI_FAILURE;
+  }
   if (small2 && !hip_ok(zmi_launch_gemm_group_decode(op2, E, H, e2, s), "Op2 decode-shaped GEMM launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;
   upload_fence();
