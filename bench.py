@@ -31,7 +31,7 @@ INT8_PEAK_TOPS = 5000.0
 K_DEC, N_DEC = 4096, 14336
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
 # size), measured with the commands recorded in profiles/zmi_gemm_decode_kernel_decode_M16_K4096_N14336.md
-DECODE_TRAFFIC_BYTES = 60274290
+DECODE_TRAFFIC_BYTES = 60293616
 
 
 def main():
@@ -205,7 +205,7 @@ def main():
             out["mfma_i8_" + name] = {"TOPS": round(tops.value, 1), "shader_MHz": round(mhz.value, 0),
                                       "pct_of_nominal": round(100 * tops.value / INT8_PEAK_TOPS, 1)}
         out["mfma_i8_what"] = ("a loop of nothing but v_mfma_i32_32x32x32_i8, 4 wavefronts per workgroup on every compute "
-                               "unit, ~0.2 ms per launch; 'varying': consecutive instructions get different random int8 operand "
+                               "unit, about 1 ms per timed launch; 'varying': consecutive instructions get different random int8 operand "
                                "fragments, as in a GEMM on random data (the multipliers' toggling sets the power, the clock follows)")
         return out
 
