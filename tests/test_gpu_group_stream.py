@@ -18,13 +18,16 @@ pytestmark = pytest.mark.gpu
 TOP128, TOP256 = str(128 | 0x10000), str(256 | 0x10000)
 
 
-def _with_kernel(monkeypatch, top):
+def _with_kernel(monkeypatch, top, slices=None):
     monkeypatch.delenv("ZMI_NO_GROUP_STREAM", raising=False)
     monkeypatch.delenv("ZMI_GROUP_STREAM_TOP", raising=False)
+    monkeypatch.delenv("ZMI_GROUP_STREAM_SLICES", raising=False)
     if top is None:
         monkeypatch.setenv("ZMI_NO_GROUP_STREAM", "1")
     else:
         monkeypatch.setenv("ZMI_GROUP_STREAM_TOP", top)
+        if slices:
+            monkeypatch.setenv("ZMI_GROUP_STREAM_SLICES", str(slices))
 
 
 def _grouped(Ms, K, N, dst_dt, post=None, bias=False, gated=None, rng=None, static_u8=False):
@@ -174,3 +177,45 @@ def test_the_kernel_takes_a_large_enough_launch_by_itself(monkeypatch):
         run, _ = _grouped([100] * 8, 512, 2 * I, capi.DT_BF16, rng=rng, gated=capi.ACT_SILU_AND_MUL)
         _, names[I] = run()
     assert "ring" in names[4096] and "stream" in names[8192]
+
+
+@pytest.mark.parametrize("top", [TOP128, TOP256])    # (the 256-row build ignores the request and runs unsliced)
+@pytest.mark.parametrize("slices", [2, 3, 4])
+@pytest.mark.parametrize("dst_dt,post", [(capi.DT_BF16, capi.PO_SWISH), (capi.DT_F32, None)])
+def test_k_slices_leave_every_bit_where_it_was(zo, monkeypatch, top, slices, dst_dt, post):
+    """Plain grouped launches cut into K slices (int32 partial tiles in a workspace, a second kernel adds them and
+    finishes the elements): bit-identical to the unsliced MFMA-bound kernel; K_pad / 64 = 12 stages, so 3 and 4 slices
+    divide evenly and unevenly, and the row counts leave row fragments and whole row blocks without rows."""
+    rng = np.random.default_rng(slices * 10 + (post or 0))
+    Ms, K, N = [100, 0, 129, 40, 300], 704, 600
+    run, _ = _grouped(Ms, K, N, dst_dt, post=post, bias=True, rng=rng)
+    _with_kernel(monkeypatch, None)
+    ref, _ = run()
+    _with_kernel(monkeypatch, top, slices)
+    got, name = run()
+    assert "stream" in name
+    for e, m in enumerate(Ms):
+        assert np.array_equal(got[e], ref[e]), f"expert {e} ({m} rows)"
+
+
+def test_fused_block_with_a_sliced_down_projection(zo, monkeypatch):
+    """The device-routed block whose down projection has few tiles and a long K takes K slices by itself
+    (8 experts x ~32 rows, 2048 -> 512: 16 tiles of 128 rows on a device that holds hundreds of workgroups)."""
+    c = MH.make_case(0x5EED0F00, 128, 512, 2048, 8, 2)
+    outs = {}
+    for which in (None, "auto"):
+        monkeypatch.delenv("ZMI_GROUP_STREAM_TOP", raising=False)
+        monkeypatch.delenv("ZMI_GROUP_STREAM_SLICES", raising=False)
+        monkeypatch.delenv("ZMI_NO_GROUP_STREAM", raising=False)
+        if which is None:
+            monkeypatch.setenv("ZMI_NO_GROUP_STREAM", "1")
+        d = MH.DeviceMoe(c)
+        w13b = [H.prepack(w, c.H, 2 * c.I) for w in d.w13]
+        w2b = [H.prepack(w, c.I, c.H) for w in d.w2]
+        out2 = torch.zeros((c.T, c.H), dtype=torch.bfloat16, device=H.DEV)
+        st = lowoha.moe_fused_device(d.x, H.to_dev(c.ids), d.topk_w, w13b, w2b, d.s13, d.s2, c.I, capi.ACT_SILU_AND_MUL, out2)
+        assert st == capi.SUCCESS, lowoha.last_error()
+        outs[which] = H.to_host(out2)
+    assert np.array_equal(outs[None], outs["auto"])
+    want = MH.oracle_moe(zo, c, list(range(c.T)))
+    MH.check_moe_out(outs["auto"], want, flipped_rows=2)

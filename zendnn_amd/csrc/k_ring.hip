@@ -666,7 +666,7 @@ hipError_t zmi_launch_ring_table(const ZmiProblem *probs_dev, int n_prob, int to
   return hipGetLastError();
 }
 
-static int ring_cu_count() {
+int zmi_cu_count() {
   static const int n_cu = [] {
     int dev = 0, n = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
@@ -697,7 +697,7 @@ static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int
   if (n_items <= 0) return hipSuccess;
   n_items *= split.slices;
   // at most one workgroup per CU anyway: let it have the whole LDS for its ring
-  const int n_cu = ring_cu_count();
+  const int n_cu = zmi_cu_count();
   (void)exact;   // a bound that fits one workgroup per CU is as good as the exact count
   static const bool force_deep = getenv("ZMI_RING_DEEP") != nullptr;   // EXPERIMENT
   if (BM != 256 && (n_items <= n_cu || force_deep))
@@ -739,7 +739,7 @@ ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices) {
   const int64_t tiles_n = (N + 255) / 256;
   plan.tiles = (int)(((M + plan.top - 1) / plan.top) * tiles_n);
   if (M <= 0) return plan;
-  const int n_cu = ring_cu_count();
+  const int n_cu = zmi_cu_count();
   const int nk = (int)(zmi_blob_kpad(K) / 64);
   const int top = M <= 64 ? 64 : 128;
   const int64_t tiles = ((M + top - 1) / top) * tiles_n;

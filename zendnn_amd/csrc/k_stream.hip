@@ -23,12 +23,17 @@
 //     scales were parked in LDS, decoded, behind the first stages;
 //   * an element is finished with the arithmetic of the MFMA-bound kernel's epilogue, so which of the two kernels
 //     takes an expert does not change a bit of its result.
+// K slices (128-row build, plain epilogues): a launch that would leave workgroup slots empty (few tiles, long K: a down
+// projection) gives every tile to 2 .. 4 workgroups, each over its share of K; they leave int32 partial tiles in a
+// workspace and zmi_stream_reduce_kernel adds them (integers: exact in any order) and finishes the elements with the
+// same arithmetic.  The 256-row build has no registers to spare for it (it spilled 128 of them when it was tried, and
+// two workgroups on the halves of one tile's K stream were measured slower than the MFMA-bound kernel on the same launch).
 // Two builds: 128-row tiles with two workgroups per compute unit (one's start-up and epilogue run under the other's
 // stream; 230 registers), and 256-row tiles with one (an expert of 129 .. 256 rows stays one row block, so its
 // weights pass once).  Measured on MI355X, 8 experts of K = 4096 -> 28672 gated and 14336 -> 4096, whole fused
 // block in ms, MFMA-bound kernel / this one: 11 .. 20 rows 0.358 / 0.333, 52 .. 78 rows 0.397 / 0.351,
 // 88 .. 122 rows 0.391 / 0.376 (128-row tiles); 109 .. 150 rows 0.444 / 0.421, 173 .. 218 rows 0.554 / 0.479
-// (256-row tiles).  In its main loop the kernel moves 5.8 TB/s of weights; what is left on the table is the
+// (256-row tiles); with the down projection in K slices: 11 .. 20 rows 0.371 / 0.298, 52 .. 78 rows 0.398 / 0.343.  In its main loop the kernel moves 5.8 TB/s of weights; what is left on the table is the
 // start-up and the epilogue of every tile (17 of 63 us on a 256-row tile), which a single workgroup per compute
 // unit cannot hide.
 #include <type_traits>
@@ -71,10 +76,10 @@ __device__ __forceinline__ void zmi_s_static_for(F &&f) {
 
 }  // namespace
 
-template <int MI, int D, bool GATED, int OCC>
+template <int MI, int D, bool GATED, int OCC, bool SPLIT>
 __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const ZmiProblem *probs, int n_prob, int n_items,
                                                                        const int *tile_tab, int bm_idx, int top_flags,
-                                                                       ZmiEpilogue epi) {
+                                                                       ZmiRingSplit split, ZmiEpilogue epi) {
   constexpr int BM = 32 * MI;
   constexpr int NPA = MI / 4;                  // row-fragment pairs a wavefront moves per stage
   constexpr int OPS = 2 * NPA + 4;             // memory operations of a wavefront per stage
@@ -90,11 +95,14 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
 
   // ---- which tile (the numbering of the MFMA-bound kernel's grouped launches) ----
-  n_items = tile_tab[bm_idx];
+  // (K slices of one tile are neighbours: the same XCD, their partial sums meet in one L2)
+  const int n_slice = SPLIT ? split.slices : 1;   // (the 256-row build has no registers to spare for the sliced form)
+  n_items = tile_tab[bm_idx] * n_slice;
   const int b = blockIdx.x;
   const int per_xcd = (n_items + 7) / 8;
-  const int id = (b % 8) * per_xcd + b / 8;
-  if (b / 8 >= per_xcd || id >= n_items) return;
+  const int item = (b % 8) * per_xcd + b / 8;
+  if (b / 8 >= per_xcd || item >= n_items) return;
+  const int id = item / n_slice, slice = item % n_slice;
   ZmiProblem p;
   int tn, m0;
   {
@@ -122,7 +130,9 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
   }
   const int M = p.M, N = p.N, K = p.K;
   const int K_pad = (int)zmi_blob_kpad(K);
-  const int nk = K_pad / 64;
+  const int nk_all = K_pad / 64;
+  const int k_first = (int)((int64_t)slice * nk_all / n_slice);            // this slice's stages of 64 k
+  const int nk = (int)((int64_t)(slice + 1) * nk_all / n_slice) - k_first;
   const int64_t frow_bytes = (int64_t)K_pad * 32;
   const uint8_t *Afr = (const uint8_t *)p.A;
   const uint8_t *Bfr = p.blob + zmi_blob_tiles_off(N);
@@ -166,7 +176,8 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
       for (int j = 0; j < 16; ++j) acc[ni][mi][j] = 0;
 
   auto issue_rows = [&](int stage, int slot) {
-    const uint32_t voff = lane16 + (uint32_t)stage * 2048u;
+    const int st_abs = k_first + stage < nk_all ? k_first + stage : nk_all - 1;   // (a slice without stages reads valid memory)
+    const uint32_t voff = lane16 + (uint32_t)(st_abs > 0 ? st_abs : 0) * 2048u;
 #pragma unroll
     for (int j = 0; j < NPA; ++j) zmi_s_dma_pair(abase[j], voff, a_lds[j] + slot * SLOT);
   };
@@ -174,7 +185,8 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
   // only wait there is (the compiler cannot count the global -> LDS loads and would wait for more than it must);
   // their registers are not touched until that wait has covered them.
   auto issue_weights = [&](int u, int stage) {
-    const uint32_t voff = lane16 + (uint32_t)stage * 2048u;
+    const int st_abs = k_first + stage < nk_all ? k_first + stage : nk_all - 1;   // (a slice without stages reads valid memory)
+    const uint32_t voff = lane16 + (uint32_t)(st_abs > 0 ? st_abs : 0) * 2048u;
 #pragma unroll
     for (int ni = 0; ni < 2; ++ni) {
       asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(bw[u][ni][0]) : "v"(voff), "s"(bsrc[ni]) : "memory");
@@ -185,7 +197,7 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
   // ---- prologue: D stages in flight (stages past the end re-read the last one: uniform counts) ----
 #pragma unroll
   for (int s = 0; s < D; ++s) {
-    const int st = s < nk ? s : nk - 1;
+    const int st = s < nk ? s : (nk > 0 ? nk - 1 : 0);
     issue_rows(st, s);
     issue_weights(s, st);
   }
@@ -201,8 +213,10 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
       n = tn * 256 + tid;
       lim = N;
     }
-    cst[tid] = zmi_col_ctx(epi, p, colsum, n, lim);
-    if (tid < BM) rsc[tid] = m0 + tid < M ? zmi_row_scale(epi, p, m0 + tid) : 1.0f;
+    if (n_slice == 1) {
+      cst[tid] = zmi_col_ctx(epi, p, colsum, n, lim);
+      if (tid < BM) rsc[tid] = m0 + tid < M ? zmi_row_scale(epi, p, m0 + tid) : 1.0f;
+    }
   }
   // row fragments of this tile that hold rows at all (the others are skipped: their MFMAs and LDS reads)
   const int n_mi = __builtin_amdgcn_readfirstlane((M - m0 + 31) / 32 < MI ? (M - m0 + 31) / 32 : MI);
@@ -263,6 +277,25 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
     for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) asm volatile("" ::"v"(bw[u][ni][kb]));
+
+  // ---- K slices: every slice leaves its int32 partial tile in the workspace, in register order (16 bytes per lane
+  // and store: whole cache lines), and is done; zmi_stream_reduce_kernel adds the slices and finishes the elements.
+  if (SPLIT && n_slice > 1) {
+    constexpr int CH = 2 * MI * 4;   // 16-byte chunks per lane
+    int32_t *mine = split.partial + (((int64_t)id * n_slice + slice) * 4 + wave) * (int64_t)(CH * 256) + lane * 4;
+    zmi_s_static_for<0, MI>([&](auto mic) {
+      constexpr int mi = decltype(mic)::value;
+      if (mi >= n_mi) return;   // (row fragments without rows are never read back)
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const v4i o = {acc[ni][mi][g * 4], acc[ni][mi][g * 4 + 1], acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]};
+          *zmi_global<v4i>(mine + ((ni * MI + mi) * 4 + g) * 256) = o;
+        }
+    });
+    return;
+  }
 
   // ---- epilogue.  Lane l holds row l % 32 of every 32-row fragment and, per 32-column fragment, four runs of four
   // consecutive columns starting at g * 8 + (l / 32) * 4. ----
@@ -355,6 +388,66 @@ __global__ __launch_bounds__(S_THREADS, OCC) void zmi_gemm_stream_kernel(const Z
   });
 }
 
+// Second step of a K-sliced launch (plain epilogues only: gated launches are never sliced): adds the slices' partial
+// tiles and finishes the elements.  One wavefront per 16-byte chunk column of a tile: lane l of chunk (wave w, ni, mi, g)
+// holds row mi * 32 + l % 32 and the four columns from w * 64 + ni * 32 + g * 8 + (l / 32) * 4 of the tile.
+template <int MI>
+__global__ __launch_bounds__(S_THREADS) void zmi_stream_reduce_kernel(const ZmiProblem *probs, int n_prob, const int *tile_tab,
+                                                                      int bm_idx, int top_flags, ZmiRingSplit split,
+                                                                      ZmiEpilogue epi) {
+  constexpr int BM = 32 * MI, CH = 2 * MI * 4;
+  const int top = top_flags & 0xffff;
+  const int lane = threadIdx.x % 64;
+  constexpr int units_per_tile = 4 * CH;
+  const int unit = blockIdx.x * (S_THREADS / 64) + threadIdx.x / 64;
+  const int id = unit / units_per_tile;
+  if (id >= tile_tab[bm_idx]) return;
+  const int *starts = tile_tab + 4 + bm_idx * n_prob;
+  int e = -1;
+  for (int e0 = 0; e0 < n_prob; e0 += 64) {
+    const int ee = e0 + lane;
+    const int st = ee < n_prob ? starts[ee] : 0x7fffffff;
+    const int c = __popcll(__ballot(st <= id));
+    if (c > 0) e = e0 + c - 1;
+    if (c < 64) break;
+  }
+  e = __builtin_amdgcn_readfirstlane(e);
+  if (e < 0) return;
+  const ZmiProblem p = probs[e];
+  int full; bool rem;
+  zmi_ring_rows<BM>(p.M, top_flags, full, rem);
+  const int tiles_m = full + (rem ? 1 : 0);
+  if (tiles_m <= 0) return;
+  const int r = id - starts[e];
+  const int tm = r % tiles_m, tn = r / tiles_m;
+  const int m0 = tm < full ? tm * top : (p.M / top) * top;
+
+  int u = unit % units_per_tile;
+  const int g = u % 4; u /= 4;
+  const int mi = u % MI; u /= MI;
+  const int ni = u % 2; u /= 2;
+  const int w = u;
+  const int m = m0 + mi * 32 + lane % 32;
+  if (m0 + mi * 32 >= p.M) return;        // (a fragment without rows: the slices stored nothing there)
+  const int n0 = tn * 256 + w * 64 + ni * 32 + g * 8 + (lane / 32) * 4;
+  v4i sum = {0, 0, 0, 0};
+  for (int sl = 0; sl < split.slices; ++sl) {
+    const int32_t *base = split.partial + (((int64_t)id * split.slices + sl) * 4 + w) * (int64_t)(CH * 256) + lane * 4;
+    const v4i a = *zmi_global<const v4i>(base + ((ni * MI + mi) * 4 + g) * 256);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum[j] += a[j];
+  }
+  if (m >= p.M) return;
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+  const float rs = zmi_row_scale(epi, p, m);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + j;
+    if (n >= p.N) break;
+    zmi_finish_element_ring(p, epi, zmi_col_ctx(epi, p, colsum, n, p.N), rs, sum[j], m, n);
+  }
+}
+
 // True when the streaming kernel can stand in for the MFMA-bound kernel on a grouped launch with this epilogue.
 bool zmi_group_stream_takes(const ZmiEpilogue &epi, int N, int top_flags) {
   const int top = top_flags & 0xffff;
@@ -364,35 +457,35 @@ bool zmi_group_stream_takes(const ZmiEpilogue &epi, int N, int top_flags) {
   return getenv("ZMI_NO_GROUP_STREAM") == nullptr;
 }
 
-template <int MI, int D, int OCC>
+template <int MI, int D, int OCC, bool SPLIT>
 static hipError_t stream_launch(const ZmiProblem *probs_dev, int n_prob, int n_items, const int *tab, int top,
-                                const ZmiEpilogue &epi, hipStream_t stream) {
+                                const ZmiRingSplit &split, const ZmiEpilogue &epi, hipStream_t stream) {
+  if (!SPLIT && split.slices > 1) return hipErrorInvalidValue;
   const size_t smem = 256 * 16 + (size_t)MI * 32 * 4 + (size_t)(D + 1) * MI * 2048;
-  const int grid = (n_items + 7) / 8 * 8;
+  const int grid = (n_items * split.slices + 7) / 8 * 8;
   const int bm_idx = MI == 8 ? 0 : 1;
   if (epi.gated_act != 0) {
-    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_stream_kernel<MI, D, true, OCC>, (int)smem);
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_stream_kernel<MI, D, true, OCC, false>, (int)smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((zmi_gemm_stream_kernel<MI, D, true, OCC>), dim3(grid), dim3(S_THREADS), smem, stream, probs_dev, n_prob,
-                       n_items, tab, bm_idx, top, epi);
+    hipLaunchKernelGGL((zmi_gemm_stream_kernel<MI, D, true, OCC, false>), dim3(grid), dim3(S_THREADS), smem, stream, probs_dev,
+                       n_prob, n_items, tab, bm_idx, top, split, epi);
   } else {
-    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_stream_kernel<MI, D, false, OCC>, (int)smem);
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_stream_kernel<MI, D, false, OCC, SPLIT>, (int)smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((zmi_gemm_stream_kernel<MI, D, false, OCC>), dim3(grid), dim3(S_THREADS), smem, stream, probs_dev, n_prob,
-                       n_items, tab, bm_idx, top, epi);
+    hipLaunchKernelGGL((zmi_gemm_stream_kernel<MI, D, false, OCC, SPLIT>), dim3(grid), dim3(S_THREADS), smem, stream, probs_dev,
+                       n_prob, n_items, tab, bm_idx, top, split, epi);
+    if (SPLIT && split.slices > 1) {
+      const int units = n_items * 4 * (2 * MI * 4);
+      hipLaunchKernelGGL((zmi_stream_reduce_kernel<MI>), dim3((units + S_THREADS / 64 - 1) / (S_THREADS / 64)), dim3(S_THREADS), 0,
+                         stream, probs_dev, n_prob, tab, bm_idx, top, split, epi);
+    }
   }
   return hipGetLastError();
 }
 
-// Same contract as zmi_launch_gemm_ring_group for top = 128 | ZMI_RING_PAD or 256 | ZMI_RING_PAD (one launch, every
-// problem's remainder rows in a partly filled tile); tab_dev must already hold the tile table (zmi_launch_ring_table
-// or the kernel that built the problems).
-hipError_t zmi_launch_gemm_stream_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob, int top,
-                                        int64_t worst_rows, int worst_cols, const int *tab_dev, const ZmiEpilogue &epi,
-                                        hipStream_t stream) {
-  const bool gated = epi.gated_act != 0;
+// Tiles of a launch (an upper bound when the row counts live on the device: probs_host null).
+int zmi_stream_items(const ZmiProblem *probs_host, int n_prob, int top, int64_t worst_rows, int worst_cols, bool gated) {
   const int th = top & 0xffff;
-  if (!tab_dev || !(top & ZMI_RING_PAD) || (th != 128 && th != 256)) return hipErrorInvalidValue;
   int items = 0;
   if (probs_host) {
     for (int e = 0; e < n_prob; ++e) {
@@ -405,8 +498,34 @@ hipError_t zmi_launch_gemm_stream_group(const ZmiProblem *probs_host, const ZmiP
     const int ncols = gated ? worst_cols / 2 : worst_cols;
     items = (int)(worst_rows / th + n_prob) * ((ncols + per - 1) / per);
   }
+  return items;
+}
+// Workspace of a K-sliced launch: every (tile, slice) leaves a th x 256 int32 tile.
+size_t zmi_stream_partial_bytes(int items, int slices, int top) {
+  return slices > 1 ? (size_t)items * slices * (top & 0xffff) * 256 * sizeof(int32_t) : 0;
+}
+
+// Same contract as zmi_launch_gemm_ring_group for top = 128 | ZMI_RING_PAD or 256 | ZMI_RING_PAD (one launch, every
+// problem's remainder rows in a partly filled tile); tab_dev must already hold the tile table (zmi_launch_ring_table
+// or the kernel that built the problems).  split (may be null): K slices per tile and their workspace of
+// zmi_stream_partial_bytes bytes; plain epilogues only.
+hipError_t zmi_launch_gemm_stream_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob, int top,
+                                        int64_t worst_rows, int worst_cols, const int *tab_dev, const ZmiRingSplit *split,
+                                        const ZmiEpilogue &epi, hipStream_t stream) {
+  const bool gated = epi.gated_act != 0;
+  const int th = top & 0xffff;
+  if (!tab_dev || !(top & ZMI_RING_PAD) || (th != 128 && th != 256)) return hipErrorInvalidValue;
+  ZmiRingSplit sp = {1, nullptr};
+  if (split && split->slices > 1) {
+    if (gated || !split->partial) return hipErrorInvalidValue;
+    sp = *split;
+  }
+  const int items = zmi_stream_items(probs_host, n_prob, top, worst_rows, worst_cols, gated);
   if (items <= 0) return hipSuccess;
-  if (th == 256) return stream_launch<8, 6, 1>(probs_dev, n_prob, items, tab_dev, top, epi, stream);
+  if (th == 256) {
+    sp.slices = 1;   // (not sliced: see the kernel)
+    return stream_launch<8, 6, 1, false>(probs_dev, n_prob, items, tab_dev, top, sp, epi, stream);
+  }
   // two workgroups per compute unit: one's epilogue and start-up run under the other's stream
-  return stream_launch<4, 4, 2>(probs_dev, n_prob, items, tab_dev, top, epi, stream);
+  return stream_launch<4, 4, 2, true>(probs_dev, n_prob, items, tab_dev, top, sp, epi, stream);
 }

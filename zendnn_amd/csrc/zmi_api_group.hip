@@ -246,18 +246,38 @@ int group_top(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated) {
   return zmi_ring_pick_top_group(rows, n_prob, K, N, gated);
 }
 
-// Tile height (with ZMI_RING_PAD) when the weight-traffic-bound kernel should take a grouped launch whose largest
-// expert has max_rows rows (for a launch whose row counts live on the device: a class derived from the average),
-// 0 when the MFMA-bound kernel keeps it.  Up to 256 rows an expert is one row block: its weights pass once, and
-// the MFMA work of 256 rows takes about as long as its weights need to arrive.  A launch with fewer tiles than two
-// per compute unit stays with the MFMA-bound kernel, whose deep-ring build does better on a half-empty chip
-// (8 experts x 14336 -> 4096: 136 against 157 us).
-int group_stream_top(int max_rows, const ZmiEpilogue &epi, int N, int64_t tiles) {
+// Whether the weight-traffic-bound kernel takes a grouped launch, and how: top = tile height (with ZMI_RING_PAD; 0: the
+// MFMA-bound kernel keeps the launch), slices = K slices per tile.  max_rows: rows of the largest expert (for a launch
+// whose row counts live on the device: a class derived from the average); tiles: (expected) number of tiles at that height.
+// Up to 256 rows an expert is one row block: its weights pass once, and the MFMA work of 256 rows takes about as
+// long as its weights need to arrive.  A launch needs two tiles per compute unit to be worth it; a plain (not gated)
+// launch of 128-row tiles that would leave workgroup slots empty gets there by K slices (8 experts x 28 .. 36 rows,
+// 14336 -> 4096: 128 tiles in 4 slices each).
+struct StreamPlan { int top, slices; };
+// room for the workspace of a K-sliced grouped launch: such a launch has at most 2 x (compute units) items of 128 rows
+// or (compute units) items of 256 rows (64 MiB on 256 compute units), twice that for the slack of a launch sized by
+// a bound; a launch that would need more runs unsliced
+size_t stream_partial_bound() { return (size_t)zmi_cu_count() * 2 * 256 * 256 * sizeof(int32_t); }
+StreamPlan group_stream_plan(int max_rows, const ZmiEpilogue &epi, int N, int K, int64_t tiles) {
+  StreamPlan plan = {0, 1};
+  if ((max_rows <= 16 || max_rows > 256) && !std::getenv("ZMI_GROUP_STREAM_TOP")) return plan;
+  const int th = max_rows <= 128 ? 128 : 256;
+  const int64_t slots = th == 128 ? 2 * (int64_t)zmi_cu_count() : zmi_cu_count();   // workgroups the device holds at once
+  const int nk = (int)(zmi_blob_kpad(K) / 64);
+  int slices = 1;
+  // (256-row tiles are not sliced: two workgroups on the halves of one tile's K stream at 4.1 TB/s together where the
+  // MFMA-bound kernel's deep-ring build reaches the same end sooner: 115 + 35 us against 136 us on config 4's Op2)
+  if (epi.gated_act == 0 && th == 128 && tiles > 0 && tiles * 2 <= slots) slices = (int)std::min<int64_t>(4, slots / tiles);
+  while (slices > 1 && nk / slices < 16) --slices;
+  if (const char *env = std::getenv("ZMI_GROUP_STREAM_SLICES")) slices = std::max(1, std::atoi(env));
+  if (epi.gated_act != 0) slices = 1;
   int top = 0;
-  if (max_rows > 16 && max_rows <= 256 && tiles >= 512) top = (max_rows <= 128 ? 128 : 256) | ZMI_RING_PAD;
+  if (tiles >= slots || slices > 1) top = th | ZMI_RING_PAD;
   if (const char *env = std::getenv("ZMI_GROUP_STREAM_TOP")) top = std::atoi(env);   // (0 switches the kernel off)
-  if (!top || !zmi_group_stream_takes(epi, N, top)) return 0;
-  return top;
+  if (!top || !zmi_group_stream_takes(epi, N, top)) return plan;
+  plan.top = top;
+  plan.slices = slices;
+  return plan;
 }
 
 // Every expert's activations are fragment-major.  Experts with more than 16 rows: one launch of the MFMA-bound
@@ -285,19 +305,27 @@ int32_t launch_stage(const Stage &st, const char *what) {
   const bool split = small > 0 && small_ok && (small >= large || force_split);
   int top = group_top(rows, n, kmax, cols, gated);
   // experts of at most 256 rows are a stream of their weights: the kernel built for that takes the launch
-  int64_t tiles128 = 0;
+  int64_t tiles_th = 0;
   for (const ZmiProblem &q : st.probs)
-    if (q.M > 16) tiles128 += zmi_ring_items<128>(q.M, q.N, 128 | ZMI_RING_PAD, gated);
-  const int stream_top = group_stream_top(max_rows, st.epi, cols, max_rows <= 128 ? tiles128 : 2 * tiles128);
-  if (stream_top) top = stream_top;
+    if (q.M > 16)
+      tiles_th += max_rows <= 128 ? zmi_ring_items<128>(q.M, q.N, 128 | ZMI_RING_PAD, gated) : zmi_ring_items<256>(q.M, q.N, 256 | ZMI_RING_PAD, gated);
+  const StreamPlan sp = group_stream_plan(max_rows, st.epi, cols, kmax, tiles_th);
+  if (sp.top) top = sp.top;
   if (split) top |= ZMI_RING_SKIP_SMALL;
   if (large > 0 || !split) {
     int *tab = (int *)arena().alloc(sizeof(int) * (4 + 3 * (size_t)n));
     if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
-    st.streamed = stream_top != 0;
-    if (stream_top) {
+    st.streamed = sp.top != 0;
+    if (sp.top) {
+      ZmiRingSplit rs = {1, nullptr};
+      if (sp.slices > 1) {
+        const int items = zmi_stream_items(st.probs.data(), n, top, 0, 0, gated);
+        rs.slices = sp.slices;
+        rs.partial = (int32_t *)arena().alloc(zmi_stream_partial_bytes(items, sp.slices, top));
+        if (!rs.partial) rs.slices = 1;   // (no room: the unsliced launch is as right)
+      }
       if (!hip_ok(zmi_launch_ring_table(dev, n, top, gated, tab, stream()), what)) return ZMI_FAILURE;
-      if (!hip_ok(zmi_launch_gemm_stream_group(st.probs.data(), dev, n, top, 0, 0, tab, st.epi, stream()), what)) return ZMI_FAILURE;
+      if (!hip_ok(zmi_launch_gemm_stream_group(st.probs.data(), dev, n, top, 0, 0, tab, &rs, st.epi, stream()), what)) return ZMI_FAILURE;
     } else if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) {
       return ZMI_FAILURE;
     }
@@ -537,6 +565,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       need += Arena::padded(tbl);
     }
     need += 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * num_ops));
+    need += 2 * Arena::padded(stream_partial_bound());   // K-sliced grouped launches (one workspace per GEMM stage)
     if (!arena().begin(need)) return ZMI_FAILURE;
 
     // ---- stage 1: sources (dynamic per-token quantization of every expert in one launch)
@@ -793,6 +822,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   need += Arena::padded((size_t)Rp * kpI) + Arena::padded(sizeof(float) * Rp);       // A2, s2
   need += Arena::padded((size_t)Rp * H * 2);                                         // Y bf16
   need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * (size_t)E));
+  need += Arena::padded(stream_partial_bound());   // Op2 in K slices
   const size_t hist_ints = zmi_moe_route_scratch_ints(R, E);
   need += Arena::padded(hist_ints * sizeof(int32_t));
   if (!arena().begin(need)) return ZMI_FAILURE;
@@ -852,11 +882,13 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   const int avg_rows = (int)((R + E - 1) / E);
   ZmiEpilogue probe1 = probe;
   probe.gated_act = 0;
-  // (an average of up to 96 rows: taken to be at most 128 everywhere; up to 224: at most 256)
+  // (an average of up to 96 rows: taken to be at most 128 everywhere; up to 224: at most 256; the expected tile count
+  // takes every expert to have rows)
   const int row_class = avg_rows <= 96 ? 128 : (avg_rows <= 224 ? 256 : 0);
-  const int64_t blocks = R / 128 + E;
-  const int stream1 = group_stream_top(row_class, probe1, 2 * I, blocks * ((I + 127) / 128));
-  const int stream2 = group_stream_top(row_class, probe, H, blocks * ((H + 255) / 256));
+  const int64_t blocks = row_class ? std::max<int64_t>(R / row_class, std::min<int64_t>(E, R)) : 0;
+  const StreamPlan sp1 = group_stream_plan(row_class, probe1, 2 * I, H, blocks * ((I + 127) / 128));
+  const StreamPlan sp2 = group_stream_plan(row_class, probe, H, I, blocks * ((H + 255) / 256));
+  const int stream1 = sp1.top, stream2 = sp2.top;
   if (stream1) top1 = stream1;
   if (stream2) top2 = stream2;
   if (small1) top1 |= ZMI_RING_SKIP_SMALL;
@@ -871,7 +903,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   ZmiEpilogue e2 = e1;
   e1.gated_act = d->gated_act;
   if (stream1) {
-    if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
+    if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, nullptr, e1, s), "Op1 GEMM launch")) return ZMI_FAILURE;
   } else if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op1, E, top1, R, 2 * I, tile_tab1, true, e1, s), "Op1 GEMM launch")) {
     return ZMI_FAILURE;
   }
@@ -879,7 +911,13 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
   if (stream2) {
-    if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op2, E, top2, R, H, tile_tab2, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
+    ZmiRingSplit rs = {1, nullptr};
+    if (sp2.slices > 1) {
+      rs.slices = sp2.slices;
+      rs.partial = (int32_t *)arena().alloc(zmi_stream_partial_bytes(zmi_stream_items(nullptr, E, top2, R, H, false), sp2.slices, top2));
+      if (!rs.partial) rs.slices = 1;
+    }
+    if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op2, E, top2, R, H, tile_tab2, &rs, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
   } else if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s), "Op2 GEMM launch")) {
     return ZMI_FAILURE;
   }

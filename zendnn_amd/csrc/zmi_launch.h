@@ -92,9 +92,12 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
 bool zmi_group_decode_takes(const ZmiEpilogue &epi, int N);
 // Weight-traffic-bound grouped launch on the MFMA-bound kernel's tiles (k_stream.hip)
 bool zmi_group_stream_takes(const ZmiEpilogue &epi, int N, int top_flags);
+int zmi_cu_count();   // compute units of the current device
+int zmi_stream_items(const ZmiProblem *probs_host, int n_prob, int top, int64_t worst_rows, int worst_cols, bool gated);
+size_t zmi_stream_partial_bytes(int items, int slices, int top);
 hipError_t zmi_launch_gemm_stream_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob, int top,
-                                        int64_t worst_rows, int worst_cols, const int *tab_dev, const ZmiEpilogue &epi,
-                                        hipStream_t stream);
+                                        int64_t worst_rows, int worst_cols, const int *tab_dev, const ZmiRingSplit *split,
+                                        const ZmiEpilogue &epi, hipStream_t stream);
 // Fills the tile table of a grouped launch (4 + 3 * n_prob ints) from the problems' row counts on the device
 hipError_t zmi_launch_ring_table(const ZmiProblem *probs_dev, int n_prob, int top, bool gated, int *tab_dev, hipStream_t stream);
 hipError_t zmi_launch_gemm_group_decode(const ZmiProblem *probs_dev, int n_prob, int max_out_cols, const ZmiEpilogue &epi,
