@@ -17,17 +17,26 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "..", "zendnn_amd", "csrc")
 
 
-@pytest.fixture(scope="module")
-def isa():
+def _compile(source):
     from zendnn_amd import build
     with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "k_stream.s")
+        out = os.path.join(tmp, source.replace(".hip", ".s"))
         flags = [f for f in build.HIPCC_FLAGS if f != "-fPIC"]
         cmd = ["hipcc"] + flags + ["-I", os.path.join(HERE, "..", "include"), "-S", "--cuda-device-only",
-                                   os.path.join(CSRC, "k_stream.hip"), "-o", out]
+                                   os.path.join(CSRC, source), "-o", out]
         r = subprocess.run(cmd, capture_output=True, text=True)
         assert r.returncode == 0, r.stderr[-2000:]
         return open(out).read()
+
+
+@pytest.fixture(scope="module")
+def isa():
+    return _compile("k_stream.hip")
+
+
+@pytest.fixture(scope="module")
+def isa_pgring():
+    return _compile("k_pgring.hip")
 
 
 def _kernels(isa):
@@ -71,3 +80,41 @@ def test_in_flight_registers_are_touched_by_mfmas_only(isa):
                 regs.add(int(m.group(1)))
             assert not (regs & inflight) or op.startswith("v_mfma"), f"{name}: {line}"
         assert n_loads >= 16 and len(inflight) >= 64, name
+
+
+def test_pergroup_tiled_kernel_has_no_spills_and_interleaves_its_fold(isa_pgring):
+    """k_pgring.hip: two wavefronts share a SIMD, so every variant must fit 256 registers without scratch (a spill in
+    the k loop costs more than the kernel gains); and in the variants that fold every block, the loop must issue
+    the fold's VALU instructions between the MFMAs (never two MFMAs in a row, never a run of 3 x 64 fold
+    instructions): that order is what lets the MFMAs run under the fold."""
+    metas = [m for m in re.split(r"\n\s*- \.agpr_count", isa_pgring)[1:] if "zmi_gemm_pgring_kernel" in m]
+    assert len(metas) == 8
+    for meta in metas:
+        name = re.search(r"\.name:\s+(\S+)", meta).group(1)
+        assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", meta).group(1)) == 0, name
+        assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", meta).group(1)) == 0, name
+        assert int(re.search(r"\.vgpr_count:\s+(\d+)", meta).group(1)) <= 256, name
+    bodies = re.split(r"\n(?=_Z22zmi_gemm_pgring_kernel)", isa_pgring)[1:]
+    checked = 0
+    for body in bodies:
+        name = body.split(":")[0]
+        if "Lb1E" in name:          # groups of several blocks: the fold is not pipelined
+            continue
+        body = body.split("s_endpgm")[0]
+        start = body.index("Inner Loop Header")
+        loop = body[start:body.index("s_cbranch_scc", start)]
+        ops = [ln.split()[0] for ln in loop.split("\n") if ln.startswith("\t") and ln.strip() and not ln.strip().startswith(";")]
+        seq = [o for o in ops if o.startswith("v_mfma") or o.startswith(("v_cvt_f32_i32", "v_mul_f32", "v_add_f32"))]
+        run_valu = run_mfma = worst_valu = worst_mfma = 0
+        for o in seq:
+            if o.startswith("v_mfma"):
+                run_mfma += 1
+                run_valu = 0
+            else:
+                run_valu += 1
+                run_mfma = 0
+            worst_valu, worst_mfma = max(worst_valu, run_valu), max(worst_mfma, run_mfma)
+        assert sum(o.startswith("v_mfma") for o in seq) in (8, 16), name
+        assert worst_mfma == 1 and worst_valu <= 64, (name, worst_mfma, worst_valu)
+        checked += 1
+    assert checked == 6

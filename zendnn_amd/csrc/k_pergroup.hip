@@ -621,6 +621,97 @@ hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64
   return hipGetLastError();
 }
 
+// The same quantization for the large-M per-group GEMM: s8 rows in MFMA fragment order (zmi_afrag_off), groups of
+// 32, 64 or 128.  A lane owns 16 consecutive k of one row (one 32- or 64-byte run in, one 16-byte piece of a fragment
+// out); lane l of a wavefront takes row l % 8 of its 8 rows and chunk l / 8 of its 8 chunks, so that the 8 rows of a
+// chunk are 128 contiguous bytes of the fragment, and a group's 2, 4 or 8 lanes meet through cross-lane exchanges.
+template <bool BF16>
+__global__ __launch_bounds__(256) void zmi_quant_groups_frag_kernel(const void *x, int64_t ldx, int M, int K, int G,
+                                                                    int8_t *q, int64_t k_pad, float *scales,
+                                                                    void *user_scales, int32_t user_dt) {
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int gs = K / G, L = gs / 16;                 // lanes per group: 2, 4 or 8
+  const int row = (blockIdx.y * 4 + wave) * 8 + lane % 8;
+  const int chunk = blockIdx.x * 8 + lane / 8;
+  const int k0 = chunk * 16;
+  const bool live = row < M && k0 < K;               // (K is a multiple of 16 and of the group size)
+  float v[16];
+  if (live) {
+    if (BF16) {
+      const uint16_t *src = (const uint16_t *)x + (int64_t)row * ldx + k0;
+      const v4i a = *(const v4i *)src, b = *(const v4i *)(src + 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float((uint32_t)a[j] << 16);
+        v[2 * j + 1] = __uint_as_float((uint32_t)a[j] & 0xffff0000u);
+        v[8 + 2 * j] = __uint_as_float((uint32_t)b[j] << 16);
+        v[8 + 2 * j + 1] = __uint_as_float((uint32_t)b[j] & 0xffff0000u);
+      }
+    } else {
+      const float *src = (const float *)x + (int64_t)row * ldx + k0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const v4f t = *(const v4f *)(src + 4 * j);
+        v[4 * j] = t[0]; v[4 * j + 1] = t[1]; v[4 * j + 2] = t[2]; v[4 * j + 3] = t[3];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = 0.0f;
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const float a = fabsf(v[j]);
+    if ((__float_as_uint(a) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a);
+  }
+  // the group's lanes are 8 apart: chunks (l / 8) of one aligned run of L
+  for (int o = 8; o < 8 * L; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (amax < 1e-10f) amax = 1e-10f;
+  float s = __fdiv_rn(amax, 127.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, s);
+  if (!live) return;
+  if ((lane / 8) % L == 0) {
+    const int64_t item = (int64_t)row * G + k0 / gs;
+    scales[item] = user_dt == ZMI_DT_BF16 ? zmi_bf16_to_f32(zmi_f32_to_bf16_rne(s)) : s;
+    if (user_scales) {
+      if (user_dt == ZMI_DT_BF16) ((uint16_t *)user_scales)[item] = zmi_f32_to_bf16_rne(s);
+      else ((float *)user_scales)[item] = s;
+    }
+  }
+  v4i o;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    uint32_t pk = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pk |= ((uint32_t)(uint8_t)zmi_quant_elem(v[w * 4 + j], s, inv)) << (8 * j);
+    o[w] = (int)pk;
+  }
+  *(v4i *)(q + zmi_afrag_off(row, k0, k_pad)) = o;
+}
+
+bool zmi_quant_groups_frag_ok(const void *x, int32_t x_dt, int64_t K, int64_t ldx, int64_t G) {
+  if (G <= 0 || K % G != 0) return false;
+  const int64_t gs = K / G, es = x_dt == ZMI_DT_BF16 ? 2 : 4;
+  if (x_dt != ZMI_DT_BF16 && x_dt != ZMI_DT_F32) return false;
+  return (gs == 32 || gs == 64 || gs == 128) && ((uintptr_t)x) % 16 == 0 && (ldx * es) % 16 == 0;
+}
+
+hipError_t zmi_launch_quant_groups_frag(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
+                                        float *scales, void *user_scales, int32_t user_dt, hipStream_t stream) {
+  if (M <= 0) return hipSuccess;
+  if (!zmi_quant_groups_frag_ok(x, x_dt, K, ldx, G)) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((K / 16 + 7) / 8), (unsigned)((M + 31) / 32));
+  if (x_dt == ZMI_DT_BF16)
+    hipLaunchKernelGGL(zmi_quant_groups_frag_kernel<true>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q,
+                       zmi_blob_kpad(K), scales, user_scales, user_dt);
+  else
+    hipLaunchKernelGGL(zmi_quant_groups_frag_kernel<false>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q,
+                       zmi_blob_kpad(K), scales, user_scales, user_dt);
+  return hipGetLastError();
+}
+
 // ---- 4-bit tiles for the decode-shaped kernel --------------------------------------------------
 // From the blob of widened s8 weights (every byte a code in -8 .. 7): per 32-column block, the 2 KiB of chunk
 // 2c and of chunk 2c + 1 become one 2 KiB piece, high nibble = even chunk, low nibble = odd chunk.

@@ -699,8 +699,7 @@ static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int
   // at most one workgroup per CU anyway: let it have the whole LDS for its ring
   const int n_cu = zmi_cu_count();
   (void)exact;   // a bound that fits one workgroup per CU is as good as the exact count
-  static const bool force_deep = getenv("ZMI_RING_DEEP") != nullptr;   // EXPERIMENT
-  if (BM != 256 && (n_items <= n_cu || force_deep))
+  if (BM != 256 && n_items <= n_cu)
     return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
   return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
 }

@@ -317,6 +317,15 @@ bool use_ring_kernel(int M, int N, int K) {
   return M > 128 || (M > 64 && wide_output(M, N));
 }
 
+// rows from which the per-group GEMM takes the MFMA-tiled kernel (ZMI_PGRING_MIN_M overrides; 0 turns it off)
+int pgring_min_rows() {
+  if (const char *env = std::getenv("ZMI_PGRING_MIN_M")) {
+    const int v = std::atoi(env);
+    return v > 0 ? v : 0x7fffffff;
+  }
+  return 160;
+}
+
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
   return transA || (K % 16) != 0 || (lda % 16) != 0 || (((uintptr_t)A) % 16) != 0;
 }
@@ -509,6 +518,12 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     plan = plan_ring_gemm(M, N, K);
     need += Arena::padded(plan.partial_bytes);
   }
+  // per-group scales at large M: fragment-order rows, f32 weight scales in padded rows, f32 source scales
+  const bool pgring = pg_groups && M >= pgring_min_rows() && zmi_pgring_takes(M, N, K, K / pg_groups);
+  if (pgring)
+    need += Arena::padded((size_t)zmi_afrag_bytes(M, K)) +
+            Arena::padded(sizeof(float) * (size_t)pg_groups * (size_t)zmi_pgring_ws_cols(N)) +
+            Arena::padded(sizeof(float) * (size_t)M * (size_t)pg_groups);
   if (!arena().begin(need)) return ZMI_FAILURE;
 
   // ---- weights ----
@@ -549,6 +564,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
   ZmiFusedQuant fused;
   std::memset(&fused, 0, sizeof(fused));
   bool use_fused = false;
+  int8_t *a_frag = nullptr;   // per-group GEMM at large M: the rows in fragment order, once they exist
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
     int8_t *q = (int8_t *)arena().alloc(a_bytes);
@@ -572,6 +588,12 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
         fused.q = q; fused.ldq = K16; fused.scales = sc;
         fused.user_scales = (void *)p.src_scale.buff; fused.user_dt = sdt;
         use_fused = true;
+      } else if (pgring && zmi_quant_groups_frag_ok(src, p.dt_src, K, lda, pg_groups)) {
+        // large M: the quantized rows go straight into MFMA fragment order
+        a_frag = (int8_t *)arena().alloc((size_t)zmi_afrag_bytes(M, K));
+        if (!hip_ok(zmi_launch_quant_groups_frag(src, p.dt_src, M, K, lda, pg_groups, a_frag, sc, (void *)p.src_scale.buff, sdt,
+                                                 stream()), "per-group quant launch"))
+          return ZMI_FAILURE;
       } else if (!hip_ok(zmi_launch_quant_groups(src, p.dt_src, M, K, lda, pg_groups, q, K16, sc, (void *)p.src_scale.buff,
                                                  sdt, stream()), "per-group quant launch")) {
         return ZMI_FAILURE;
@@ -655,7 +677,22 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
   ZmiEpilogue epi;
   int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
   if (st != ZMI_SUCCESS) return st;
-  if (epi.n_groups > 0) {
+  if (epi.n_groups > 0 && pgring && !use_fused) {
+    const int64_t G = epi.n_groups, np = zmi_pgring_ws_cols(N);
+    int8_t *af = a_frag ? a_frag : (int8_t *)arena().alloc((size_t)zmi_afrag_bytes(M, K));
+    float *wsp = (float *)arena().alloc(sizeof(float) * (size_t)G * (size_t)np);
+    const float *ssp = (const float *)prob.src_scale_ptr;
+    bool ok = (a_frag || hip_ok(zmi_launch_repack_frag(prob.A, M, K, prob.lda, 0, 0, af, stream()), "repack launch")) &&
+              hip_ok(zmi_launch_pgring_scales(prob.wei_scale_ptr, epi.wei_scale_dt, G, N, np, wsp, stream()), "scale launch");
+    if (ok && epi.src_scale_dt != ZMI_DT_F32) {
+      float *wide = (float *)arena().alloc(sizeof(float) * (size_t)M * (size_t)G);
+      ok = hip_ok(zmi_launch_pgring_scales(prob.src_scale_ptr, epi.src_scale_dt, M, G, G, wide, stream()), "scale launch");
+      ssp = wide;
+    }
+    prob.A = af;
+    set_kernel_name("pergroup_ring_mfma32x32x32");
+    st = ok && hip_ok(zmi_launch_gemm_pgring(prob, epi, ssp, wsp, stream()), "per-group GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
+  } else if (epi.n_groups > 0) {
     const bool s4_stream = tiles_s4 && zmi_pergroup_s4_shape(prob, epi.n_groups);
     set_kernel_name(s4_stream ? (use_fused ? (fused.per_row ? "pergroup_decode_s4_mfma16x16x64 (fused per-token quant)" : "pergroup_decode_s4_mfma16x16x64 (fused per-group quant)") : "pergroup_decode_s4_mfma16x16x64")
                     : use_fused ? "pergroup_decode_mfma16x16x64 (fused per-group quant)"

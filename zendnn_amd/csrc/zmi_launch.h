@@ -141,6 +141,21 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
 bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G);
 // true when it would stream 4-bit tiles if it had them
 bool zmi_pergroup_s4_shape(const ZmiProblem &p, int G);
+// the same with the s8 rows written in MFMA fragment order (groups of 32, 64 or 128, 16-byte aligned rows)
+bool zmi_quant_groups_frag_ok(const void *x, int32_t x_dt, int64_t K, int64_t ldx, int64_t G);
+hipError_t zmi_launch_quant_groups_frag(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
+                                        float *scales, void *user_scales, int32_t user_dt, hipStream_t stream);
+// k_pgring.hip: the per-group GEMM at large M (fragment-order rows, MFMA 32x32x32, scales through LDS);
+// group sizes 32 (K a multiple of 64), 64 and multiples of 128
+bool zmi_pgring_takes(int64_t M, int64_t N, int64_t K, int64_t gs);
+int64_t zmi_pgring_ws_cols(int64_t N);
+// scales {rows, cols} (f32 / bf16) -> f32 rows of out_cols columns: the weight scales {G, N} with
+// out_cols = zmi_pgring_ws_cols(N); bf16 source scales {M, G} with out_cols = G
+hipError_t zmi_launch_pgring_scales(const void *src, int32_t dt, int64_t rows, int64_t cols, int64_t out_cols, float *out,
+                                    hipStream_t stream);
+// p.A: s8 rows in fragment order; ss: {M, G} f32 source scales; ws: the padded f32 weight scales
+hipError_t zmi_launch_gemm_pgring(const ZmiProblem &p, const ZmiEpilogue &epi, const float *ss, const float *ws,
+                                  hipStream_t stream);
 // 4-bit tiles of a blob of widened s4 weights (zmi_s4_tiles_bytes(K, N) bytes)
 hipError_t zmi_launch_s4_tiles(const uint8_t *blob, int64_t K, int64_t N, uint8_t *out, hipStream_t stream);
 // per (row, group) dynamic quantization of bf16 / f32 rows: s8 rows (ld ldq), f32 scales {M,G} and an
