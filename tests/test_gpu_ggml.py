@@ -26,7 +26,8 @@ def _weights(rng, N, K):
     return rows, d16, _pack(rows, d16)
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 64, 16), (16, 4096, 96), (5, 512, 33), (40, 256, 70), (130, 1024, 48), (7, 32, 50)])
+@pytest.mark.parametrize("M,K,N", [(1, 64, 16), (16, 4096, 96), (5, 512, 33), (40, 256, 70), (130, 1024, 48), (7, 32, 50),
+                                   (300, 512, 260)])   # (the last one: the MFMA-tiled per-group kernel, groups of 32)
 @pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_BF16])
 def test_static_s8_rows_with_q8_0_weights(zo, M, K, N, dst_dt):
     rng = np.random.default_rng(M + K + N)
@@ -53,7 +54,7 @@ def test_static_s8_rows_with_q8_0_weights(zo, M, K, N, dst_dt):
     capi.load().zmi_clear_weight_cache()
 
 
-@pytest.mark.parametrize("M,K,N", [(16, 4096, 256), (3, 128, 40), (70, 512, 64), (20, 32, 36)])
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 256), (3, 128, 40), (70, 512, 64), (20, 32, 36), (257, 1024, 130)])
 def test_dynamic_bf16_rows_with_q8_0_weights(zo, M, K, N):
     rng = np.random.default_rng(M * 3 + K + N)
     G = K // 32
@@ -76,6 +77,8 @@ def test_dynamic_bf16_rows_with_q8_0_weights(zo, M, K, N):
     assert st == capi.SUCCESS
     assert np.array_equal(H.to_host(scales_d), scales)
     H.check_bf16(H.to_host(dst), want, max_frac=1e-2)
+    if M >= 160:
+        assert lowoha.last_kernel() == "pergroup_ring_mfma32x32x32"
     capi.load().zmi_clear_weight_cache()
 
 

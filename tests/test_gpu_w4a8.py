@@ -74,7 +74,8 @@ def _run(zo, M, K, N, G, sdims, *, transB=False, const=True, postop=None, bias=F
 
 
 @pytest.mark.parametrize("M,K,N,G", [(16, 4096, 512, 32), (4, 4096, 14336, 32), (1, 4096, 96, 128), (16, 1024, 100, 16),
-                                     (5, 256, 33, 4), (40, 512, 70, 8), (130, 1024, 48, 32), (3, 128, 16, 8)])
+                                     (5, 256, 33, 4), (40, 512, 70, 8), (130, 1024, 48, 32), (3, 128, 16, 8),
+                                     (260, 1024, 200, 8), (192, 512, 64, 16)])   # (the MFMA-tiled per-group kernel)
 @pytest.mark.parametrize("kind", ["tensor", "token", "group"])
 def test_w4a8_scale_granularities(zo, M, K, N, G, kind):
     sdims = {"tensor": (1, 1), "token": (M, 1), "group": (M, G)}[kind]
