@@ -218,7 +218,7 @@ typedef struct zmi_prepack_params_t {
 typedef struct zmi_reorder_params_t {
   int32_t src_dtype, dst_dtype;
   zmi_quant_t scale;        /* dynamic mode: device buffer the scales are WRITTEN to */
-  zmi_quant_t zero_point;   /* must be empty: only symmetric quantization */
+  zmi_quant_t zero_point;   /* empty: symmetric (s8 rows); an s32 buffer with the scale's dims: asymmetric (u8 rows), {M,1} or {M,G} */
   int32_t algo;             /* reorder_algo_t: -1 none, 0 DT, 1 native, 2 reference */
   int32_t num_threads;
   int32_t n_src_shape;   int64_t src_shape[ZMI_MAX_DIMS];

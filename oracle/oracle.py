@@ -46,6 +46,9 @@ def lib():
         L.zo_quant_per_group.restype = None
         L.zo_quant_per_group.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                                          C.c_void_p, C.c_int64, C.c_void_p]
+        L.zo_quant_asym.restype = None
+        L.zo_quant_asym.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                    C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
         L.zo_fp16_to_f32.restype = C.c_float
         L.zo_fp16_to_f32.argtypes = [C.c_uint16]
         L.zo_ggml_q8_0_unpack.restype = None
@@ -119,6 +122,17 @@ def quant_per_group(src, src_dt, G):
     s = np.empty((M, G), dtype=np.float32)
     lib().zo_quant_per_group(_p(src), src_dt, M, K, G, K, _p(q), K, _p(s))
     return q, s
+
+
+def quant_asym(src, src_dt, G=1):
+    """src [M,K] (float32, or uint16 bf16 bits) -> (q uint8 [M,K], scales f32 [M,G], zero-points int32 [M,G])."""
+    src = np.ascontiguousarray(src)
+    M, K = src.shape
+    q = np.empty((M, K), dtype=np.uint8)
+    s = np.empty((M, G), dtype=np.float32)
+    z = np.empty((M, G), dtype=np.int32)
+    lib().zo_quant_asym(_p(src), src_dt, M, K, G, K, _p(q), K, _p(s), _p(z))
+    return q, s, z
 
 
 def ggml_q8_0_unpack(blocks, N, K):

@@ -35,6 +35,9 @@
  *                                restatement on random buffers, both orientations with padded ldb
  *   zo_quant_per_group           per-group constants (closed form), == zo_quant_per_token on the
  *                                [M*G, K/G] view
+ *   zo_quant_asym                closed forms (rows k * 2^-e: scale, zero-point and every code known exactly;
+ *                                constant and non-finite rows), dequantization within half a step, codes of
+ *                                the row minimum / maximum, zero-point against Python fractions
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
  *   prepack layout, weight_prepack_size values: parity unpinned (opaque by the
  *     reference's contract; only the round trip matmul(prepack(B)) == matmul(B)
@@ -189,6 +192,52 @@ ZO_EXPORT void zo_quant_per_group(const void *src, int32_t src_dt, int64_t M, in
       for (int64_t j = 0; j < gs; ++j) {
         float v = zo_read_f32(src, src_dt, m * ld_src + g * gs + j);
         dst[m * ld_dst + g * gs + j] = isfinite(v) ? (int8_t)(int32_t)nearbyintf(v / scale) : 0;
+      }
+    }
+  }
+}
+
+/* Dynamic quantization, asymmetric (u8 rows + s32 zero-points), per token (G == 1) or per group:
+ * lowoha_operators/reorder/reorder_data_type/dynamic_quant_impl/per_token_avx512_f32_fma_kernel.cpp:89-116
+ * (compute_asymmetric_scale_zp: min / max over finite values, an empty or non-finite range becomes [0, 0], a range
+ * of width 0 becomes [min, min + 1], scale = (max - min) / 255 clamped to >= 1e-10, zp = round(-min / scale) in
+ * double, half away from zero, clamped to the s32 range) and :636-680 (q = clamp(nearbyint(v / scale) + zp, 0, 255)
+ * with the true division, non-finite elements -> 0 as the scalar tail :672-677 and the file's notes say; the
+ * reference's vector loop gets there through VCVTPS2DQ's 0x80000000 plus a wrapping add, which gives 255 instead
+ * when zp < 0, and its tail casts quotients beyond s32, which C leaves undefined: here the sum is taken in 64
+ * bits, which agrees with both wherever both are defined); the per-group kernels apply the same rule to every slice
+ * of a row (per_group_avx512_f32_fma_kernel.cpp:91-115, :694-760).  scales, zps: {M,G} row-major. */
+ZO_EXPORT void zo_quant_asym(const void *src, int32_t src_dt, int64_t M, int64_t K, int64_t G, int64_t ld_src,
+                             uint8_t *dst, int64_t ld_dst, float *scales, int32_t *zps) {
+  const int64_t gs = K / G;
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t g = 0; g < G; ++g) {
+      float lo = INFINITY, hi = -INFINITY;
+      for (int64_t j = 0; j < gs; ++j) {
+        float v = zo_read_f32(src, src_dt, m * ld_src + g * gs + j);
+        if (isfinite(v)) {
+          if (v < lo) lo = v;
+          if (v > hi) hi = v;
+        }
+      }
+      if (lo > hi || !isfinite(lo) || !isfinite(hi)) lo = hi = 0.0f;
+      if (hi <= lo) hi = lo + 1.0f;
+      float scale = (hi - lo) / 255.0f;
+      if (scale < 1e-10f) scale = 1e-10f;
+      double zd = round((double)(-lo) / (double)scale);
+      int32_t zp = zd < -2147483648.0 ? INT32_MIN : zd > 2147483647.0 ? INT32_MAX : (int32_t)zd;
+      scales[m * G + g] = scale;
+      zps[m * G + g] = zp;
+      if (!dst) continue;
+      for (int64_t j = 0; j < gs; ++j) {
+        float v = zo_read_f32(src, src_dt, m * ld_src + g * gs + j);
+        if (!isfinite(v)) { dst[m * ld_dst + g * gs + j] = 0; continue; }
+        float t = nearbyintf(v / scale);
+        if (t > 4e9f) t = 4e9f;
+        if (t < -4e9f) t = -4e9f;
+        int64_t q = (int64_t)t + (int64_t)zp;
+        dst[m * ld_dst + g * gs + j] = (uint8_t)(q < 0 ? 0 : q > 255 ? 255 : q);
       }
     }
   }

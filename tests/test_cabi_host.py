@@ -155,8 +155,19 @@ def test_reorder_dynamic_validation():
     rp.scale = lowoha.QuantParam(None, capi.DT_F32, (4, 1))
     assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE          # no scale buffer
     rp.scale = lowoha.QuantParam(FAKE, capi.DT_F32, (4, 1))
+    # a zero-point buffer selects the asymmetric form (reference: validate_dynamic_quant_params,
+    # reorder/lowoha_reorder_utils.cpp:549-580): u8 destination, s32 zero-points, dims given
     rp.zero_point = lowoha.QuantParam(FAKE, capi.DT_S32, (4, 1))
-    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.UNIMPLEMENTED    # asymmetric
+    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE          # asymmetric needs a u8 destination
+    rp.dst_dtype = capi.DT_U8
+    rp.zero_point = lowoha.QuantParam(FAKE, capi.DT_S8, (4, 1))
+    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE          # zero-points are s32
+    rp.zero_point = lowoha.QuantParam(FAKE, capi.DT_S32, ())
+    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE          # zero_point dims are required
+    rp.zero_point = lowoha.QuantParam()
+    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE          # symmetric needs an s8 destination
+    rp.dst_dtype = capi.DT_BF16
+    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE          # s8 or u8 only
     rp2 = lowoha.ReorderParams()                                          # static conversion modes
     assert lowoha.reorder_direct(FAKE, FAKE, rp2) == capi.UNIMPLEMENTED
 

@@ -242,6 +242,63 @@ def test_reorder_direct_per_group_needs_divisible_k(zo):
     assert lowoha.reorder_direct(x_d, q_d, rp) == capi.FAILURE
 
 
+@pytest.mark.parametrize("M,K,G", [(1, 64, 1), (7, 515, 1), (33, 4096, 1), (5, 20000, 1), (9, 512, 16), (300, 1408, 11)])
+@pytest.mark.parametrize("src_dt", [capi.DT_BF16, capi.DT_F32])
+def test_reorder_direct_asymmetric_dynamic_quantization_bit_exact(zo, M, K, G, src_dt):
+    """reorder_direct with a zero-point buffer: u8 rows, f32 (or bf16) scales and s32 zero-points per token ({M,1}) or
+    per group ({M,G}) equal the oracle's (reference: compute_asymmetric_scale_zp and the u8 kernels,
+    dynamic_quant_impl/per_token_avx512_f32_fma_kernel.cpp:89-116, :565-680), with constant slices, shifted rows, NaN
+    and infinities."""
+    rng = np.random.default_rng(M * 17 + K + G)
+    xf = (rng.standard_normal((M, K)) * rng.uniform(0.01, 30, (M, 1)) + rng.uniform(-40, 40, (M, 1))).astype(np.float32)
+    gs = K // G
+    xf[0, :gs] = 2.5                         # a constant slice: its range is widened to 1
+    xf[M - 1, K - 1] = np.inf
+    xf[M // 2, 1] = np.nan
+    if M > 3:
+        xf[3, :] = np.nan                    # nothing finite: range [0, 1], zero-point 0, codes 0
+    x = H.bf16_bits(xf) if src_dt == capi.DT_BF16 else xf
+    x_d = H.to_dev(x)
+    q, s, z = zo.quant_asym(x, src_dt, G)
+
+    def params(scale_buf, scale_dt, zp_buf):
+        rp = lowoha.ReorderParams()
+        rp.src_dtype, rp.dst_dtype = src_dt, capi.DT_U8
+        rp.dynamic_quant = True
+        rp.algo = 1
+        rp.src_shape = rp.dst_shape = (M, K)
+        rp.scale = lowoha.QuantParam(scale_buf, scale_dt, (M, G))
+        rp.zero_point = lowoha.QuantParam(zp_buf, capi.DT_S32, (M, G))
+        return rp
+
+    q_d = torch.zeros((M, K), dtype=torch.uint8, device=H.DEV)
+    s_d = torch.zeros(M * G, dtype=torch.float32, device=H.DEV)
+    z_d = torch.zeros(M * G, dtype=torch.int32, device=H.DEV)
+    st = lowoha.reorder_direct(x_d, q_d, params(s_d, capi.DT_F32, z_d))
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert lowoha.last_kernel() == ("quant_asym_per_token" if G == 1 else "quant_asym_groups")
+    assert np.array_equal(H.to_host(s_d).reshape(M, G), s)
+    assert np.array_equal(H.to_host(z_d).reshape(M, G), z)
+    assert np.array_equal(H.to_host(q_d), q)
+    # bf16 scales: the f32 scale narrowed for the caller, the rows quantized with the f32 scale; scales only
+    sb_d = torch.zeros(M * G, dtype=torch.bfloat16, device=H.DEV)
+    z2_d = torch.zeros(M * G, dtype=torch.int32, device=H.DEV)
+    q2_d = torch.zeros((M, K), dtype=torch.uint8, device=H.DEV)
+    st = lowoha.reorder_direct(x_d, q2_d, params(sb_d, capi.DT_BF16, z2_d))
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert np.array_equal(H.to_host(sb_d).reshape(M, G), H.bf16_bits(s))
+    assert torch.equal(q2_d, q_d) and torch.equal(z2_d, z_d)
+    s3 = torch.zeros(M * G, dtype=torch.float32, device=H.DEV)
+    z3 = torch.zeros(M * G, dtype=torch.int32, device=H.DEV)
+    st = lowoha.reorder_direct(x_d, None, params(s3, capi.DT_F32, z3))
+    assert st == capi.SUCCESS and torch.equal(s3, s_d) and torch.equal(z3, z_d)
+    # scale and zero-point dims must agree
+    bad = params(s_d, capi.DT_F32, z_d)
+    bad.zero_point = lowoha.QuantParam(z_d, capi.DT_S32, (M * G, 1) if G > 1 else (1, M))
+    if bad.zero_point.dims != bad.scale.dims:
+        assert lowoha.reorder_direct(x_d, q_d, bad) == capi.FAILURE
+
+
 @pytest.mark.parametrize("G", [1, 8])
 def test_group_dynamic_quant_per_token_and_per_group(zo, G):
     """group_dynamic_quant (lowoha_reorder.cpp:279-404) through the C ABI: several matrices, one with no rows, padded

@@ -376,6 +376,63 @@ def test_quant_per_group_closed_form_and_per_token_view(zo):
     assert q[1, 40] == 0 and q[2, 3] == 0
 
 
+def test_asymmetric_quant_closed_forms_and_properties(zo):
+    """zo_quant_asym (u8 rows + s32 zero-points; reference: compute_asymmetric_scale_zp,
+    per_token_avx512_f32_fma_kernel.cpp:89-116, quantization :636-680).  Rows of integers times a power of two make
+    every step exact, so scale, zero-point and every code are known without evaluating the formula; the other checks
+    are properties (dequantization within half a step, the codes of the row's extremes, the zero-point against exact
+    fractions)."""
+    from fractions import Fraction
+    # rows k * s, k = lo .. lo + 255: range 255 s, scale = s exactly, zp = -lo, code = k - lo
+    for lo, e in ((0, -3), (-100, -5), (-255, 0), (-17, -10)):
+        s_ = np.float32(2.0 ** e)
+        k = np.arange(lo, lo + 256, dtype=np.int64)
+        rng = np.random.default_rng(lo + 1000)
+        row = (rng.permutation(k).astype(np.float32) * s_)[None, :]
+        q, sc, zp = zo.quant_asym(row, capi.DT_F32)
+        assert sc[0, 0] == s_ and zp[0, 0] == -lo
+        assert np.array_equal(q[0].astype(np.int64), np.rint(row[0] / s_).astype(np.int64) - lo)
+    # a constant row: the range becomes [c, c + 1] (c = 0.25: c + 1 and the width are exact), scale = 1/255 as f32,
+    # every code is 0 (c * 255 = 63.75 is no tie)
+    row = np.full((1, 40), 0.25, dtype=np.float32)
+    q, sc, zp = zo.quant_asym(row, capi.DT_F32)
+    assert sc[0, 0] == np.float32(1.0) / np.float32(255.0) and np.all(q == 0)
+    assert zp[0, 0] == -round(Fraction(0.25) / Fraction(float(sc[0, 0]))) == -64
+    # no finite value at all: range [0, 1], zero-point 0, every code 0; non-finite elements of a mixed row give 0
+    row = np.array([[np.nan, np.inf, -np.inf, np.nan]], dtype=np.float32)
+    q, sc, zp = zo.quant_asym(row, capi.DT_F32)
+    assert sc[0, 0] == np.float32(1.0) / np.float32(255.0) and zp[0, 0] == 0 and np.all(q == 0)
+    row = np.array([[1.0, np.nan, 3.0, np.inf, 2.0, -np.inf]], dtype=np.float32)
+    q, sc, zp = zo.quant_asym(row, capi.DT_F32)
+    assert sc[0, 0] == np.float32(2.0) / np.float32(255.0)
+    assert q[0, 0] == 0 and q[0, 2] == 255 and q[0, 1] == 0 and q[0, 3] == 0 and q[0, 5] == 0
+    # random rows, bf16 and f32, per token and per group
+    rng = np.random.default_rng(3)
+    for src_dt, G in ((capi.DT_F32, 1), (capi.DT_BF16, 1), (capi.DT_F32, 4), (capi.DT_BF16, 8)):
+        M, K = 13, 256
+        xf = (rng.standard_normal((M, K)) * rng.uniform(0.01, 20, (M, 1)) + rng.uniform(-5, 5, (M, 1))).astype(np.float32)
+        x = zo.f32_to_bf16(xf) if src_dt == capi.DT_BF16 else xf
+        v = zo.bf16_to_f32(x) if src_dt == capi.DT_BF16 else xf
+        q, sc, zp = zo.quant_asym(x, src_dt, G)
+        vg = v.reshape(M, G, K // G)
+        qg = q.reshape(M, G, K // G).astype(np.int64)
+        lo, hi = vg.min(axis=2), vg.max(axis=2)
+        assert np.array_equal(sc, ((hi - lo) / np.float32(255.0)).astype(np.float32))     # one f32 subtraction, one division
+        for m in range(M):
+            for g in range(G):
+                exact = Fraction(float(-lo[m, g])) / Fraction(float(sc[m, g]))
+                # (round half away from zero of the double quotient: within 1 of the exact quotient's rounding)
+                assert abs(int(zp[m, g]) - round(exact)) <= 1
+        back = (qg - zp[:, :, None]).astype(np.float64) * sc[:, :, None].astype(np.float64)
+        assert np.all(np.abs(back - vg) <= 0.5001 * sc[:, :, None] + 1e-12)                  # within half a step
+        at_lo = np.take_along_axis(qg, vg.argmin(axis=2)[:, :, None], axis=2)[:, :, 0]
+        at_hi = np.take_along_axis(qg, vg.argmax(axis=2)[:, :, None], axis=2)[:, :, 0]
+        assert np.all(at_lo <= 1) and np.all(at_hi >= 254)
+        # per group == per token on the [M * G, K / G] view
+        q2, sc2, zp2 = zo.quant_asym(np.ascontiguousarray(x.reshape(M * G, K // G)), src_dt, 1)
+        assert np.array_equal(q2.reshape(M, K), q) and np.array_equal(sc2.reshape(M, G), sc) and np.array_equal(zp2.reshape(M, G), zp)
+
+
 def test_chain_dynamic_quant_per_group(zo):
     rng = np.random.default_rng(24)
     M, K, N, G = 4, 128, 6, 4

@@ -621,6 +621,80 @@ hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64
   return hipGetLastError();
 }
 
+// ---- asymmetric dynamic quantization: u8 rows + s32 zero-points, per token (G == 1) or per group ----
+// Reference: compute_asymmetric_scale_zp (zendnnl/src/lowoha_operators/reorder/reorder_data_type/dynamic_quant_impl/
+// per_token_avx512_f32_fma_kernel.cpp:89-116; the per-group twin per_group_avx512_f32_fma_kernel.cpp:91-115) and the
+// quantization loops (:636-680): min / max over the finite values of the row (slice), [0, 0] when there is none, a
+// range of width 0 widened to 1, scale = (max - min) / 255 clamped to >= 1e-10, zp = round(-min / scale) in double
+// (half away from zero, clamped to s32), q = clamp(nearbyint(v / scale) + zp, 0, 255) with the true division,
+// non-finite elements -> 0.  One wavefront per (row, group).
+template <bool BF16>
+__global__ __launch_bounds__(256) void zmi_quant_asym_kernel(const void *x, int64_t ldx, int M, int K, int G, uint8_t *q,
+                                                             int64_t ldq, float *scales, int32_t *zps, void *user_scales,
+                                                             int32_t user_dt) {
+  const int lane = threadIdx.x % 64;
+  const int64_t item = (int64_t)blockIdx.x * 4 + threadIdx.x / 64;
+  if (item >= (int64_t)M * G) return;
+  const int m = (int)(item / G), g = (int)(item % G);
+  const int gs = K / G;
+  const int64_t base = (int64_t)m * ldx + (int64_t)g * gs;
+  auto ld = [&](int k) { return BF16 ? zmi_bf16_to_f32(((const uint16_t *)x)[base + k]) : ((const float *)x)[base + k]; };
+  const float inf = __uint_as_float(0x7f800000u);
+  float lo = inf, hi = -inf;
+  for (int k = lane; k < gs; k += 64) {
+    const float v = ld(k);
+    if ((__float_as_uint(v) & 0x7f800000u) != 0x7f800000u) {
+      lo = fminf(lo, v);
+      hi = fmaxf(hi, v);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    lo = fminf(lo, __shfl_xor(lo, o));
+    hi = fmaxf(hi, __shfl_xor(hi, o));
+  }
+  if (lo > hi) lo = hi = 0.0f;                       // (no finite value; finite bounds are finite by construction)
+  if (hi <= lo) hi = __fadd_rn(lo, 1.0f);
+  float s = __fdiv_rn(__fsub_rn(hi, lo), 255.0f);
+  if (s < 1e-10f) s = 1e-10f;
+  const double zd = round((double)(-lo) / (double)s);
+  const int32_t zp = zd < -2147483648.0 ? (int32_t)0x80000000 : zd > 2147483647.0 ? 0x7fffffff : (int32_t)zd;
+  if (lane == 0) {
+    scales[item] = s;
+    zps[item] = zp;
+    if (user_scales && user_dt == ZMI_DT_BF16) ((uint16_t *)user_scales)[item] = zmi_f32_to_bf16_rne(s);
+  }
+  if (!q) return;
+  uint8_t *dst = q + (int64_t)m * ldq + (int64_t)g * gs;
+  for (int k = lane; k < gs; k += 64) {
+    const float v = ld(k);
+    uint8_t out = 0;
+    if ((__float_as_uint(v) & 0x7f800000u) != 0x7f800000u) {
+      float t = rintf(__fdiv_rn(v, s));
+      t = fminf(fmaxf(t, -4e9f), 4e9f);
+      const long long qq = (long long)t + (long long)zp;
+      out = (uint8_t)(qq < 0 ? 0 : qq > 255 ? 255 : qq);
+    }
+    dst[k] = out;
+  }
+}
+
+// scales: f32 {M,G} (the caller's buffer when its dtype is f32, else scratch with the bf16 copy going to user_scales)
+hipError_t zmi_launch_quant_asym(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, uint8_t *q,
+                                 int64_t ldq, float *scales, int32_t *zps, void *user_scales, int32_t user_dt,
+                                 hipStream_t stream) {
+  if (M <= 0) return hipSuccess;
+  if (G <= 0 || K % G != 0 || (x_dt != ZMI_DT_BF16 && x_dt != ZMI_DT_F32) || !scales || !zps) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((M * G + 3) / 4));
+  if (x_dt == ZMI_DT_BF16)
+    hipLaunchKernelGGL(zmi_quant_asym_kernel<true>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q, ldq, scales,
+                       zps, user_scales, user_dt);
+  else
+    hipLaunchKernelGGL(zmi_quant_asym_kernel<false>, grid, dim3(256), 0, stream, x, ldx, (int)M, (int)K, (int)G, q, ldq, scales,
+                       zps, user_scales, user_dt);
+  return hipGetLastError();
+}
+
 // The same quantization for the large-M per-group GEMM: s8 rows in MFMA fragment order (zmi_afrag_off), groups of
 // 32, 64 or 128.  A lane owns 16 consecutive k of one row (one 32- or 64-byte run in, one 16-byte piece of a fragment
 // out); lane l of a wavefront takes row l % 8 of its 8 rows and chunk l / 8 of its 8 chunks, so that the 8 rows of a

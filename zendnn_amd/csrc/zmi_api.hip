@@ -836,11 +836,23 @@ static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t 
   }
   const int64_t M = rp.src_shape[0], K = rp.src_shape[1];
   if (M <= 0 || K <= 0) { set_error("reorder: non-positive shape"); return ZMI_FAILURE; }
-  if (!(rp.src_dtype == ZMI_DT_BF16 || rp.src_dtype == ZMI_DT_F32) || rp.dst_dtype != ZMI_DT_S8) {
-    set_error("dynamic quantization: only bf16/f32 -> s8 is implemented");
+  if (rp.dst_dtype != ZMI_DT_S8 && rp.dst_dtype != ZMI_DT_U8) {
+    set_error("dynamic quantization: the destination must be s8 or u8");
+    return ZMI_FAILURE;
+  }
+  if (!(rp.src_dtype == ZMI_DT_BF16 || rp.src_dtype == ZMI_DT_F32)) {
+    set_error("dynamic quantization: only bf16 / f32 sources are implemented");
     return ZMI_UNIMPLEMENTED;
   }
-  if (rp.zero_point.buff) { set_error("dynamic quantization: only symmetric (no zero-point buffer)"); return ZMI_UNIMPLEMENTED; }
+  // a zero-point buffer selects the asymmetric form (reference: validate_dynamic_quant_params,
+  // reorder/lowoha_reorder_utils.cpp:549-580: without one the destination must be s8, with one u8, s32 zero-points)
+  const bool asym = rp.zero_point.buff != nullptr;
+  if (!asym && rp.dst_dtype != ZMI_DT_S8) { set_error("dynamic quantization without a zero-point buffer is symmetric: s8 destination"); return ZMI_FAILURE; }
+  if (asym) {
+    if (rp.zero_point.ndims == 0) { set_error("asymmetric dynamic quantization: zero_point dims are required"); return ZMI_FAILURE; }
+    if (rp.zero_point.dt != ZMI_DT_S32) { set_error("asymmetric dynamic quantization: zero-points are s32"); return ZMI_FAILURE; }
+    if (rp.dst_dtype != ZMI_DT_U8) { set_error("asymmetric dynamic quantization: u8 destination"); return ZMI_FAILURE; }
+  }
   if (!rp.scale.buff) { set_error("dynamic quantization: scale buffer is required"); return ZMI_FAILURE; }
   const int32_t sdt = rp.scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : rp.scale.dt;
   if (sdt != ZMI_DT_F32 && sdt != ZMI_DT_BF16) { set_error("dynamic quantization: scale must be f32 or bf16"); return ZMI_FAILURE; }
@@ -854,6 +866,33 @@ static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t 
   }
   const int64_t sn = nelems(rp.scale);
   if (!ensure_device()) return ZMI_FAILURE;
+  if (asym) {
+    // scale and zero-point share granularity and dims (lowoha_reorder_utils.cpp:644-658); per token {M,1} or per
+    // group {M,G} along K
+    if (rp.zero_point.ndims != rp.scale.ndims ||
+        std::memcmp(rp.zero_point.dims, rp.scale.dims, sizeof(rp.scale.dims[0]) * rp.scale.ndims) != 0) {
+      set_error("asymmetric dynamic quantization: scale and zero_point dims differ");
+      return ZMI_FAILURE;
+    }
+    if (!(rp.scale.ndims == 2 && rp.scale.dims[0] == M && rp.scale.dims[1] >= 1 && rp.scale.dims[1] != K)) {
+      set_error("asymmetric dynamic quantization: {M,1} and {M,G} scale dims are implemented");
+      return ZMI_UNIMPLEMENTED;
+    }
+    const int64_t G = rp.scale.dims[1];
+    if (K % G != 0) { set_error("dynamic quantization: per-group scale needs K divisible by the number of groups"); return ZMI_FAILURE; }
+    float *sc = (float *)rp.scale.buff;
+    void *user = nullptr;
+    if (sdt != ZMI_DT_F32) {
+      if (!arena().begin(Arena::padded(sizeof(float) * (size_t)(M * G)))) return ZMI_FAILURE;
+      sc = (float *)arena().alloc(sizeof(float) * (size_t)(M * G));
+      user = (void *)rp.scale.buff;
+    }
+    if (!hip_ok(zmi_launch_quant_asym(src, rp.src_dtype, M, K, ld, G, (uint8_t *)dst, K, sc, (int32_t *)rp.zero_point.buff, user,
+                                      sdt, stream()), "asymmetric quant launch"))
+      return ZMI_FAILURE;
+    set_kernel_name(G == 1 ? "quant_asym_per_token" : "quant_asym_groups");
+    return ZMI_SUCCESS;
+  }
   if (rp.scale.ndims == 2 && rp.scale.dims[0] == M && rp.scale.dims[1] == 1) {
     if (!hip_ok(zmi_launch_quant_rows(src, rp.src_dtype, M, K, ld, (int8_t *)dst, K, 0, (void *)rp.scale.buff, sdt, stream()),
                 "quant launch"))

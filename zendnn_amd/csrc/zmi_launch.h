@@ -141,6 +141,11 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
 bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G);
 // true when it would stream 4-bit tiles if it had them
 bool zmi_pergroup_s4_shape(const ZmiProblem &p, int G);
+// asymmetric form: u8 rows, f32 scales {M,G} and s32 zero-points {M,G} (G == 1: per token); a bf16 copy of the
+// scales goes to user_scales when user_dt says so
+hipError_t zmi_launch_quant_asym(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, uint8_t *q,
+                                 int64_t ldq, float *scales, int32_t *zps, void *user_scales, int32_t user_dt,
+                                 hipStream_t stream);
 // the same with the s8 rows written in MFMA fragment order (groups of 32, 64 or 128, 16-byte aligned rows)
 bool zmi_quant_groups_frag_ok(const void *x, int32_t x_dt, int64_t K, int64_t ldx, int64_t G);
 hipError_t zmi_launch_quant_groups_frag(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, int64_t G, int8_t *q,
