@@ -77,7 +77,7 @@ def test_dynamic_bf16_rows_with_q8_0_weights(zo, M, K, N):
     assert st == capi.SUCCESS
     assert np.array_equal(H.to_host(scales_d), scales)
     H.check_bf16(H.to_host(dst), want, max_frac=1e-2)
-    if M >= 160:
+    if M >= 129:
         assert lowoha.last_kernel() == "pergroup_ring_mfma32x32x32"
     capi.load().zmi_clear_weight_cache()
 

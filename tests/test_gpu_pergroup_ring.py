@@ -17,7 +17,7 @@ RING = "pergroup_ring_mfma32x32x32"
 
 @pytest.fixture(autouse=True)
 def _tiled_kernel_from_96_rows(monkeypatch):
-    """The library takes the tiled kernel from 160 rows (below that its few tiles leave most compute units idle);
+    """The library takes the tiled kernel from 129 rows (below that its few tiles leave most compute units idle);
     these tests reach its 128-row tile and ragged single tiles by lowering the switch."""
     monkeypatch.setenv("ZMI_PGRING_MIN_M", "96")
 
@@ -168,9 +168,9 @@ def test_binary_post_ops_and_rows_below_the_switch(zo, monkeypatch):
     st, want, _, _ = zo.matmul_int8(a, w, ph.flat(keep), M, N, K)
     assert st == capi.SUCCESS
     assert np.array_equal(H.to_host(dst), want)
-    # the default switch: 160 rows
+    # the default switch: 129 rows
     monkeypatch.delenv("ZMI_PGRING_MIN_M")
-    for rows, name in ((159, "pergroup_mfma16x16x64"), (160, RING)):
+    for rows, name in ((128, "pergroup_mfma16x16x64"), (129, RING)):
         pr = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
         ssr = rng.uniform(0.005, 0.03, (rows, G)).astype(np.float32)
         ssr_d = H.to_dev(ssr)

@@ -22,7 +22,7 @@
 
 #define PG_WAVES 2
 
-// RB: 16-row blocks per wavefront; D: chunks per operand set; SUB: groups per 64-k chunk (1: groups of whole
+// RB: 16-row blocks per wavefront (1, 2 or 4); D: chunks per operand set (RB * D == 8); SUB: groups per 64-k chunk (1: groups of whole
 // chunks); CPG: chunks per group when that is 1 or 2 (groups of 64 / 128), 0: any other multiple of 64,
 // taken from gs at run time
 template <int RB, int D, int SUB, int CPG>
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
   // ---- scales: this wavefront's slices ({G,16} weight scales, {16 RB, G} source scales) are staged in its own
   // LDS area GB groups at a time, all requests in flight at once; a fold then needs no global load.  (Fetching
   // them one group ahead from global memory made every fold wait for a full memory latency.) ----
-  constexpr int GB = RB == 1 ? 128 : 32;           // groups per staged block: 16 KiB / 10 KiB per wavefront
+  constexpr int GB = RB == 1 ? 128 : RB == 2 ? 64 : 32;   // groups per staged block: 16 / 12 / 10 KiB per wavefront
   __shared__ float scale_lds[PG_WAVES][(16 + 16 * RB) * GB];
   float *ws_l = scale_lds[wave], *ss_l = scale_lds[wave] + 16 * GB;
   auto stage_scales = [&](int gb0) {
@@ -532,7 +532,9 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
   }
   if (fq) return hipErrorInvalidValue;   // fused quantization exists for the decode-shaped kernel only
   const int n_cb = (int)(zmi_blob_npad(p.N) / 16);
-  const int rb = p.M <= 16 ? 1 : 4;
+  // 16-row blocks per wavefront: 32 rows keep four times as many wavefronts in flight as 64 and are faster up to
+  // ~96 rows (M = 64, groups of 128 / 32: 48 -> 36 us, 105 -> 63 us); beyond that the weights' re-reads from L2 win
+  const int rb = p.M <= 16 ? 1 : p.M <= 96 ? 2 : 4;
   const int n_rb = (p.M + 16 * rb - 1) / (16 * rb);
   const int n_items = n_cb * n_rb;
   const dim3 grid((n_items + PG_WAVES - 1) / PG_WAVES), block(PG_WAVES * 64);
@@ -543,6 +545,9 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
   if (rb == 1) {
     if (sub == 2) PG_LAUNCH(1, 8, 2, 1); else if (sub == 4) PG_LAUNCH(1, 8, 4, 1);
     else if (cpg == 1) PG_LAUNCH(1, 8, 1, 1); else if (cpg == 2) PG_LAUNCH(1, 8, 1, 2); else PG_LAUNCH(1, 8, 1, 0);
+  } else if (rb == 2) {
+    if (sub == 2) PG_LAUNCH(2, 4, 2, 1); else if (sub == 4) PG_LAUNCH(2, 4, 4, 1);
+    else if (cpg == 1) PG_LAUNCH(2, 4, 1, 1); else if (cpg == 2) PG_LAUNCH(2, 4, 1, 2); else PG_LAUNCH(2, 4, 1, 0);
   } else {
     if (sub == 2) PG_LAUNCH(4, 2, 2, 1); else if (sub == 4) PG_LAUNCH(4, 2, 4, 1);
     else if (cpg == 1) PG_LAUNCH(4, 2, 1, 1); else if (cpg == 2) PG_LAUNCH(4, 2, 1, 2); else PG_LAUNCH(4, 2, 1, 0);

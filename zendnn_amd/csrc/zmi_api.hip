@@ -323,7 +323,7 @@ int pgring_min_rows() {
     const int v = std::atoi(env);
     return v > 0 ? v : 0x7fffffff;
   }
-  return 160;
+  return 129;
 }
 
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA) {
