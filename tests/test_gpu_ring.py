@@ -225,3 +225,36 @@ def test_k_slices_chosen_for_a_problem_with_few_tiles(zo):
     ph.src_scale = lowoha.QuantParam(None, capi.DT_F32, (len(sel), 1))
     want, _, _ = _oracle(zo, ph, np.ascontiguousarray(x[sel]), w, len(sel), N, K)
     H.check_bf16(H.to_host(dst)[sel], want)
+
+
+def test_remainder_tiles_beside_the_256_row_tiles_keep_stream_order(zo, monkeypatch):
+    """With 256-row tiles the remainder rows' tiles are a launch of their own on the library's side stream, between a
+    fork and a join on the caller's stream.  Calls that reuse one destination back to back, with a torch kernel
+    on the same stream in between, must see each other's results in stream order."""
+    monkeypatch.setenv("ZMI_GEMM_TOP", "256")
+    rng = np.random.default_rng(21)
+    K, N = 320, 300
+    w = H.gen_weights(rng, K, N)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    w_d, ws_d = H.to_dev(w), H.to_dev(ws)
+    ss = np.array([0.02], dtype=np.float32)
+    Ms = (300, 257, 600, 449)     # remainders of 44, 1, 88 and 193 rows (64-, 64-, 128- and 256-row tiles)
+    dst = torch.zeros((max(Ms), N), dtype=torch.float32, device=H.DEV)
+    for rep in range(3):
+        for M in Ms:
+            a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+            p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32)
+            p.src_scale = lowoha.QuantParam(ss.ctypes.data, capi.DT_F32, (1,))
+            p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+            dst.fill_(7.0)                    # (a torch kernel on the same stream between the calls)
+            st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(a), K, w_d, N, None, 0.0, dst, N, True, p)
+            assert st == capi.SUCCESS, lowoha.last_error()
+            assert lowoha.last_kernel() == "ring_mfma32x32x32_top256"
+            got = dst[:M].clone()             # (reads the destination on the same stream, right behind the call)
+            ph = H.host_params(p, src_scale=ss, wei_scale=ws)
+            keep = []
+            st, want, _, _ = zo.matmul_int8(a, w, ph.flat(keep), M, N, K)
+            assert st == capi.SUCCESS
+            assert np.array_equal(H.to_host(got), want), (rep, M)
+            assert torch.all(dst[M:] == 7.0)
+    capi.load().zmi_clear_weight_cache()

@@ -693,21 +693,34 @@ static hipError_t ring_launch_cfg(const ZmiProblem &p0, const ZmiProblem *probs,
 template <int BM>
 static hipError_t ring_launch(const ZmiProblem &p0, const ZmiProblem *probs, int n_prob, int n_items, bool exact,
                               const int *tile_tab, int top, const ZmiRingSplit &split, const ZmiEpilogue &epi,
-                              hipStream_t stream) {
+                              hipStream_t stream, bool shares_cus = false) {
   if (n_items <= 0) return hipSuccess;
   n_items *= split.slices;
-  // at most one workgroup per CU anyway: let it have the whole LDS for its ring
+  // at most one workgroup per CU anyway: let it have the whole LDS for its ring -- unless the launch runs beside
+  // another one and has only the CUs that one leaves free (two workgroups on each of them then)
   const int n_cu = zmi_cu_count();
   (void)exact;   // a bound that fits one workgroup per CU is as good as the exact count
-  if (BM != 256 && n_items <= n_cu)
+  if (BM != 256 && n_items <= n_cu && !shares_cus)
     return ring_launch_cfg<BM, (BM != 256)>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
   return ring_launch_cfg<BM, false>(p0, probs, n_prob, n_items, tile_tab, top, split, epi, stream);
 }
 
 // Largest tile height for a problem set: 256-row tiles once they fill the chip,
 // 128-row tiles for smaller problems (more tiles, two workgroups per CU).
+// Tile height of a single problem.  128-row tiles run two workgroups per CU (one's epilogue under the other's main
+// loop) and, while all of them fit the CUs' slots at once, take ragged row counts as one launch with a partly filled
+// last tile; 256-row tiles halve the operand traffic per multiply-add and win once their count fills the CUs.
+// Measured on MI355X, K = 4096, N = 14336, whole call in us, 128- / 256-row tiles: M = 769 68 / 77, 900 72 / 70,
+// 1024 74 / 70, 1025 78 / 83, 1100 80 / 94, 1536 113 / 119, 2048 134 / 127, 4096 - / 242.
 int zmi_ring_pick_top(int64_t rows, int64_t out_cols) {
-  const int64_t t256 = ((rows + 255) / 256) * ((out_cols + 255) / 256);
+  const int64_t tn = (out_cols + 255) / 256;
+  const int64_t t256 = ((rows + 255) / 256) * tn, t128 = ((rows + 127) / 128) * tn;
+  const int n_cu = zmi_cu_count();
+  if (t128 <= 2 * n_cu) {
+    // one round either way: 256-row tiles only when they are whole and cover most CUs
+    const bool whole256 = rows % 256 == 0 && t256 <= n_cu && t256 * 100 >= 85 * n_cu;
+    return whole256 ? 256 : 128;
+  }
   return t256 >= 192 ? 256 : 128;
 }
 
@@ -746,7 +759,19 @@ ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices) {
   if (force_slices > 0) slices = force_slices;
   else if (tiles * 4 <= n_cu && nk >= 16) slices = 4;
   if (slices > nk) slices = nk;
-  if (slices < 2) return plan;
+  if (slices < 2) {
+    // A remainder of rows would be a launch of its own behind the full tiles' launch, each with too few tiles to
+    // fill the CUs (M = 129 .. 255, N = 14336: 38 us for 128 rows + 25 us for the rest).  While the padded count
+    // still fits the CUs' workgroup slots at once, the remainder is a partly filled 128-row tile of the one launch.
+    if ((plan.top & 0xffff) == 128 && M > 128 && M % 128 != 0) {
+      const int64_t padded = ((M + 127) / 128) * tiles_n;
+      if (padded <= 2 * n_cu) {
+        plan.top = 128 | ZMI_RING_PAD;
+        plan.tiles = (int)padded;
+      }
+    }
+    return plan;
+  }
   plan.top = top | ZMI_RING_PAD;
   plan.slices = slices;
   plan.tiles = (int)tiles;
@@ -756,7 +781,7 @@ ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices) {
 
 // One problem, M rows in fragment-major order at p.A.
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, const ZmiRingSplit *split,
-                                hipStream_t stream) {
+                                hipStream_t stream, const ZmiRingSide *side) {
   if (p.M <= 0) return hipSuccess;
   const bool gated = epi.gated_act != 0;
   ZmiRingSplit sp = {1, nullptr};
@@ -767,13 +792,29 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
     sp = *split;
   }
   hipError_t e = hipSuccess;
+  // the remainder rows of a 256-row launch: on the side stream when there is one (the two launches write disjoint rows)
+  hipStream_t rem_stream = stream;
+  bool forked = false;
   if ((top & 0xffff) == 256) {
+    const int rem_items = zmi_ring_items<128>(p.M, p.N, top, gated) + zmi_ring_items<64>(p.M, p.N, top, gated);
+    if (side && side->stream && rem_items > 0 && zmi_ring_items<256>(p.M, p.N, top, gated) > 0 && sp.slices == 1) {
+      e = hipEventRecord(side->fork, stream);
+      if (e == hipSuccess) e = hipStreamWaitEvent(side->stream, side->fork, 0);
+      if (e != hipSuccess) return e;
+      rem_stream = side->stream;
+      forked = true;
+    }
     e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
     if (e != hipSuccess) return e;
   }
-  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
+  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, rem_stream, forked);
   if (e != hipSuccess) return e;
-  e = ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
+  e = ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, rem_stream, forked);
+  if (forked) {
+    hipError_t j = hipEventRecord(side->join, side->stream);
+    if (j == hipSuccess) j = hipStreamWaitEvent(stream, side->join, 0);
+    if (e == hipSuccess) e = j;
+  }
   if (e != hipSuccess || sp.slices == 1) return e;
   // the slices' partial tiles -> finished elements
   const int th = top & 0xffff;

@@ -300,7 +300,8 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")
                                      : (th == 256 ? "ring_mfma32x32x32_top256" : "ring_mfma32x32x32_top128"));
-    if (!hip_ok(zmi_launch_gemm_ring(prob, epi, plan->top, &split, stream()), "MFMA GEMM launch")) return ZMI_FAILURE;
+    const ZmiRingSide side = side_stream();
+    if (!hip_ok(zmi_launch_gemm_ring(prob, epi, plan->top, &split, stream(), &side), "MFMA GEMM launch")) return ZMI_FAILURE;
   }
   return ZMI_SUCCESS;
 }

@@ -23,6 +23,10 @@ bool hip_ok(hipError_t e, const char *what);
 // Makes sure a GPU is usable and the per-device state exists.
 bool ensure_device();
 
+// The calling thread's side stream (default priority, created on first use) with a fork and a join event, for work
+// that may run beside the stream's own; null fields when it cannot be had or ZMI_NO_SIDE_STREAM is set.
+ZmiRingSide side_stream();
+
 // ---- scratch arena ------------------------------------------------------------
 // Grow-only device buffer owned by the calling thread.  begin() sizes it for
 // one API call (synchronising the stream only when it has to grow); alloc()

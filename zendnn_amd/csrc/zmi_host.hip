@@ -36,6 +36,10 @@ struct ThreadCtx {
   // stream hand-over (zmi_set_stream): work of this thread may still be queued on `stream`
   bool enqueued = false;
   hipEvent_t handover = nullptr;
+  // side stream (see side_stream())
+  hipStream_t side = nullptr;
+  hipEvent_t side_fork = nullptr, side_join = nullptr;
+  bool side_tried = false;
 };
 thread_local ThreadCtx tctx;
 
@@ -79,6 +83,24 @@ bool hip_ok(hipError_t e, const char *what) {
   set_error(std::string(what) + ": " + hipGetErrorString(e));
   (void)hipGetLastError();
   return false;
+}
+
+ZmiRingSide side_stream() {
+  auto &c = tctx;
+  if (!c.side_tried) {
+    c.side_tried = true;
+    if (!std::getenv("ZMI_NO_SIDE_STREAM")) {
+      bool ok = hipStreamCreateWithFlags(&c.side, hipStreamNonBlocking) == hipSuccess &&
+                hipEventCreateWithFlags(&c.side_fork, hipEventDisableTiming) == hipSuccess &&
+                hipEventCreateWithFlags(&c.side_join, hipEventDisableTiming) == hipSuccess;
+      if (!ok) {
+        (void)hipGetLastError();
+        c.side = nullptr;
+      }
+    }
+  }
+  ZmiRingSide s = {c.side, c.side_fork, c.side_join};
+  return s;
 }
 
 bool ensure_device() {

@@ -81,8 +81,15 @@ struct ZmiRingPlan {
 // top_hint: tile height to use when the launch is not sliced (0: zmi_ring_pick_top);
 // force_slices: 0 = choose, n = that many slices where the shape allows it.
 ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices);
+// side (optional): a second stream with two events.  An unsliced launch with 256-row tiles puts the remainder rows'
+// tiles (their own kernel: 64- or 128-row tiles) on it, between a fork and a join on `stream`, so that they run on
+// the CUs the 256-row tiles leave free instead of behind them.
+struct ZmiRingSide {
+  hipStream_t stream;
+  hipEvent_t fork, join;
+};
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, const ZmiRingSplit *split,
-                                hipStream_t stream);
+                                hipStream_t stream, const ZmiRingSide *side = nullptr);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
                                       const ZmiEpilogue &epi, hipStream_t stream);
