@@ -123,6 +123,62 @@ def _fused_call(M, K, N, rng):
     return x, w, ws, p, dst, call, keep
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("K,N", [(4160, 96), (8192, 1000), (14336, 333), (20000, 64)])
+@pytest.mark.parametrize("mode", ["arrivals", "reduce_kernel"])
+def test_long_k_in_slices_bit_exact(zo, M, K, N, mode, monkeypatch):
+    """K beyond 4096 with at most 16 rows: the 16-row kernel in K slices (2, 2, 4 and 5 of them; K that is no multiple
+    of 64), finished by the last slice to arrive or, without the arrival words, by a reduction kernel.  Raw s32 sums
+    against the integer product, the f32 chain and dynamically quantized bf16 rows against the oracle; repeated
+    calls (the arrival words must be zero again)."""
+    if mode == "reduce_kernel":
+        monkeypatch.setenv("ZMI_NO_SLICE_ARRIVALS", "1")
+    rng = np.random.default_rng(M * 1000 + K + N)
+    for u8 in (False, True):
+        a, w, _, _, _, zp, p, _ = _static_call(M, K, N, u8, capi.DT_S32, rng)
+        want = (a.astype(np.int64) - (131 if u8 else 0)) @ w.astype(np.int64)
+        a_d, w_d = H.to_dev(a), H.to_dev(w)
+        for rep in range(2):
+            dst = torch.full((M, N), -7, dtype=torch.int32, device=H.DEV)
+            st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, a_d, K, w_d, N, None, 0.0, dst, N, True, p)
+            assert st == capi.SUCCESS, lowoha.last_error()
+            assert lowoha.last_kernel() == "decode16_ksliced_dma_rows_mfma16x16x64"
+            assert np.array_equal(H.to_host(dst).astype(np.int64), want), (u8, rep)
+        capi.load().zmi_clear_weight_cache()
+    # f32 chain with bias, rows given
+    a, w, ws, ss, b, zp, p, dev = _static_call(M, K, N, False, capi.DT_F32, rng, bias=True)
+    dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(a), K, H.to_dev(w), N, H.to_dev(b), 0.0, dst, N, False, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    ph = H.host_params(p, src_scale=ss if M > 1 else ss[:1], wei_scale=ws)
+    keep = []
+    st, want, _, _ = zo.matmul_int8(a, w, ph.flat(keep), M, N, K, bias=b)
+    assert st == capi.SUCCESS and np.array_equal(H.to_host(dst), want)
+    # bf16 rows quantized per token by the call (a launch of its own in front of the sliced kernel)
+    x = H.gen_bf16_normal(rng, (M, K), std=2.0)
+    ws_d = H.to_dev(ws)
+    sc_d = torch.zeros(M, dtype=torch.float32, device=H.DEV)
+    pd = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_F32, compute=capi.DT_S8)
+    pd.dynamic_quant = True
+    pd.src_scale = lowoha.QuantParam(sc_d, capi.DT_F32, (M, 1))
+    pd.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    dst = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(x), K, H.to_dev(w), N, None, 0.0, dst, N, False, pd)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert lowoha.last_kernel() == "decode16_ksliced_dma_rows_mfma16x16x64"
+    ph = H.host_params(pd, src_scale=None, wei_scale=ws)
+    keep = []
+    st, want, _, scales = zo.matmul_int8(x, w, ph.flat(keep), M, N, K, want_scales=True, n_scales=M)
+    assert st == capi.SUCCESS
+    assert np.array_equal(H.to_host(sc_d), scales[:M]) and np.array_equal(H.to_host(dst), want)
+    # the small-M kernel on the same call (environment switch): the same bits
+    monkeypatch.setenv("ZMI_NO_DECODE_SLICED", "1")
+    dst2 = torch.zeros((M, N), dtype=torch.float32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(x), K, H.to_dev(w), N, None, 0.0, dst2, N, False, pd)
+    assert st == capi.SUCCESS and lowoha.last_kernel().startswith("smallm_splitk")
+    assert torch.equal(dst2, dst)
+
+
 @pytest.mark.parametrize("M,K,N", [(16, 4096, 2048), (4, 512, 320), (40, 1024, 256)])
 def test_handoff_timeout_fails_loudly_and_recovers(zo, M, K, N, monkeypatch):
     """A streaming workgroup whose wait for the quantized rows runs out computes nothing: the output keeps its

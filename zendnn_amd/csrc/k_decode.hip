@@ -300,14 +300,27 @@ __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkm
 
 #define D16_W_FIRST 2    // chunks of weights requested ahead of the rows
 
-__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi) {
+// K beyond 4096 (n_slices > 1, blockIdx.y = slice): the workgroups of a column block take up to 64 chunks of K each
+// (their rows' share fits LDS as before) and leave their int32 sums in `partial` ([slice][16][N]); integers, so the
+// order of the slices does not matter.  More workgroups at once is the point as much as the LDS: K = 14336,
+// N = 4096 is 128 column blocks on 256 CUs (the kernel moves 4 .. 5 TB/s there, the split-K small-M kernel 2.3).
+// With `arrivals` (a zeroed word per column block, zero again when the launch is over) the slice that arrives last
+// at its column block's word adds the slices and finishes the elements itself: every slice writes its sums through
+// to device scope (word stores that bypass the caches) and waits for their acknowledgement before it counts itself
+// in, and the last one reads them with loads of the same scope.  No fence: a release fence at device scope writes
+// back the whole L2, once per workgroup (90 us per call instead of 16).  Without `arrivals`
+// zmi_decode16_reduce_kernel finishes the elements in a launch of its own (+2 us).
+__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi, int n_slices,
+                                                                           int32_t *partial, unsigned int *arrivals) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int M = p.M, N = p.N, K = p.K;
   const int K_pad = (int)zmi_blob_kpad(K);
-  const int nchunks = K_pad / 64;
   const int blk = (int)blockIdx.x;
+  const int slice = (int)blockIdx.y;
+  const int c0 = (int)((int64_t)slice * (K_pad / 64) / n_slices);               // this workgroup's chunks of 64 k
+  const int nchunks = (int)((int64_t)(slice + 1) * (K_pad / 64) / n_slices) - c0;
 
   // one chunk of rows -> LDS
   const int G = ((K + 15) & ~15) / 16;      // readable 16-byte granules per row
@@ -318,11 +331,11 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     const int gran = c * 4 + a_kg;
     const uint32_t voff = a_row_off + (uint32_t)(gran < G ? gran : G - 1) * 16u;
     if (a_r < M)
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(c * 1024), "v"(voff), "s"(p.A) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"((c - c0) * 1024), "v"(voff), "s"(p.A) : "memory", "m0");
   };
 
-  const int c_begin = wave * nchunks / DEC_WAVES;
-  const int c_end = (wave + 1) * nchunks / DEC_WAVES;
+  const int c_begin = c0 + wave * nchunks / DEC_WAVES;
+  const int c_end = c0 + (wave + 1) * nchunks / DEC_WAVES;
   const int c16 = lane % 16, g = lane / 16;
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const uint8_t *bsrc[2];
@@ -361,7 +374,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   for (int u = 0; u < 8; ++u) {
     const bool live = c_begin + u < c_end;
     const int c = live ? c_begin + u : c_begin;
-    v4i a = *(const v4i *)(lds + c * 1024 + (c16 * 4 + (g ^ ((c16 >> 2) & 3))) * 16);
+    v4i a = *(const v4i *)(lds + (c - c0) * 1024 + (c16 * 4 + (g ^ ((c16 >> 2) & 3))) * 16);
     a[0] ^= xm; a[1] ^= xm; a[2] ^= xm; a[3] ^= xm;   // u8 rows enter the MFMA as (a - 128)
     if (!live) a = (v4i){0, 0, 0, 0};   // whatever b holds then adds nothing
     acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[0], 0, 0, 0);
@@ -376,21 +389,65 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     #pragma unroll
     for (int q = 0; q < 4; ++q) red[wave * 512 + (h * 4 + q) * 64 + lane] = acc[h][q];
   zmi_lds_barrier();
-  if (e_n >= N || e_row >= M) return;
+  const bool e_live = e_n < N && e_row < M;
+  if (!e_live && !(n_slices > 1 && arrivals)) return;
 
   // acc[h][q] of lane l is row (l/16)*4 + q, column h*16 + l%16
   const int off = ((e_col / 16) * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_col % 16;
   int32_t s = 0;
   #pragma unroll
   for (int w = 0; w < DEC_WAVES; ++w) s += red[w * 512 + off];
+  if (n_slices > 1) {
+    if (!arrivals) {
+      if (e_live) partial[((int64_t)slice * 16 + e_row) * N + e_n] = s;
+      return;
+    }
+    if (e_live) __hip_atomic_store(partial + ((int64_t)slice * 16 + e_row) * N + e_n, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    zmi_lds_barrier();                       // (also: everybody has read its sums out of `red`)
+    if (tid == 0) {
+      const unsigned int before = __hip_atomic_fetch_add(arrivals + blk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = before == (unsigned int)(n_slices - 1);
+      if (last) __hip_atomic_store(arrivals + blk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      red[0] = last ? 1 : 0;
+    }
+    zmi_lds_barrier();
+    if (red[0] == 0 || !e_live) return;
+    s = 0;   // (loads that bypass this CU's and this XCD's caches: what the other slices wrote through)
+    for (int sl = 0; sl < n_slices; ++sl)
+      s += __hip_atomic_load(partial + ((int64_t)sl * 16 + e_row) * N + e_n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   const ZmiColCtx cc0 = zmi_col_ctx_raw(epi, p, craw, zp_word, e_n, n_ok, N);
   zmi_finish_element(p, epi, cc0, zmi_row_scale_from_raw(epi, p, rs_word, m_ok), s, e_row, e_n);
+}
+
+__global__ __launch_bounds__(256) void zmi_decode16_reduce_kernel(ZmiProblem p, ZmiEpilogue epi, int n_slices,
+                                                                 const int32_t *partial) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int N = p.N;
+  if (e >= (int64_t)p.M * N) return;
+  const int row = (int)(e / N), n = (int)(e % N);
+  int32_t s = 0;
+  for (int sl = 0; sl < n_slices; ++sl) s += partial[((int64_t)sl * 16 + row) * N + n];
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+  zmi_finish_element(p, epi, zmi_col_ctx(epi, p, colsum, n, N), zmi_row_scale(epi, p, row), s, row, n);
 }
 
 int zmi_decode_grid(const ZmiProblem &p) { return (int)(zmi_blob_npad(p.N) / 32); }
 
 bool zmi_decode_kernel_fits(const ZmiProblem &p) {
   return p.M > 0 && p.M <= 128 && zmi_blob_kpad(p.K) <= 4096;
+}
+
+// K slices of the 16-row kernel for K beyond 4096 (0: the shape is not its: more than 16 rows, or rows it cannot address)
+int zmi_decode16_slices(int M, int64_t K, int64_t lda) {
+  const int64_t nchunks = zmi_blob_kpad(K) / 64;
+  if (M <= 0 || M > 16 || nchunks <= 64 || lda * 16 >= ((int64_t)1 << 31) || getenv("ZMI_DECODE_ROWGROUP_KERNEL")) return 0;
+  return (int)((nchunks + 63) / 64);
+}
+size_t zmi_decode16_partial_bytes(int M, int N, int64_t K) {
+  const int64_t nchunks = zmi_blob_kpad(K) / 64;
+  return M <= 16 && nchunks > 64 ? (size_t)((nchunks + 63) / 64) * 16 * (size_t)N * sizeof(int32_t) : 0;
 }
 
 // Rows given as s8 / u8, at most 16 of them: the kernel without anything in front of the weight stream.
@@ -400,10 +457,27 @@ bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant) {
 }
 
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
-                                  hipStream_t stream) {
-  if (!zmi_decode_kernel_fits(p)) return hipErrorInvalidValue;
+                                  hipStream_t stream, int32_t *partial, unsigned int *arrivals) {
   if (epi.gated_act != 0) return hipErrorInvalidValue;   // gated GEMMs are grouped launches: the large-M kernel
   const int n_blk = zmi_decode_grid(p);
+  if (!zmi_decode_kernel_fits(p)) {
+    // K beyond 4096: up to 16 given rows, in K slices
+    const int slices = fq ? 0 : zmi_decode16_slices(p.M, p.K, p.lda);
+    if (slices < 2 || !partial) return hipErrorInvalidValue;
+    if (n_blk <= 0) return hipSuccess;
+    const int64_t per = (zmi_blob_kpad(p.K) / 64 + slices - 1) / slices + 1;   // chunks of the longest slice, rounded up
+    const size_t op = (size_t)(per < 64 ? per : 64) * 1024;
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel, 4096 * 16);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(zmi_gemm_decode16_kernel, dim3(n_blk, slices), dim3(DEC_THREADS), op > DEC_RED_BYTES ? op : DEC_RED_BYTES,
+                       stream, p, epi, slices, partial, arrivals);
+    e = hipGetLastError();
+    if (e != hipSuccess || arrivals) return e;
+    const int64_t elems = (int64_t)p.M * p.N;
+    hipLaunchKernelGGL(zmi_decode16_reduce_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, stream, p, epi, slices,
+                       partial);
+    return hipGetLastError();
+  }
   if (n_blk <= 0) return hipSuccess;
   ZmiFusedQuant none = {};
   if (zmi_decode_16row_kernel(p, fq != nullptr)) {
@@ -411,7 +485,7 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel, 4096 * 16);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(zmi_gemm_decode16_kernel, dim3(n_blk), dim3(DEC_THREADS), op > DEC_RED_BYTES ? op : DEC_RED_BYTES, stream,
-                       p, epi);
+                       p, epi, 1, (int32_t *)nullptr, (unsigned int *)nullptr);
     return hipGetLastError();
   }
   // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at

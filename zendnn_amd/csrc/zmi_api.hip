@@ -267,6 +267,16 @@ static bool decode_kernel_allowed(int M, int N, int K) {
   return M <= 64 || !wide_output(M, N);
 }
 
+// Up to 16 rows with K beyond the decode kernel's 4096: its 16-row form in K slices (partial sums + a small reduction).
+// (ZMI_NO_DECODE_SLICED: the small-M kernel instead, as before the sliced form existed.)
+static bool decode_sliced_allowed(int M, int N, int K) {
+  (void)N;
+  int max_m = 16;
+  if (const char *env = std::getenv("ZMI_DECODE_MAX_M")) max_m = std::min(max_m, std::atoi(env));
+  if (std::getenv("ZMI_NO_DECODE_KERNEL") || std::getenv("ZMI_NO_DECODE_SLICED")) max_m = 0;
+  return M <= max_m && zmi_blob_kpad(K) > 4096 && zmi_decode16_slices(M, K, zmi_round_up(K, 16)) >= 2;
+}
+
 // Tile height and K slices of a one-problem ring launch.  ZMI_GEMM_TOP (128 / 256) and
 // ZMI_RING_SPLITK (1 = never slice, n = n slices) override the choice; the tests use them
 // to reach every kernel configuration with small shapes.
@@ -284,6 +294,14 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
   if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
     set_kernel_name(zmi_decode_16row_kernel(prob, false) ? "decode16_dma_rows_mfma16x16x64" : "decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
+  } else if (decode_sliced_allowed(prob.M, prob.N, prob.K) && zmi_decode16_slices(prob.M, prob.K, prob.lda) >= 2) {
+    // (the scratch arena was sized for the partial sums by the caller)
+    int32_t *partial = (int32_t *)arena().alloc(zmi_decode16_partial_bytes(prob.M, prob.N, prob.K));
+    if (!partial) { set_error("no scratch for the K-sliced decode GEMM"); return ZMI_FAILURE; }
+    set_kernel_name("decode16_ksliced_dma_rows_mfma16x16x64");
+    if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream(), partial, slice_arrivals(zmi_blob_npad(prob.N) / 32)),
+                "decode GEMM launch"))
+      return ZMI_FAILURE;
   } else if (!use_ring_kernel(prob.M, prob.N, prob.K)) {
     set_kernel_name("smallm_splitk_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_smallm(prob, epi, stream()), "small-M GEMM launch")) return ZMI_FAILURE;
@@ -309,12 +327,16 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
 // Problems with more rows than the small-M kernels take run on the MFMA-bound
 // kernel, which reads the activations in fragment-major order.
 bool use_ring_kernel(int M, int N, int K) {
-  if (decode_kernel_allowed(M, N, K)) return false;
+  if (decode_kernel_allowed(M, N, K) || decode_sliced_allowed(M, N, K)) return false;
   // ZMI_RING_MIN_M overrides the choice (the tests reach the 64-row tile through it)
   if (const char *env = std::getenv("ZMI_RING_MIN_M")) {
     const int min_m = std::atoi(env);
     if (min_m > 0) return M >= min_m;
   }
+  // (33 .. 128 rows with K beyond the decode kernel's: the small-M kernel multiplies every weight chunk by up to
+  // eight row blocks out of L2 and falls behind the K-sliced tiles: K = 14336, N = 4096: M = 64 48 us against 35,
+  // M = 128 93 against 41)
+  if (zmi_blob_kpad(K) > 4096) return M > 32;
   return M > 128 || (M > 64 && wide_output(M, N));
 }
 
@@ -519,6 +541,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     plan = plan_ring_gemm(M, N, K);
     need += Arena::padded(plan.partial_bytes);
   }
+  if (!pg_groups && decode_sliced_allowed(M, N, K)) need += Arena::padded(zmi_decode16_partial_bytes(M, N, K));
   // per-group scales at large M: fragment-order rows, f32 weight scales in padded rows, f32 source scales
   const bool pgring = pg_groups && M >= pgring_min_rows() && zmi_pgring_takes(M, N, K, K / pg_groups);
   if (pgring)
@@ -616,7 +639,9 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
     } else if (per_token && !bcast_src && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
-        !std::getenv("ZMI_NO_FUSED_QUANT")) {
+               !decode_sliced_allowed(M, N, K) && !std::getenv("ZMI_NO_FUSED_QUANT")) {
+      // (the K-sliced decode kernel takes quantized rows: with the quantization of 14336-element rows inside the
+      // launch its workgroups wait longer than the separate launch costs -- 32 against 22 us)
       if (!fused_handoff(&fused)) return ZMI_FAILURE;
       fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
       fused.q = q; fused.ldq = K16; fused.scales = sc;
@@ -625,7 +650,8 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       ep.src_scale.buff = sc;
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = 1;
-    } else if (dyn_scale_n == M && M > 1) {
+    } else if (dyn_scale_n == M && (M > 1 || decode_sliced_allowed(M, N, K))) {
+      // (one row in front of the K-sliced decode kernel: the row kernel, one launch, instead of the per-tensor pair)
       void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
       // (without a caller buffer the scales live in scratch, in the dtype the params name: the reference allocates
       // its own buffer of that dtype, reorder_quantization.cpp:103-117, and its GEMM reads the narrowed values back)

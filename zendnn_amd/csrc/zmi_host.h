@@ -23,6 +23,10 @@ bool hip_ok(hipError_t e, const char *what);
 // Makes sure a GPU is usable and the per-device state exists.
 bool ensure_device();
 
+// Zeroed device words (one per 32-column block, at least n of them) that K-sliced launches count their arrivals in and
+// leave zeroed; null when they cannot be had or ZMI_NO_SLICE_ARRIVALS is set (the launch then ends in a reduction kernel).
+unsigned int *slice_arrivals(int64_t n);
+
 // The calling thread's side stream (default priority, created on first use) with a fork and a join event, for work
 // that may run beside the stream's own; null fields when it cannot be had or ZMI_NO_SIDE_STREAM is set.
 ZmiRingSide side_stream();

@@ -36,6 +36,9 @@ struct ThreadCtx {
   // stream hand-over (zmi_set_stream): work of this thread may still be queued on `stream`
   bool enqueued = false;
   hipEvent_t handover = nullptr;
+  // arrival words of K-sliced launches (see slice_arrivals())
+  unsigned int *arrivals = nullptr;
+  int64_t n_arrivals = 0;
   // side stream (see side_stream())
   hipStream_t side = nullptr;
   hipEvent_t side_fork = nullptr, side_join = nullptr;
@@ -83,6 +86,30 @@ bool hip_ok(hipError_t e, const char *what) {
   set_error(std::string(what) + ": " + hipGetErrorString(e));
   (void)hipGetLastError();
   return false;
+}
+
+unsigned int *slice_arrivals(int64_t n) {
+  auto &c = tctx;
+  if (std::getenv("ZMI_NO_SLICE_ARRIVALS")) return nullptr;
+  if (n > c.n_arrivals) {
+    // (launches still in flight count in the old words)
+    if (c.arrivals) {
+      if (hipStreamSynchronize(c.stream) != hipSuccess || hipFree(c.arrivals) != hipSuccess) (void)hipGetLastError();
+      c.arrivals = nullptr;
+      c.n_arrivals = 0;
+    }
+    const int64_t want = n < 4096 ? 4096 : n * 2;
+    void *d = nullptr;
+    if (hipMalloc(&d, (size_t)want * sizeof(unsigned int)) != hipSuccess ||
+        hipMemset(d, 0, (size_t)want * sizeof(unsigned int)) != hipSuccess) {
+      (void)hipGetLastError();
+      if (d) (void)hipFree(d);
+      return nullptr;
+    }
+    c.arrivals = (unsigned int *)d;
+    c.n_arrivals = want;
+  }
+  return c.arrivals;
 }
 
 ZmiRingSide side_stream() {

@@ -178,8 +178,13 @@ hipError_t zmi_launch_quant_groups(const void *x, int32_t x_dt, int64_t M, int64
 // k_decode.hip: single problem, M <= 128, K_pad <= 4096
 bool zmi_decode_kernel_fits(const ZmiProblem &p);
 // fq != null: the launch also quantizes the M source rows (its grid must be resident at once)
+// partial: int32 workspace of zmi_decode16_partial_bytes() for the K-sliced form (K beyond 4096, up to 16 given rows);
+// arrivals: one zeroed word per 32-column block (left zeroed) -- with it the last slice of a block finishes the
+// elements, without it a second kernel does
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
-                                  hipStream_t stream);
+                                  hipStream_t stream, int32_t *partial = nullptr, unsigned int *arrivals = nullptr);
+int zmi_decode16_slices(int M, int64_t K, int64_t lda);
+size_t zmi_decode16_partial_bytes(int M, int N, int64_t K);
 int zmi_decode_grid(const ZmiProblem &p);
 // true when the launch above takes the 16-row kernel (rows fetched by global->LDS loads behind the first weights)
 bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant);
