@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0
 K_DEC, N_DEC = 4096, 14336
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
-# size), measured with the commands recorded in profiles/zmi_gemm_decode_kernel_decode_M16_K4096_N14336.md
+# size), measured with the commands recorded in profiles/zmi_gemm_decode16_kernel_decode_M16_K4096_N14336.md
 DECODE_TRAFFIC_BYTES = 60293616
 
 
@@ -255,7 +255,7 @@ def main():
             "config": {"workload": "matmul_direct decode: M=16 K=4096 N=14336, bf16 -> per-token s8, "
                                    "prepacked s8 weights, per-channel scales, SiLU, bf16 out",
                        "weight_sets_rotated": n_sets, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1)},
-            "roofline": {"bound": "hbm", "kernel": "zmi_gemm_decode_kernel: " + (step_kernel if fused else gemm_kernel),
+            "roofline": {"bound": "hbm", "kernel": "zmi_gemm_decode16_kernel: " + (step_kernel if fused else gemm_kernel),
                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": DECODE_TRAFFIC_BYTES,
                          "algorithmic_bytes_per_launch": decode_bytes(M) if fused else kbytes,

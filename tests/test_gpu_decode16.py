@@ -123,6 +123,31 @@ def _fused_call(M, K, N, rng):
     return x, w, ws, p, dst, call, keep
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("K,N", [(4096, 14336), (4096, 1000), (1000, 333), (64, 32), (24, 70), (2048, 4096)])
+def test_fused_quantization_on_the_16_row_kernel_bit_exact(zo, M, K, N, monkeypatch):
+    """bf16 rows quantized per token inside the launch of the 16-row kernel (the wait for the rows goes through the
+    scalar unit): bit-identical to the oracle on repeated calls (a fresh launch number each), and to the row-group
+    kernel's form of the same call."""
+    rng = np.random.default_rng(M * 100 + K + N)
+    x, w, ws, p, dst, call, keep = _fused_call(M, K, N, rng)
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    ph.mem_format_b = "n"
+    hk = []
+    st, want, _, _ = zo.matmul_int8(x, w, ph.flat(hk), M, N, K)
+    assert st == capi.SUCCESS
+    for rep in range(3):
+        dst.fill_(12345.0)
+        assert call() == capi.SUCCESS, lowoha.last_error()
+        assert lowoha.last_kernel() == "decode16_dma_rows_mfma16x16x64 (fused per-token quant)"
+        assert np.array_equal(H.to_host(dst), want), rep
+    monkeypatch.setenv("ZMI_DECODE_ROWGROUP_KERNEL", "1")
+    dst.fill_(12345.0)
+    assert call() == capi.SUCCESS, lowoha.last_error()
+    assert lowoha.last_kernel() == "decode_lds_rows_mfma16x16x64 (fused per-token quant)"
+    assert np.array_equal(H.to_host(dst), want)
+
+
 @pytest.mark.parametrize("M", [1, 7, 16])
 @pytest.mark.parametrize("K,N", [(4160, 96), (8192, 1000), (14336, 333), (20000, 64)])
 @pytest.mark.parametrize("mode", ["arrivals", "reduce_kernel"])

@@ -293,9 +293,7 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
 // zero weights and are fetched from the row's last 16 bytes.
 // (Measured and dropped: the rows by helper wavefronts -- their requests end up behind the weights of
 // the whole compute unit; at most 2 .. 6 chunks of weights in flight per wavefront; neighbouring
-// workgroups starting at different slices of K; rows and weights requested alternately; the
-// quantization of bf16 rows inside this kernel behind helper wavefronts that wait for the quantizing
-// workgroups -- 15.8 us against 14.6 us for the row-group kernel's form.)
+// workgroups starting at different slices of K; rows and weights requested alternately.)
 __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 #define D16_W_FIRST 2    // chunks of weights requested ahead of the rows
@@ -310,14 +308,38 @@ __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkm
 // in, and the last one reads them with loads of the same scope.  No fence: a release fence at device scope writes
 // back the whole L2, once per workgroup (90 us per call instead of 16).  Without `arrivals`
 // zmi_decode16_reduce_kernel finishes the elements in a launch of its own (+2 us).
-__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi, int n_slices,
-                                                                           int32_t *partial, unsigned int *arrivals) {
+//
+// FQ: the per-token quantization of bf16 / f32 rows is part of the launch (K up to 4096).  M workgroups at the head
+// of the grid quantize one row each and stamp its flag; every other wavefront requests ALL its weights, then waits
+// for the flags through the scalar unit, then requests the rows (they return behind the weights, which the MFMAs
+// need as well) and the constants.  The scalar unit's loads do not stand in the compute unit's queue of vector
+// memory requests: behind the weight stream a vector load of the flags only returns with the stream (microseconds),
+// which is why the row-group kernel holds a quarter of its weights back until its wait is over.  M = 16,
+// N = 14336: 14.6 us per call against 15.9 us for the row-group kernel's form and 12.8 us with rows that are given.
+// What is left of the difference (timestamps inside the kernel): the rows are published 5 us after the launch
+// starts (2.4 us to read and quantize a row, 1.1 us until its stores are acknowledged, 1.5 us for the flag, all
+// behind the weight requests of the workgroup that shares the compute unit), a waiting wavefront sees that 1 us
+// later, and its row requests then stand at the end of its compute unit's queue: the last workgroups end 11.6 us
+// after they started against 9.7 us.  Requesting the rows ahead of the last quarter of the weights changes 0.3 us;
+// sixteen copies of the flags on different memory channels bring the wait forward by 1.3 us and the end by nothing.
+template <bool FQ>
+__global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi, ZmiFusedQuant fq,
+                                                                           int n_slices, int32_t *partial,
+                                                                           unsigned int *arrivals) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int M = p.M, N = p.N, K = p.K;
   const int K_pad = (int)zmi_blob_kpad(K);
-  const int blk = (int)blockIdx.x;
+  int blk = (int)blockIdx.x;
+  if (FQ) {
+    if (blk < M) {   // (producers wait for nothing and are dispatched first)
+      zmi_fused_quant_row(fq, blk, K, reinterpret_cast<float *>(lds));
+      zmi_fq_publish(fq, blk);
+      return;
+    }
+    blk -= M;
+  }
   const int slice = (int)blockIdx.y;
   const int c0 = (int)((int64_t)slice * (K_pad / 64) / n_slices);               // this workgroup's chunks of 64 k
   const int nchunks = (int)((int64_t)(slice + 1) * (K_pad / 64) / n_slices) - c0;
@@ -349,13 +371,25 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     b[u][0] = __builtin_nontemporal_load((const v4i *)(bsrc[0] + (int64_t)c * 2048));
     b[u][1] = __builtin_nontemporal_load((const v4i *)(bsrc[1] + (int64_t)c * 2048));
   };
-  #pragma unroll
-  for (int u = 0; u < D16_W_FIRST; ++u) load_b(u);
-  #pragma unroll
-  for (int u = 0; u < 8; ++u)
-    if (c_begin + u < c_end) stage_chunk(c_begin + u);
-  #pragma unroll
-  for (int u = D16_W_FIRST; u < 8; ++u) load_b(u);
+  bool rows_ok = true;
+  if (!FQ) {
+    #pragma unroll
+    for (int u = 0; u < D16_W_FIRST; ++u) load_b(u);
+    #pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (c_begin + u < c_end) stage_chunk(c_begin + u);
+    #pragma unroll
+    for (int u = D16_W_FIRST; u < 8; ++u) load_b(u);
+  } else {
+    #pragma unroll
+    for (int u = 0; u < 8; ++u) load_b(u);
+    rows_ok = zmi_fq_wait_scalar(fq, M);   // (every wavefront for itself: there is no barrier before the MFMAs)
+    if (rows_ok) {
+      #pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (c_begin + u < c_end) stage_chunk(c_begin + u);
+    }
+  }
   // this thread's output element (row tid / 32, column tid % 32) and its constants, as raw words
   const int e_row = tid / 32, e_col = tid % 32;
   const int e_n = blk * 32 + e_col;
@@ -366,7 +400,8 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   const uint32_t rs_word = zmi_row_scale_raw(epi, p, colsum, m_ok);
   // requests complete in order: once the rows are in LDS, at most the weight requests that followed them
   // and the 5 constant words are outstanding
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (8 - D16_W_FIRST) + 5) : "memory");
+  if (FQ) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (8 - D16_W_FIRST) + 5) : "memory");
   const uint32_t xm = p.a_is_u8 ? 0x80808080u : 0u;
 
   v4i acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
@@ -388,7 +423,14 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   for (int h = 0; h < 2; ++h)
     #pragma unroll
     for (int q = 0; q < 4; ++q) red[wave * 512 + (h * 4 + q) * 64 + lane] = acc[h][q];
+  if (FQ && lane == 0) red[DEC_WAVES * 512 + wave] = rows_ok ? 1 : 0;
   zmi_lds_barrier();
+  if (FQ) {   // a wavefront whose wait ran out staged no rows: the workgroup stores nothing
+    int all = 1;
+    #pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) all &= red[DEC_WAVES * 512 + w];
+    if (!all) return;
+  }
   const bool e_live = e_n < N && e_row < M;
   if (!e_live && !(n_slices > 1 && arrivals)) return;
 
@@ -453,7 +495,8 @@ size_t zmi_decode16_partial_bytes(int M, int N, int64_t K) {
 // Rows given as s8 / u8, at most 16 of them: the kernel without anything in front of the weight stream.
 // (ZMI_DECODE_ROWGROUP_KERNEL: the tests reach the row-group kernel with few rows through it.)
 bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant) {
-  return !fused_quant && p.M <= 16 && (int64_t)p.lda * 16 < ((int64_t)1 << 31) && !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
+  (void)fused_quant;
+  return p.M <= 16 && (int64_t)p.lda * 16 < ((int64_t)1 << 31) && !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
 }
 
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
@@ -467,10 +510,10 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     if (n_blk <= 0) return hipSuccess;
     const int64_t per = (zmi_blob_kpad(p.K) / 64 + slices - 1) / slices + 1;   // chunks of the longest slice, rounded up
     const size_t op = (size_t)(per < 64 ? per : 64) * 1024;
-    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel, 4096 * 16);
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel<false>, 4096 * 16);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(zmi_gemm_decode16_kernel, dim3(n_blk, slices), dim3(DEC_THREADS), op > DEC_RED_BYTES ? op : DEC_RED_BYTES,
-                       stream, p, epi, slices, partial, arrivals);
+    hipLaunchKernelGGL(zmi_gemm_decode16_kernel<false>, dim3(n_blk, slices), dim3(DEC_THREADS),
+                       op > DEC_RED_BYTES ? op : DEC_RED_BYTES, stream, p, epi, ZmiFusedQuant{}, slices, partial, arrivals);
     e = hipGetLastError();
     if (e != hipSuccess || arrivals) return e;
     const int64_t elems = (int64_t)p.M * p.N;
@@ -481,11 +524,18 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
   if (n_blk <= 0) return hipSuccess;
   ZmiFusedQuant none = {};
   if (zmi_decode_16row_kernel(p, fq != nullptr)) {
+    // (the operand area, reused by the partial tiles, and with the quantization in the launch a word per wavefront)
     const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
-    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel, 4096 * 16);
+    const size_t smem = (op > DEC_RED_BYTES ? op : DEC_RED_BYTES) + (fq ? 64 : 0);
+    const void *f = fq ? (const void *)zmi_gemm_decode16_kernel<true> : (const void *)zmi_gemm_decode16_kernel<false>;
+    hipError_t e = zmi_func_smem_once(f, 4096 * 16 + 64);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(zmi_gemm_decode16_kernel, dim3(n_blk), dim3(DEC_THREADS), op > DEC_RED_BYTES ? op : DEC_RED_BYTES, stream,
-                       p, epi, 1, (int32_t *)nullptr, (unsigned int *)nullptr);
+    if (fq)
+      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<true>, dim3(n_blk + p.M), dim3(DEC_THREADS), smem, stream, p, epi, *fq, 1,
+                         (int32_t *)nullptr, (unsigned int *)nullptr);
+    else
+      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<false>, dim3(n_blk), dim3(DEC_THREADS), smem, stream, p, epi, ZmiFusedQuant{},
+                         1, (int32_t *)nullptr, (unsigned int *)nullptr);
     return hipGetLastError();
   }
   // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at

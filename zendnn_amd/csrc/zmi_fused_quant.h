@@ -67,6 +67,33 @@ static __device__ __forceinline__ bool zmi_fq_wait(const ZmiFusedQuant &fq, int 
   return ok;
 }
 
+// The same wait through the scalar unit, called by a whole wavefront: a scalar load does not stand in the compute
+// unit's queue of vector memory requests, so a wavefront may have its whole weight stream in flight while it waits
+// (behind the stream, a vector load of the flags returns with the stream).  A scalar load cannot ask for device
+// scope; the flags lie in uncached device memory for it (in cached memory the XCD's L2 would keep answering with
+// the line it fetched first), and `glc` makes the load miss in the scalar cache.
+static __device__ __forceinline__ bool zmi_fq_wait_scalar(const ZmiFusedQuant &fq, int rows) {
+  typedef unsigned int zmi_u16v __attribute__((ext_vector_type(16)));
+  const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+  bool ok = false;
+  if (fq.wait_ticks != 0) {
+    for (;;) {
+      bool all = true;
+      for (int r0 = 0; r0 < rows; r0 += 16) {   // (rows <= 128: at most 8 loads of 16 flags)
+        zmi_u16v v;
+        asm volatile("s_load_dwordx16 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=&s"(v) : "s"(fq.flags + r0) : "memory");
+#pragma unroll
+        for (int i = 0; i < 16; ++i) all &= (r0 + i >= rows) | (v[i] == fq.epoch);
+      }
+      if (all) { ok = true; break; }
+      if (__builtin_amdgcn_s_memrealtime() - t0 > (uint64_t)fq.wait_ticks) break;
+      __builtin_amdgcn_s_sleep(2);
+    }
+  }
+  if (!ok && threadIdx.x % 64 == 0) __hip_atomic_store(fq.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  return ok;
+}
+
 static __device__ void zmi_fused_quant_row(const ZmiFusedQuant &fq, int row, int K, float *red) {
   const int t = threadIdx.x, nt = blockDim.x;
   const bool bf16 = fq.x_dt == ZMI_DT_BF16;

@@ -252,7 +252,9 @@ bool fused_handoff(ZmiFusedQuant *fq) {
   ThreadCtx &c = tctx;
   if (!c.fq_flags) {
     void *d = nullptr, *h = nullptr, *hd = nullptr;
-    if (!hip_ok(hipMalloc(&d, 512), "hipMalloc(hand-off words)")) return false;
+    // (uncached: the waiting side may read the flags through the scalar unit, which cannot ask for device scope;
+    // never freed -- memory of this kind that a kernel has read stays allocated until the process ends)
+    if (!hip_ok(hipExtMallocWithFlags(&d, 512, hipDeviceMallocUncached), "hipExtMallocWithFlags(hand-off words)")) return false;
     if (!hip_ok(hipMemset(d, 0, 512), "hipMemset(hand-off words)")) return false;
     if (!hip_ok(hipHostMalloc(&h, 64, hipHostMallocMapped), "hipHostMalloc(error word)")) return false;
     std::memset(h, 0, 64);
