@@ -42,6 +42,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
     ap.add_argument("--only", default=None,
                     choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "decode_M16_w4a8_group128", "decode_M16_w4a8_group128_per_token_rows", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
+                             "decode_M16_K14336_N4096", "prefill_N14336_per_group128", "prefill_N14336_per_group32",
                              "moe_decode_T16", "moe_config4", "moe_config5"],
                     help="run one of the other configs alone and print its entry (for profiler runs)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -348,19 +349,48 @@ def main():
         capi.load().zmi_clear_weight_cache()
         return out
 
-    def run_prefill(N):
+    def run_decode_down(m):
+        # the down projection of the same block at decode: K = 14336, N = 4096, bf16 rows quantized per token by the
+        # call (a launch of its own), then the 16-row kernel in K slices; bytes = weights + rows + scales + output
+        K, N = N_DEC, K_DEC
+        blobs = [prepack(rand_w(K, N), K, N) for _ in range(n_sets)]
+        ws = torch.rand(N, device=dev, generator=g) * 0.009 + 0.001
+        x = torch.randn((m, K), device=dev, generator=g).to(torch.bfloat16)
+        dst = torch.zeros((m, N), dtype=torch.bfloat16, device=dev)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (m, 1))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        calls = [lowoha.prepared_matmul("r", False, False, m, N, K, 1.0, x, K, blob, N, None, 0.0, dst, N, True, p)[0]
+                 for blob in blobs]
+        state = {"i": 0}
+
+        def step():
+            st = calls[state["i"] % n_sets]()
+            state["i"] += 1
+            if st != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+
+        t = ev_time(step, 100, 10)
+        nbytes = K * N + m * K * 2 + m * 4 + N * 4 + m * N * 2
+        return {"GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2), "kernel": lowoha.last_kernel()}
+
+    def run_prefill(N, gs=None):
         # config 3: whole call = per-token quantization launch (rows written in MFMA fragment order) + GEMM launch;
         # the per-kernel split is in the rocprofv3 summaries under profiles/
+        # gs: per-group scales instead ({M, K/gs} source scales computed by the call, {K/gs, N} weight scales)
         Mp, K = 2048, 4096
         blob = prepack(rand_w(K, N), K, N)
-        ws = torch.rand(N, device=dev, generator=g) * 0.009 + 0.001
+        ws = torch.rand(N if gs is None else (K // gs, N), device=dev, generator=g) * 0.009 + 0.001
         bias = torch.randn(N, device=dev, generator=g) * 0.1
         x = torch.randn((Mp, K), device=dev, generator=g).to(torch.bfloat16)
         dst = torch.zeros((Mp, N), dtype=torch.bfloat16, device=dev)
         p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32, compute=capi.DT_S8)
         p.dynamic_quant = True
-        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (Mp, 1))
-        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (Mp, 1) if gs is None else (Mp, K // gs))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N) if gs is None else (K // gs, N))
         p.postop_ = [lowoha.PostOp(capi.PO_GELU_TANH)]
         p.mem_format_b = "r"
         p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
@@ -443,6 +473,10 @@ def main():
         "prefill_N4096": lambda: run_prefill(4096),
         "prefill_N14336": lambda: run_prefill(14336),
         "config1_u8s8_M128": run_config1,
+        "decode_M16_K14336_N4096": lambda: run_decode_down(16),
+        # config 3's shape with per-group scales (the VALU-bound tiled kernel: every group's sums are scaled and added in f32)
+        "prefill_N14336_per_group128": lambda: run_prefill(14336, 128),
+        "prefill_N14336_per_group32": lambda: run_prefill(14336, 32),
         # a decode step of configuration 4's block: 16 tokens, every expert has a handful of rows (decode-shaped grouped kernel)
         "moe_decode_T16": lambda: run_moe(16, 4096, 14336, 8, 2, False),
         "moe_config4": lambda: run_moe(512, 4096, 14336, 8, 2, False),

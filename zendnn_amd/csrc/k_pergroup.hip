@@ -214,6 +214,10 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
   // ---- alpha / beta, then the common tail; acc element q of lane l is row (l / 16) * 4 + q, column l % 16 ----
   if (col >= N) return;
   const float bias = p.bias ? zmi_ld_f32(p.bias, epi.bias_dt, col) : 0.0f;
+  // one straight-line activation into a bf16 store: the form of the tiled kernel for more rows (k_pgring.hip), so
+  // that a row's bits do not depend on how many rows the call has
+  const bool fast_act = epi.dst_dt == ZMI_DT_BF16 && epi.fast_kind != ZMI_EK_GENERIC && epi.fast_kind != ZMI_EK_NONE;
+  if (fast_act) zmi_set_f32_flush();
 #pragma unroll
   for (int j = 0; j < RB; ++j)
 #pragma unroll
@@ -222,6 +226,10 @@ __global__ __launch_bounds__(PG_WAVES * 64) void zmi_gemm_pergroup_kernel(ZmiPro
       if (m >= M) continue;
       const int64_t o = (int64_t)m * p.ldc + col;
       float y = sum[j][q];
+      if (fast_act) {
+        ((uint16_t *)p.dst)[o] = (uint16_t)zmi_pack_bf16(zmi_act_bf16_kind(epi.fast_kind, __fadd_rn(y, bias)), 0.0f);
+        continue;
+      }
       if (epi.alpha != 1.0f) y = __fmul_rn(y, epi.alpha);
       if (epi.beta != 0.0f) y = __fadd_rn(y, __fmul_rn(zmi_ld_f32(p.dst, epi.dst_dt, o), epi.beta));
       zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_tail(epi, y, bias, m, col));
@@ -437,6 +445,13 @@ __global__ __launch_bounds__(PGD_THREADS) void zmi_gemm_decode_pergroup_kernel(Z
   if (!e_live) return;
   const int64_t o = (int64_t)e_row * p.ldc + e_n;
   float y = sum;
+  if (epi.dst_dt == ZMI_DT_BF16 && epi.fast_kind != ZMI_EK_GENERIC && epi.fast_kind != ZMI_EK_NONE) {
+    // (the same form as with more rows, see zmi_gemm_pergroup_kernel)
+    const float b = p.bias ? zmi_ld_f32(p.bias, epi.bias_dt, e_n) : 0.0f;
+    zmi_set_f32_flush();
+    ((uint16_t *)p.dst)[o] = (uint16_t)zmi_pack_bf16(zmi_act_bf16_kind(epi.fast_kind, __fadd_rn(y, b)), 0.0f);
+    return;
+  }
   if (epi.alpha != 1.0f) y = __fmul_rn(y, epi.alpha);
   if (epi.beta != 0.0f) y = __fadd_rn(y, __fmul_rn(zmi_ld_f32(p.dst, epi.dst_dt, o), epi.beta));
   const float bias = p.bias ? zmi_ld_f32(p.bias, epi.bias_dt, e_n) : 0.0f;

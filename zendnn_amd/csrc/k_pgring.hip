@@ -448,8 +448,13 @@ __global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pgring_kernel(ZmiProbl
   const int dst_dt = epi.dst_dt;
   const int es = dst_dt == ZMI_DT_BF16 ? 2 : 4;
   const bool vec_ok = (((uintptr_t)p.dst) % 16 == 0) && ((p.ldc * es) % 16 == 0);
-  const bool plain = epi.n_po == 0 && !epi.has_dst_q && epi.alpha == 1.0f && epi.beta == 0.0f &&
-                     (dst_dt == ZMI_DT_BF16 || dst_dt == ZMI_DT_F32);
+  // straight-line forms: bias (+ one activation in the MFMA-bound kernel's hardware exp / reciprocal form when the
+  // store is bf16: the sums are final, so the wavefront may flush f32 denormals from here on, which makes the
+  // hardware bf16 conversion the reference's) and 8- / 16-byte stores; everything else goes through the interpreter
+  const bool plain = epi.fast_kind != ZMI_EK_GENERIC &&
+                     (dst_dt == ZMI_DT_BF16 || (dst_dt == ZMI_DT_F32 && epi.fast_kind == ZMI_EK_NONE));
+  const int act = epi.fast_kind;
+  if (plain && dst_dt == ZMI_DT_BF16) zmi_set_f32_flush();
   const int nc = n0 + wn * 64 + c16 * 4;           // this lane's four output columns
   float bias[4];
 #pragma unroll
@@ -477,6 +482,10 @@ __global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pgring_kernel(ZmiProbl
         float y[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) y[j] = __fadd_rn(a[j], bias[j]);
+        if (act != ZMI_EK_NONE) {   // (uniform; bf16 stores only)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) y[j] = zmi_act_bf16_kind(act, y[j]);
+        }
         if (vec_ok && nc + 3 < N) {
           if (dst_dt == ZMI_DT_BF16) {
             const v2u v = {zmi_pack_bf16(y[0], y[1]), zmi_pack_bf16(y[2], y[3])};

@@ -487,6 +487,17 @@ __device__ __forceinline__ float zmi_act_bf16(float x) {
   return x;
 }
 
+// A straight-line epilogue kind applied to a finished f32 value that goes to a bf16 store (callers: the kernels
+// whose value is already the scaled sum plus bias, with the wavefront in the flush mode above).
+__device__ __forceinline__ float zmi_act_bf16_kind(int fast_kind, float y) {
+  switch (fast_kind) {
+  case ZMI_EK_SWISH: return zmi_act_bf16<ZMI_EK_SWISH>(y);
+  case ZMI_EK_GELU_TANH: return zmi_act_bf16<ZMI_EK_GELU_TANH>(y);
+  case ZMI_EK_RELU: return zmi_act_bf16<ZMI_EK_RELU>(y);
+  default: return y;
+  }
+}
+
 // Store conversions (reference: store_output,
 // zendnnl/src/operators/matmul/matmul_ref_kernel.cpp:154-254).
 __device__ __forceinline__ void zmi_store(void *dst, int dt, int64_t i, float y) {
