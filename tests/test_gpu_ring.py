@@ -127,10 +127,14 @@ def env():
 
 # 64-row tiles (M <= 64) and 128-row tiles; K not a multiple of the slice count, fewer
 # 64-k stages than slices asked for (K = 100: two stages), several row and column tiles
+# finished by the slice that arrives last at its tile's word, or (without the arrival words) by a reduction launch
+@pytest.mark.parametrize("arrivals", [True, False])
 @pytest.mark.parametrize("slices", [2, 3, 8])
 @pytest.mark.parametrize("M,K,N", [(20, 256, 256), (64, 1000, 700), (100, 100, 300), (129, 512, 256), (300, 640, 515)])
-def test_k_sliced_s32_accumulators_bit_exact(zo, env, M, K, N, slices):
+def test_k_sliced_s32_accumulators_bit_exact(zo, env, M, K, N, slices, arrivals):
     env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=slices)
+    if not arrivals:
+        env(ZMI_NO_SLICE_ARRIVALS=1)
     rng = np.random.default_rng(M + K + N)
     a = rng.integers(0, 256, (M, K), dtype=np.uint8)
     w = H.gen_weights(rng, K, N)
@@ -147,10 +151,13 @@ def test_k_sliced_s32_accumulators_bit_exact(zo, env, M, K, N, slices):
         assert np.array_equal(H.to_host(dst).astype(np.int64), want)
 
 
+@pytest.mark.parametrize("arrivals", [True, False])
 @pytest.mark.parametrize("po", [None, capi.PO_SWISH, capi.PO_GELU_TANH])
 @pytest.mark.parametrize("M,K,N,ldc_pad", [(48, 512, 320, 0), (200, 384, 322, 3)])
-def test_k_sliced_bf16_epilogues(zo, env, po, M, K, N, ldc_pad):
+def test_k_sliced_bf16_epilogues(zo, env, po, M, K, N, ldc_pad, arrivals):
     env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=3)
+    if not arrivals:
+        env(ZMI_NO_SLICE_ARRIVALS=1)
     rng = np.random.default_rng(M + N + (po or 0))
     a = rng.integers(-128, 128, (M, K), dtype=np.int8)
     w = H.gen_weights(rng, K, N)

@@ -374,7 +374,50 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   // ---- K slices: every slice leaves its int32 partial tile in the workspace, in register
   // order (16 bytes per lane and store: whole cache lines), and is done;
   // zmi_ring_reduce_kernel adds the slices of a tile and runs the epilogue on all CUs.
-  if (BM != 256 && n_slice > 1) {   // (256-row tiles are chosen only when they cover the CUs)
+  // With arrival words the slices write their tiles through to device scope (word stores that bypass the caches,
+  // 256 contiguous bytes per instruction), wait for the acknowledgements and count themselves in at the tile's word;
+  // the slice that arrives last reads the others' tiles with loads of the same scope into its own accumulators and
+  // goes on to the epilogue.  No fence (a release fence at device scope writes back the whole L2) and no second
+  // launch: M = 128, K = 4096, N = 14336 in four slices 38.2 -> 36.4 us per call (the last slice's loads are one
+  // compute unit's: 384 KiB at its own rate).
+  if (BM != 256 && n_slice > 1 && split.arrivals) {
+    constexpr int CH = NI * MI * 4;
+    auto words = [&](int s) { return (unsigned int *)split.partial + (((int64_t)id * n_slice + s) * 4 + wave) * (CH * 256) + lane; };
+    unsigned int *mine = words(slice);
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          __hip_atomic_store(mine + ((ni * MI + mi) * 16 + e) * 64, (unsigned int)acc[ni][mi][e], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    zmi_wait_vm<0>();
+    zmi_wg_barrier();
+    int *flag = reinterpret_cast<int *>(smem);   // (the ring is free)
+    if (tid == 0) {
+      const unsigned int before = __hip_atomic_fetch_add(split.arrivals + id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = before == (unsigned int)(n_slice - 1);
+      if (last) __hip_atomic_store(split.arrivals + id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *flag = last ? 1 : 0;
+    }
+    zmi_wg_barrier();
+    const bool last = *flag != 0;
+    zmi_wg_barrier();   // (everybody has read the word before the epilogue reuses the ring)
+    if (!last) return;
+    for (int s = 0; s < n_slice; ++s) {
+      if (s == slice) continue;
+      const unsigned int *theirs = words(s);
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            acc[ni][mi][e] += (int32_t)__hip_atomic_load(theirs + ((ni * MI + mi) * 16 + e) * 64, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else if (BM != 256 && n_slice > 1) {   // (256-row tiles are chosen only when they cover the CUs)
     constexpr int CH = NI * MI * 4;   // 16-byte chunks per lane
     int32_t *mine = split.partial + (((int64_t)id * n_slice + slice) * 4 + wave) * (CH * 256) + lane * 4;
 #pragma unroll
@@ -784,7 +827,7 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
                                 hipStream_t stream, const ZmiRingSide *side) {
   if (p.M <= 0) return hipSuccess;
   const bool gated = epi.gated_act != 0;
-  ZmiRingSplit sp = {1, nullptr};
+  ZmiRingSplit sp = {1, nullptr, nullptr};
   if (split && split->slices > 1) {
     // sliced launches are one launch: the remainder rows stay with the top-height kernel
     if (!(top & ZMI_RING_PAD) || (top & 0xffff) == 256 || !split->partial || gated) return hipErrorInvalidValue;
@@ -815,7 +858,7 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
     if (j == hipSuccess) j = hipStreamWaitEvent(stream, side->join, 0);
     if (e == hipSuccess) e = j;
   }
-  if (e != hipSuccess || sp.slices == 1) return e;
+  if (e != hipSuccess || sp.slices == 1 || sp.arrivals) return e;
   // the slices' partial tiles -> finished elements
   const int th = top & 0xffff;
   const int tiles = th == 128 ? zmi_ring_items<128>(p.M, p.N, top, gated) : zmi_ring_items<64>(p.M, p.N, top, gated);

@@ -515,7 +515,7 @@ hipError_t zmi_launch_gemm_stream_group(const ZmiProblem *probs_host, const ZmiP
   const bool gated = epi.gated_act != 0;
   const int th = top & 0xffff;
   if (!tab_dev || !(top & ZMI_RING_PAD) || (th != 128 && th != 256)) return hipErrorInvalidValue;
-  ZmiRingSplit sp = {1, nullptr};
+  ZmiRingSplit sp = {1, nullptr, nullptr};
   if (split && split->slices > 1) {
     if (gated || !split->partial) return hipErrorInvalidValue;
     sp = *split;

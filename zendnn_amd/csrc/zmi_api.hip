@@ -308,12 +308,13 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
   } else {
     // prob.A is fragment-major here (see use_ring_kernel)
     if (!plan) { set_error("ring GEMM without a launch plan"); return ZMI_FAILURE; }
-    ZmiRingSplit split = {1, nullptr};
+    ZmiRingSplit split = {1, nullptr, nullptr};
     if (plan->slices > 1) {
       // (the scratch arena was sized for the partial tiles by the caller)
       split.slices = plan->slices;
       split.partial = (int32_t *)arena().alloc(plan->partial_bytes);
       if (!split.partial) { set_error("no scratch for the K-sliced GEMM"); return ZMI_FAILURE; }
+      split.arrivals = slice_arrivals(plan->tiles);   // (null: a reduction launch finishes the elements)
     }
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")

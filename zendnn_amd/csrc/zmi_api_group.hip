@@ -317,7 +317,7 @@ int32_t launch_stage(const Stage &st, const char *what) {
     if (!tab) { set_error("scratch exhausted (tile table)"); return ZMI_FAILURE; }
     st.streamed = sp.top != 0;
     if (sp.top) {
-      ZmiRingSplit rs = {1, nullptr};
+      ZmiRingSplit rs = {1, nullptr, nullptr};
       if (sp.slices > 1) {
         const int items = zmi_stream_items(st.probs.data(), n, top, 0, 0, gated);
         rs.slices = sp.slices;
@@ -911,7 +911,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   // idle slots between experts are quantized too (their values are never read back)
   if (!hip_ok(zmi_launch_quant_rows(act, ZMI_DT_BF16, Rp, I, I, A2, kpI, kpI, s2, ZMI_DT_F32, s), "Op2 quant launch")) return ZMI_FAILURE;
   if (stream2) {
-    ZmiRingSplit rs = {1, nullptr};
+    ZmiRingSplit rs = {1, nullptr, nullptr};
     if (sp2.slices > 1) {
       rs.slices = sp2.slices;
       rs.partial = (int32_t *)arena().alloc(zmi_stream_partial_bytes(zmi_stream_items(nullptr, E, top2, R, H, false), sp2.slices, top2));

@@ -71,6 +71,9 @@ int zmi_ring_pick_top_group(int64_t rows, int n_prob, int64_t K, int64_t N, bool
 struct ZmiRingSplit {
   int slices;              // 1: no slicing, the pointer is unused
   int32_t *partial;        // tiles * slices * tile rows * 256 words
+  unsigned int *arrivals;  // null, or a zeroed word per tile (zero again after the launch): the slice that arrives last
+                           // at its tile's word adds the others' partial tiles to its own and finishes the elements,
+                           // and there is no reduction launch
 };
 struct ZmiRingPlan {
   int top;                 // tile height (with ZMI_RING_PAD when slices > 1)
