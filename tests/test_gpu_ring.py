@@ -177,6 +177,35 @@ def test_k_sliced_bf16_epilogues(zo, env, po, M, K, N, ldc_pad, arrivals):
     assert np.all(got[:, N:] == 0)
 
 
+@pytest.mark.parametrize("M,K,N", [(100, 256, 6200), (200, 192, 3300), (256, 320, 3100)])
+def test_unsliced_64_row_tiles_for_a_wide_problem_with_few_rows(zo, env, M, K, N):
+    """65 .. 256 rows against many weight columns and a short K: the launch plan takes 64-row tiles, unsliced (a
+    partly filled last tile included).  Raw s32 sums against the integer product, bf16 + SiLU against the oracle."""
+    env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17)
+    rng = np.random.default_rng(M + K + N)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    want = a.astype(np.int64) @ w.astype(np.int64)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_S32)
+    dst = torch.zeros((M, N), dtype=torch.int32, device=H.DEV)
+    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, H.to_dev(a), K, H.to_dev(w), N, None, 0.0, dst, N, False, p)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    assert lowoha.last_kernel() == "ring_mfma32x32x32_top64"
+    assert np.array_equal(H.to_host(dst).astype(np.int64), want)
+    ss = rng.uniform(0.01, 0.03, M).astype(np.float32)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    ss_d, ws_d = H.to_dev(ss), H.to_dev(ws)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+    p.weight_cache_type = 0
+    got, want = _run_both(zo, p, a, w, M, N, K, bias=bias, host_bufs={"src_scale": ss, "wei_scale": ws})
+    assert lowoha.last_kernel() == "ring_mfma32x32x32_top64"
+    H.check_bf16(got, want, max_frac=5e-3)
+
+
 @pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_S8, capi.DT_U8])
 def test_k_sliced_f32_exact_and_quantized_destinations(zo, env, dst_dt):
     env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=4)
@@ -205,11 +234,11 @@ def test_k_sliced_f32_exact_and_quantized_destinations(zo, env, dst_dt):
 
 
 def test_k_slices_chosen_for_a_problem_with_few_tiles(zo):
-    """M = 192, N = 4096, K = 4096 (32 tiles): the launch plan slices K without being told to,
+    """M = 192, N = 2048, K = 4096 (16 tiles): the launch plan slices K without being told to,
     and the dynamic-quantization call agrees with the oracle."""
     from tests.test_gpu_matmul import _oracle
     rng = np.random.default_rng(5)
-    M, K, N = 192, 4096, 4096
+    M, K, N = 192, 4096, 2048
     x = H.gen_bf16_normal(rng, (M, K))
     w = H.gen_weights(rng, K, N)
     ws = rng.uniform(0.001, 0.01, N).astype(np.float32)

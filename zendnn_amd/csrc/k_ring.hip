@@ -792,9 +792,25 @@ ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices) {
   plan.slices = 1;
   plan.partial_bytes = 0;
   const int64_t tiles_n = (N + 255) / 256;
-  plan.tiles = (int)(((M + plan.top - 1) / plan.top) * tiles_n);
+  plan.tiles = (int)(((M + (plan.top & 0xffff) - 1) / (plan.top & 0xffff)) * tiles_n);
   if (M <= 0) return plan;
   const int n_cu = zmi_cu_count();
+  if ((plan.top & 0xffff) == 64 && force_slices <= 0) return plan;
+  // 65 .. 256 rows or so against a wide weight matrix: 64-row tiles, unsliced, while they fit the CUs at once.  A
+  // workgroup's weight stream runs at what one compute unit keeps in flight (about 60 GB/s), so the call is as long
+  // as one tile's stream (256 columns x K) whatever the tile height: more, lower tiles put more CUs to work without
+  // the partial tiles of the K slices (their int32 traffic is half the weights' at 128 rows).  Measured, us per
+  // call, this / before: K = 4096, N = 14336: 96 rows 31.5 / 36.7, 256 rows 34.2 / 38.7; K = 2048, N = 11008:
+  // 128 rows 20.6 / 28.2; K = 4096, N = 4096: 256 rows 28.9 / 32.1.  Long K (8192 and more) and two rounds of tiles
+  // (384 rows at N = 14336: 48.5 / 41.7) stay with the sliced and the 128-row forms.
+  if (!top_hint && force_slices <= 0 && M > 64) {
+    const int64_t t64 = ((M + 63) / 64) * tiles_n;
+    if (t64 >= 48 && t64 <= n_cu && zmi_blob_kpad(K) <= 6144) {
+      plan.top = 64 | ZMI_RING_PAD;
+      plan.tiles = (int)t64;
+      return plan;
+    }
+  }
   const int nk = (int)(zmi_blob_kpad(K) / 64);
   const int top = M <= 64 ? 64 : 128;
   const int64_t tiles = ((M + top - 1) / top) * tiles_n;

@@ -285,6 +285,7 @@ ZmiRingPlan plan_ring_gemm(int M, int N, int K) {
   if (const char *env = std::getenv("ZMI_GEMM_TOP")) {
     const int v = std::atoi(env);
     if (v == 128 || v == 256) top_hint = v;
+    if (v == 64) top_hint = 64 | 0x10000;   // (ZMI_RING_PAD)
   }
   if (const char *env = std::getenv("ZMI_RING_SPLITK")) force = std::atoi(env);
   return zmi_ring_plan(M, N, K, top_hint, force);
@@ -318,7 +319,8 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
     }
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")
-                                     : (th == 256 ? "ring_mfma32x32x32_top256" : "ring_mfma32x32x32_top128"));
+                                     : (th == 256 ? "ring_mfma32x32x32_top256"
+                                                  : th == 64 ? "ring_mfma32x32x32_top64" : "ring_mfma32x32x32_top128"));
     const ZmiRingSide side = side_stream();
     if (!hip_ok(zmi_launch_gemm_ring(prob, epi, plan->top, &split, stream(), &side), "MFMA GEMM launch")) return ZMI_FAILURE;
   }
