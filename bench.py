@@ -229,10 +229,10 @@ def main():
         value = decode_bytes(M) / (ms * 1e-3) / 1e9
         ms_k = ev_time(kernel_only, args.steps, args.warmup)
         gemm_kernel = lowoha.last_kernel()
-        # One step is ONE launch: the decode kernel with the per-token quantization fused in (its
-        # first M workgroups quantize, the rest stream the weights).  The timed region above is
-        # therefore already "that kernel launched back to back between two events on its stream".
-        fused = "fused" in step_kernel
+        # One step is ONE launch: the decode kernel with the per-token quantization inside it (by the
+        # workgroups that use the rows, or by quantizing workgroups at the head of the grid).  The timed region
+        # above is therefore already "that kernel launched back to back between two events on its stream".
+        fused = "fused" in step_kernel or "selfquant" in step_kernel
         achieved = value if fused else None
         # the same kernel on rows that are already s8 (no quantization part), for comparison
         kbytes = K_DEC * N_DEC + M * K_DEC + M * 4 + N_DEC * 4 + M * N_DEC * 2
@@ -256,7 +256,8 @@ def main():
             "config": {"workload": "matmul_direct decode: M=16 K=4096 N=14336, bf16 -> per-token s8, "
                                    "prepacked s8 weights, per-channel scales, SiLU, bf16 out",
                        "weight_sets_rotated": n_sets, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1)},
-            "roofline": {"bound": "hbm", "kernel": "zmi_gemm_decode16_kernel: " + (step_kernel if fused else gemm_kernel),
+            "roofline": {"bound": "hbm", "kernel": ("zmi_gemm_decode16_selfq_kernel: " if "selfquant" in step_kernel and fused
+                                                      else "zmi_gemm_decode16_kernel: ") + (step_kernel if fused else gemm_kernel),
                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": DECODE_TRAFFIC_BYTES,
                          "algorithmic_bytes_per_launch": decode_bytes(M) if fused else kbytes,

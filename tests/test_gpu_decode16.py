@@ -123,12 +123,20 @@ def _fused_call(M, K, N, rng):
     return x, w, ws, p, dst, call, keep
 
 
+FUSED_NAMES = {
+    "selfq": "decode16x2_selfquant_mfma16x16x64 (per-token quant in the workgroup)",
+    "handoff16": "decode16_dma_rows_mfma16x16x64 (fused per-token quant)",
+    "rowgroup": "decode_lds_rows_mfma16x16x64 (fused per-token quant)",
+}
+
+
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
-@pytest.mark.parametrize("K,N", [(4096, 14336), (4096, 1000), (1000, 333), (64, 32), (24, 70), (2048, 4096)])
-def test_fused_quantization_on_the_16_row_kernel_bit_exact(zo, M, K, N, monkeypatch):
-    """bf16 rows quantized per token inside the launch of the 16-row kernel (the wait for the rows goes through the
-    scalar unit): bit-identical to the oracle on repeated calls (a fresh launch number each), and to the row-group
-    kernel's form of the same call."""
+@pytest.mark.parametrize("K,N", [(4096, 14336), (4096, 1000), (1000, 333), (64, 32), (24, 70), (2048, 4096), (4096, 2080)])
+def test_fused_quantization_three_forms_bit_exact(zo, M, K, N, monkeypatch):
+    """bf16 rows quantized per token inside the decode launch, in its three forms: by the workgroups that use the
+    rows (16 wavefronts, two column blocks; odd block counts included), by quantizing workgroups whose rows the
+    16-row kernel waits for through the scalar unit, and the row-group kernel's hand-off.  Each bit-identical to the
+    oracle on repeated calls; rows with NaN / infinite elements (they count as zero) give the same bits in all three."""
     rng = np.random.default_rng(M * 100 + K + N)
     x, w, ws, p, dst, call, keep = _fused_call(M, K, N, rng)
     ph = H.host_params(p, src_scale=None, wei_scale=ws)
@@ -136,16 +144,46 @@ def test_fused_quantization_on_the_16_row_kernel_bit_exact(zo, M, K, N, monkeypa
     hk = []
     st, want, _, _ = zo.matmul_int8(x, w, ph.flat(hk), M, N, K)
     assert st == capi.SUCCESS
-    for rep in range(3):
-        dst.fill_(12345.0)
+    xbad = x.copy()
+    xbad[0, 0] = 0x7f80          # +inf
+    xbad[M - 1, K - 1] = 0xffc0  # NaN
+    xbad[M // 2, K // 2] = 0xff80  # -inf
+    xbad_d = H.to_dev(xbad)
+    bad = []
+    for mode in ("selfq", "handoff16", "rowgroup"):
+        monkeypatch.delenv("ZMI_NO_DECODE_SELFQ", raising=False)
+        monkeypatch.delenv("ZMI_DECODE_ROWGROUP_KERNEL", raising=False)
+        monkeypatch.setenv("ZMI_DECODE_SELFQ_MIN_WGS", "1")
+        monkeypatch.setenv("ZMI_DECODE_SELFQ_MAX_M", "16")
+        if mode != "selfq":
+            monkeypatch.setenv("ZMI_NO_DECODE_SELFQ", "1")
+        if mode == "rowgroup":
+            monkeypatch.setenv("ZMI_DECODE_ROWGROUP_KERNEL", "1")
+        for rep in range(2):
+            dst.fill_(12345.0)
+            assert call() == capi.SUCCESS, lowoha.last_error()
+            assert lowoha.last_kernel() == FUSED_NAMES[mode]
+            assert np.array_equal(H.to_host(dst), want), (mode, rep)
+        d2 = torch.full((M, N), 12345.0, dtype=torch.float32, device=H.DEV)
+        st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, xbad_d, K, keep["blob"], N, None, 0.0, d2, N, True, p)
+        assert st == capi.SUCCESS, lowoha.last_error()
+        bad.append(H.to_host(d2))
+    assert np.array_equal(bad[0], bad[1]) and np.array_equal(bad[1], bad[2])
+    assert np.all(np.isfinite(bad[0]))
+
+
+def test_fused_quantization_default_form_by_width(zo, monkeypatch):
+    """Which form a call takes by itself: up to 12 rows and an output wide enough for 64 two-block workgroups (at
+    most one per compute unit) quantize in the workgroups, the others keep the hand-off."""
+    monkeypatch.delenv("ZMI_DECODE_SELFQ_MIN_WGS", raising=False)
+    monkeypatch.delenv("ZMI_DECODE_SELFQ_MAX_M", raising=False)
+    rng = np.random.default_rng(3)
+    for M, N, mode in ((8, 14336, "selfq"), (12, 4096, "selfq"), (13, 14336, "handoff16"), (16, 14336, "handoff16"),
+                       (4, 2048, "handoff16"), (1, 20480, "handoff16")):
+        x, w, ws, p, dst, call, keep = _fused_call(M, 512, N, rng)
         assert call() == capi.SUCCESS, lowoha.last_error()
-        assert lowoha.last_kernel() == "decode16_dma_rows_mfma16x16x64 (fused per-token quant)"
-        assert np.array_equal(H.to_host(dst), want), rep
-    monkeypatch.setenv("ZMI_DECODE_ROWGROUP_KERNEL", "1")
-    dst.fill_(12345.0)
-    assert call() == capi.SUCCESS, lowoha.last_error()
-    assert lowoha.last_kernel() == "decode_lds_rows_mfma16x16x64 (fused per-token quant)"
-    assert np.array_equal(H.to_host(dst), want)
+        assert lowoha.last_kernel() == FUSED_NAMES[mode], N
+        capi.load().zmi_clear_weight_cache()
 
 
 @pytest.mark.parametrize("M", [1, 7, 16])

@@ -463,6 +463,237 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   zmi_finish_element(p, epi, cc0, zmi_row_scale_from_raw(epi, p, rs_word, m_ok), s, e_row, e_n);
 }
 
+// ---------------------------------------------------------------------------------------
+// Up to 16 bf16 rows, quantized per token by the workgroups that use them: no second kind of workgroup, nothing
+// handed from one workgroup to another, no wait.  A workgroup of 16 wavefronts owns TWO column blocks (wavefronts
+// 0 .. 7 the even one, 8 .. 15 the odd one, each streaming an eighth of K of its block as in the 16-row kernel) and
+// one copy of the rows in LDS: wavefront r requests bf16 row r first (it is there long before the weights), then all
+// its weights, then the constants; while the weights are on their way it takes the row's absolute maximum (a
+// wavefront reduction: a row is a wavefront's), quantizes the row with the arithmetic of k_quant.hip and writes the
+// s8 bytes into LDS in the order the 16-row kernel's global->LDS loads leave them.  One barrier, then every wavefront
+// multiplies its slice.  A compute unit holds one such workgroup: its 16 rows are fetched and quantized once per
+// compute unit (half the row traffic of two 8-wavefront workgroups), about 450 VALU instructions per wavefront, all
+// of them under the weight stream.  The scales go to the caller's buffer from workgroup 0 and to the epilogue
+// through LDS.  (Measured times: at zmi_decode_selfq_takes.)
+#define DQ_WAVES 16
+#ifndef DQ_LATE
+#define DQ_LATE 2
+#endif
+#define DQ_THREADS (DQ_WAVES * 64)
+__global__ __launch_bounds__(DQ_THREADS, 1) void zmi_gemm_decode16_selfq_kernel(ZmiProblem p, ZmiEpilogue epi, ZmiFusedQuant fq,
+                                                                              int n_blk) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int half = wave / DEC_WAVES, w8 = wave % DEC_WAVES;
+  const int M = p.M, N = p.N, K = p.K;
+  const int K_pad = (int)zmi_blob_kpad(K);
+  const int nchunks = K_pad / 64;
+  const int blk_raw = (int)blockIdx.x * 2 + half;
+  const bool blk_live = blk_raw < n_blk;
+  const int blk = blk_live ? blk_raw : n_blk - 1;   // (an odd block count: the last workgroup's second half repeats a block, stores nothing)
+  const int rows_bytes = nchunks * 1024;
+  // LDS: the s8 rows (reused by the partial tiles) | DQ_LATE chunks of weights per wavefront | a scale per row
+  const int wl_off = rows_bytes > 2 * DEC_RED_BYTES ? rows_bytes : 2 * DEC_RED_BYTES;
+  float *rs_lds = reinterpret_cast<float *>(lds + wl_off + DQ_WAVES * DQ_LATE * 2048);
+
+  // ---- requests, in this order (a wavefront's loads return in order, so the wait below can count): the column
+  // constants of this thread's output element as raw words (4 loads, nothing waits for them early), this
+  // wavefront's bf16 row (8 loads of a KiB), its weights (4 global->LDS requests, 12 loads into registers) ----
+  const int t2 = tid % DEC_THREADS;
+  const int e_row = t2 / 32, e_col = t2 % 32;
+  const int e_n = blk * 32 + e_col;
+  const int32_t *colsum = (const int32_t *)(p.blob + zmi_blob_colsum_off());
+  const int n_ok = e_n < N ? e_n : N - 1;
+  const ZmiColRaw craw = zmi_col_raw(epi, p, colsum, n_ok);
+  const int32_t zp_word = zmi_zp_raw(p, colsum);
+  const int c_begin = w8 * nchunks / DEC_WAVES;
+  const int c_end = (w8 + 1) * nchunks / DEC_WAVES;
+  const int c16 = lane % 16, g = lane / 16;
+  const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
+  // The row comes FIRST in the wavefront's queue (loads return in order: behind a weight request it would arrive with
+  // the weights, microseconds later on the compute units memory serves last) and by loads the compiler does not
+  // count (inline assembly; the wait below is explicit and hands the registers on), so that the global->LDS
+  // requests behind them do not turn the compiler's own waits for the row into waits for weights.
+  asm volatile("" ::: "memory");
+  const int NG = K / 8;                       // granules of 8 bf16 per row
+  const bool row_live = wave < M;
+  const uint16_t *xrow = (const uint16_t *)fq.x + (size_t)(row_live ? wave : 0) * fq.ldx;
+  v4i xr[8];
+  // (rows are 8 KiB apart and every workgroup wants the same ones at the same moment: each wavefront starts at a
+  // different KiB of its row, or the requests of the whole device meet in one L2 channel after the other)
+  const int rot = (wave + (int)blockIdx.x) & 7;
+  #pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int gi = lane + 64 * ((i + rot) & 7);
+    const uint32_t voff = (uint32_t)(gi < NG ? gi : NG - 1) * 16u;   // (past the row's end: its last granule, not written below)
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(xr[i]) : "v"(voff), "s"(xrow) : "memory");
+  }
+  asm volatile("" ::: "memory");
+  const uint8_t *wbase = tiles + (int64_t)blk * zmi_blob_nb_stride(K);
+  const uint32_t wlane = (uint32_t)((g / 2) * 1024 + ((g % 2) * 32 + c16) * 16);
+  #pragma unroll
+  for (int u = 8 - DQ_LATE; u < 8; ++u) {
+    const int c = c_begin + u < c_end ? c_begin + u : c_begin;
+    #pragma unroll
+    for (int h = 0; h < 2; ++h)
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   ::"s"(wl_off + (wave * DQ_LATE + (u - (8 - DQ_LATE))) * 2048 + h * 1024),
+                     "v"(wlane + (uint32_t)c * 2048u + (uint32_t)h * 256u), "s"(wbase)
+                   : "memory", "m0");
+  }
+  asm volatile("" ::: "memory");
+  const uint8_t *bsrc[2];
+  #pragma unroll
+  for (int h = 0; h < 2; ++h)
+    bsrc[h] = tiles + (int64_t)blk * zmi_blob_nb_stride(K) + (g / 2) * 1024 + ((g % 2) * 32 + h * 16 + c16) * 16;
+  // (128 registers per lane at 16 wavefronts: the row's 32 and 48 of weights; the last DQ_LATE chunks of the slice
+  // land in LDS instead, global->LDS loads in the lanes' own order, and are read back as MFMA operands)
+  v4i b[8 - DQ_LATE][2];
+  #pragma unroll
+  for (int u = 0; u < 8 - DQ_LATE; ++u) {
+    const int c = c_begin + u < c_end ? c_begin + u : c_begin;   // (past the slice: a valid chunk, result unused)
+    b[u][0] = __builtin_nontemporal_load((const v4i *)(bsrc[0] + (int64_t)c * 2048));
+    b[u][1] = __builtin_nontemporal_load((const v4i *)(bsrc[1] + (int64_t)c * 2048));
+  }
+
+  // (behind the row: the 2 * DQ_LATE global->LDS requests and the 2 * (8 - DQ_LATE) register loads = 16)
+  asm volatile("s_waitcnt vmcnt(16)"
+               : "+v"(xr[0]), "+v"(xr[1]), "+v"(xr[2]), "+v"(xr[3]), "+v"(xr[4]), "+v"(xr[5]), "+v"(xr[6]), "+v"(xr[7])
+               :: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+  // maximum of the absolute values: the 15-bit patterns of |bf16| order like the values, so a packed 16-bit maximum
+  // over the raw words does two elements per instruction; a result in the NaN / infinity range means the row holds
+  // non-finite elements, which count as zero (in the maximum and below): they are zeroed in the registers, rarely
+  typedef unsigned short dq_u16x2 __attribute__((ext_vector_type(2)));
+  auto row_max = [&]() {
+    dq_u16x2 m = {0, 0};
+    #pragma unroll
+    for (int i = 0; i < 8; ++i)
+      #pragma unroll
+      for (int j = 0; j < 4; ++j)
+        m = __builtin_elementwise_max(m, __builtin_bit_cast(dq_u16x2, (uint32_t)xr[i][j] & 0x7fff7fffu));
+    uint32_t v = m[0] > m[1] ? m[0] : m[1];
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t t = (uint32_t)__shfl_xor((int)v, o);
+      v = t > v ? t : v;
+    }
+    return v;
+  };
+  uint32_t mbits = row_max();
+  if (mbits >= 0x7f80u) {   // (uniform)
+    #pragma unroll
+    for (int i = 0; i < 8; ++i)
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t raw = (uint32_t)xr[i][j];
+        if ((raw & 0x7f80u) == 0x7f80u) raw &= 0xffff0000u;
+        if ((raw & 0x7f800000u) == 0x7f800000u) raw &= 0x0000ffffu;
+        xr[i][j] = (int)raw;
+      }
+    mbits = row_max();
+  }
+  float amax = __uint_as_float(mbits << 16);
+  if (amax < 1e-10f) amax = 1e-10f;
+  float sc = __fdiv_rn(amax, 127.0f);
+  if (sc < 1e-10f) sc = 1e-10f;
+  const float inv = __fdiv_rn(1.0f, sc);
+  if (lane == 0 && row_live) {
+    rs_lds[wave] = zmi_fused_scale_as_stored(fq, sc);
+    if (blockIdx.x == 0) {
+      fq.scales[wave] = zmi_fused_scale_as_stored(fq, sc);
+      if (fq.user_scales) {
+        if (fq.user_dt == ZMI_DT_BF16) ((uint16_t *)fq.user_scales)[wave] = zmi_f32_to_bf16_rne(sc);
+        else ((float *)fq.user_scales)[wave] = sc;
+      }
+    }
+  }
+  // the s8 bytes: x * (1 / scale) rounded, and the exact quotient for the elements whose product lies within 1e-4
+  // of a half-integer (the arithmetic of zmi_quant_elem: one in a thousand, looked for once per eight elements)
+#ifdef DQ_SKIPQ
+  if (row_live && inv == 12345.0f) {
+#else
+  if (row_live) {
+#endif
+    const int r = wave;
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int gi = lane + 64 * ((i + rot) & 7);
+      uint32_t w2[2];
+      #pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {   // (four elements at a time: the temporaries of eight do not fit the registers)
+        float x[4], t[4], q[4];
+        bool redo = false;
+        #pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          x[2 * j] = __uint_as_float(((uint32_t)xr[i][hh * 2 + j]) << 16);
+          x[2 * j + 1] = __uint_as_float(((uint32_t)xr[i][hh * 2 + j]) & 0xffff0000u);
+        }
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          t[e] = __fmul_rn(x[e], inv);
+          q[e] = rintf(t[e]);
+          redo |= fabsf(t[e] - q[e]) > 0.4999f;
+        }
+        if (__builtin_expect(redo, 0)) {
+          #pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (fabsf(t[e] - q[e]) > 0.4999f) q[e] = rintf(__fdiv_rn(x[e], sc));
+        }
+        w2[hh] = ((uint32_t)(int32_t)q[0] & 0xffu) | (((uint32_t)(int32_t)q[1] & 0xffu) << 8) |
+                 (((uint32_t)(int32_t)q[2] & 0xffu) << 16) | ((uint32_t)(int32_t)q[3] << 24);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // granule gi = 8 k: chunk gi / 8, 16-byte k group (gi % 8) / 2, its half gi % 2
+      const int c = gi >> 3, kg = (gi & 7) >> 1;
+      if (gi < NG) *(v2u *)(lds + c * 1024 + (r * 4 + (kg ^ ((r >> 2) & 3))) * 16 + (gi & 1) * 8) = (v2u){w2[0], w2[1]};
+      __builtin_amdgcn_sched_barrier(0);   // (one granule at a time: interleaved, their temporaries do not fit the registers)
+    }
+  }
+  // (k past K inside the last written chunks and rows past M: whatever LDS holds meets zero weights or rows that are not stored)
+  zmi_lds_barrier();   // (long before the weights are there: every wavefront then waits for its own only)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  v4i acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  #pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const bool live = c_begin + u < c_end;
+    const int c = live ? c_begin + u : c_begin;
+    v4i a = *(const v4i *)(lds + c * 1024 + (c16 * 4 + (g ^ ((c16 >> 2) & 3))) * 16);
+    if (!live) a = (v4i){0, 0, 0, 0};
+    v4i b0, b1;
+    if (u < 8 - DQ_LATE) {
+      b0 = b[u][0];
+      b1 = b[u][1];
+    } else {
+      const uint8_t *wl = lds + wl_off + (wave * DQ_LATE + (u - (8 - DQ_LATE))) * 2048 + lane * 16;
+      b0 = *(const v4i *)wl;
+      b1 = *(const v4i *)(wl + 1024);
+    }
+    acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b0, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b1, acc[1], 0, 0, 0);
+  }
+
+  // ---- cross-wavefront reduction through LDS (reuses the operand area; one 16 KiB area per half) ----
+  const float rs = rs_lds[e_row < M ? e_row : 0];
+  zmi_lds_barrier();
+  int32_t *red = (int32_t *)lds + half * (DEC_RED_BYTES / 4);
+  #pragma unroll
+  for (int h = 0; h < 2; ++h)
+    #pragma unroll
+    for (int q = 0; q < 4; ++q) red[w8 * 512 + (h * 4 + q) * 64 + lane] = acc[h][q];
+  zmi_lds_barrier();
+  if (!(blk_live && e_n < N && e_row < M)) return;
+  const int off = ((e_col / 16) * 4 + e_row % 4) * 64 + (e_row / 4) * 16 + e_col % 16;
+  int32_t s = 0;
+  #pragma unroll
+  for (int w = 0; w < DEC_WAVES; ++w) s += red[w * 512 + off];
+  const ZmiColCtx cc0 = zmi_col_ctx_raw(epi, p, craw, zp_word, e_n, n_ok, N);
+  zmi_finish_element(p, epi, cc0, rs, s, e_row, e_n);
+}
+
+
 __global__ __launch_bounds__(256) void zmi_decode16_reduce_kernel(ZmiProblem p, ZmiEpilogue epi, int n_slices,
                                                                  const int32_t *partial) {
   const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -499,6 +730,26 @@ bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant) {
   return p.M <= 16 && (int64_t)p.lda * 16 < ((int64_t)1 << 31) && !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
 }
 
+// bf16 rows quantized by the workgroups that use them (zmi_gemm_decode16_selfq_kernel): rows of whole 16-byte
+// granules, K up to 4096, and a block count whose workgroups (two blocks each, one per compute unit) are all resident.
+// Up to 12 rows: every compute unit quantizes all the rows (about 75 VALU instructions per 8 elements, 4 cycles
+// each), and with a wavefront per row the work of 13 .. 16 rows is four wavefronts deep on every SIMD and no longer
+// hides under the weight stream.  Measured, us per call (bf16 rows, K = 4096, rotating weights), this form / the
+// hand-off through the scalar unit: N = 14336: 1 row 12.06 / 12.60, 4 rows 12.09 / 12.86, 8 rows 12.71 / 13.26,
+// 12 rows 13.34 / 14.02, 16 rows 15.27 / 14.58; N = 11008: 1 row 10.36 / 11.72, 8 rows 10.63 / 12.23, 16 rows
+// 13.60 / 13.57; N = 4096: 1 row 8.97 / 9.25, 16 rows 11.87 / 9.15.
+// ZMI_NO_DECODE_SELFQ, ZMI_DECODE_SELFQ_MAX_M, ZMI_DECODE_SELFQ_MIN_WGS: the tests reach every form through them.
+bool zmi_decode_selfq_takes(const ZmiProblem &p, const ZmiFusedQuant *fq) {
+  if (!fq || !fq->x || fq->x_dt != ZMI_DT_BF16 || p.M > 16 || p.a_is_u8 || !zmi_decode_kernel_fits(p)) return false;
+  if (p.K % 8 != 0 || ((uintptr_t)fq->x % 16) != 0 || (fq->ldx * 2) % 16 != 0) return false;
+  const int wgs = (zmi_decode_grid(p) + 1) / 2;
+  int min_wgs = 64, max_m = 12;
+  if (const char *e = getenv("ZMI_DECODE_SELFQ_MIN_WGS")) min_wgs = atoi(e);
+  if (const char *e = getenv("ZMI_DECODE_SELFQ_MAX_M")) max_m = atoi(e);
+  return p.M <= max_m && wgs <= zmi_cu_count() && wgs >= min_wgs && !getenv("ZMI_NO_DECODE_SELFQ") &&
+         !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
+}
+
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
                                   hipStream_t stream, int32_t *partial, unsigned int *arrivals) {
   if (epi.gated_act != 0) return hipErrorInvalidValue;   // gated GEMMs are grouped launches: the large-M kernel
@@ -523,6 +774,15 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
   }
   if (n_blk <= 0) return hipSuccess;
   ZmiFusedQuant none = {};
+  if (zmi_decode_selfq_takes(p, fq)) {
+    // (the s8 rows, reused by the two halves' partial tiles, and a scale per row)
+    const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
+    const size_t smem = (op > 2 * DEC_RED_BYTES ? op : 2 * DEC_RED_BYTES) + DQ_WAVES * DQ_LATE * 2048 + 64;
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_selfq_kernel, 4096 * 16 + DQ_WAVES * DQ_LATE * 2048 + 64);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(zmi_gemm_decode16_selfq_kernel, dim3((n_blk + 1) / 2), dim3(DQ_THREADS), smem, stream, p, epi, *fq, n_blk);
+    return hipGetLastError();
+  }
   if (zmi_decode_16row_kernel(p, fq != nullptr)) {
     // (the operand area, reused by the partial tiles, and with the quantization in the launch a word per wavefront)
     const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;

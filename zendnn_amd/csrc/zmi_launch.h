@@ -191,6 +191,9 @@ size_t zmi_decode16_partial_bytes(int M, int N, int64_t K);
 int zmi_decode_grid(const ZmiProblem &p);
 // true when the launch above takes the 16-row kernel (rows fetched by global->LDS loads behind the first weights)
 bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant);
+struct ZmiFusedQuant;
+// true when a launch with these rows quantizes them inside the workgroups that use them (no hand-off)
+bool zmi_decode_selfq_takes(const ZmiProblem &p, const ZmiFusedQuant *fq);
 
 // k_moe.hip
 struct ZmiActMat {
