@@ -623,6 +623,9 @@ __global__ __launch_bounds__(DQ_THREADS, 1) void zmi_gemm_decode16_selfq_kernel(
       uint32_t w2[2];
       #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {   // (four elements at a time: the temporaries of eight do not fit the registers)
+        // q + 128 as a float: x * (1 / scale) + 128 in one fused step, rounded.  That differs from x / scale + 128 by
+        // less than 5e-5 (the product's 3.8e-5 and half a unit in the last place at 256), so away from the
+        // half-integers the rounded value IS rint(x / scale) + 128, and within 1e-4 of one the exact quotient decides
         float x[4], t[4], q[4];
         bool redo = false;
         #pragma unroll
@@ -632,17 +635,21 @@ __global__ __launch_bounds__(DQ_THREADS, 1) void zmi_gemm_decode16_selfq_kernel(
         }
         #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          t[e] = __fmul_rn(x[e], inv);
+          t[e] = __builtin_fmaf(x[e], inv, 128.0f);
           q[e] = rintf(t[e]);
           redo |= fabsf(t[e] - q[e]) > 0.4999f;
         }
         if (__builtin_expect(redo, 0)) {
           #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (fabsf(t[e] - q[e]) > 0.4999f) q[e] = rintf(__fdiv_rn(x[e], sc));
+            if (fabsf(t[e] - q[e]) > 0.4999f) q[e] = __fadd_rn(rintf(__fdiv_rn(x[e], sc)), 128.0f);
         }
-        w2[hh] = ((uint32_t)(int32_t)q[0] & 0xffu) | (((uint32_t)(int32_t)q[1] & 0xffu) << 8) |
-                 (((uint32_t)(int32_t)q[2] & 0xffu) << 16) | ((uint32_t)(int32_t)q[3] << 24);
+        // (the hardware's float -> byte conversion inserts the byte; the values are whole numbers in 1 .. 255)
+        uint32_t w = __builtin_amdgcn_cvt_pk_u8_f32(q[0], 0, 0);
+        w = __builtin_amdgcn_cvt_pk_u8_f32(q[1], 1, w);
+        w = __builtin_amdgcn_cvt_pk_u8_f32(q[2], 2, w);
+        w = __builtin_amdgcn_cvt_pk_u8_f32(q[3], 3, w);
+        w2[hh] = w ^ 0x80808080u;
         __builtin_amdgcn_sched_barrier(0);
       }
       // granule gi = 8 k: chunk gi / 8, 16-byte k group (gi % 8) / 2, its half gi % 2
