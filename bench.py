@@ -282,10 +282,11 @@ def main():
     def run_decode_m(m):
         s_, k_, kp_ = decode_setup(m, n_sets)
         t = ev_time(s_, 100, 10)
+        step_name = lowoha.last_kernel()
         tk = ev_time(k_, 100, 10)
         return {"GBps": round(decode_bytes(m) / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2),
                 "gemm_only_GBps": round((K_DEC * N_DEC + m * K_DEC + m * 4 + N_DEC * 4 + m * N_DEC * 2) / (tk * 1e-3) / 1e9, 1),
-                "kernel": lowoha.last_kernel()}
+                "kernel": step_name, "gemm_only_kernel": lowoha.last_kernel()}
 
     def run_decode_per_group(m, gs):
         # the decode call with per-group scales: {M,G} source scales computed by the library, {G,N} weight scales,
