@@ -611,11 +611,7 @@ __global__ __launch_bounds__(DQ_THREADS, 1) void zmi_gemm_decode16_selfq_kernel(
   }
   // the s8 bytes: x * (1 / scale) rounded, and the exact quotient for the elements whose product lies within 1e-4
   // of a half-integer (the arithmetic of zmi_quant_elem: one in a thousand, looked for once per eight elements)
-#ifdef DQ_SKIPQ
-  if (row_live && inv == 12345.0f) {
-#else
   if (row_live) {
-#endif
     const int r = wave;
     #pragma unroll
     for (int i = 0; i < 8; ++i) {
