@@ -116,6 +116,8 @@ typedef struct zmi_matmul_params_t {
   int32_t n_postops;
   const zmi_post_op_t *postops;
   zmi_quant_t src_scale, wei_scale, dst_scale, src_zp, wei_zp, dst_zp;
+                              /* wei_zp: one zero-point for the weight tensor (s8 / u8 / s32, host or device), single
+                               * problems with s8 / u8 sources (aocl_kernel.cpp:982-985, lru_cache/lowoha_cache.hpp:151-232) */
   char mem_format_a;          /* 'n' */
   char mem_format_b;          /* 'n' plain weights, 'r' blob from zmi_reorder_direct */
   int32_t lowoha_algo;        /* enum zmi_matmul_algo */

@@ -22,7 +22,8 @@
  *                                ties-to-even), |q|<=127, max|q|==127
  *   zo_gemm_s32                  int64 brute force, all-ones closed form, the
  *                                reference example's deterministic recipe
- *   zp compensation              integer identity sum((a-zp)w) == sum(aw)-zp*sum(w)
+ *   zp compensation              integer identity sum((a-zp)w) == sum(aw)-zp*sum(w); with a weight zero-point the
+ *                                product of the shifted operands in Python integers (u8 / s8, transposed A)
  *   dequant chain / bias         special cases (unit scales, equal per-channel
  *                                scales == per-tensor), op order from source
  *   post-ops                     libm double evaluation within 2 f32 ulp
@@ -677,6 +678,23 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
     comp = (int32_t *)malloc(sizeof(int32_t) * (size_t)N);
     zo_zp_comp((const int8_t *)weight, transB, ldb, K, N, src_zp, comp);
   }
+  /* a weight zero-point (per tensor): the 2-D compensation of cache_or_compute_zp_compensation,
+   * lowoha_operators/matmul/lru_cache/lowoha_cache.hpp:151-232:
+   * comp[m,n] = -src_zp * colsum[n] - wei_zp * rowsum[m] + src_zp * wei_zp * K, rowsum over the source as given
+   * (u8 or s8); its column term is `comp` above, the rest is one int32 per row */
+  int32_t wei_zp = p->wei_zp.buff ? zo_read_s32(p->wei_zp.buff, p->wei_zp.dt, 0) : 0;
+  int32_t *rowc = NULL;
+  if (wei_zp) {
+    rowc = (int32_t *)malloc(sizeof(int32_t) * (size_t)M);
+    for (int64_t m = 0; m < M; ++m) {
+      int32_t rs = 0;
+      for (int64_t k = 0; k < K; ++k) {
+        const int64_t i = transA ? k * lda + m : m * lda + k;
+        rs += a_dt == ZMI_DT_U8 ? (int32_t)((const uint8_t *)A)[i] : (int32_t)((const int8_t *)A)[i];
+      }
+      rowc[m] = -wei_zp * rs + src_zp * wei_zp * (int32_t)K;
+    }
+  }
   const int per_token = (src_scale_n == M && M > 1);
   const int64_t wei_scale_n = p->wei_scale.buff ? zo_nelems(&p->wei_scale) : 0;
   const float dst_scale = p->dst_scale.buff ? zo_read_f32(p->dst_scale.buff, p->dst_scale.dt, 0) : 1.0f;
@@ -689,7 +707,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
       float y = (float)acc[m * N + n];
       if (c->alpha != 1.0f) y *= c->alpha;
       if (c->beta != 0.0f) y += zo_read_f32(c->dst, p->dt_dst, m * (int64_t)c->ldc + n) * c->beta;
-      if (comp) y += (float)comp[n];
+      if (comp || rowc) y += (float)((comp ? comp[n] : 0) + (rowc ? rowc[m] : 0));
       if (src_scale_n) y *= zo_read_f32(src_scale, src_scale_dt, per_token ? m : 0);
       if (wei_scale_n) y *= zo_read_f32(p->wei_scale.buff, p->wei_scale.dt, n % wei_scale_n);
       if (c->bias) y += zo_read_f32(c->bias, p->dt_bias == ZMI_DT_NONE ? ZMI_DT_F32 : p->dt_bias, n);
@@ -711,7 +729,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
       zo_store(c->dst, p->dt_dst, m * (int64_t)c->ldc + n, y);
     }
   }
-  free(acc); free(comp); free(qbuf); free(sbuf); free(ggml_rows); free(ggml_scales);
+  free(acc); free(comp); free(rowc); free(qbuf); free(sbuf); free(ggml_rows); free(ggml_scales);
   return ZMI_SUCCESS;
 }
 

@@ -185,6 +185,28 @@ def test_zp_identity(zo):
     assert np.all(comp0 == 0)
 
 
+@pytest.mark.parametrize("u8", [False, True])
+@pytest.mark.parametrize("transA", [False, True])
+def test_weight_zero_point_is_the_integer_product_of_the_shifted_operands(zo, u8, transA):
+    """(A - a_zp)(W - w_zp) evaluated in Python integers equals the oracle's s32 result with a source and a weight
+    zero-point (either alone as well): the 2-D compensation's three terms, none dropped, no sign wrong."""
+    rng = np.random.default_rng(12 + int(u8) + 2 * int(transA))
+    M, K, N = 7, 45, 13
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8) if u8 else rng.integers(-128, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    src = np.ascontiguousarray(A.T) if transA else A
+    for a_zp, w_zp, w_dt in ((0, 5, np.int8), (3 if not u8 else 131, -7, np.int32), (-2 if not u8 else 17, 0, np.int8)):
+        azp = np.array([a_zp], dtype=np.int32)
+        wzp = np.array([w_zp], dtype=w_dt)
+        p = _params(dt_src=capi.DT_U8 if u8 else capi.DT_S8, dt_wei=capi.DT_S8, dt_dst=capi.DT_S32,
+                    src_zp=capi.quant(azp.ctypes.data, capi.DT_S32, (1,)) if a_zp else capi.quant(),
+                    wei_zp=capi.quant(wzp.ctypes.data, capi.DT_S8 if w_dt == np.int8 else capi.DT_S32, (1,)) if w_zp else capi.quant())
+        st, dst, _, _ = zo.matmul_int8(src, B, p, M, N, K, transA=transA, lda=M if transA else K)
+        assert st == capi.SUCCESS
+        want = (A.astype(np.int64) - a_zp) @ (B.astype(np.int64) - w_zp)
+        assert np.array_equal(dst[:, :N].astype(np.int64), want), (a_zp, w_zp)
+
+
 # ------------------------------------------------------ dequant chain
 def _params(**kw):
     p = capi.MatmulParamsT()

@@ -161,3 +161,37 @@ hipError_t zmi_launch_narrow_scales(float *sc, int64_t n, void *user_bf16, int64
                      (uint16_t *)user_bf16, n_user);
   return hipGetLastError();
 }
+
+
+// ---- weight zero-point: one compensation word per source row ------------------------------------------
+// row_comp[m] = -wei_zp * sum_k A[m, k] + src_zp * wei_zp * K in int32 (two's complement wrap), the source as the
+// caller gave it (u8 / s8, row- or column-major).  Reference: cache_or_compute_zp_compensation,
+// lowoha_operators/matmul/lru_cache/lowoha_cache.hpp:151-232 (its column term is the blob's colsum).  One wavefront per row.
+__global__ __launch_bounds__(256) void zmi_row_comp_kernel(const void *A, int64_t lda, int transA, int is_u8, int M, int K,
+                                                           int32_t wei_zp_val, const void *wei_zp_ptr, int32_t wei_zp_dt,
+                                                           int32_t src_zp_val, const int32_t *src_zp_ptr, int32_t *out) {
+  const int lane = threadIdx.x % 64;
+  const int m = blockIdx.x * 4 + threadIdx.x / 64;
+  if (m >= M) return;
+  int32_t wz = wei_zp_val;
+  if (wei_zp_ptr) wz = wei_zp_dt == ZMI_DT_S8 ? (int32_t)*(const int8_t *)wei_zp_ptr
+                     : wei_zp_dt == ZMI_DT_U8 ? (int32_t)*(const uint8_t *)wei_zp_ptr : *(const int32_t *)wei_zp_ptr;
+  const int32_t sz = src_zp_ptr ? *src_zp_ptr : src_zp_val;
+  uint32_t sum = 0;
+  for (int k = lane; k < K; k += 64) {
+    const int64_t i = transA ? (int64_t)k * lda + m : (int64_t)m * lda + k;
+    sum += is_u8 ? (uint32_t)((const uint8_t *)A)[i] : (uint32_t)(int32_t)((const int8_t *)A)[i];
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += (uint32_t)__shfl_xor((int)sum, o);
+  if (lane == 0) out[m] = (int32_t)((uint32_t)sz * (uint32_t)wz * (uint32_t)K - (uint32_t)wz * sum);
+}
+
+hipError_t zmi_launch_row_comp(const void *A, int64_t lda, bool transA, bool is_u8, int M, int K, int32_t wei_zp_val,
+                               const void *wei_zp_ptr, int32_t wei_zp_dt, int32_t src_zp_val, const int32_t *src_zp_ptr,
+                               int32_t *out, hipStream_t stream) {
+  if (M <= 0) return hipSuccess;
+  hipLaunchKernelGGL(zmi_row_comp_kernel, dim3((M + 3) / 4), dim3(256), 0, stream, A, lda, transA ? 1 : 0, is_u8 ? 1 : 0, M, K,
+                     wei_zp_val, wei_zp_ptr, wei_zp_dt, src_zp_val, src_zp_ptr, out);
+  return hipGetLastError();
+}

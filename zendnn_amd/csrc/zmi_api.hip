@@ -99,7 +99,7 @@ bool is_dynamic_quant_config(const zmi_matmul_params_t &p) {
 // kernels' shared epilogue descriptor (*out) and the per-problem operands
 // (scale / zero-point / bias fields of *prob).  Returns a ZMI_* status.
 int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, float beta, const void *bias,
-                       ZmiEpilogue *out, ZmiProblem *prob) {
+                       ZmiEpilogue *out, ZmiProblem *prob, bool allow_wei_zp) {
   ZmiEpilogue e;
   std::memset(&e, 0, sizeof(e));
   e.alpha = alpha;
@@ -174,8 +174,23 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
     return ZMI_FAILURE;
   }
   if (p.wei_zp.buff) {
-    set_error("weight zero-points are not implemented (symmetric s8 weights only)");
-    return ZMI_UNIMPLEMENTED;
+    // one zero-point for the whole weight tensor, read as an integer whatever its dtype (reference: read_and_cast in
+    // aocl_kernel.cpp:982-985); a single matmul_direct problem with s8 / u8 rows only
+    if (!allow_wei_zp || e.n_groups > 0) {
+      set_error("a weight zero-point is implemented for single problems with s8 / u8 sources and per-tensor or per-channel scales");
+      return ZMI_UNIMPLEMENTED;
+    }
+    if (p.wei_zp.dt != ZMI_DT_S8 && p.wei_zp.dt != ZMI_DT_U8 && p.wei_zp.dt != ZMI_DT_S32) {
+      set_error("weight zero-point: s8, u8 or s32");
+      return ZMI_FAILURE;
+    }
+    prob->wei_zp_dt = p.wei_zp.dt;
+    if (is_device_pointer(p.wei_zp.buff)) {
+      prob->wei_zp_ptr = p.wei_zp.buff;
+    } else {
+      prob->wei_zp_val = p.wei_zp.dt == ZMI_DT_S8 ? (int32_t)*(const int8_t *)p.wei_zp.buff
+                         : p.wei_zp.dt == ZMI_DT_U8 ? (int32_t)*(const uint8_t *)p.wei_zp.buff : *(const int32_t *)p.wei_zp.buff;
+    }
   }
   if (p.src_zp.buff) {
     if (!scalar_param_s32(p.src_zp.buff, p.src_zp.dt, &prob->src_zp_val, &prob->src_zp_ptr)) return ZMI_FAILURE;
@@ -315,7 +330,9 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
       split.slices = plan->slices;
       split.partial = (int32_t *)arena().alloc(plan->partial_bytes);
       if (!split.partial) { set_error("no scratch for the K-sliced GEMM"); return ZMI_FAILURE; }
-      split.arrivals = slice_arrivals(plan->tiles);   // (null: a reduction launch finishes the elements)
+      // (null: a reduction launch finishes the elements -- also with a weight zero-point, whose per-row term only
+      // the reduction's element-finishing code adds)
+      split.arrivals = prob.row_comp ? nullptr : slice_arrivals(plan->tiles);
     }
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")
@@ -539,9 +556,18 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
   if (bcast_src) need += Arena::padded(sizeof(float) * (size_t)M * (size_t)pg_groups);
   if (dyn) need += Arena::padded(a_bytes) + Arena::padded(sizeof(float) * (size_t)M * (size_t)(pg_groups ? pg_groups : 1)) + 256;
   if (repack_a) need += Arena::padded(a_bytes);
+  // a weight zero-point: one compensation word per row, and the kernels that finish their elements through
+  // zmi_finish_element (the decode and small-M kernels; the large-M kernel in K slices with its reduction launch)
+  const bool wzp = p.wei_zp.buff != nullptr;
+  if (wzp && (dyn || pg_groups || ggml || w4a8)) {
+    set_error("a weight zero-point is implemented for s8 / u8 sources and per-tensor or per-channel scales");
+    return ZMI_UNIMPLEMENTED;
+  }
+  if (wzp) need += Arena::padded(sizeof(int32_t) * (size_t)M);
   ZmiRingPlan plan = {};
   if (ring) {
     plan = plan_ring_gemm(M, N, K);
+    if (wzp && plan.slices < 2) plan = zmi_ring_plan(M, N, K, 0, 2);
     need += Arena::padded(plan.partial_bytes);
   }
   if (!pg_groups && decode_sliced_allowed(M, N, K)) need += Arena::padded(zmi_decode16_partial_bytes(M, N, K));
@@ -705,8 +731,16 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
   }
 
   ZmiEpilogue epi;
-  int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob);
+  int32_t st = build_epilogue(ep, M, N, alpha, beta, bias, &epi, &prob, true);
   if (st != ZMI_SUCCESS) return st;
+  if (wzp && (prob.wei_zp_ptr || prob.wei_zp_val != 0)) {
+    int32_t *rc = (int32_t *)arena().alloc(sizeof(int32_t) * (size_t)M);
+    if (!rc) { set_error("no scratch for the weight zero-point compensation"); return ZMI_FAILURE; }
+    if (!hip_ok(zmi_launch_row_comp(src, lda, transA != 0, p.dt_src == ZMI_DT_U8, M, K, prob.wei_zp_val, prob.wei_zp_ptr,
+                                    prob.wei_zp_dt, prob.src_zp_val, prob.src_zp_ptr, rc, stream()), "zero-point compensation launch"))
+      return ZMI_FAILURE;
+    prob.row_comp = rc;
+  }
   if (epi.n_groups > 0 && pgring && !use_fused) {
     const int64_t G = epi.n_groups, np = zmi_pgring_ws_cols(N);
     int8_t *af = a_frag ? a_frag : (int8_t *)arena().alloc((size_t)zmi_afrag_bytes(M, K));

@@ -145,6 +145,15 @@ struct ZmiProblem {
   float src_scale_val;         // ZMI_SS_VALUE
   float wei_scale_val;
   int32_t src_zp_val;
+  // weight zero-point (per tensor): the kernels see it as one int32 per row that joins the accumulator's
+  // compensation, row_comp[m] = -wei_zp * sum_k A[m, k] + src_zp * wei_zp * K (reference: the 2-D compensation of
+  // cache_or_compute_zp_compensation, lowoha_operators/matmul/lru_cache/lowoha_cache.hpp:151-232, without its
+  // column term, which is the blob's colsum).  Only the kernels that finish elements through zmi_finish_element
+  // read it; the API keeps calls with a weight zero-point on those.
+  const int32_t *row_comp;     // null: no weight zero-point
+  int32_t wei_zp_val;          // host-side planning only (value, or a device pointer and its dtype)
+  int32_t wei_zp_dt;
+  const void *wei_zp_ptr;
 };
 
 #ifdef __HIPCC__
@@ -524,8 +533,10 @@ __device__ __forceinline__ bool zmi_epilogue_is_raw_s32(const ZmiEpilogue &e, co
 
 // One finished output element: accumulator -> epilogue -> store at dst[m * ldc + n].  The
 // kernels that produce one element per thread (decode, the K-slice reduction) end here.
-__device__ __forceinline__ void zmi_finish_element(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &c,
+__device__ __forceinline__ void zmi_finish_element(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiColCtx &c_in,
                                                    float rs, int32_t s, int m, int n) {
+  ZmiColCtx c = c_in;
+  if (p.row_comp) c.comp += p.row_comp[m];   // (a weight zero-point: see ZmiProblem)
   const bool has_rs = epi.src_scale_mode != ZMI_SS_NONE, has_ws = epi.wei_scale_mode != 0;
   const bool has_bias = p.bias != nullptr;
   const int64_t o = (int64_t)m * p.ldc + n;

@@ -103,6 +103,10 @@ bool zmi_group_decode_takes(const ZmiEpilogue &epi, int N);
 // Weight-traffic-bound grouped launch on the MFMA-bound kernel's tiles (k_stream.hip)
 bool zmi_group_stream_takes(const ZmiEpilogue &epi, int N, int top_flags);
 int zmi_cu_count();   // compute units of the current device
+// k_util.hip: the per-row compensation of a weight zero-point (see ZmiProblem::row_comp)
+hipError_t zmi_launch_row_comp(const void *A, int64_t lda, bool transA, bool is_u8, int M, int K, int32_t wei_zp_val,
+                               const void *wei_zp_ptr, int32_t wei_zp_dt, int32_t src_zp_val, const int32_t *src_zp_ptr,
+                               int32_t *out, hipStream_t stream);
 int zmi_stream_items(const ZmiProblem *probs_host, int n_prob, int top, int64_t worst_rows, int worst_cols, bool gated);
 size_t zmi_stream_partial_bytes(int items, int slices, int top);
 hipError_t zmi_launch_gemm_stream_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob, int top,
