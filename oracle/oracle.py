@@ -51,6 +51,8 @@ def lib():
                                     C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
         L.zo_fp16_to_f32.restype = C.c_float
         L.zo_fp16_to_f32.argtypes = [C.c_uint16]
+        L.zo_f32_to_f16.restype = C.c_uint16
+        L.zo_f32_to_f16.argtypes = [C.c_float]
         L.zo_ggml_q8_0_unpack.restype = None
         L.zo_ggml_q8_0_unpack.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.zo_s4_to_s8.restype = None
@@ -88,7 +90,7 @@ def _p(a):
 
 
 NP_OF_DT = {capi.DT_F32: np.float32, capi.DT_BF16: np.uint16, capi.DT_S32: np.int32,
-            capi.DT_S8: np.int8, capi.DT_U8: np.uint8}
+            capi.DT_S8: np.int8, capi.DT_U8: np.uint8, capi.DT_F16: np.uint16}
 
 
 def f32_to_bf16(x, ctor=True):

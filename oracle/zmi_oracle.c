@@ -30,6 +30,8 @@
  *   per-group scales             closed form (all-ones operands, power-of-two scales: every step exact),
  *                                equal power-of-two group scales == per-token chain bit for bit,
  *                                numpy float32 brute force on small random cases
+ *   zo_f32_to_f16                round trip of all 65536 half values, numpy float16 on 4 million random bit patterns and
+ *                                on every tie / boundary case (except the documented carry case, which has known answers)
  *   zo_fp16_to_f32, Q8_0 unpack  all 65536 half values against numpy float16; block layout by construction
  *                                of the packed buffer from known rows and scales (numpy), bf16 via torch
  *   zo_s4_to_s8 (W4A8 widening)  every nibble value in both positions (known answers), numpy shift/mask
@@ -112,9 +114,13 @@ static int64_t zo_nelems(const zmi_quant_t *q) {
 }
 
 /* read_and_cast<float> of the reference for the dtypes this path uses. */
+ZO_EXPORT float zo_fp16_to_f32(uint16_t h);
+ZO_EXPORT uint16_t zo_f32_to_f16(float f);
+
 static float zo_read_f32(const void *p, int32_t dt, int64_t i) {
   switch (dt) {
   case ZMI_DT_F32: return ((const float *)p)[i];
+  case ZMI_DT_F16: return zo_fp16_to_f32(((const uint16_t *)p)[i]);
   case ZMI_DT_BF16: return zo_bf16_to_f32(((const uint16_t *)p)[i]);
   case ZMI_DT_S32: return (float)((const int32_t *)p)[i];
   case ZMI_DT_S8: return (float)((const int8_t *)p)[i];
@@ -408,6 +414,7 @@ static void zo_store(void *dst, int32_t dt, int64_t i, float val) {
     ((int32_t *)dst)[i] = val >= 2147483648.0f ? INT32_MAX : (int32_t)nearbyintf(val);
     break;
   case ZMI_DT_BF16: ((uint16_t *)dst)[i] = zo_f32_to_bf16_ctor(val); break;
+  case ZMI_DT_F16: ((uint16_t *)dst)[i] = zo_f32_to_f16(val); break;
   default: ((float *)dst)[i] = val; break;
   }
 }
@@ -431,6 +438,41 @@ ZO_EXPORT float zo_fp16_to_f32(uint16_t h) {
   float f;
   memcpy(&f, &u, 4);
   return f;
+}
+
+/* float16_t(float), common/float16.cpp:124-205: round to nearest even into half precision.  f32 zeros and
+ * subnormals, and magnitudes that round below the smallest half subnormal, give a signed zero; magnitudes from
+ * 65520 up give infinity; NaN keeps the top ten mantissa bits and is made quiet.  A half-subnormal result whose
+ * rounding carries into the exponent (magnitudes in [2^-14 - 2^-25, 2^-14)) loses the carry, because the
+ * reference masks that result with the mantissa field: it stores a signed zero there, and so does this. */
+ZO_EXPORT uint16_t zo_f32_to_f16(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  const uint32_t e = (u >> 23) & 0xffu, m = u & 0x7fffffu;
+  if (e == 0) return sign;
+  if (e == 255) return m ? (uint16_t)(sign | 0x7c00u | (m >> 13) | 0x200u) : (uint16_t)(sign | 0x7c00u);
+  int32_t he = (int32_t)e - 112;                     /* exponent bias 127 -> 15 */
+  if (he >= 31) return (uint16_t)(sign | 0x7c00u);
+  if (he <= 0) {
+    if (he < -10) return sign;
+    const uint32_t full = m | 0x800000u;             /* with the implicit one */
+    const int shift = 14 - he;
+    const uint32_t half = 1u << (shift - 1);
+    uint32_t q = full >> shift;
+    if ((full & half) && ((full & (half - 1u)) || (q & 1u))) q += 1u;
+    return (uint16_t)(sign | (q & 0x3ffu));
+  }
+  uint32_t q = m >> 13;
+  if ((m & 0x1000u) && ((m & 0xfffu) || (q & 1u))) {
+    q += 1u;
+    if (q > 0x3ffu) {
+      q = 0;
+      he += 1;
+      if (he >= 31) return (uint16_t)(sign | 0x7c00u);
+    }
+  }
+  return (uint16_t)(sign | ((uint32_t)he << 10) | q);
 }
 
 /* fp32_to_bf16 of ggml_weight_unpack.cpp:66-73: NaN quieted, else round to nearest even (no flush). */

@@ -484,6 +484,44 @@ def _q8_0_pack(rows, d16):
     return blk.reshape(-1)
 
 
+def test_f32_to_fp16_round_trip_numpy_and_the_reference_carry_case(zo):
+    """Narrowing to half precision: every half value survives the round trip; 300 000 random f32 bit patterns and
+    every tie / boundary neighbourhood agree with numpy's float16 (IEEE round to nearest even), except where the
+    reference's own code departs from IEEE: magnitudes in [2^-14 - 2^-25, 2^-14) round up to the smallest normal
+    half in IEEE and to a signed zero in the reference (it masks the carried mantissa) -- known answers there."""
+    L = zo.lib()
+    conv = np.frompyfunc(lambda v: L.zo_f32_to_f16(float(v)), 1, 1)
+    halves = np.arange(65536, dtype=np.uint16)
+    vals = halves.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(vals)
+    got = conv(vals[ok]).astype(np.uint16)
+    assert np.array_equal(got, halves[ok])
+    rng = np.random.default_rng(7)
+    bits = rng.integers(0, 2 ** 32, 300000, dtype=np.uint64).astype(np.uint32)
+    # neighbourhoods of every half value's midpoints (ties) and of the range ends
+    mid = ((halves[ok].astype(np.uint32) & 0x7fff) < 0x7bff)
+    h32 = vals[ok][mid].view(np.uint32)
+    h64 = h32.astype(np.int64)
+    ties = np.concatenate([h64 + 0x1000 + d for d in (-1, 0, 1)] + [np.array([0x477fe000 + d for d in range(-3, 4)], dtype=np.int64)])
+    x = np.concatenate([bits, ties.astype(np.uint32)]).view(np.float32)
+    x = x[~np.isnan(x)]
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = conv(x).astype(np.uint16)
+    a = np.abs(x.astype(np.float64))
+    carry = (a >= 2.0 ** -14 - 2.0 ** -25) & (a < 2.0 ** -14)
+    tiny = a < 2.0 ** -126          # f32 subnormals: signed zero in both
+    assert np.array_equal(got[~carry], want[~carry])
+    assert np.all(got[tiny] == (x[tiny].view(np.uint32) >> 16 & 0x8000))
+    # the carry case: IEEE gives the smallest normal, the reference a signed zero
+    for v in (np.float32(2.0 ** -14 - 2.0 ** -25), np.float32(2.0 ** -14 - 2.0 ** -26), np.float32(-(2.0 ** -14) * (1 - 2.0 ** -13))):
+        assert np.float16(v).view(np.uint16) & 0x7fff == 0x0400
+        assert L.zo_f32_to_f16(float(v)) == (0x8000 if v < 0 else 0)
+    # NaN: quiet, sign and top mantissa bits kept
+    nan = np.array([0x7fa00000], dtype=np.uint32).view(np.float32)[0]
+    assert L.zo_f32_to_f16(float(nan)) & 0x7e00 == 0x7e00
+
+
 def test_fp16_conversion_against_numpy_for_every_half_value(zo):
     h = np.arange(65536, dtype=np.uint16)
     want = h.view(np.float16).astype(np.float32)

@@ -192,9 +192,48 @@ __device__ __forceinline__ uint16_t zmi_f32_to_bf16_rne(float f) {
   return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
 }
 
+// half precision <-> f32 (reference: float16_t, common/float16.cpp:77-205).  Widening is exact (the hardware
+// conversion).  Narrowing rounds to nearest even like the hardware does, except where the reference's own code does
+// something else: f32 subnormals become signed zeros whatever the mode, NaN keeps its top mantissa bits and is made
+// quiet, and a half-subnormal result whose rounding carries into the exponent (magnitudes in [2^-14 - 2^-25, 2^-14))
+// is stored as a signed zero, because the reference masks it with the mantissa field.  Integer code, so that the
+// result does not depend on the wavefront's denormal mode.
+__device__ __forceinline__ float zmi_f16_to_f32(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+__device__ __forceinline__ uint16_t zmi_f32_to_f16(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t sign = (u >> 16) & 0x8000u;
+  const uint32_t e = (u >> 23) & 0xffu, m = u & 0x7fffffu;
+  if (e == 0) return (uint16_t)sign;
+  if (e == 255) return (uint16_t)(m ? (sign | 0x7c00u | (m >> 13) | 0x200u) : (sign | 0x7c00u));
+  int he = (int)e - 112;
+  if (he >= 31) return (uint16_t)(sign | 0x7c00u);
+  if (he <= 0) {
+    if (he < -10) return (uint16_t)sign;
+    const uint32_t full = m | 0x800000u;
+    const int shift = 14 - he;
+    const uint32_t half = 1u << (shift - 1);
+    uint32_t q = full >> shift;
+    if ((full & half) && ((full & (half - 1u)) || (q & 1u))) q += 1u;
+    return (uint16_t)(sign | (q & 0x3ffu));
+  }
+  uint32_t q = m >> 13;
+  if ((m & 0x1000u) && ((m & 0xfffu) || (q & 1u))) {
+    q += 1u;
+    if (q > 0x3ffu) {
+      q = 0;
+      he += 1;
+      if (he >= 31) return (uint16_t)(sign | 0x7c00u);
+    }
+  }
+  return (uint16_t)(sign | ((uint32_t)he << 10) | q);
+}
+
 __device__ __forceinline__ float zmi_ld_f32(const void *p, int dt, int64_t i) {
   switch (dt) {
   case ZMI_DT_BF16: return zmi_bf16_to_f32(((const uint16_t *)p)[i]);
+  case ZMI_DT_F16: return zmi_f16_to_f32(((const uint16_t *)p)[i]);
   case ZMI_DT_S32: return (float)((const int32_t *)p)[i];
   case ZMI_DT_S8: return (float)((const int8_t *)p)[i];
   case ZMI_DT_U8: return (float)((const uint8_t *)p)[i];
@@ -512,6 +551,7 @@ __device__ __forceinline__ float zmi_act_bf16_kind(int fast_kind, float y) {
 __device__ __forceinline__ void zmi_store(void *dst, int dt, int64_t i, float y) {
   switch (dt) {
   case ZMI_DT_BF16: ((uint16_t *)dst)[i] = zmi_f32_to_bf16(y); break;
+  case ZMI_DT_F16: ((uint16_t *)dst)[i] = zmi_f32_to_f16(y); break;
   case ZMI_DT_S32: {
     float v = fminf(fmaxf(y, -2147483648.0f), 2147483648.0f);
     ((int32_t *)dst)[i] = v >= 2147483648.0f ? 2147483647 : (int32_t)rintf(v);
