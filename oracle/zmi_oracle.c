@@ -803,6 +803,7 @@ ZO_EXPORT void zo_gated_act(int32_t act, void *buf, int32_t dt, int64_t M, int64
         else r = (g * 0.5f * (1.0f + erff(g * 0.7071067811865476f))) * u;
       }
       if (dt == ZMI_DT_BF16) ((uint16_t *)buf)[m * ld + n] = zo_f32_to_bf16_ctor(r);
+      else if (dt == ZMI_DT_F16) ((uint16_t *)buf)[m * ld + n] = zo_f32_to_f16(r);   /* :165-182 */
       else ((float *)buf)[m * ld + n] = r;
     }
   }
@@ -827,6 +828,7 @@ ZO_EXPORT void zo_moe_reduce(const void *const *row_ptrs, const float *w, int32_
         acc = (k == 0) ? wk * x : fmaf(wk, x, acc);
       }
       if (dt == ZMI_DT_BF16) ((uint16_t *)out)[t * ldo + d] = zo_f32_to_bf16_rne(acc);
+      else if (dt == ZMI_DT_F16) ((uint16_t *)out)[t * ldo + d] = zo_f32_to_f16(acc);   /* store_from_f32, :84-100 */
       else ((float *)out)[t * ldo + d] = acc;
     }
   }

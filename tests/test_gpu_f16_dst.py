@@ -59,3 +59,52 @@ def test_f16_destination_bit_identical_to_the_oracle(zo, M, K, N, u8, beta):
         assert np.isinf(f).any()
     if M == 24 and beta == 0.0:
         assert ((f > 0) & (f < 6.0e-5)).any()
+
+
+@pytest.mark.parametrize("act", [capi.ACT_SILU_AND_MUL, capi.ACT_SWIGLU_OAI_MUL])
+def test_group_call_with_f16_destinations_gated_activation_and_weighted_reduce(zo, act):
+    """group_matmul_direct with half-precision expert outputs: the GEMMs, the gated activation (float16_t(value),
+    group_matmul_moe_act.cpp:165-182) and the weighted reduce over half-precision rows (store_from_f32,
+    group_matmul_moe_postop.cpp:84-100).  Before, the activation and the reduce treated f16 as f32 words."""
+    rng = np.random.default_rng(31 + act)
+    E, T, K, I = 3, 10, 192, 40
+    N = 2 * I
+    Ms = [T, T, T]
+    srcs = [rng.integers(-128, 128, (T, K), dtype=np.int8) for _ in range(E)]
+    ws = [H.gen_weights(rng, K, N) for _ in range(E)]
+    sscale = np.array([0.01], dtype=np.float32)
+    wscale = [rng.uniform(0.001, 0.004, N).astype(np.float32) for _ in range(E)]
+    src_d = [H.to_dev(s) for s in srcs]
+    w_d = [H.to_dev(w) for w in ws]
+    wsc_d = [H.to_dev(x) for x in wscale]
+    dst = [torch.zeros((T, N), dtype=torch.int16, device=H.DEV) for _ in range(E)]
+    params = []
+    for e in range(E):
+        p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F16)
+        p.src_scale = lowoha.QuantParam(sscale.ctypes.data, capi.DT_F32, (1,))
+        p.wei_scale = lowoha.QuantParam(wsc_d[e], capi.DT_F32, (1, N))
+        params.append(p)
+    ids = [(t % E, (t + 1) % E) for t in range(T)]
+    rp = [dst[e].data_ptr() + t * N * 2 for t in range(T) for e in ids[t]]
+    tw_h = rng.uniform(0.2, 0.8, (T, 2)).astype(np.float32)
+    tw = H.to_dev(tw_h)
+    out = torch.zeros((T, N), dtype=torch.int16, device=H.DEV)   # (without fused_moe the reduce takes whole rows)
+    pp = lowoha.MoePostop(T, 2, out, N, tw, rp)
+    st = lowoha.group_matmul_direct(
+        ["r"] * E, [False] * E, [False] * E, Ms, [N] * E, [K] * E, [1.0] * E,
+        src_d, [K] * E, w_d, [N] * E, [None] * E, [0.0] * E, dst, [N] * E, [True] * E, params,
+        gated_act=act, moe_postop=pp)
+    assert st == capi.SUCCESS, lowoha.last_error()
+    got = [_f16_host(d) for d in dst]
+    for e in range(E):
+        ph = H.host_params(params[e], wei_scale=wscale[e])
+        keep = []
+        st, y, _, _ = zo.matmul_int8(srcs[e], ws[e], ph.flat(keep), T, N, K)
+        assert st == capi.SUCCESS
+        zo.gated_act(act, y, capi.DT_F16)
+        d = np.abs(got[e][:, :I].view(np.int16).astype(np.int32) - y[:, :I].view(np.int16).astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() < 5e-3, (e, d.max())
+    # the reduce over the device's own rows: bit-identical
+    rows = [got[e][t].copy() for t in range(T) for e in ids[t]]
+    want = zo.moe_reduce(rows, tw_h, capi.DT_F16, N)
+    assert np.array_equal(_f16_host(out), want)

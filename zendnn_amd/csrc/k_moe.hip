@@ -43,6 +43,7 @@ __global__ __launch_bounds__(256) void zmi_gated_act_kernel(ZmiActMat m0, const 
   __syncthreads();
   for (int n = threadIdx.x; n < dim; n += blockDim.x) {
     if (dt == ZMI_DT_BF16) ((uint16_t *)m.buf)[base + n] = zmi_f32_to_bf16(res[n]);
+    else if (dt == ZMI_DT_F16) ((uint16_t *)m.buf)[base + n] = zmi_f32_to_f16(res[n]);   // (float16_t(value), group_matmul_moe_act.cpp:165-182)
     else ((float *)m.buf)[base + n] = res[n];
   }
 }
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(256) void zmi_moe_combine_kernel(const void *const 
                                                               const float *weights, int skip_weighted, int topk,
                                                               int D, int dt, void *out, int64_t ldo) {
   const int t = blockIdx.x;
-  const size_t es = dt == ZMI_DT_BF16 ? 2 : 4;
+  const size_t es = dt == ZMI_DT_BF16 || dt == ZMI_DT_F16 ? 2 : 4;
   auto row_of = [&](int k) -> const void * {
     const int s = t * topk + k;
     return row_ptrs ? row_ptrs[s] : (const void *)((const char *)rows_base + (int64_t)slot_of[s] * row_ld * es);
@@ -115,6 +116,7 @@ __global__ __launch_bounds__(256) void zmi_moe_combine_kernel(const void *const 
       acc = (k == 0) ? __fmul_rn(w, x) : __builtin_fmaf(w, x, acc);
     }
     if (dt == ZMI_DT_BF16) ((uint16_t *)out)[(int64_t)t * ldo + d] = zmi_f32_to_bf16_rne(acc);
+    else if (dt == ZMI_DT_F16) ((uint16_t *)out)[(int64_t)t * ldo + d] = zmi_f32_to_f16(acc);   // (store_from_f32, group_matmul_moe_postop.cpp:84-100)
     else ((float *)out)[(int64_t)t * ldo + d] = acc;
   }
 }

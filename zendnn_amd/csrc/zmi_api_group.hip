@@ -512,7 +512,7 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       return ZMI_UNIMPLEMENTED;
     }
     if (dyn && p0.dt_compute == ZMI_DT_U8) { set_error("dynamic u8 quantization is not implemented"); return ZMI_UNIMPLEMENTED; }
-    const int dst_es = p0.dt_dst == ZMI_DT_BF16 ? 2 : (p0.dt_dst == ZMI_DT_F32 || p0.dt_dst == ZMI_DT_S32 ? 4 : 1);
+    const int dst_es = p0.dt_dst == ZMI_DT_BF16 || p0.dt_dst == ZMI_DT_F16 ? 2 : (p0.dt_dst == ZMI_DT_F32 || p0.dt_dst == ZMI_DT_S32 ? 4 : 1);
     if (fused_moe && !(p0.dt_dst == ZMI_DT_BF16 || p0.dt_dst == ZMI_DT_F32)) { set_error("fused_moe needs a bf16 or f32 dst"); return ZMI_UNIMPLEMENTED; }
     if (fused_moe && !dyn) { set_error("fused_moe is implemented for dynamic_quant int8 only"); return ZMI_UNIMPLEMENTED; }
     for (size_t i = 0; i < num_ops; ++i) {
@@ -758,7 +758,7 @@ postop_only:
     if (!ensure_device()) return ZMI_FAILURE;
     const int D = fused_moe ? fused_moe->N_down[0] : a.N[0];
     const int dt = a.params[0].dt_dst;
-    if (dt != ZMI_DT_BF16 && dt != ZMI_DT_F32) { set_error("moe_postop: f16 is not implemented"); return ZMI_UNIMPLEMENTED; }
+    if (dt != ZMI_DT_BF16 && dt != ZMI_DT_F32 && dt != ZMI_DT_F16) { set_error("moe_postop: rows of f32, bf16 or f16"); return ZMI_FAILURE; }
     const size_t tbl = sizeof(void *) * (size_t)moe_postop->num_tokens * moe_postop->topk;
     const void *const *rp = (const void *const *)upload(moe_postop->row_ptrs, tbl);
     if (!rp) return ZMI_FAILURE;
