@@ -235,6 +235,11 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
       if (!po.buff) { set_error("binary post-op without operand"); return ZMI_FAILURE; }
       d.buff = po.buff;
       d.dtype = po.dtype == ZMI_DT_NONE ? ZMI_DT_F32 : po.dtype;
+      if (d.dtype != ZMI_DT_F32 && d.dtype != ZMI_DT_BF16 && d.dtype != ZMI_DT_F16 && d.dtype != ZMI_DT_S32 &&
+          d.dtype != ZMI_DT_S8 && d.dtype != ZMI_DT_U8) {
+        set_error("binary post-op operand: f32, bf16, f16, s32, s8 or u8");
+        return ZMI_UNIMPLEMENTED;
+      }
       d.ld = po.leading_dim > 0 ? po.leading_dim : N;
       const bool row = (po.ndims == 2 && po.dims[0] == 1 && po.dims[1] == N) || (po.ndims == 1 && po.dims[0] == N);
       const bool full = po.ndims == 2 && po.dims[0] == M && po.dims[1] == N;
