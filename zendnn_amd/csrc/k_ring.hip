@@ -796,23 +796,32 @@ ZmiRingPlan zmi_ring_plan(int M, int N, int K, int top_hint, int force_slices) {
   if (M <= 0) return plan;
   const int n_cu = zmi_cu_count();
   if ((plan.top & 0xffff) == 64 && force_slices <= 0) return plan;
-  // 65 .. 256 rows or so against a wide weight matrix: 64-row tiles, unsliced, while they fit the CUs at once.  A
-  // workgroup's weight stream runs at what one compute unit keeps in flight (about 60 GB/s), so the call is as long
-  // as one tile's stream (256 columns x K) whatever the tile height: more, lower tiles put more CUs to work without
-  // the partial tiles of the K slices (their int32 traffic is half the weights' at 128 rows).  Measured, us per
-  // call, this / before: K = 4096, N = 14336: 96 rows 31.5 / 36.7, 256 rows 34.2 / 38.7; K = 2048, N = 11008:
-  // 128 rows 20.6 / 28.2; K = 4096, N = 4096: 256 rows 28.9 / 32.1.  Long K (8192 and more) and two rounds of tiles
-  // (384 rows at N = 14336: 48.5 / 41.7) stay with the sliced and the 128-row forms.
+  // More than 64 rows whose 64-row tiles fit the CUs at once.  A workgroup's weight stream runs at what one compute
+  // unit keeps in flight (the LDS ring: about 60 GB/s at the loaded latency), so such a call lasts as long as ONE
+  // workgroup's stream whatever the tile height: lower tiles put more CUs to work, and K slices shorten the stream
+  // while slices x tiles still fit the CUs (one workgroup each: a second round costs more than it saves) and a slice
+  // keeps 24 stages of 64 k; the slice that arrives last adds the partial tiles (64 KiB each at this height).
+  // Measured, us per call, this / 128-row tiles (in four slices when few): K = 4096, N = 14336: 96 rows 29.4 / 36.7,
+  // 256 rows 33.5 / 38.7; K = 8192, N = 8192: 128 rows 32.6 / 37.1, 256 rows 39.1 / 43.7; K = 14336, N = 4096:
+  // 128 rows 38.2 / 47.1; K = 4096, N = 4096: 256 rows 25.7 / 32.1; K = 2048, N = 11008: 128 rows 21.0 / 28.2.
   if (!top_hint && force_slices <= 0 && M > 64) {
     const int64_t t64 = ((M + 63) / 64) * tiles_n;
-    if (t64 >= 48 && t64 <= n_cu && zmi_blob_kpad(K) <= 6144) {
-      plan.top = 64 | ZMI_RING_PAD;
-      plan.tiles = (int)t64;
-      return plan;
+    const int nk64 = (int)(zmi_blob_kpad(K) / 64);
+    if (t64 <= n_cu) {
+      int sl = 1;
+      if (t64 * 4 <= n_cu && nk64 / 4 >= 24) sl = 4;
+      else if (t64 * 2 <= n_cu && nk64 / 2 >= 24) sl = 2;
+      if (sl > 1 || (t64 >= 48 && zmi_blob_kpad(K) <= 6144)) {
+        plan.top = 64 | ZMI_RING_PAD;
+        plan.tiles = (int)t64;
+        plan.slices = sl;
+        plan.partial_bytes = sl > 1 ? (size_t)t64 * sl * 64 * 256 * sizeof(int32_t) : 0;
+        return plan;
+      }
     }
   }
   const int nk = (int)(zmi_blob_kpad(K) / 64);
-  const int top = M <= 64 ? 64 : 128;
+  const int top = M <= 64 || (top_hint & 0xffff) == 64 ? 64 : 128;
   const int64_t tiles = ((M + top - 1) / top) * tiles_n;
   int slices = 1;
   if (force_slices > 0) slices = force_slices;
