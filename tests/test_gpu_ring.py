@@ -206,6 +206,38 @@ def test_unsliced_64_row_tiles_for_a_wide_problem_with_few_rows(zo, env, M, K, N
     H.check_bf16(got, want, max_frac=5e-3)
 
 
+@pytest.mark.parametrize("M,K,N,slices", [(100, 3100, 1500, 2), (130, 6200, 700, 4), (257, 1600, 2600, 1)])
+def test_plan_takes_64_row_tiles_in_k_slices_by_itself(zo, env, M, K, N, slices):
+    """More than 64 rows, few tiles: the plan picks 64-row tiles and as many K slices (4, 2 or 1) as leave a slice 24
+    stages of 64 k; partly filled last row tile, K that is no multiple of 64.  s32 sums against the integer product,
+    the f32 chain with a bias against the oracle, twice (the arrival words must be zero again)."""
+    env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17)
+    rng = np.random.default_rng(M + K + N)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = H.gen_weights(rng, K, N)
+    want = a.astype(np.int64) @ w.astype(np.int64)
+    a_d, w_d = H.to_dev(a), H.to_dev(w)
+    name = "ring_mfma32x32x32_top64_ksliced" if slices > 1 else "ring_mfma32x32x32_top64"
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_S32)
+    for rep in range(2):
+        dst = torch.zeros((M, N), dtype=torch.int32, device=H.DEV)
+        st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, a_d, K, w_d, N, None, 0.0, dst, N, True, p)
+        assert st == capi.SUCCESS, lowoha.last_error()
+        assert lowoha.last_kernel() == name
+        assert np.array_equal(H.to_host(dst).astype(np.int64), want), rep
+    ss = rng.uniform(0.01, 0.03, M).astype(np.float32)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    ss_d, ws_d = H.to_dev(ss), H.to_dev(ws)
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_F32, bias=capi.DT_F32)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.weight_cache_type = 0
+    got, want = _run_both(zo, p, a, w, M, N, K, bias=bias, host_bufs={"src_scale": ss, "wei_scale": ws})
+    assert lowoha.last_kernel() == name
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("dst_dt", [capi.DT_F32, capi.DT_S8, capi.DT_U8])
 def test_k_sliced_f32_exact_and_quantized_destinations(zo, env, dst_dt):
     env(ZMI_DECODE_MAX_M=16, ZMI_RING_MIN_M=17, ZMI_RING_SPLITK=4)
