@@ -786,7 +786,7 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     hipLaunchKernelGGL(zmi_gemm_decode16_selfq_kernel, dim3((n_blk + 1) / 2), dim3(DQ_THREADS), smem, stream, p, epi, *fq, n_blk);
     return hipGetLastError();
   }
-  if (zmi_decode_16row_kernel(p, fq != nullptr)) {
+  if (zmi_decode_16row_kernel(p, fq != nullptr) && (!fq || fq->flags_uncached)) {
     // (the operand area, reused by the partial tiles, and with the quantization in the launch a word per wavefront)
     const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
     const size_t smem = (op > DEC_RED_BYTES ? op : DEC_RED_BYTES) + (fq ? 64 : 0);

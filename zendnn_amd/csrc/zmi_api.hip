@@ -773,7 +773,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     if (epi.src_scale_mode == ZMI_SS_TENSOR_PTR) epi.src_scale_mode = ZMI_SS_TOKEN_PTR;
     if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
       set_kernel_name(zmi_decode_selfq_takes(prob, &fused) ? "decode16x2_selfquant_mfma16x16x64 (per-token quant in the workgroup)"
-                      : zmi_decode_16row_kernel(prob, true) ? "decode16_dma_rows_mfma16x16x64 (fused per-token quant)"
+                      : zmi_decode_16row_kernel(prob, true) && fused.flags_uncached ? "decode16_dma_rows_mfma16x16x64 (fused per-token quant)"
                                                             : "decode_lds_rows_mfma16x16x64 (fused per-token quant)");
       st = hip_ok(zmi_launch_gemm_decode(prob, epi, &fused, stream()), "fused decode GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
     } else {

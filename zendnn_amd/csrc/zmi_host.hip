@@ -30,6 +30,7 @@ struct ThreadCtx {
   int next = 0;
   // hand-off words of the launches that quantize their own rows (ZmiFusedQuant::sync / error)
   unsigned int *fq_flags = nullptr;      // device: one flag per row, holding the epoch of the launch that published it
+  bool fq_flags_uncached = false;
   unsigned int fq_epoch = 0;             // name of this thread's latest launch of that kind
   unsigned int *fq_err_host = nullptr;   // pinned host word the kernels set when a wait ran out
   unsigned int *fq_err_dev = nullptr;    // the same word as the device addresses it
@@ -253,8 +254,16 @@ bool fused_handoff(ZmiFusedQuant *fq) {
   if (!c.fq_flags) {
     void *d = nullptr, *h = nullptr, *hd = nullptr;
     // (uncached: the waiting side may read the flags through the scalar unit, which cannot ask for device scope;
-    // never freed -- memory of this kind that a kernel has read stays allocated until the process ends)
-    if (!hip_ok(hipExtMallocWithFlags(&d, 512, hipDeviceMallocUncached), "hipExtMallocWithFlags(hand-off words)")) return false;
+    // never freed -- memory of this kind that a kernel has read stays allocated until the process ends;
+    // a device that refuses the uncached kind gets ordinary memory and the waits that read it with device-scope loads)
+    if (hipExtMallocWithFlags(&d, 512, hipDeviceMallocUncached) != hipSuccess) {
+      (void)hipGetLastError();
+      d = nullptr;
+      if (!hip_ok(hipMalloc(&d, 512), "hipMalloc(hand-off words)")) return false;
+      c.fq_flags_uncached = false;
+    } else {
+      c.fq_flags_uncached = true;
+    }
     if (!hip_ok(hipMemset(d, 0, 512), "hipMemset(hand-off words)")) return false;
     if (!hip_ok(hipHostMalloc(&h, 64, hipHostMallocMapped), "hipHostMalloc(error word)")) return false;
     std::memset(h, 0, 64);
@@ -264,6 +273,7 @@ bool fused_handoff(ZmiFusedQuant *fq) {
     c.fq_err_dev = (unsigned int *)hd;
   }
   fq->flags = c.fq_flags;
+  fq->flags_uncached = c.fq_flags_uncached ? 1 : 0;
   if (++c.fq_epoch == 0) c.fq_epoch = 1;   // (0 is what the flags hold before the first launch)
   fq->epoch = c.fq_epoch;
   fq->error = c.fq_err_dev;

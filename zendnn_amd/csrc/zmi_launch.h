@@ -136,6 +136,7 @@ struct ZmiFusedQuant {
   unsigned int *error;    // host-visible word, set to 1 by a wavefront whose wait ran out
   uint32_t wait_ticks;    // limit of the wait in ticks of the 100 MHz real-time counter; 0: give up at once
   int32_t per_row;        // per-group kernels only: one scale per row (scales[row]) stands for all its groups
+  int32_t flags_uncached; // the flags lie in uncached device memory: the wait through the scalar unit may be used
 };
 
 int zmi_smallm_grid(const ZmiProblem &p);
