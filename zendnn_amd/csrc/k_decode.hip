@@ -297,6 +297,9 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
 __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 #define D16_W_FIRST 2    // chunks of weights requested ahead of the rows
+// ... ahead of the wait for rows that are quantized inside the launch (us per call at M = 16, N = 14336, one box:
+// 4 chunks 14.40, 5 chunks 14.17, 6 chunks 14.41, 7 chunks 14.68, all 8 14.67)
+#define D16_FQ_FIRST 5
 
 // K beyond 4096 (n_slices > 1, blockIdx.y = slice): the workgroups of a column block take up to 64 chunks of K each
 // (their rows' share fits LDS as before) and leave their int32 sums in `partial` ([slice][16][N]); integers, so the
@@ -309,20 +312,22 @@ __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkm
 // back the whole L2, once per workgroup (90 us per call instead of 16).  Without `arrivals`
 // zmi_decode16_reduce_kernel finishes the elements in a launch of its own (+2 us).
 //
-// FQ: the per-token quantization of bf16 / f32 rows is part of the launch (K up to 4096).  M workgroups at the head
-// of the grid quantize one row each and stamp its flag; every other wavefront requests ALL its weights, then waits
-// for the flags through the scalar unit, then requests the rows (they return behind the weights, which the MFMAs
-// need as well) and the constants.  The scalar unit's loads do not stand in the compute unit's queue of vector
+// FQ (= chunks of weights requested ahead of the wait, 0: rows that are given): the per-token quantization of
+// bf16 / f32 rows is part of the launch (K up to 4096).  M workgroups at the head of the grid quantize one row each
+// and stamp its flag (in every copy of the flag words); every other wavefront requests most of its weights, waits
+// for the flags through the scalar unit (at a copy of its own: the waiters of the device spread over the copies'
+// memory channels), then requests the rows, the rest of the weights and the constants.  The scalar unit's loads do not stand in the compute unit's queue of vector
 // memory requests: behind the weight stream a vector load of the flags only returns with the stream (microseconds),
 // which is why the row-group kernel holds a quarter of its weights back until its wait is over.  M = 16,
-// N = 14336: 14.6 us per call against 15.9 us for the row-group kernel's form and 12.8 us with rows that are given.
+// N = 14336: 14.2 us per call against 15.9 us for the row-group kernel's form and 12.8 us with rows that are given.
 // What is left of the difference (timestamps inside the kernel): the rows are published 5 us after the launch
 // starts (2.4 us to read and quantize a row, 1.1 us until its stores are acknowledged, 1.5 us for the flag, all
 // behind the weight requests of the workgroup that shares the compute unit), a waiting wavefront sees that 1 us
 // later, and its row requests then stand at the end of its compute unit's queue: the last workgroups end 11.6 us
-// after they started against 9.7 us.  Requesting the rows ahead of the last quarter of the weights changes 0.3 us;
-// sixteen copies of the flags on different memory channels bring the wait forward by 1.3 us and the end by nothing.
-template <bool FQ>
+// after they started against 9.7 us.  Sixteen copies of the flags on different memory channels bring the end of the
+// wait forward by 1.3 us, and with the rows then requested ahead of the last three chunks of weights the call takes
+// 14.2 us (either change alone: nothing, or 0.3 us).
+template <int FQ>
 __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi, ZmiFusedQuant fq,
                                                                            int n_slices, int32_t *partial,
                                                                            unsigned int *arrivals) {
@@ -335,7 +340,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   if (FQ) {
     if (blk < M) {   // (producers wait for nothing and are dispatched first)
       zmi_fused_quant_row(fq, blk, K, reinterpret_cast<float *>(lds));
-      zmi_fq_publish(fq, blk);
+      zmi_fq_publish(fq, blk, fq.n_copies);
       return;
     }
     blk -= M;
@@ -382,13 +387,17 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     for (int u = D16_W_FIRST; u < 8; ++u) load_b(u);
   } else {
     #pragma unroll
-    for (int u = 0; u < 8; ++u) load_b(u);
-    rows_ok = zmi_fq_wait_scalar(fq, M);   // (every wavefront for itself: there is no barrier before the MFMAs)
+    for (int u = 0; u < FQ; ++u) load_b(u);
+    // (every wavefront for itself: there is no barrier before the MFMAs; the copies of the flags are ZMI_FQ_COPIES
+    // pages apart, so that the waiting wavefronts of the device do not all read one memory channel)
+    rows_ok = zmi_fq_wait_scalar(fq, M, fq.flags + (fq.n_copies > 1 ? ((blk * DEC_WAVES + wave) % fq.n_copies) * 1024 : 0));
     if (rows_ok) {
       #pragma unroll
       for (int u = 0; u < 8; ++u)
         if (c_begin + u < c_end) stage_chunk(c_begin + u);
     }
+    #pragma unroll
+    for (int u = FQ; u < 8; ++u) load_b(u);
   }
   // this thread's output element (row tid / 32, column tid % 32) and its constants, as raw words
   const int e_row = tid / 32, e_col = tid % 32;
@@ -400,7 +409,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   const uint32_t rs_word = zmi_row_scale_raw(epi, p, colsum, m_ok);
   // requests complete in order: once the rows are in LDS, at most the weight requests that followed them
   // and the 5 constant words are outstanding
-  if (FQ) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  if (FQ) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (8 - (FQ ? FQ : 8)) + 5) : "memory");
   else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (8 - D16_W_FIRST) + 5) : "memory");
   const uint32_t xm = p.a_is_u8 ? 0x80808080u : 0u;
 
@@ -764,9 +773,9 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     if (n_blk <= 0) return hipSuccess;
     const int64_t per = (zmi_blob_kpad(p.K) / 64 + slices - 1) / slices + 1;   // chunks of the longest slice, rounded up
     const size_t op = (size_t)(per < 64 ? per : 64) * 1024;
-    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel<false>, 4096 * 16);
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel<0>, 4096 * 16);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(zmi_gemm_decode16_kernel<false>, dim3(n_blk, slices), dim3(DEC_THREADS),
+    hipLaunchKernelGGL(zmi_gemm_decode16_kernel<0>, dim3(n_blk, slices), dim3(DEC_THREADS),
                        op > DEC_RED_BYTES ? op : DEC_RED_BYTES, stream, p, epi, ZmiFusedQuant{}, slices, partial, arrivals);
     e = hipGetLastError();
     if (e != hipSuccess || arrivals) return e;
@@ -790,14 +799,14 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     // (the operand area, reused by the partial tiles, and with the quantization in the launch a word per wavefront)
     const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
     const size_t smem = (op > DEC_RED_BYTES ? op : DEC_RED_BYTES) + (fq ? 64 : 0);
-    const void *f = fq ? (const void *)zmi_gemm_decode16_kernel<true> : (const void *)zmi_gemm_decode16_kernel<false>;
+    const void *f = fq ? (const void *)zmi_gemm_decode16_kernel<D16_FQ_FIRST> : (const void *)zmi_gemm_decode16_kernel<0>;
     hipError_t e = zmi_func_smem_once(f, 4096 * 16 + 64);
     if (e != hipSuccess) return e;
     if (fq)
-      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<true>, dim3(n_blk + p.M), dim3(DEC_THREADS), smem, stream, p, epi, *fq, 1,
-                         (int32_t *)nullptr, (unsigned int *)nullptr);
+      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<D16_FQ_FIRST>, dim3(n_blk + p.M), dim3(DEC_THREADS), smem, stream, p, epi, *fq,
+                         1, (int32_t *)nullptr, (unsigned int *)nullptr);
     else
-      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<false>, dim3(n_blk), dim3(DEC_THREADS), smem, stream, p, epi, ZmiFusedQuant{},
+      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<0>, dim3(n_blk), dim3(DEC_THREADS), smem, stream, p, epi, ZmiFusedQuant{},
                          1, (int32_t *)nullptr, (unsigned int *)nullptr);
     return hipGetLastError();
   }

@@ -23,10 +23,13 @@ static __device__ __forceinline__ float zmi_fused_scale_as_stored(const ZmiFused
 // ---- hand-off --------------------------------------------------------------------------
 // Producer side, called by every thread of a workgroup that has just quantized row `row`: the
 // row's flag takes the launch's epoch once all the workgroup's write-through stores have landed.
-static __device__ __forceinline__ void zmi_fq_publish(const ZmiFusedQuant &fq, int row) {
+// (copies > 1: the flag goes to that many copies of the flag words, a page apart; waiters through the scalar unit
+// spread over them, everybody else reads copy 0)
+static __device__ __forceinline__ void zmi_fq_publish(const ZmiFusedQuant &fq, int row, int copies = 1) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(&fq.flags[row], fq.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if ((int)threadIdx.x < copies)
+    __hip_atomic_store(&fq.flags[threadIdx.x * 1024 + row], fq.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Consumer side, called by whole wavefronts (every lane): polls the flags of rows 0 .. rows-1
@@ -72,7 +75,7 @@ static __device__ __forceinline__ bool zmi_fq_wait(const ZmiFusedQuant &fq, int 
 // (behind the stream, a vector load of the flags returns with the stream).  A scalar load cannot ask for device
 // scope; the flags lie in uncached device memory for it (in cached memory the XCD's L2 would keep answering with
 // the line it fetched first), and `glc` makes the load miss in the scalar cache.
-static __device__ __forceinline__ bool zmi_fq_wait_scalar(const ZmiFusedQuant &fq, int rows) {
+static __device__ __forceinline__ bool zmi_fq_wait_scalar(const ZmiFusedQuant &fq, int rows, const unsigned int *flags) {
   typedef unsigned int zmi_u16v __attribute__((ext_vector_type(16)));
   const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
   bool ok = false;
@@ -81,7 +84,7 @@ static __device__ __forceinline__ bool zmi_fq_wait_scalar(const ZmiFusedQuant &f
       bool all = true;
       for (int r0 = 0; r0 < rows; r0 += 16) {   // (rows <= 128: at most 8 loads of 16 flags)
         zmi_u16v v;
-        asm volatile("s_load_dwordx16 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=&s"(v) : "s"(fq.flags + r0) : "memory");
+        asm volatile("s_load_dwordx16 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=&s"(v) : "s"(flags + r0) : "memory");
 #pragma unroll
         for (int i = 0; i < 16; ++i) all &= (r0 + i >= rows) | (v[i] == fq.epoch);
       }

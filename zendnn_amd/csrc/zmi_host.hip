@@ -249,6 +249,9 @@ void upload_fence() {
   }
 }
 
+// copies of the hand-off flags, a page apart (the waiters of a launch spread over them)
+constexpr int kFqCopies = 16;
+
 bool fused_handoff(ZmiFusedQuant *fq) {
   ThreadCtx &c = tctx;
   if (!c.fq_flags) {
@@ -256,7 +259,7 @@ bool fused_handoff(ZmiFusedQuant *fq) {
     // (uncached: the waiting side may read the flags through the scalar unit, which cannot ask for device scope;
     // never freed -- memory of this kind that a kernel has read stays allocated until the process ends;
     // a device that refuses the uncached kind gets ordinary memory and the waits that read it with device-scope loads)
-    if (hipExtMallocWithFlags(&d, 512, hipDeviceMallocUncached) != hipSuccess) {
+    if (hipExtMallocWithFlags(&d, kFqCopies * 4096, hipDeviceMallocUncached) != hipSuccess) {
       (void)hipGetLastError();
       d = nullptr;
       if (!hip_ok(hipMalloc(&d, 512), "hipMalloc(hand-off words)")) return false;
@@ -264,7 +267,7 @@ bool fused_handoff(ZmiFusedQuant *fq) {
     } else {
       c.fq_flags_uncached = true;
     }
-    if (!hip_ok(hipMemset(d, 0, 512), "hipMemset(hand-off words)")) return false;
+    if (!hip_ok(hipMemset(d, 0, c.fq_flags_uncached ? kFqCopies * 4096 : 512), "hipMemset(hand-off words)")) return false;
     if (!hip_ok(hipHostMalloc(&h, 64, hipHostMallocMapped), "hipHostMalloc(error word)")) return false;
     std::memset(h, 0, 64);
     if (!hip_ok(hipHostGetDevicePointer(&hd, h, 0), "hipHostGetDevicePointer(error word)")) return false;
@@ -274,6 +277,7 @@ bool fused_handoff(ZmiFusedQuant *fq) {
   }
   fq->flags = c.fq_flags;
   fq->flags_uncached = c.fq_flags_uncached ? 1 : 0;
+  fq->n_copies = c.fq_flags_uncached ? kFqCopies : 1;
   if (++c.fq_epoch == 0) c.fq_epoch = 1;   // (0 is what the flags hold before the first launch)
   fq->epoch = c.fq_epoch;
   fq->error = c.fq_err_dev;

@@ -137,6 +137,7 @@ struct ZmiFusedQuant {
   uint32_t wait_ticks;    // limit of the wait in ticks of the 100 MHz real-time counter; 0: give up at once
   int32_t per_row;        // per-group kernels only: one scale per row (scales[row]) stands for all its groups
   int32_t flags_uncached; // the flags lie in uncached device memory: the wait through the scalar unit may be used
+  int32_t n_copies;       // copies of the flag words, 1024 words apart (1: just flags[0 .. M))
 };
 
 int zmi_smallm_grid(const ZmiProblem &p);
