@@ -73,6 +73,11 @@ def lib():
         L.zo_eltwise.argtypes = [C.c_int32, C.c_float, C.c_float, C.c_float]
         L.zo_matmul_int8.restype = C.c_int32
         L.zo_matmul_int8.argtypes = [C.POINTER(MatmulCall)]
+        L.zo_matmul_woq.restype = C.c_int32
+        L.zo_matmul_woq.argtypes = [C.POINTER(MatmulCall), C.c_int32]
+        L.zo_woq_dequant.restype = None
+        L.zo_woq_dequant.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32,
+                                     C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]
         L.zo_gated_act.restype = None
         L.zo_gated_act.argtypes = [C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64]
         L.zo_moe_reduce.restype = None
@@ -199,6 +204,41 @@ def matmul_int8(src, weight, params, M, N, K, *, bias=None, dst=None, lda=None, 
     call.scale_out = _p(scales)
     st = lib().zo_matmul_int8(C.byref(call))
     return st, dst, acc, scales
+
+
+def woq_dequant(packed, K, N, wei_dt, scales, scale_dt, zp=None, zp_dt=0, ldb=None, transposed=False):
+    """4-bit codes -> the bf16 weight matrix [K, N] (bits) the weight-only path multiplies with."""
+    packed = np.ascontiguousarray(packed)
+    out = np.empty((K, N), dtype=np.uint16)
+    ldb = ldb if ldb is not None else (K if transposed else N)
+    lib().zo_woq_dequant(_p(packed), K, N, ldb, int(transposed), wei_dt, _p(scales), scales.size, scale_dt,
+                         _p(zp), 0 if zp is None else zp.size, zp_dt, _p(out))
+    return out
+
+
+def matmul_woq(src, weight, params, M, N, K, *, bias=None, dst=None, lda=None, ldb=None, ldc=None,
+               transA=False, transB=False, alpha=1.0, beta=0.0, is_weights_const=True):
+    """The oracle's matmul_direct for a bf16 source with s4 / u4 weights (weight-only quantization) on host
+    arrays.  Returns (status, dst array)."""
+    src = np.ascontiguousarray(src)
+    weight = np.ascontiguousarray(weight)
+    lda = lda if lda is not None else src.shape[-1]
+    ldb = ldb if ldb is not None else (K if transB else N)
+    ldc = ldc if ldc is not None else N
+    if dst is None:
+        dst = np.zeros((M, ldc), dtype=NP_OF_DT[params.dt_dst])
+    call = MatmulCall()
+    call.layout = b"r"
+    call.transA, call.transB = int(transA), int(transB)
+    call.M, call.N, call.K = M, N, K
+    call.alpha, call.beta = alpha, beta
+    call.src, call.lda = _p(src), lda
+    call.weight, call.ldb = _p(weight), ldb
+    call.bias = _p(bias)
+    call.dst, call.ldc = _p(dst), ldc
+    call.params = C.pointer(params)
+    st = lib().zo_matmul_woq(C.byref(call), int(is_weights_const))
+    return st, dst
 
 
 def gated_act(act, buf, dt):

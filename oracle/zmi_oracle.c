@@ -775,6 +775,100 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
   return ZMI_SUCCESS;
 }
 
+/* ---- weight-only quantization ---------------------------------------------------------- */
+
+/* cvt_int4_to_bf16, lowoha_operators/matmul/backends/aocl/aocl_kernel.cpp:43-139: every 4-bit code of the K x N
+ * weight matrix (physical nibble index row * ldb + col, or col * ldb + row when transposed; even index = low nibble;
+ * s4 codes sign-extended, u4 codes as they are) becomes one bf16 value,
+ *   f = float(code); f = (f - zp) * scale, or for u4 codes with a bf16 zero-point f = (f - 8) * scale + zp;
+ *   out[row * N + col] = bfloat16_t(f),
+ * the scale / zero-point read per tensor (1 element), per column (N elements) or per K group and column
+ * (element count / N groups of K / groups rows each: index group * N + col). */
+ZO_EXPORT void zo_woq_dequant(const void *packed, int64_t K, int64_t N, int64_t ldb, int32_t transposed, int32_t wei_dt,
+                              const void *scales, int64_t scale_n, int32_t scale_dt,
+                              const void *zp, int64_t zp_n, int32_t zp_dt, uint16_t *out) {
+  const uint8_t *w = (const uint8_t *)packed;
+  const int float_domain_u4 = zp_dt == ZMI_DT_BF16 && wei_dt == ZMI_DT_U4;
+  int64_t group_size = K;
+  if (scale_n > 1 && scale_n != N) {
+    const int64_t groups = scale_n / N;
+    if (groups > 0) group_size = K / groups;
+  }
+  for (int64_t row = 0; row < K; ++row)
+    for (int64_t col = 0; col < N; ++col) {
+      const int64_t idx = transposed ? col * ldb + row : row * ldb + col;
+      const uint8_t byte = w[idx / 2];
+      int32_t v = (idx % 2 == 0) ? (byte & 0x0F) : (byte >> 4);
+      if (wei_dt == ZMI_DT_S4 && (v & 0x08)) v -= 16;
+      float f = (float)v;
+      const int64_t so = scale_n <= 1 ? 0 : scale_n == N ? col : (row / group_size) * N + col;
+      const float scale = scale_n ? zo_read_f32(scales, scale_dt, so) : 1.0f;
+      float zpv = 0.0f;
+      if (zp_n >= 1) zpv = zo_read_f32(zp, zp_dt, zp_n == 1 ? 0 : zp_n == N ? col : (row / group_size) * N + col);
+      if (float_domain_u4) {
+        f = (f - 8) * scale;
+        f = f + zpv;
+      } else {
+        f = (f - zpv) * scale;
+      }
+      out[row * N + col] = zo_f32_to_bf16_ctor(f);
+    }
+}
+
+/* matmul_direct with a bf16 source, s4 / u4 weights and no dynamic_quant.  Rules: validate_matmul_direct_inputs,
+ * lowoha_operators/matmul/lowoha_matmul_utils.cpp:214-328 (constant weights, no source / destination quantization
+ * parameters, u4 weights need a bf16 or s8 zero-point, a bf16 source does not store f16).  Arithmetic: the weights
+ * become bf16 once (zo_woq_dequant), then the bf16 GEMM with f32 accumulation in k order and the tail of
+ * compute_matmul, operators/matmul/matmul_ref_kernel.cpp:877-896: sum *= alpha (if != 1); sum += C * beta (if beta);
+ * sum += bias; then the post-ops in order and the store (no destination quantization on this path, :499-502).
+ * The reference's own GEMM on the bf16 matrix is AOCL's, whose summation order is not part of its contract: results
+ * are compared with this function to a tolerance, not bit for bit. */
+ZO_EXPORT int32_t zo_matmul_woq(const zo_matmul_call *c, int32_t is_weights_const) {
+  const zmi_matmul_params_t *p = c->params;
+  const int64_t M = c->M, N = c->N, K = c->K;
+  if (!(p->dt_src == ZMI_DT_BF16 && (p->dt_wei == ZMI_DT_S4 || p->dt_wei == ZMI_DT_U4) && !p->dynamic_quant))
+    return ZMI_UNIMPLEMENTED;
+  if (!is_weights_const) return ZMI_FAILURE;
+  if (p->src_scale.buff || p->dst_scale.buff || p->src_zp.buff || p->dst_zp.buff) return ZMI_FAILURE;
+  if (p->dt_wei == ZMI_DT_U4 && (!p->wei_zp.buff || (p->wei_zp.dt != ZMI_DT_BF16 && p->wei_zp.dt != ZMI_DT_S8)))
+    return ZMI_FAILURE;
+  if (p->dt_dst == ZMI_DT_F16 || !p->wei_scale.buff) return ZMI_FAILURE;
+  const int64_t ns = zo_nelems(&p->wei_scale), nz = p->wei_zp.buff ? zo_nelems(&p->wei_zp) : 0;
+  if (!(ns == 1 || ns == N || (ns > N && ns % N == 0 && K % (ns / N) == 0))) return ZMI_FAILURE;
+  if (nz && !(nz == 1 || nz == N || nz == ns)) return ZMI_FAILURE;
+  uint16_t *wb = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)K * N);
+  zo_woq_dequant(c->weight, K, N, c->ldb, c->transB, p->dt_wei, p->wei_scale.buff, ns,
+                 p->wei_scale.dt == ZMI_DT_NONE ? ZMI_DT_F32 : p->wei_scale.dt, p->wei_zp.buff, nz, p->wei_zp.dt, wb);
+  const uint16_t *A = (const uint16_t *)c->src;
+  #pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      float sum = 0.0f;
+      for (int64_t k = 0; k < K; ++k)
+        sum += zo_bf16_to_f32(A[c->transA ? k * c->lda + m : m * c->lda + k]) * zo_bf16_to_f32(wb[k * N + n]);
+      float y = sum;
+      const int64_t o = m * (int64_t)c->ldc + n;
+      if (c->alpha != 1.0f) y *= c->alpha;
+      if (c->beta != 0.0f) y += zo_read_f32(c->dst, p->dt_dst, o) * c->beta;
+      if (c->bias) y += zo_read_f32(c->bias, p->dt_bias == ZMI_DT_NONE ? ZMI_DT_F32 : p->dt_bias, n);
+      for (int i = 0; i < p->n_postops; ++i) {
+        const zmi_post_op_t *po = &p->postops[i];
+        if (po->po_type == ZMI_PO_BINARY_ADD || po->po_type == ZMI_PO_BINARY_MUL) {
+          int64_t ld = po->leading_dim > 0 ? po->leading_dim : N;
+          int rowb = (po->ndims == 2 && po->dims[0] == 1) || po->ndims == 1;
+          float t = zo_read_f32(po->buff, po->dtype, rowb ? n : m * ld + n);
+          y = po->po_type == ZMI_PO_BINARY_ADD ? y + t : y * t;
+        } else {
+          y = zo_eltwise(po->po_type, y, po->alpha, po->beta);
+        }
+      }
+      zo_store(c->dst, p->dt_dst, o, y);
+    }
+  }
+  free(wb);
+  return ZMI_SUCCESS;
+}
+
 /* ---- gated activation ----------------------------------------------------- */
 
 /* silu_and_mul_row_scalar_{bf16,f32}, gelu_and_mul_*, swiglu_oai_mul_*,

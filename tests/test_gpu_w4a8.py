@@ -135,7 +135,7 @@ def test_w4a8_rejections(zo):
     assert call(src=capi.DT_F32) == capi.FAILURE
     assert call(dst_dt=capi.DT_F32) == capi.FAILURE
     assert call(compute=capi.DT_BF16) == capi.FAILURE
-    assert call(dyn=False) == capi.UNIMPLEMENTED           # weight-only quantization is another path
+    assert call(dyn=False) == capi.SUCCESS                 # weight-only quantization: another path (test_gpu_woq.py)
     assert call(sdims=(M, 3)) == capi.FAILURE
     assert call(wdims=(G, N - 1)) == capi.FAILURE
     assert call(wdims=(3, N)) == capi.FAILURE

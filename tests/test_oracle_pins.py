@@ -760,3 +760,127 @@ def test_moe_reduce_closed_form_and_brute_force(zo):
     ones = zo.moe_reduce(rows, w, capi.DT_BF16, D, skip_weighted=True)
     t0 = sum(zo.bf16_to_f32(rows[k]).astype(np.float64) for k in range(topk))
     assert np.abs(zo.bf16_to_f32(ones[0]) - t0).max() < 0.05
+
+
+# ------------------------------------------------- weight-only quantization
+def _nib_pack(flat):
+    flat = np.asarray(flat, dtype=np.int64) & 15
+    if flat.size % 2:
+        flat = np.append(flat, 0)
+    return (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)
+
+
+def test_woq_nibble_order_sign_extension_and_orientation(zo):
+    # byte 0x21 holds index 0 -> 1 (low nibble) and index 1 -> 2; 0xF8 holds 8 -> -8 (s4) / 8 (u4) and 15 -> -1 / 15
+    packed = np.array([0x21, 0xF8], dtype=np.uint8)
+    one = np.ones(1, dtype=np.float32)
+    got = zo.bf16_to_f32(zo.woq_dequant(packed, 2, 2, capi.DT_S4, one, capi.DT_F32))
+    assert got.tolist() == [[1.0, 2.0], [-8.0, -1.0]]
+    got = zo.bf16_to_f32(zo.woq_dequant(packed, 2, 2, capi.DT_U4, one, capi.DT_F32))
+    assert got.tolist() == [[1.0, 2.0], [8.0, 15.0]]
+    # transposed: element (row, col) sits at nibble col * ldb + row
+    got = zo.bf16_to_f32(zo.woq_dequant(packed, 2, 2, capi.DT_S4, one, capi.DT_F32, transposed=True))
+    assert got.tolist() == [[1.0, -8.0], [2.0, -1.0]]
+    # a leading dimension of 3 nibbles: rows start at nibbles 0 and 3
+    packed = _nib_pack([1, 2, 7, 3, 4, 7])
+    got = zo.bf16_to_f32(zo.woq_dequant(packed, 2, 2, capi.DT_S4, one, capi.DT_F32, ldb=3))
+    assert got.tolist() == [[1.0, 2.0], [3.0, 4.0]]
+
+
+def test_woq_dequantization_formulas_where_every_step_is_exact(zo):
+    # scales and zero-points that keep every operation exact: the two formulas give different, known values
+    codes = np.arange(16).reshape(16, 1)
+    packed = _nib_pack(np.repeat(codes, 2, axis=1).reshape(-1))     # [16, 2], both columns the same code
+    scale = np.array([0.25], dtype=np.float32)
+    zp8 = np.array([3], dtype=np.int8)
+    zpf = zo.f32_to_bf16(np.array([0.5], dtype=np.float32))
+    u = np.arange(16, dtype=np.float64)
+    s = np.where(u >= 8, u - 16, u)
+    col = lambda a: zo.bf16_to_f32(a)[:, 0].astype(np.float64)
+    assert np.array_equal(col(zo.woq_dequant(packed, 16, 2, capi.DT_S4, scale, capi.DT_F32)), s * 0.25)
+    assert np.array_equal(col(zo.woq_dequant(packed, 16, 2, capi.DT_S4, scale, capi.DT_F32, zp8, capi.DT_S8)), (s - 3) * 0.25)
+    assert np.array_equal(col(zo.woq_dequant(packed, 16, 2, capi.DT_U4, scale, capi.DT_F32, zp8, capi.DT_S8)), (u - 3) * 0.25)
+    # u4 codes with a bf16 zero-point: the midpoint 8 comes off, the zero-point is added after the scale
+    assert np.array_equal(col(zo.woq_dequant(packed, 16, 2, capi.DT_U4, scale, capi.DT_F32, zpf, capi.DT_BF16)), (u - 8) * 0.25 + 0.5)
+    # s4 codes with a bf16 zero-point stay on the first formula
+    assert np.array_equal(col(zo.woq_dequant(packed, 16, 2, capi.DT_S4, scale, capi.DT_F32, zpf, capi.DT_BF16)), (s - 0.5) * 0.25)
+
+
+def test_woq_dequantization_granularities_and_rounding_against_torch(zo):
+    # bf16-valued scales: (code - zp) * scale has at most 14 significant bits, so the f32 product is exact and the
+    # one rounding left is the bf16 one, which torch does from the exact double product
+    rng = np.random.default_rng(77)
+    K, N, G = 48, 10, 3
+    codes = rng.integers(-8, 8, (K, N))
+    packed = _nib_pack(codes.reshape(-1))
+    for dims in ((1, 1), (1, N), (G, N)):
+        sc_bits = zo.f32_to_bf16(rng.uniform(0.01, 0.3, dims).astype(np.float32))
+        sc = zo.bf16_to_f32(sc_bits).astype(np.float64)
+        zp = rng.integers(-4, 5, dims).astype(np.int8)
+        rows = np.arange(K) // (K // dims[0]) if dims[0] > 1 else np.zeros(K, dtype=np.int64)
+        sc_full = np.broadcast_to(sc, (dims[0], N))[rows]
+        zp_full = np.broadcast_to(zp, (dims[0], N))[rows].astype(np.float64)
+        exact = (codes - zp_full) * sc_full
+        want = torch.from_numpy(exact).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        got = zo.woq_dequant(packed, K, N, capi.DT_S4, sc_bits.reshape(-1), capi.DT_BF16, zp.reshape(-1), capi.DT_S8)
+        assert np.array_equal(got, want), dims
+
+
+def test_woq_product_is_the_double_precision_product_of_the_bf16_operands(zo):
+    rng = np.random.default_rng(78)
+    M, K, N, G = 6, 96, 20, 4
+    codes = rng.integers(0, 16, (K, N))
+    packed = _nib_pack(codes.reshape(-1))
+    sc = rng.uniform(0.01, 0.1, (G, N)).astype(np.float32)
+    zp = zo.f32_to_bf16(rng.uniform(-0.2, 0.2, (G, N)).astype(np.float32))
+    x = zo.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    bias = rng.standard_normal(N).astype(np.float32)
+    c0 = rng.standard_normal((M, N)).astype(np.float32)
+    p = _params(dt_src=capi.DT_BF16, dt_wei=capi.DT_U4, dt_dst=capi.DT_F32, dt_bias=capi.DT_F32,
+                wei_scale=capi.quant(sc.ctypes.data, capi.DT_F32, (G, N)),
+                wei_zp=capi.quant(zp.ctypes.data, capi.DT_BF16, (G, N)))
+    st, got = zo.matmul_woq(x, packed, p, M, N, K, bias=bias, dst=c0.copy(), alpha=0.5, beta=2.0)
+    assert st == capi.SUCCESS
+    wb = zo.bf16_to_f32(zo.woq_dequant(packed, K, N, capi.DT_U4, sc.reshape(-1), capi.DT_F32, zp.reshape(-1), capi.DT_BF16))
+    xf = zo.bf16_to_f32(x).astype(np.float64)
+    want = 0.5 * (xf @ wb.astype(np.float64)) + 2.0 * c0 + bias
+    mag = 0.5 * (np.abs(xf) @ np.abs(wb.astype(np.float64))) + 2.0 * np.abs(c0) + np.abs(bias)
+    assert (np.abs(got - want) <= 2e-6 * mag).all()
+    # integer-valued operands and a power-of-two scale: every partial sum is exact in f32, any order gives this
+    xi = zo.f32_to_bf16(rng.integers(-4, 5, (M, K)).astype(np.float32))
+    half = np.array([0.5], dtype=np.float32)
+    z8 = np.array([7], dtype=np.int8)
+    p = _params(dt_src=capi.DT_BF16, dt_wei=capi.DT_U4, dt_dst=capi.DT_F32,
+                wei_scale=capi.quant(half.ctypes.data, capi.DT_F32, (1, 1)), wei_zp=capi.quant(z8.ctypes.data, capi.DT_S8, (1, 1)))
+    st, got = zo.matmul_woq(xi, packed, p, M, N, K)
+    assert st == capi.SUCCESS
+    assert np.array_equal(got, zo.bf16_to_f32(xi).astype(np.float64) @ ((codes - 7) * 0.5))
+
+
+def test_woq_rejections_follow_the_reference_validator(zo):
+    M, K, N, G = 2, 32, 4, 2
+    x = np.zeros((M, K), dtype=np.uint16)
+    packed = np.zeros(K * N // 2, dtype=np.uint8)
+    ws = np.ones((G, N), dtype=np.float32)
+    z8 = np.zeros((G, N), dtype=np.int8)
+
+    def call(wei=capi.DT_S4, dst=capi.DT_BF16, const=True, zp=None, zp_dt=capi.DT_S8, extra=None, scale=True, dyn=0):
+        kw = dict(dt_src=capi.DT_BF16, dt_wei=wei, dt_dst=dst, dynamic_quant=dyn)
+        if scale:
+            kw["wei_scale"] = capi.quant(ws.ctypes.data, capi.DT_F32, (G, N))
+        if zp is not None:
+            kw["wei_zp"] = capi.quant(zp.ctypes.data, zp_dt, (G, N))
+        if extra:
+            kw[extra] = capi.quant(ws.ctypes.data, capi.DT_F32, (1, 1))
+        return zo.matmul_woq(x, packed, _params(**kw), M, N, K, is_weights_const=const)[0]
+
+    assert call() == capi.SUCCESS
+    assert call(wei=capi.DT_U4, zp=z8) == capi.SUCCESS
+    assert call(const=False) == capi.FAILURE
+    assert call(extra="src_scale") == capi.FAILURE
+    assert call(extra="dst_scale") == capi.FAILURE
+    assert call(wei=capi.DT_U4) == capi.FAILURE                      # u4 without a zero-point
+    assert call(wei=capi.DT_U4, zp=z8, zp_dt=capi.DT_S32) == capi.FAILURE
+    assert call(dst=capi.DT_F16) == capi.FAILURE
+    assert call(scale=False) == capi.FAILURE
+    assert call(dyn=1) == capi.UNIMPLEMENTED                         # W4A8: zo_matmul_int8's

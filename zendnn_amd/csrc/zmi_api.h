@@ -11,4 +11,9 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan);
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA);
 bool use_ring_kernel(int M, int N, int K);
+// weight-only quantization (zmi_api_woq.hip): bf16 source, s4 / u4 weights, no dynamic_quant
+bool is_woq_config(const zmi_matmul_params_t &p);
+int32_t matmul_woq(char layout, int32_t transA, int32_t transB, int32_t M, int32_t N, int32_t K, float alpha,
+                   const void *src, int32_t lda, const void *weight, int32_t ldb, const void *bias, float beta, void *dst,
+                   int32_t ldc, int32_t is_weights_const, const zmi_matmul_params_t &p);
 }  // namespace zmi

@@ -388,7 +388,7 @@ int32_t validate_w4a8(const zmi_matmul_params_t &p, int M, int N, int K) {
   if (p.dt_src == ZMI_DT_U8 && (p.src_scale.buff || p.dynamic_quant)) { set_error("s4 weights with a u8 source: the 4-bit path is symmetric and starts from bf16"); return ZMI_FAILURE; }
   const bool entry = p.dynamic_quant && p.dt_src == ZMI_DT_BF16;
   if (entry && p.dt_compute != ZMI_DT_S8) { set_error("s4 weights with dynamic_quant: dt_compute must be s8"); return ZMI_FAILURE; }
-  if (!entry) { set_error("s4 weights: only W4A8 (bf16 source, dynamic_quant, s8 compute) is implemented, not weight-only quantization"); return ZMI_UNIMPLEMENTED; }
+  if (!entry) { set_error("s4 weights go with a bf16 source: with dynamic_quant and s8 compute (W4A8), or without dynamic_quant (weight-only quantization)"); return ZMI_FAILURE; }
   if (p.dt_dst != ZMI_DT_BF16) { set_error("s4 weights with dynamic_quant: dt_dst must be bf16"); return ZMI_FAILURE; }
   if (p.wei_zp.buff || p.src_zp.buff) { set_error("s4 weights with dynamic_quant: zero-points are not taken (weights and source are symmetric)"); return ZMI_FAILURE; }
   const zmi_quant_t &ws = p.wei_scale;
@@ -442,6 +442,8 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
                              const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
                              const zmi_matmul_params_t &p) {
   const int Batch_A = 1, Batch_B = 1;
+  if (is_woq_config(p))
+    return matmul_woq(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc, is_weights_const, p);
   const bool w4a8 = p.dt_wei == ZMI_DT_S4;
   if (w4a8) {
     // (the shape rules of this path keep the kernels inside their buffers: checked whatever the diagnostics switch says)
@@ -457,7 +459,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     return ZMI_FAILURE;
   }
   // ---- what this library implements of matmul_direct: the int8 path ----
-  if (p.dt_wei != ZMI_DT_S8 && !w4a8) { set_error("only s8 and (W4A8) s4 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+  if (p.dt_wei != ZMI_DT_S8 && !w4a8) { set_error("weights: s8, s4 (W4A8, or weight-only with a bf16 source) or u4 (weight-only with a bf16 source)"); return ZMI_UNIMPLEMENTED; }
   if (layout != 'r' && layout != 'R') { set_error("only row-major layout is implemented"); return ZMI_UNIMPLEMENTED; }
   const bool ggml = p.pack_format_b == 1;
   if (p.pack_format_b != 0 && !ggml) { set_error("unknown pack_format_b"); return ZMI_FAILURE; }

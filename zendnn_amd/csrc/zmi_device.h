@@ -64,6 +64,10 @@ static inline __host__ __device__ int64_t zmi_s4_nb_stride(int64_t K) { return z
 static inline __host__ __device__ int64_t zmi_s4_tiles_bytes(int64_t K, int64_t N) {
   return zmi_s4_nb_stride(K) * (zmi_blob_npad(N) / 32);
 }
+// 4-bit tiles of the weight-only path (k_woq.hip): [ceil(N/32)][ceil(K/64)] pieces of 1 KiB
+static inline __host__ __device__ int64_t zmi_woq_tiles_bytes(int64_t K, int64_t N) {
+  return ((N + 31) / 32) * ((K + 63) / 64) * 1024;
+}
 static inline __host__ __device__ int64_t zmi_blob_bytes(int64_t K, int64_t N) {
   return zmi_blob_tiles_off(N) + zmi_blob_nb_stride(K) * (zmi_blob_npad(N) / 32);
 }

@@ -90,6 +90,10 @@ const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const 
 // *tiles_s4 receives the 4-bit tiles kept behind a cached blob (null when not cached: a one-off pack streams s8).
 const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
                                  void *widen_slot, void *arena_slot, const uint8_t **tiles_s4);
+// packed s4 / u4 weights of the weight-only path: the codes in the kernel's tile order (zmi_woq_tiles_bytes(K, N)
+// bytes), cached like the others or written into arena_slot.
+const uint32_t *packed_woq_tiles(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
+                                 void *arena_slot);
 void clear_weight_cache();
 
 // Checks (once per pointer) that a caller-supplied blob carries the header of a

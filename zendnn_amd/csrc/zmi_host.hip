@@ -474,6 +474,41 @@ const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64
   return (const uint8_t *)blob;
 }
 
+// Weight-only quantization: the 4-bit codes in the order the kernel's wavefronts read them (reference:
+// woqReorderAndCacheWeightsAocl, matmul/backends/aocl/aocl_kernel.cpp:640-702, which caches the dequantized bf16
+// matrix; the codes stay 4-bit here).  The key's leading dimension is stored negated and far below W4A8's.
+const uint32_t *packed_woq_tiles(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
+                                 void *arena_slot) {
+  if (!use_cache) {
+    if (!hip_ok(zmi_launch_woq_tiles(weight, K, N, ldb, transB, (uint32_t *)arena_slot, stream()), "4-bit tiles launch"))
+      return nullptr;
+    return (const uint32_t *)arena_slot;
+  }
+  std::lock_guard<std::mutex> lk(g_mu);
+  CacheKey key{weight, K, N, -ldb - ((int64_t)1 << 40), transB};
+  auto it = g_cache.find(key);
+  if (it != g_cache.end()) {
+    g_lru.splice(g_lru.begin(), g_lru, it->second.lru);
+    return (const uint32_t *)it->second.blob;
+  }
+  void *blob = nullptr;
+  if (!hip_ok(hipMalloc(&blob, (size_t)zmi_woq_tiles_bytes(K, N)), "hipMalloc(4-bit tiles)")) return nullptr;
+  if (!hip_ok(zmi_launch_woq_tiles(weight, K, N, ldb, transB, (uint32_t *)blob, stream()), "4-bit tiles launch")) {
+    (void)hipFree(blob);
+    return nullptr;
+  }
+  g_lru.push_front(key);
+  g_cache[key] = CacheVal{(uint8_t *)blob, g_lru.begin()};
+  while (g_cache.size() > cache_capacity()) {
+    (void)hipDeviceSynchronize();
+    CacheKey old = g_lru.back();
+    g_lru.pop_back();
+    (void)hipFree(g_cache[old].blob);
+    g_cache.erase(old);
+  }
+  return (const uint32_t *)blob;
+}
+
 void clear_weight_cache() {
   std::lock_guard<std::mutex> lk(g_mu);
   if (!g_cache.empty()) (void)hipDeviceSynchronize();

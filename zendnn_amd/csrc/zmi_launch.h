@@ -177,6 +177,35 @@ hipError_t zmi_launch_pgring_scales(const void *src, int32_t dt, int64_t rows, i
 // p.A: s8 rows in fragment order; ss: {M, G} f32 source scales; ws: the padded f32 weight scales
 hipError_t zmi_launch_gemm_pgring(const ZmiProblem &p, const ZmiEpilogue &epi, const float *ss, const float *ws,
                                   hipStream_t stream);
+// Weight-only quantization (k_woq.hip): bf16 rows x 4-bit weights dequantized to bf16 in registers, f32 accumulation.
+struct ZmiWoqProblem {
+  const void *A;            // bf16 [M, lda] (or [K, lda] when transA)
+  int64_t lda;
+  int32_t transA;
+  int32_t a_fast;           // rows can be read 16 bytes at a time (no transA, K, lda multiples of 8, 16-byte aligned base)
+  const uint32_t *tiles;    // zmi_woq_tiles_bytes(K, N) bytes from zmi_launch_woq_tiles
+  void *dst;
+  int64_t ldc;
+  int32_t M, N, K;
+  int32_t is_u4;            // codes 0 .. 15 instead of -8 .. 7
+  int32_t has_zp;
+  int32_t zp_float_domain;  // u4 codes with a bf16 zero-point: (code - 8) * scale + zp
+  // scale / zero-point: mode 0 = one value (the pointer, or the value when it is null), 1 = one per column,
+  // 2 = one per K group and column, {n_groups, N}
+  const void *scale;
+  const void *zp;
+  int32_t scale_dt, scale_mode;
+  int32_t zp_dt, zp_mode;
+  float scale_val, zp_val;
+  int32_t group_size;       // K / n_groups
+  int32_t n_groups;
+  const void *bias;
+};
+hipError_t zmi_launch_woq_tiles(const void *packed, int64_t K, int64_t N, int64_t ldb, bool transB, uint32_t *out,
+                                hipStream_t stream);
+// (of the epilogue descriptor only alpha, beta, bias_dt, the post-ops and dst_dt are read)
+hipError_t zmi_launch_gemm_woq(const ZmiWoqProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+
 // 4-bit tiles of a blob of widened s4 weights (zmi_s4_tiles_bytes(K, N) bytes)
 hipError_t zmi_launch_s4_tiles(const uint8_t *blob, int64_t K, int64_t N, uint8_t *out, hipStream_t stream);
 // per (row, group) dynamic quantization of bf16 / f32 rows: s8 rows (ld ldq), f32 scales {M,G} and an
