@@ -41,7 +41,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configs and the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "decode_M16_w4a8_group128", "decode_M16_w4a8_group128_per_token_rows", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
+                    choices=["decode_M1", "decode_M4", "decode_M64", "decode_M128", "decode_M16_per_group128", "decode_M16_per_group32", "decode_M16_w4a8_group128", "decode_M16_w4a8_group128_per_token_rows", "decode_M16_woq_s4_group128", "decode_M16_woq_u4_group128", "decode_M1_woq_s4_group128", "prefill_N4096", "prefill_N14336", "config1_u8s8_M128",
                              "decode_M16_K14336_N4096", "prefill_N14336_per_group128", "prefill_N14336_per_group32",
                              "moe_decode_T16", "moe_config4", "moe_config5"],
                     help="run one of the other configs alone and print its entry (for profiler runs)")
@@ -351,6 +351,39 @@ def main():
         capi.load().zmi_clear_weight_cache()
         return out
 
+    def run_decode_woq(m, gs, u4):
+        # weight-only quantization at decode: bf16 rows as they are, packed s4 (or u4 with bf16 zero-points) weights with
+        # {G,N} scales, dequantized to bf16 in registers in front of the bf16 MFMA; the 4-bit tiles are made and cached
+        # on the first call per weight pointer (outside the timed region).  bytes = 4-bit weights + rows + scales
+        # (+ zero-points) + output.
+        G = K_DEC // gs
+        ws4 = [torch.randint(0, 256, (K_DEC * N_DEC // 2,), dtype=torch.uint8, device=dev, generator=g) for _ in range(n_sets)]
+        ws = torch.rand((G, N_DEC), device=dev, generator=g) * 0.009 + 0.001
+        zp = (torch.rand((G, N_DEC), device=dev, generator=g) * 0.1).to(torch.bfloat16)
+        x = torch.randn((m, K_DEC), device=dev, generator=g).to(torch.bfloat16)
+        dst = torch.zeros((m, N_DEC), dtype=torch.bfloat16, device=dev)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_U4 if u4 else capi.DT_S4, dst=capi.DT_BF16)
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (G, N_DEC))
+        if u4:
+            p.wei_zp = lowoha.QuantParam(zp, capi.DT_BF16, (G, N_DEC))
+        p.postop_ = [lowoha.PostOp(capi.PO_SWISH)]
+        calls = [lowoha.prepared_matmul("r", False, False, m, N_DEC, K_DEC, 1.0, x, K_DEC, w4, N_DEC, None, 0.0,
+                                        dst, N_DEC, True, p)[0] for w4 in ws4]
+        state = {"i": 0}
+
+        def step():
+            st = calls[state["i"] % n_sets]()
+            state["i"] += 1
+            if st != capi.SUCCESS:
+                raise RuntimeError(lowoha.last_error())
+
+        t = ev_time(step, 100, 2 * n_sets)
+        nbytes = K_DEC * N_DEC // 2 + m * K_DEC * 2 + G * N_DEC * (6 if u4 else 4) + m * N_DEC * 2
+        out = {"GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "us_per_call": round(t * 1e3, 2), "group_size": gs,
+               "weights": "u4, bf16 zero-points" if u4 else "s4", "kernel": lowoha.last_kernel()}
+        capi.load().zmi_clear_weight_cache()
+        return out
+
     def run_decode_down(m):
         # the down projection of the same block at decode: K = 14336, N = 4096, bf16 rows quantized per token by the
         # call (a launch of its own), then the 16-row kernel in K slices; bytes = weights + rows + scales + output
@@ -472,6 +505,9 @@ def main():
         "decode_M16_per_group32": lambda: run_decode_per_group(16, 32),
         "decode_M16_w4a8_group128": lambda: run_decode_w4a8(16, 128, False),
         "decode_M16_w4a8_group128_per_token_rows": lambda: run_decode_w4a8(16, 128, True),
+        "decode_M16_woq_s4_group128": lambda: run_decode_woq(16, 128, False),
+        "decode_M16_woq_u4_group128": lambda: run_decode_woq(16, 128, True),
+        "decode_M1_woq_s4_group128": lambda: run_decode_woq(1, 128, False),
         "prefill_N4096": lambda: run_prefill(4096),
         "prefill_N14336": lambda: run_prefill(14336),
         "config1_u8s8_M128": run_config1,

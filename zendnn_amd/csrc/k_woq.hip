@@ -5,7 +5,7 @@
 //   f = float(code); f = (f - zp) * scale, or (f - 8) * scale + zp for u4 codes with a bf16 zero-point;
 //   w = bfloat16_t(f)), caches the bf16 matrix and runs a bf16 GEMM with f32 accumulation on it.  Here the weights stay
 // 4-bit in memory (a quarter of the bf16 matrix, the bound of a decode-shaped call) and every workgroup makes the
-// same bf16 values in registers, with the same three f32 operations and the same rounding, right before the MFMA.
+// same bf16 values in registers, with f32 operations that round like the reference's, right before the MFMA.
 //
 // Tiles: [N/32][K/64] pieces of 1 KiB; lane l of a wavefront owns 16 bytes of a piece = 4 dwords, dword t holding the
 // 8 codes (k = 64*kc + 16*t + 8*(l/32) + j, j = 0..7 from the low nibble up; n = 32*nb + l%32): the B operand of four
@@ -17,12 +17,15 @@
 // loop after it).
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../../include/zmi_lowoha.h"
 #include "zmi_device.h"
 #include "zmi_launch.h"
 
 typedef __bf16 woq_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float woq_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t woq_u32x4 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------------------------------------------- tiles
 __global__ __launch_bounds__(256) void zmi_woq_tiles_kernel(const uint8_t *packed, int64_t K, int64_t N, int64_t ldb,
@@ -54,64 +57,113 @@ hipError_t zmi_launch_woq_tiles(const void *packed, int64_t K, int64_t N, int64_
   return hipGetLastError();
 }
 
+// Scales and zero-points as f32, one per K group and column ([n_groups][N]), whatever their type and granularity were:
+// they belong to the weights and are kept with the tiles (the reference bakes them into its cached bf16 matrix).
+__global__ __launch_bounds__(256) void zmi_woq_params_kernel(ZmiWoqParamSrc s, ZmiWoqParamSrc z, int64_t G, int64_t N,
+                                                             float *sf, float *zf) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= G * N) return;
+  const int64_t g = i / N, n = i % N;
+  sf[i] = s.ptr ? zmi_ld_f32(s.ptr, s.dt, s.mode == 0 ? 0 : s.mode == 1 ? n : g * N + n) : s.val;
+  zf[i] = z.ptr ? zmi_ld_f32(z.ptr, z.dt, z.mode == 0 ? 0 : z.mode == 1 ? n : g * N + n) : z.val;
+}
+
+hipError_t zmi_launch_woq_params(const ZmiWoqParamSrc &s, const ZmiWoqParamSrc &z, int64_t G, int64_t N, float *sf,
+                                 float *zf, hipStream_t stream) {
+  hipLaunchKernelGGL(zmi_woq_params_kernel, dim3((unsigned)((G * N + 255) / 256)), dim3(256), 0, stream, s, z, G, N, sf, zf);
+  return hipGetLastError();
+}
+
 // ---------------------------------------------------------------------------------------------------- GEMM
 // Q: 0 = s4 codes, no zero-point; 1 = s4 codes with a zero-point; 2 = u4 codes, (code - zp) * scale;
 //    3 = u4 codes, (code - 8) * scale + zp
+// 8 codes of one dword -> 8 bf16 values.  Q = 1 takes the codes one by one (signed field, conversion, subtraction,
+// multiplication).  The others go through the byte conversions: the even and the odd nibbles are spread over the bytes
+// of two words, each byte converted exactly (s4 codes after flipping their top bits: code + 8); then
+//   Q = 0: fma(code + 8, s, -8 s) -- the exact product code * s rounded once, which is the reference's multiplication
+//          (-8 s is exact: a power of two);
+//   Q = 2: (code - zp) * s as written;  Q = 3: fma(code, s, -8 s) = the rounded (code - 8) * s, then + zp.
+// byte B of a word as f32 (the conversion instruction that names its byte: the compiler finds it only for byte 0
+// once it knows that the bytes hold nibbles)
+template <int B>
+__device__ __forceinline__ float woq_byte_f32(uint32_t x) {
+  float f;
+  if (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(x));
+  else if (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(x));
+  else if (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(x));
+  else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(x));
+  return f;
+}
+
 template <int Q>
 __device__ __forceinline__ woq_bf16x8 woq_dequant(uint32_t d, float s, float z) {
   uint32_t o[4];
+  if (Q == 1) {
 #pragma unroll
-  for (int jj = 0; jj < 4; ++jj) {
-    float f[2];
+    for (int jj = 0; jj < 4; ++jj) {
+      float f[2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int j = 2 * jj + h;
-      const int v = Q >= 2 ? (int)((d >> (4 * j)) & 15u) : ((int)(d << (28 - 4 * j)) >> 28);
-      float x = (float)v;
-      if (Q == 0) x = __fmul_rn(x, s);
-      else if (Q == 3) x = __fadd_rn(__fmul_rn(__fsub_rn(x, 8.0f), s), z);
-      else x = __fmul_rn(__fsub_rn(x, z), s);
-      f[h] = x;
+      for (int h = 0; h < 2; ++h) {
+        const int j = 2 * jj + h;
+        f[h] = __fmul_rn(__fsub_rn((float)((int)(d << (28 - 4 * j)) >> 28), z), s);
+      }
+      o[jj] = zmi_pack_bf16(f[0], f[1]);
     }
+  } else {
+    if (Q == 0) d ^= 0x88888888u;
+    const uint32_t ev = d & 0x0f0f0f0fu, od = (d >> 4) & 0x0f0f0f0fu;
+    const float c = __fmul_rn(s, -8.0f);
     // (round to nearest even; f32 subnormals count as zero in this mode, as in the reference's bfloat16_t(float))
-    o[jj] = zmi_pack_bf16(f[0], f[1]);
+    auto pair = [&](float f0, float f1) {
+      float f[2] = {f0, f1};
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        if (Q == 0) f[h] = __builtin_fmaf(f[h], s, c);
+        else if (Q == 2) f[h] = __fmul_rn(__fsub_rn(f[h], z), s);
+        else f[h] = __fadd_rn(__builtin_fmaf(f[h], s, c), z);
+      }
+      return zmi_pack_bf16(f[0], f[1]);
+    };
+    o[0] = pair(woq_byte_f32<0>(ev), woq_byte_f32<0>(od));
+    o[1] = pair(woq_byte_f32<1>(ev), woq_byte_f32<1>(od));
+    o[2] = pair(woq_byte_f32<2>(ev), woq_byte_f32<2>(od));
+    o[3] = pair(woq_byte_f32<3>(ev), woq_byte_f32<3>(od));
   }
   uint4 r = {o[0], o[1], o[2], o[3]};
   return __builtin_bit_cast(woq_bf16x8, r);
 }
 
+// The main loop below has no branches: a load under a branch makes the compiler wait for every load in flight where
+// the paths meet.  Rows beyond M and chunks beyond K read an address that exists; rows beyond M are never stored and
+// values of k beyond K are replaced by zeros (which also makes a whole chunk beyond K add nothing).
 __device__ __forceinline__ uint4 woq_load_a(const ZmiWoqProblem &p, int row, int k) {
-  uint4 r = {0u, 0u, 0u, 0u};
-  if (row >= p.M || k >= p.K) return r;
   const uint16_t *a = (const uint16_t *)p.A;
-  if (p.a_fast) return *(const uint4 *)(a + (int64_t)row * p.lda + k);
+  row = min(row, p.M - 1);
   uint32_t e[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const int kk = k + j;
-    e[j] = kk < p.K ? (uint32_t)a[p.transA ? (int64_t)kk * p.lda + row : (int64_t)row * p.lda + kk] : 0u;
+    const int kk = min(k + j, p.K - 1);
+    const uint32_t v = a[p.transA ? (int64_t)kk * p.lda + row : (int64_t)row * p.lda + kk];
+    e[j] = k + j < p.K ? v : 0u;
   }
+  uint4 r;
   r.x = e[0] | (e[1] << 16); r.y = e[2] | (e[3] << 16); r.z = e[4] | (e[5] << 16); r.w = e[6] | (e[7] << 16);
   return r;
 }
 
-__device__ __forceinline__ float woq_param(const void *ptr, int dt, int mode, float val, int g, int n, int N) {
-  if (!ptr) return val;
-  return zmi_ld_f32(ptr, dt, mode == 0 ? 0 : mode == 1 ? (int64_t)n : (int64_t)g * N + n);
-}
-
 template <int MT> struct WoqWaves { static constexpr int W = MT <= 2 ? 8 : 4; };
 
-template <int MT, int Q>
-__global__ __launch_bounds__(WoqWaves<MT>::W * 64) void zmi_gemm_woq_kernel(ZmiWoqProblem p, ZmiEpilogue epi) {
+// GENERAL = false: rows read 16 bytes at a time, one scale per 64-value chunk (scale groups are multiples of 64, or
+// there are none).  GENERAL = true: rows element by element (any stride, transposed sources, K not a multiple of 8),
+// scales looked up per 8 values.
+template <int MT, int Q, bool GENERAL>
+__global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1) void zmi_gemm_woq_kernel(ZmiWoqProblem p, ZmiEpilogue epi) {
   constexpr int W = WoqWaves<MT>::W, U = 8;
   extern __shared__ float woq_red[];   // [W][MT * 16][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nb = blockIdx.x, m0 = blockIdx.y * 32 * MT;
   const int nc = min(nb * 32 + (lane & 31), p.N - 1), kh = lane >> 5;
   const int nkc = (p.K + 63) / 64;
-  const uint4 *wt = (const uint4 *)p.tiles + (int64_t)nb * nkc * 64 + lane;
-  const bool fine = p.scale_mode == 2 && (p.group_size & 63) != 0;
 
   woq_f32x16 acc[MT];
 #pragma unroll
@@ -119,45 +171,93 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64) void zmi_gemm_woq_kernel(ZmiW
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
 
+  // Requests run ahead of their use: a wavefront's next 8 chunks of weights (the whole K up to 4096), and the rows and
+  // scales of the chunk after the one being multiplied (loads come back in the order they were asked for, so a
+  // chunk's rows are asked for before anything that is needed later).  Addresses are a base every lane shares (kept
+  // in scalar registers) plus a 32-bit offset per lane that never changes.
+  constexpr int RING = !GENERAL && MT <= 2 ? 2 : 1;
+  constexpr int NS = GENERAL ? 4 : 1;
   uint4 wq[U];
+  float sw[RING][NS], zw[RING][NS];
+  uint4 af[RING][4][MT];
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const char *wbase = (const char *)p.tiles + (int64_t)nb * nkc * 1024;
+  const uint32_t woff = lane * 16, noff = nc * 4;
+  uint32_t aoff[MT];
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int kc = wave + u * W;
-    wq[u] = kc < nkc ? wt[(int64_t)kc * 64] : uint4{0u, 0u, 0u, 0u};
+  for (int i = 0; i < MT; ++i) {
+    // rows beyond M get an offset outside the buffer: such a lane reads zeros and asks memory for nothing
+    const int row = m0 + 32 * i + (lane & 31);
+    aoff[i] = row < p.M ? (uint32_t)((row * (int)p.lda + kh * 8) * 2) : 0x80000000u;
   }
-  zmi_set_f32_flush();
-  for (int kc0 = wave; kc0 < nkc; kc0 += U * W) {
+  // the rows as a buffer of M * lda bf16 values (untyped, 32-bit offsets, range-checked)
+  const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.A, 0, GENERAL ? 0 : p.M * (int)p.lda * 2, 0x00020000);
+  auto load_weights = [&](int kc) { return *(const uint4 *)(wbase + (int64_t)min(kc, nkc - 1) * 1024 + woff); };
+  // TAIL = false: every value of the chunk lies inside K
+  auto load_rows = [&](auto tail, int slot, int kc) {
+    constexpr bool TAIL = decltype(tail)::value;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        if (GENERAL) {
+          af[slot][t][i] = woq_load_a(p, m0 + 32 * i + (lane & 31), kc * 64 + t * 16 + kh * 8);
+        } else {
+          const int k0 = kc * 64 + t * 16;
+          // (with the tail handling a lane whose 8 values lie beyond K reads the last 8 inside it instead)
+          const woq_u32x4 rb = TAIL ? __builtin_amdgcn_raw_buffer_load_b128(arsrc, aoff[i] - kh * 16 + min(k0 + kh * 8, p.K - 8) * 2, 0, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(arsrc, aoff[i], k0 * 2, 0);
+          uint4 r = {rb[0], rb[1], rb[2], rb[3]};
+          if (TAIL) {
+            const bool in = k0 + kh * 8 < p.K;
+            r.x = in ? r.x : 0u; r.y = in ? r.y : 0u; r.z = in ? r.z : 0u; r.w = in ? r.w : 0u;
+          }
+          af[slot][t][i] = r;
+        }
+      }
+#pragma unroll
+    for (int t = 0; t < NS; ++t) {
+      if (GENERAL) {
+        const int64_t gi = (int64_t)min((kc * 64 + t * 16 + kh * 8) / p.group_size, p.n_groups - 1) * p.N + nc;
+        sw[slot][t] = p.sf[gi];
+        zw[slot][t] = Q == 0 ? 0.0f : p.zf[gi];
+      } else {
+        const int64_t go = (int64_t)min((kc * 64) / p.group_size, p.n_groups - 1) * p.N * 4;
+        sw[slot][t] = *(const float *)((const char *)p.sf + go + noff);
+        zw[slot][t] = Q == 0 ? 0.0f : *(const float *)((const char *)p.zf + go + noff);
+      }
+    }
+  };
+  auto pass = [&](auto tail, int kc0) {
+    constexpr bool TAIL = decltype(tail)::value;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int kc = kc0 + u * W;
-      if (kc >= nkc) break;
-      // this chunk's rows and parameters are requested ahead of the next chunk of weights for this slot: loads come
-      // back in the order they were asked for
-      uint4 af[4][MT];
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int i = 0; i < MT; ++i) af[t][i] = woq_load_a(p, m0 + 32 * i + (lane & 31), kc * 64 + t * 16 + kh * 8);
-      int g = min((kc * 64) / p.group_size, p.n_groups - 1);
-      float s = woq_param(p.scale, p.scale_dt, p.scale_mode, p.scale_val, g, nc, p.N);
-      float z = Q == 0 ? 0.0f : woq_param(p.zp, p.zp_dt, p.zp_mode, p.zp_val, g, nc, p.N);
+      // (a chunk beyond K that a pass without the tail handling asks for ahead is never multiplied)
+      if (RING == 1) load_rows(tail, 0, kc);
+      else load_rows(tail, (u + 1) % RING, TAIL ? kc + W : min(kc + W, nkc - 1));
       const uint4 w = wq[u];
-      const int kn = kc + U * W;
-      if (kn < nkc) wq[u] = wt[(int64_t)kn * 64];
+      wq[u] = load_weights(kc + U * W);
       const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        if (fine) {
-          g = min((kc * 64 + t * 16 + kh * 8) / p.group_size, p.n_groups - 1);
-          s = woq_param(p.scale, p.scale_dt, p.scale_mode, p.scale_val, g, nc, p.N);
-          if (Q != 0) z = woq_param(p.zp, p.zp_dt, p.zp_mode, p.zp_val, g, nc, p.N);
-        }
-        const woq_bf16x8 b = woq_dequant<Q>(wd[t], s, z);
+        const int ts = GENERAL ? t : 0;
+        const woq_bf16x8 b = woq_dequant<Q>(wd[t], sw[u % RING][ts], zw[u % RING][ts]);
 #pragma unroll
         for (int i = 0; i < MT; ++i)
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(woq_bf16x8, af[t][i]), b, acc[i], 0, 0, 0);
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(woq_bf16x8, af[u % RING][t][i]), b, acc[i], 0, 0, 0);
       }
     }
+  };
+  if (RING > 1) load_rows(std::true_type{}, 0, wave_s);
+#pragma unroll
+  for (int u = 0; u < U; ++u) wq[u] = load_weights(wave_s + u * W);
+  zmi_set_f32_flush();
+  for (int kc0 = wave_s; kc0 < nkc; kc0 += U * W) {
+    // a pass whose 8 chunks, and the chunk it asks for ahead, lie inside K (or beyond the last chunk) needs no tail handling
+    const int last = kc0 + (U - 1) * W, ahead = kc0 + U * W;
+    if (!GENERAL && (last + 1) * 64 <= p.K && ((ahead + 1) * 64 <= p.K || ahead >= nkc)) pass(std::false_type{}, kc0);
+    else pass(std::true_type{}, kc0);
   }
   // back to IEEE subnormals for the element-wise tail (the mode the other kernels' tails run in)
   __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 3);
@@ -183,33 +283,40 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64) void zmi_gemm_woq_kernel(ZmiW
   }
 }
 
-template <int MT>
+template <int MT, bool GENERAL>
 static hipError_t woq_launch_q(const ZmiWoqProblem &p, const ZmiEpilogue &epi, int q, hipStream_t stream) {
   constexpr int W = WoqWaves<MT>::W;
   const int smem = W * MT * 16 * 64 * 4;
   const dim3 grid((unsigned)((p.N + 31) / 32), (unsigned)((p.M + 32 * MT - 1) / (32 * MT)));
-  const void *f = q == 0 ? (const void *)zmi_gemm_woq_kernel<MT, 0> : q == 1 ? (const void *)zmi_gemm_woq_kernel<MT, 1>
-                : q == 2 ? (const void *)zmi_gemm_woq_kernel<MT, 2> : (const void *)zmi_gemm_woq_kernel<MT, 3>;
+  const void *f = q == 0 ? (const void *)zmi_gemm_woq_kernel<MT, 0, GENERAL> : q == 1 ? (const void *)zmi_gemm_woq_kernel<MT, 1, GENERAL>
+                : q == 2 ? (const void *)zmi_gemm_woq_kernel<MT, 2, GENERAL> : (const void *)zmi_gemm_woq_kernel<MT, 3, GENERAL>;
   hipError_t e = zmi_func_smem_once(f, smem);
   if (e != hipSuccess) return e;
   switch (q) {
-  case 0: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 0>), grid, dim3(W * 64), smem, stream, p, epi); break;
-  case 1: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 1>), grid, dim3(W * 64), smem, stream, p, epi); break;
-  case 2: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 2>), grid, dim3(W * 64), smem, stream, p, epi); break;
-  default: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 3>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  case 0: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 0, GENERAL>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  case 1: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 1, GENERAL>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  case 2: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 2, GENERAL>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  default: hipLaunchKernelGGL((zmi_gemm_woq_kernel<MT, 3, GENERAL>), grid, dim3(W * 64), smem, stream, p, epi); break;
   }
   return hipGetLastError();
 }
 
+template <bool GENERAL>
+static hipError_t woq_launch_m(const ZmiWoqProblem &p, const ZmiEpilogue &epi, int q, hipStream_t stream) {
+  if (p.M <= 32) return woq_launch_q<1, GENERAL>(p, epi, q, stream);
+  if (p.M <= 64) return woq_launch_q<2, GENERAL>(p, epi, q, stream);
+  return woq_launch_q<4, GENERAL>(p, epi, q, stream);
+}
+
 hipError_t zmi_launch_gemm_woq(const ZmiWoqProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
-  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || !p.A || !p.tiles || !p.dst || p.group_size <= 0 || p.n_groups <= 0 ||
-      (p.scale_mode == 2 && (p.group_size % 8 != 0 || (int64_t)p.group_size * p.n_groups != p.K)) ||
-      (p.a_fast && (p.transA || p.K % 8 != 0 || p.lda % 8 != 0 || ((uintptr_t)p.A & 15) != 0)) ||
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || !p.A || !p.tiles || !p.sf || !p.zf || !p.dst || p.group_size <= 0 ||
+      p.n_groups <= 0 || (p.n_groups > 1 && (p.group_size % 8 != 0 || (int64_t)p.group_size * p.n_groups != p.K)) ||
+      (p.a_fast && (p.transA || p.K % 8 != 0 || p.K < 64 || p.lda % 8 != 0 || ((uintptr_t)p.A & 15) != 0 ||
+                    (int64_t)p.M * p.lda >= ((int64_t)1 << 30))) ||
       (p.M + 127) / 128 > 65535)
     return hipErrorInvalidValue;
   const int q = p.is_u4 ? (p.zp_float_domain ? 3 : 2) : (p.has_zp ? 1 : 0);
   if (p.is_u4 && !p.has_zp) return hipErrorInvalidValue;
-  if (p.M <= 32) return woq_launch_q<1>(p, epi, q, stream);
-  if (p.M <= 64) return woq_launch_q<2>(p, epi, q, stream);
-  return woq_launch_q<4>(p, epi, q, stream);
+  const bool general = !p.a_fast || (p.n_groups > 1 && p.group_size % 64 != 0);
+  return general ? woq_launch_m<true>(p, epi, q, stream) : woq_launch_m<false>(p, epi, q, stream);
 }

@@ -42,30 +42,28 @@ int32_t matmul_woq(char layout, int32_t transA, int32_t transB, int32_t M, int32
 
   ZmiWoqProblem w;
   std::memset(&w, 0, sizeof(w));
+  ZmiWoqParamSrc sc{nullptr, sdt, 0, 1.0f}, zp{nullptr, ZMI_DT_F32, 0, 0.0f};
   // scale granularity: one value, one per column, or {G, N} (cvt_int4_to_bf16's own reading of the element count)
   const int64_t ns = nelems(p.wei_scale);
-  w.scale_dt = sdt;
   w.n_groups = 1;
   if (ns == 1) {
-    w.scale_mode = 0;
-    if (!scalar_param_f32(p.wei_scale.buff, sdt, &w.scale_val, &w.scale)) return ZMI_FAILURE;
+    if (!scalar_param_f32(p.wei_scale.buff, sdt, &sc.val, &sc.ptr)) return ZMI_FAILURE;
   } else if (ns == N) {
-    w.scale_mode = 1;
-    w.scale = p.wei_scale.buff;
+    sc.mode = 1;
+    sc.ptr = p.wei_scale.buff;
   } else if (ns > N && ns % N == 0 && K % (ns / N) == 0) {
-    w.scale_mode = 2;
-    w.scale = p.wei_scale.buff;
+    sc.mode = 2;
+    sc.ptr = p.wei_scale.buff;
     w.n_groups = (int32_t)(ns / N);
   } else {
     set_error("wei_scale must hold 1, N or groups x N elements, with groups dividing K");
     return ZMI_FAILURE;
   }
   w.group_size = K / w.n_groups;
-  if (w.scale_mode == 2 && w.group_size % 8 != 0) {
+  if (w.n_groups > 1 && w.group_size % 8 != 0) {
     set_error("weight-only quantization: a scale group must span a multiple of 8 values of K");
     return ZMI_UNIMPLEMENTED;
   }
-  if (w.scale_mode && !is_device_pointer(w.scale)) { set_error("per-channel / per-group wei_scale must be in device memory"); return ZMI_FAILURE; }
   if (p.wei_zp.buff) {
     const int32_t zdt = p.wei_zp.dt;
     if (zdt != ZMI_DT_BF16 && zdt != ZMI_DT_S8 && zdt != ZMI_DT_U8 && zdt != ZMI_DT_S32 && zdt != ZMI_DT_F32) {
@@ -74,32 +72,35 @@ int32_t matmul_woq(char layout, int32_t transA, int32_t transB, int32_t M, int32
     }
     const int64_t nz = nelems(p.wei_zp);
     w.has_zp = 1;
-    w.zp_dt = zdt;
+    zp.dt = zdt;
     w.zp_float_domain = u4 && zdt == ZMI_DT_BF16;
     if (nz == 1) {
-      w.zp_mode = 0;
-      if (!scalar_param_f32(p.wei_zp.buff, zdt, &w.zp_val, &w.zp)) return ZMI_FAILURE;
+      if (!scalar_param_f32(p.wei_zp.buff, zdt, &zp.val, &zp.ptr)) return ZMI_FAILURE;
     } else if (nz == N) {
-      w.zp_mode = 1;
-      w.zp = p.wei_zp.buff;
-    } else if (w.scale_mode == 2 && nz == ns) {
-      w.zp_mode = 2;
-      w.zp = p.wei_zp.buff;
+      zp.mode = 1;
+      zp.ptr = p.wei_zp.buff;
+    } else if (sc.mode == 2 && nz == ns) {
+      zp.mode = 2;
+      zp.ptr = p.wei_zp.buff;
     } else {
       set_error("wei_zp must hold 1, N or as many elements as a per-group wei_scale");
       return ZMI_FAILURE;
     }
-    if (w.zp_mode && !is_device_pointer(w.zp)) { set_error("per-channel / per-group wei_zp must be in device memory"); return ZMI_FAILURE; }
   }
 
   if (!ensure_device()) return ZMI_FAILURE;
   const bool use_cache = std::min(weight_cache_env(), p.weight_cache_type) > 0;
   const size_t tile_bytes = (size_t)zmi_woq_tiles_bytes(K, N);
-  if (!arena().begin(use_cache ? 0 : Arena::padded(tile_bytes))) return ZMI_FAILURE;
-  void *slot = use_cache ? nullptr : arena().alloc(tile_bytes);
-  if (!use_cache && !slot) { set_error("no scratch for the 4-bit tiles"); return ZMI_FAILURE; }
-  w.tiles = packed_woq_tiles(weight, K, N, ldb, transB != 0, use_cache, slot);
-  if (!w.tiles) return ZMI_FAILURE;
+  const size_t blob_bytes = tile_bytes + 2 * sizeof(float) * (size_t)w.n_groups * (size_t)N;
+  if (!arena().begin(use_cache ? 0 : Arena::padded(blob_bytes))) return ZMI_FAILURE;
+  void *slot = use_cache ? nullptr : arena().alloc(blob_bytes);
+  if (!use_cache && !slot) { set_error("no scratch for the 4-bit weights"); return ZMI_FAILURE; }
+  // (a cached weight keeps the scales and zero-points it was first seen with, like the reference's cached bf16 matrix)
+  const uint8_t *blob = packed_woq_weights(weight, K, N, ldb, transB != 0, w.n_groups, sc, zp, use_cache, slot);
+  if (!blob) return ZMI_FAILURE;
+  w.tiles = (const uint32_t *)blob;
+  w.sf = (const float *)(blob + tile_bytes);
+  w.zf = w.sf + (size_t)w.n_groups * N;
 
   // alpha, beta, bias and the post-ops go the way of every other call; the quantization parameters are this path's own
   zmi_matmul_params_t ep = p;
@@ -111,7 +112,7 @@ int32_t matmul_woq(char layout, int32_t transA, int32_t transB, int32_t M, int32
   if (st != ZMI_SUCCESS) return st;
 
   w.A = src; w.lda = lda; w.transA = transA ? 1 : 0;
-  w.a_fast = !transA && K % 8 == 0 && lda % 8 == 0 && ((uintptr_t)src & 15) == 0;
+  w.a_fast = !transA && K % 8 == 0 && K >= 64 && lda % 8 == 0 && ((uintptr_t)src & 15) == 0 && (int64_t)M * lda < ((int64_t)1 << 30);
   w.dst = dst; w.ldc = ldc;
   w.M = M; w.N = N; w.K = K;
   w.is_u4 = u4 ? 1 : 0;

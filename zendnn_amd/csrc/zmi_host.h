@@ -91,9 +91,10 @@ const uint8_t *packed_ggml_q8_0(const void *weight, int64_t K, int64_t N, const 
 const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
                                  void *widen_slot, void *arena_slot, const uint8_t **tiles_s4);
 // packed s4 / u4 weights of the weight-only path: the codes in the kernel's tile order (zmi_woq_tiles_bytes(K, N)
-// bytes), cached like the others or written into arena_slot.
-const uint32_t *packed_woq_tiles(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
-                                 void *arena_slot);
+// bytes), then the scales and the zero-points as f32 [G][N] each; cached per weight pointer like the others (the
+// scales are part of the cached weights, as in the reference), or written into arena_slot.
+const uint8_t *packed_woq_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, int64_t G,
+                                  const ZmiWoqParamSrc &sc, const ZmiWoqParamSrc &zp, bool use_cache, void *arena_slot);
 void clear_weight_cache();
 
 // Checks (once per pointer) that a caller-supplied blob carries the header of a

@@ -474,26 +474,29 @@ const uint8_t *packed_s4_weights(const void *weight, int64_t K, int64_t N, int64
   return (const uint8_t *)blob;
 }
 
-// Weight-only quantization: the 4-bit codes in the order the kernel's wavefronts read them (reference:
-// woqReorderAndCacheWeightsAocl, matmul/backends/aocl/aocl_kernel.cpp:640-702, which caches the dequantized bf16
-// matrix; the codes stay 4-bit here).  The key's leading dimension is stored negated and far below W4A8's.
-const uint32_t *packed_woq_tiles(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, bool use_cache,
-                                 void *arena_slot) {
-  if (!use_cache) {
-    if (!hip_ok(zmi_launch_woq_tiles(weight, K, N, ldb, transB, (uint32_t *)arena_slot, stream()), "4-bit tiles launch"))
-      return nullptr;
-    return (const uint32_t *)arena_slot;
-  }
+// Weight-only quantization: the 4-bit codes in the order the kernel's wavefronts read them, followed by the scales and
+// the zero-points as f32 [G][N] each (reference: woqReorderAndCacheWeightsAocl, matmul/backends/aocl/aocl_kernel.cpp:
+// 640-702, which caches the dequantized bf16 matrix per weight pointer -- scales and zero-points included, as here;
+// the codes stay 4-bit).  The key's leading dimension is stored negated and far below W4A8's.
+const uint8_t *packed_woq_weights(const void *weight, int64_t K, int64_t N, int64_t ldb, bool transB, int64_t G,
+                                  const ZmiWoqParamSrc &sc, const ZmiWoqParamSrc &zp, bool use_cache, void *arena_slot) {
+  const size_t tiles = (size_t)zmi_woq_tiles_bytes(K, N), total = tiles + 2 * sizeof(float) * (size_t)(G * N);
+  auto fill = [&](uint8_t *blob) {
+    return hip_ok(zmi_launch_woq_tiles(weight, K, N, ldb, transB, (uint32_t *)blob, stream()), "4-bit tiles launch") &&
+           hip_ok(zmi_launch_woq_params(sc, zp, G, N, (float *)(blob + tiles), (float *)(blob + tiles) + G * N, stream()),
+                  "4-bit scales launch");
+  };
+  if (!use_cache) return fill((uint8_t *)arena_slot) ? (const uint8_t *)arena_slot : nullptr;
   std::lock_guard<std::mutex> lk(g_mu);
-  CacheKey key{weight, K, N, -ldb - ((int64_t)1 << 40), transB};
+  CacheKey key{weight, K, N, -ldb - ((int64_t)1 << 40) - (G << 41), transB};
   auto it = g_cache.find(key);
   if (it != g_cache.end()) {
     g_lru.splice(g_lru.begin(), g_lru, it->second.lru);
-    return (const uint32_t *)it->second.blob;
+    return it->second.blob;
   }
   void *blob = nullptr;
-  if (!hip_ok(hipMalloc(&blob, (size_t)zmi_woq_tiles_bytes(K, N)), "hipMalloc(4-bit tiles)")) return nullptr;
-  if (!hip_ok(zmi_launch_woq_tiles(weight, K, N, ldb, transB, (uint32_t *)blob, stream()), "4-bit tiles launch")) {
+  if (!hip_ok(hipMalloc(&blob, total), "hipMalloc(4-bit weights)")) return nullptr;
+  if (!fill((uint8_t *)blob)) {
     (void)hipFree(blob);
     return nullptr;
   }
@@ -506,7 +509,7 @@ const uint32_t *packed_woq_tiles(const void *weight, int64_t K, int64_t N, int64
     (void)hipFree(g_cache[old].blob);
     g_cache.erase(old);
   }
-  return (const uint32_t *)blob;
+  return (const uint8_t *)blob;
 }
 
 void clear_weight_cache() {

@@ -190,17 +190,21 @@ struct ZmiWoqProblem {
   int32_t is_u4;            // codes 0 .. 15 instead of -8 .. 7
   int32_t has_zp;
   int32_t zp_float_domain;  // u4 codes with a bf16 zero-point: (code - 8) * scale + zp
-  // scale / zero-point: mode 0 = one value (the pointer, or the value when it is null), 1 = one per column,
-  // 2 = one per K group and column, {n_groups, N}
-  const void *scale;
-  const void *zp;
-  int32_t scale_dt, scale_mode;
-  int32_t zp_dt, zp_mode;
-  float scale_val, zp_val;
+  const float *sf;          // [n_groups][N] f32 scales and zero-points (zmi_launch_woq_params)
+  const float *zf;
   int32_t group_size;       // K / n_groups
   int32_t n_groups;
   const void *bias;
 };
+// a scale / zero-point tensor as the caller gave it: mode 0 = one value (at ptr, or val when ptr is null), 1 = one
+// per column, 2 = one per K group and column, {n_groups, N}
+struct ZmiWoqParamSrc {
+  const void *ptr;
+  int32_t dt, mode;
+  float val;
+};
+hipError_t zmi_launch_woq_params(const ZmiWoqParamSrc &s, const ZmiWoqParamSrc &z, int64_t G, int64_t N, float *sf,
+                                 float *zf, hipStream_t stream);
 hipError_t zmi_launch_woq_tiles(const void *packed, int64_t K, int64_t N, int64_t ldb, bool transB, uint32_t *out,
                                 hipStream_t stream);
 // (of the epilogue descriptor only alpha, beta, bias_dt, the post-ops and dst_dt are read)
