@@ -112,12 +112,17 @@ typedef struct zmi_batch_params_t {
 /* matmul_params (matmul/lowoha_common.hpp:145-227), flattened. */
 typedef struct zmi_matmul_params_t {
   int32_t dt_src, dt_wei, dt_dst, dt_bias, dt_compute;  /* matmul_data_types; dt_wei: s8, or s4 for W4A8 (bf16 src, dynamic_quant,
-                                                          * s8 compute, bf16 dst: lowoha_matmul_utils.cpp:72-176) */
+                                                          * s8 compute, bf16 dst: lowoha_matmul_utils.cpp:72-176), or s4 / u4
+                                                          * with a bf16 src and no dynamic_quant: weight-only quantization
+                                                          * (constant weights, wei_scale of 1, N or groups x N elements, for u4
+                                                          * a wei_zp of s8 or bf16 type; bf16 / f32 dst:
+                                                          * lowoha_matmul_utils.cpp:214-250, 313-328, aocl_kernel.cpp:43-139) */
   int32_t n_postops;
   const zmi_post_op_t *postops;
   zmi_quant_t src_scale, wei_scale, dst_scale, src_zp, wei_zp, dst_zp;
                               /* wei_zp: one zero-point for the weight tensor (s8 / u8 / s32, host or device), single
-                               * problems with s8 / u8 sources (aocl_kernel.cpp:982-985, lru_cache/lowoha_cache.hpp:151-232) */
+                               * problems with s8 / u8 sources (aocl_kernel.cpp:982-985, lru_cache/lowoha_cache.hpp:151-232);
+                               * with 4-bit weight-only weights: 1, N or groups x N zero-points (device memory beyond one) */
   char mem_format_a;          /* 'n' */
   char mem_format_b;          /* 'n' plain weights, 'r' blob from zmi_reorder_direct */
   int32_t lowoha_algo;        /* enum zmi_matmul_algo */

@@ -41,6 +41,13 @@
  *   zo_quant_asym                closed forms (rows k * 2^-e: scale, zero-point and every code known exactly;
  *                                constant and non-finite rows), dequantization within half a step, codes of
  *                                the row minimum / maximum, zero-point against Python fractions
+ *   zo_woq_dequant, zo_matmul_woq  nibble order, sign extension, orientation and leading dimension on hand-built bytes;
+ *                                both dequantization formulas on operands that keep every step exact (known answers
+ *                                that tell the formulas apart); bf16-valued scales (exact f32 product) against torch's
+ *                                rounding of the exact double product, per tensor / channel / group; the product
+ *                                against numpy float64 (to 2e-6 of the magnitude sum) and exactly on integer operands.
+ *                                The reference's own GEMM on the dequantized matrix is AOCL's: its summation order is
+ *                                parity unpinned, the comparison of products is to a tolerance.
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
  *   prepack layout, weight_prepack_size values: parity unpinned (opaque by the
  *     reference's contract; only the round trip matmul(prepack(B)) == matmul(B)
