@@ -157,9 +157,14 @@ static void gpu_w4a8_example() {
   CHECK(matmul_direct('r', false, false, M, N, K, 1.0f, x_d, K, w_d, N, nullptr, 0.0f, y_d, N, true, batch_params, params) ==
         status_t::failure);
   params.dtypes.dst = data_type_t::bf16;
-  params.dynamic_quant = false;    // bf16 x s4 without dynamic quantization is weight-only quantization: not this path
+  params.dynamic_quant = false;    // bf16 x s4 without dynamic quantization is weight-only quantization: no source scale
   CHECK(matmul_direct('r', false, false, M, N, K, 1.0f, x_d, K, w_d, N, nullptr, 0.0f, y_d, N, true, batch_params, params) ==
-        status_t::unimplemented);
+        status_t::failure);
+  params.quant_params.src_scale.buff = nullptr;
+  params.quant_params.src_scale.dims.clear();
+  params.dtypes.compute = data_type_t::none;
+  CHECK(matmul_direct('r', false, false, M, N, K, 1.0f, x_d, K, w_d, N, nullptr, 0.0f, y_d, N, true, batch_params, params) ==
+        status_t::success);
   clear_matmul_weight_caches();
   hipFree(ss_d); hipFree(ws_d); hipFree(w_d); hipFree(x_d); hipFree(y_d);
 }
