@@ -30,6 +30,7 @@ CASES = {
     "per_group_scales": ("per_group", 0x5EED0006, 9, 512, 72, 8),
     "ggml_q8_0": ("ggml", 0x5EED0007, 6, 256, 40),
     "w4a8": ("w4a8", 0x5EED0008, 12, 1024, 56, 8),
+    "weight_only_4bit": ("woq", 0x5EED0009, 192, 40, 3),
 }
 
 
@@ -53,6 +54,10 @@ class _Backend:
         if self.name == "cpu":
             keep = []
             ph = H.host_params(p, **host)
+            if p.dt_wei in (capi.DT_S4, capi.DT_U4) and not p.dynamic_quant:
+                st, dst = self.zo.matmul_woq(src, weight, ph.flat(keep), M, N, K, bias=bias, transB=transB, ldb=ldb)
+                assert st == capi.SUCCESS
+                return dst[:, :N].astype(np_dt, copy=False), None
             st, dst, _, scales = self.zo.matmul_int8(src, weight, ph.flat(keep), M, N, K, bias=bias, transB=transB, ldb=ldb,
                                                      want_scales=scales_n > 0, n_scales=scales_n or None)
             assert st == capi.SUCCESS
@@ -192,6 +197,23 @@ def run(name, backend, zo=None):
                               scales_n=int(np.prod(dims)))
             out["dst_bf16_" + tag] = (y, EXACT)
             out["src_scales_" + tag] = (sc, EXACT)
+    elif kind == "woq":
+        # weight-only quantization: one-hot bf16 rows make the product the dequantized bf16 weight matrix itself
+        # (every sum is one value plus zeros, exact in any order): s4 codes with f32 {G,N} scales, and u4 codes with
+        # bf16 {G,N} zero-points, the (code - 8) * scale + zp form
+        K, N, G = spec[2:]
+        eye = np.zeros((K, K), dtype=np.uint16)
+        eye[np.arange(K), np.arange(K)] = 0x3F80
+        packed = rng.integers(0, 256, K * N // 2, dtype=np.uint8)
+        ws = rng.uniform(0.01, 0.1, (G, N)).astype(np.float32)
+        zp = H.bf16_bits(rng.uniform(-0.2, 0.2, (G, N)).astype(np.float32))
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S4, dst=capi.DT_BF16)
+        p.wei_scale = lowoha.QuantParam(None, capi.DT_F32, (G, N))
+        out["weights_bf16_s4"] = (be.matmul(p, eye, packed, K, N, K, ldb=N, host=dict(wei_scale=ws))[0], EXACT)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_U4, dst=capi.DT_F32)
+        p.wei_scale = lowoha.QuantParam(None, capi.DT_F32, (G, N))
+        p.wei_zp = lowoha.QuantParam(None, capi.DT_BF16, (G, N))
+        out["weights_f32_u4_bf16_zp"] = (be.matmul(p, eye, packed, K, N, K, ldb=N, host=dict(wei_scale=ws, wei_zp=zp))[0], EXACT)
     else:
         raise KeyError(kind)
     return out

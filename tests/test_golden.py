@@ -1,6 +1,6 @@
 """The committed golden fixtures (tests/golden/golden.json, golden_bf16.npz; written by tests/golden/make_golden.py from
 the CPU oracle) against the oracle as it is now (CPU) and against the HIP path through the C ABI (GPU): one reduced
-case per BASELINE configuration plus per-group scales, GGML Q8_0 and W4A8.  Bit-exact outputs are compared by SHA-256,
+case per BASELINE configuration plus per-group scales, GGML Q8_0, W4A8 and the dequantized weights of the weight-only path.  Bit-exact outputs are compared by SHA-256,
 activation outputs within one bf16 unit in the last place (two for the fused MoE block, whose re-quantized
 intermediate may move by one count)."""
 import json
