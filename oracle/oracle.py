@@ -21,7 +21,7 @@ class MatmulCall(C.Structure):
                 ("ldb", C.c_int32), ("bias", C.c_void_p), ("beta", C.c_float),
                 ("dst", C.c_void_p), ("ldc", C.c_int32),
                 ("params", C.POINTER(capi.MatmulParamsT)),
-                ("acc_out", C.c_void_p), ("scale_out", C.c_void_p)]
+                ("acc_out", C.c_void_p), ("scale_out", C.c_void_p), ("zp_out", C.c_void_p)]
 
 
 def lib():
@@ -177,7 +177,7 @@ def gemm_s32(A, B, transA=False, transB=False):
 
 def matmul_int8(src, weight, params, M, N, K, *, bias=None, dst=None, lda=None, ldb=None,
                 ldc=None, transA=False, transB=False, alpha=1.0, beta=0.0, want_acc=False,
-                want_scales=False, n_scales=None):
+                want_scales=False, n_scales=None, zp_out=None):
     """Runs the oracle's matmul_direct on host arrays.  params is a
     capi.MatmulParamsT whose buff pointers reference host memory.  Returns
     (status, dst array, acc or None, scales or None)."""
@@ -202,6 +202,7 @@ def matmul_int8(src, weight, params, M, N, K, *, bias=None, dst=None, lda=None, 
     call.params = C.pointer(params)
     call.acc_out = _p(acc)
     call.scale_out = _p(scales)
+    call.zp_out = _p(zp_out)   # int32 [1]: receives the zero-point of a dynamic quantization to u8
     st = lib().zo_matmul_int8(C.byref(call))
     return st, dst, acc, scales
 

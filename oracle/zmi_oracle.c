@@ -48,6 +48,9 @@
  *                                against numpy float64 (to 2e-6 of the magnitude sum) and exactly on integer operands.
  *                                The reference's own GEMM on the dequantized matrix is AOCL's: its summation order is
  *                                parity unpinned, the comparison of products is to a tolerance.
+ *   dynamic u8 (per tensor)      closed forms (values k / 4: scale 0.25, zero-point 100, codes and product known exactly;
+ *                                constant and non-finite tensors; the 2.5 * 255 tie), identity weights dequantize to the
+ *                                source within half a step; the AVX-512 kernels' reciprocal form: parity unpinned on ties
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
  *   prepack layout, weight_prepack_size values: parity unpinned (opaque by the
  *     reference's contract; only the round trip matmul(prepack(B)) == matmul(B)
@@ -402,6 +405,7 @@ typedef struct zo_matmul_call {
   const zmi_matmul_params_t *params;
   int32_t *acc_out;   /* optional [M,N]: the raw s32 accumulator (before compensation) */
   float *scale_out;   /* optional [M]: the per-token scales a dynamic_quant call computed */
+  int32_t *zp_out;    /* optional [1]: the zero-point a dynamic_quant call to u8 computed */
 } zo_matmul_call;
 
 static void zo_store(void *dst, int32_t dt, int64_t i, float val) {
@@ -592,7 +596,56 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
 
   const int dyn = p->dynamic_quant && (a_dt == ZMI_DT_BF16 || a_dt == ZMI_DT_F32) &&
                   (p->dt_compute == ZMI_DT_S8 || p->dt_compute == ZMI_DT_U8);
-  if (dyn) {
+  int32_t dyn_zp = 0;
+  if (dyn && p->dt_compute == ZMI_DT_U8) {
+    /* dynamic asymmetric quantization of the source to u8: the GEMM reads ONE source zero-point
+     * (operators/matmul/matmul_ref_kernel.cpp:935-939, backends/aocl/aocl_kernel.cpp:971-980), so the granularity that
+     * means something is per tensor: src_scale and src_zp of one element each
+     * (matmul/quantization/reorder_quantization.cpp:60-75, 208-230: dims and types required, buffers optional).
+     * Parameters: compute_scale_zp, lowoha_operators/reorder/lowoha_reorder_utils.cpp:708-765 -- min / max over the
+     * finite values ([0, 0] when there is none), max = min + 1 when max <= min, scale = (max - min) / 255,
+     * zp = round(-min / scale) in double (half away from zero, clamped to s32) with the scale as computed, and only
+     * then scale = max(scale, 1e-10).  Elements: q = clamp(int32(nearbyint(v / scale)) + zp, 0, 255)
+     * (reorder_data_type/scalar_impl/scalar_ref_kernels.cpp:36-40); non-finite elements, whose cast the reference
+     * leaves undefined, give 0 as in its per-token kernels.  The reference's AVX-512 per-tensor kernels may multiply
+     * by a reciprocal instead of dividing: parity of the last count on exact ties is unpinned. */
+    if (transA || zo_nelems(&p->src_scale) != 1 || p->src_zp.ndims <= 0 || zo_nelems(&p->src_zp) != 1 ||
+        p->src_zp.dt != ZMI_DT_S32)
+      return ZMI_UNIMPLEMENTED;
+    float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t k = 0; k < K; ++k) {
+        float v = zo_read_f32(A, a_dt, m * lda + k);
+        if (isfinite(v)) { if (v < lo) lo = v; if (v > hi) hi = v; }
+      }
+    if (lo == 3.402823466e+38f && hi == -3.402823466e+38f) lo = hi = 0.0f;
+    if (hi <= lo) hi = lo + 1.0f;
+    float s = (hi - lo) / 255.0f;
+    double zd = round((double)(-lo) / (double)s);
+    dyn_zp = zd < -2147483648.0 ? INT32_MIN : zd > 2147483647.0 ? INT32_MAX : (int32_t)zd;
+    if (s < 1e-10f) s = 1e-10f;
+    qbuf = (int8_t *)malloc((size_t)M * K);
+    sbuf = (float *)malloc(sizeof(float));
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t k = 0; k < K; ++k) {
+        float v = zo_read_f32(A, a_dt, m * lda + k);
+        int64_t q = 0;
+        if (isfinite(v)) {
+          float t = nearbyintf(v / s);
+          if (t > 4e9f) t = 4e9f;
+          if (t < -4e9f) t = -4e9f;
+          q = (int64_t)t + (int64_t)dyn_zp;
+          q = q < 0 ? 0 : q > 255 ? 255 : q;
+        }
+        ((uint8_t *)qbuf)[m * K + k] = (uint8_t)q;
+      }
+    sbuf[0] = p->src_scale.dt == ZMI_DT_BF16 ? zo_bf16_to_f32(zo_f32_to_bf16_rne(s)) : s;
+    if (c->scale_out) c->scale_out[0] = sbuf[0];
+    if (c->zp_out) c->zp_out[0] = dyn_zp;
+    pl.src_zp.buff = &dyn_zp; pl.src_zp.dt = ZMI_DT_S32;
+    A = qbuf; a_dt = ZMI_DT_U8; lda = K;
+    src_scale = sbuf; src_scale_n = 1; src_scale_dt = ZMI_DT_F32;
+  } else if (dyn) {
     if (transA) return ZMI_UNIMPLEMENTED;
     qbuf = (int8_t *)malloc((size_t)M * K);
     sbuf = (float *)malloc(sizeof(float) * (size_t)M);

@@ -884,3 +884,53 @@ def test_woq_rejections_follow_the_reference_validator(zo):
     assert call(dst=capi.DT_F16) == capi.FAILURE
     assert call(scale=False) == capi.FAILURE
     assert call(dyn=1) == capi.UNIMPLEMENTED                         # W4A8: zo_matmul_int8's
+
+
+# ------------------------------------------------- dynamic quantization to u8 (per tensor)
+def test_dynamic_u8_per_tensor_closed_forms(zo):
+    # values k / 4 for k = -100 .. 155: min -25, max 38.75, scale = 63.75 / 255 = 0.25 exactly, zp = round(25 / 0.25) = 100,
+    # codes k + 100; the product with all-ones weights and unit weight scale is then a known integer
+    M, K, N = 2, 128, 3
+    k = np.arange(-100, 156, dtype=np.float32).reshape(M, K)
+    x = k / 4
+    w = np.ones((K, N), dtype=np.int8)
+    p = _params(dt_src=capi.DT_F32, dt_wei=capi.DT_S8, dt_dst=capi.DT_S32, dt_compute=capi.DT_U8, dynamic_quant=1,
+                src_scale=capi.quant(None, capi.DT_F32, (1, 1)), src_zp=capi.quant(None, capi.DT_S32, (1, 1)))
+    zp = np.zeros(1, dtype=np.int32)
+    st, dst, acc, scales = zo.matmul_int8(x, w, p, M, N, K, want_acc=True, want_scales=True, zp_out=zp)
+    assert st == capi.SUCCESS
+    assert scales[0] == np.float32(0.25) and zp[0] == 100
+    assert np.array_equal(acc, np.repeat((k + 100).sum(axis=1).astype(np.int32)[:, None], N, axis=1))   # u8 codes k + 100
+    # minus zp * colsum, times the source scale (the chain applies it whatever the destination type)
+    assert np.array_equal(dst[:, :N], np.repeat((k.sum(axis=1) / 4).astype(np.int32)[:, None], N, axis=1))
+    # a constant tensor: range [c, c + 1], scale 1 / 255, zp = round(-c * 255); no finite value: [0, 0] -> [0, 1], zp 0
+    # (2.5 * 255 is the tie 637.5 for the real 1 / 255; the f32 scale lies above 1 / 255, so the quotient lies below it)
+    for c, want_zp in ((2.0, -510), (-1.0, 255), (0.0, 0), (2.5, -637)):
+        xc = np.full((M, K), c, dtype=np.float32)
+        st, _, _, scales = zo.matmul_int8(xc, w, p, M, N, K, want_scales=True, zp_out=zp)
+        assert st == capi.SUCCESS and scales[0] == np.float32(1.0) / np.float32(255.0)
+        assert zp[0] == want_zp, (c, zp[0])
+    xn = np.full((M, K), np.nan, dtype=np.float32)
+    st, dst, acc, scales = zo.matmul_int8(xn, w, p, M, N, K, want_acc=True, want_scales=True, zp_out=zp)
+    assert st == capi.SUCCESS and zp[0] == 0 and not acc.any()
+    # per-token dims: the GEMM has one zero-point to read
+    p2 = _params(dt_src=capi.DT_F32, dt_wei=capi.DT_S8, dt_dst=capi.DT_S32, dt_compute=capi.DT_U8, dynamic_quant=1,
+                 src_scale=capi.quant(None, capi.DT_F32, (M, 1)), src_zp=capi.quant(None, capi.DT_S32, (M, 1)))
+    assert zo.matmul_int8(x, w, p2, M, N, K)[0] == capi.UNIMPLEMENTED
+
+
+def test_dynamic_u8_dequantizes_to_the_source_within_half_a_step(zo):
+    rng = np.random.default_rng(5)
+    M, K = 6, 64
+    x = (rng.standard_normal((M, K)) * 2 + 1).astype(np.float32)
+    eye = np.eye(K, dtype=np.int8)
+    one = np.ones(1, dtype=np.float32)
+    p = _params(dt_src=capi.DT_F32, dt_wei=capi.DT_S8, dt_dst=capi.DT_F32, dt_compute=capi.DT_U8, dynamic_quant=1,
+                src_scale=capi.quant(None, capi.DT_F32, (1, 1)), src_zp=capi.quant(None, capi.DT_S32, (1, 1)),
+                wei_scale=capi.quant(one.ctypes.data, capi.DT_F32, (1,)))
+    zp = np.zeros(1, dtype=np.int32)
+    st, dst, _, scales = zo.matmul_int8(x, eye, p, M, K, K, want_scales=True, zp_out=zp)
+    assert st == capi.SUCCESS
+    # identity weights: dst = (q - zp) * scale, the dequantized source
+    assert np.abs(dst[:, :K] - x).max() <= 0.5 * scales[0] * (1 + 1e-5) + 1e-6
+    assert scales[0] == (x.max() - x.min()) / np.float32(255.0)

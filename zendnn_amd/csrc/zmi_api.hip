@@ -436,6 +436,13 @@ void zmi_reorder_params_init(zmi_reorder_params_t *p) {
   p->prepack.algo = ZMI_ALGO_NONE;
 }
 
+// groups of a dynamic call's source scale dims ({M,G} with G > 1), else 0
+static int64_t pg_groups_of(const zmi_matmul_params_t &p, int M) {
+  int64_t n = 1;
+  for (int i = 0; i < p.src_scale.ndims; ++i) n *= p.src_scale.dims[i];
+  return n > M && n % M == 0 ? n / M : 0;
+}
+
 // One matrix product (Batch_A == Batch_B == 1): everything matmul_direct does for one (src, weight, dst).
 static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_t M, int32_t N, int32_t K,
                              float alpha, const void *src, int32_t lda, const void *weight, int32_t ldb,
@@ -480,7 +487,50 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     set_error("source must be u8 / s8, or bf16 / f32 with dynamic_quant and an s8 compute type");
     return ZMI_UNIMPLEMENTED;
   }
-  if (dyn && p.dt_compute == ZMI_DT_U8) { set_error("dynamic u8 (asymmetric) quantization is not implemented"); return ZMI_UNIMPLEMENTED; }
+  if (dyn && p.dt_compute == ZMI_DT_U8) {
+    // Dynamic asymmetric quantization of the source to u8 (matmul/quantization/reorder_quantization.cpp:60-75, 208-230:
+    // scale and zero-point dims and types are required, their buffers optional).  The GEMM reads ONE source zero-point
+    // (backends/aocl/aocl_kernel.cpp:971-980), so the granularity that means something is per tensor: the source
+    // becomes u8 rows with one scale and one zero-point in device memory, and the call goes on as a static u8 call.
+    if (w4a8 || pg_groups_of(p, M) || nelems(p.src_scale) != 1 || p.src_zp.ndims <= 0 || nelems(p.src_zp) != 1) {
+      set_error("dynamic quantization to u8: one source scale and one source zero-point (dims {1} / {1,1}) are implemented");
+      return ZMI_UNIMPLEMENTED;
+    }
+    if (p.src_zp.dt != ZMI_DT_S32) { set_error("dynamic quantization to u8: src_zp.dt must be s32"); return ZMI_FAILURE; }
+    const int32_t sdt = p.src_scale.dt;
+    if (sdt != ZMI_DT_F32 && sdt != ZMI_DT_BF16) { set_error("dynamic quantization: src_scale.dt must be f32 or bf16"); return ZMI_FAILURE; }
+    if (transA) { set_error("dynamic quantization of a transposed source is not implemented"); return ZMI_UNIMPLEMENTED; }
+    if (lda < K) { set_error("leading dimension too small"); return ZMI_FAILURE; }
+    if ((p.src_scale.buff && !is_device_pointer(p.src_scale.buff)) || (p.src_zp.buff && !is_device_pointer(p.src_zp.buff))) {
+      set_error("dynamic quantization to u8 writes src_scale / src_zp: device memory (or null: the library keeps them)");
+      return ZMI_FAILURE;
+    }
+    if (!ensure_device()) return ZMI_FAILURE;
+    // (its own scratch: the static call that follows lays out the thread's arena anew)
+    static thread_local Arena rows;
+    const size_t qb = Arena::padded((size_t)M * K), lb = Arena::padded(sizeof(float) * 2 * (size_t)M);
+    if (!rows.begin(qb + lb + 3 * 256)) return ZMI_FAILURE;
+    uint8_t *q = (uint8_t *)rows.alloc(qb);
+    float *lohi = (float *)rows.alloc(lb);
+    float *s32 = (float *)rows.alloc(4);
+    void *s16 = rows.alloc(2);
+    int32_t *zp = (int32_t *)rows.alloc(4);
+    if (!q || !lohi || !s32 || !s16 || !zp) { set_error("no scratch for the quantized source"); return ZMI_FAILURE; }
+    float *scale_f32 = sdt == ZMI_DT_F32 && p.src_scale.buff ? (float *)p.src_scale.buff : s32;
+    void *scale_bf16 = sdt == ZMI_DT_BF16 ? (p.src_scale.buff ? (void *)p.src_scale.buff : s16) : nullptr;
+    int32_t *zp_out = p.src_zp.buff ? (int32_t *)p.src_zp.buff : zp;
+    if (!hip_ok(zmi_launch_quant_asym_tensor(src, p.dt_src, M, K, lda, q, K, lohi, scale_f32, zp_out, scale_bf16, sdt, stream()),
+                "asymmetric quantization launch"))
+      return ZMI_FAILURE;
+    zmi_matmul_params_t ip = p;
+    ip.dt_src = ZMI_DT_U8;
+    ip.dynamic_quant = 0;
+    ip.src_scale.buff = sdt == ZMI_DT_BF16 ? (const void *)scale_bf16 : (const void *)scale_f32;   // (the GEMM reads the narrowed value)
+    ip.src_scale.ndims = 1; ip.src_scale.dims[0] = 1;
+    ip.src_zp.buff = zp_out;
+    ip.src_zp.ndims = 1; ip.src_zp.dims[0] = 1;
+    return matmul_single(layout, 0, transB, M, N, K, alpha, q, K, weight, ldb, bias, beta, dst, ldc, is_weights_const, ip);
+  }
   if (lda < (transA ? M : K) || ldc < N || ldb < (transB ? K : N)) {
     if (p.mem_format_b != 'r' || lda < (transA ? M : K) || ldc < N) { set_error("leading dimension too small"); return ZMI_FAILURE; }
   }

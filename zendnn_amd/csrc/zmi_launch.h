@@ -177,6 +177,12 @@ hipError_t zmi_launch_pgring_scales(const void *src, int32_t dt, int64_t rows, i
 // p.A: s8 rows in fragment order; ss: {M, G} f32 source scales; ws: the padded f32 weight scales
 hipError_t zmi_launch_gemm_pgring(const ZmiProblem &p, const ZmiEpilogue &epi, const float *ss, const float *ws,
                                   hipStream_t stream);
+// Dynamic asymmetric quantization of a whole [M, K] bf16 / f32 source to u8 with one scale and one zero-point
+// (k_asym.hip).  lohi: 2 * M floats of scratch; scale / zp: one element each, device memory.
+hipError_t zmi_launch_quant_asym_tensor(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, uint8_t *q,
+                                        int64_t ldq, float *lohi, float *scale, int32_t *zp, void *user_scale,
+                                        int32_t user_dt, hipStream_t stream);
+
 // Weight-only quantization (k_woq.hip): bf16 rows x 4-bit weights dequantized to bf16 in registers, f32 accumulation.
 struct ZmiWoqProblem {
   const void *A;            // bf16 [M, lda] (or [K, lda] when transA)
