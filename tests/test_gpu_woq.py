@@ -246,3 +246,23 @@ def test_rejections():
     assert call(wdims=(16, N)) == capi.UNIMPLEMENTED                # groups of 4 values of K
     assert call(dst_dt=capi.DT_S8) == capi.UNIMPLEMENTED
     capi.load().zmi_clear_weight_cache()
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shapes_kinds_and_granularities(zo, seed):
+    rng = np.random.default_rng(9000 + seed)
+    M = int(rng.choice([1, 2, 5, 16, 17, 32, 33, 63, 64, 65, 100, 129, 200]))
+    K = int(rng.choice([8, 24, 64, 72, 120, 128, 192, 520, 1000, 1024, 1536, 4104]))
+    N = int(rng.integers(1, 150))
+    kind = list(KINDS)[int(rng.integers(0, 4))]
+    gran = ["tensor", "channel", "group"][int(rng.integers(0, 3))]
+    G = 1
+    if gran == "group":
+        divs = [g for g in (2, 3, 4, 5, 8, 13, 16, 24) if K % g == 0 and (K // g) % 8 == 0]
+        if not divs:
+            gran = "channel"
+        else:
+            G = int(rng.choice(divs))
+    _run(zo, M, K, N, kind, gran, G, ws_bf16=bool(rng.integers(0, 2)), dst_dt=[capi.DT_BF16, capi.DT_F32][int(rng.integers(0, 2))],
+         bias=bool(rng.integers(0, 2)), transB=bool(rng.integers(0, 2)), pad=int(rng.integers(0, 2)) * 2,
+         cache=bool(rng.integers(0, 4)), seed=seed)
