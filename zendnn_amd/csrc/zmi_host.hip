@@ -496,7 +496,8 @@ const uint8_t *packed_woq_weights(const void *weight, int64_t K, int64_t N, int6
   }
   void *blob = nullptr;
   if (!hip_ok(hipMalloc(&blob, total), "hipMalloc(4-bit weights)")) return nullptr;
-  if (!fill((uint8_t *)blob)) {
+  // (the entry becomes visible to threads on other streams: its contents must be there first)
+  if (!fill((uint8_t *)blob) || !hip_ok(hipStreamSynchronize(stream()), "hipStreamSynchronize(4-bit weights)")) {
     (void)hipFree(blob);
     return nullptr;
   }
