@@ -266,3 +266,24 @@ def test_random_shapes_kinds_and_granularities(zo, seed):
     _run(zo, M, K, N, kind, gran, G, ws_bf16=bool(rng.integers(0, 2)), dst_dt=[capi.DT_BF16, capi.DT_F32][int(rng.integers(0, 2))],
          bias=bool(rng.integers(0, 2)), transB=bool(rng.integers(0, 2)), pad=int(rng.integers(0, 2)) * 2,
          cache=bool(rng.integers(0, 4)), seed=seed)
+
+
+@pytest.mark.parametrize("kind", list(KINDS))
+def test_two_column_blocks_per_workgroup(zo, kind, monkeypatch):
+    # the form wide decode-shaped calls take by themselves (more than 4 rows, at least 384 column blocks), forced here
+    # on small shapes: odd block counts, one block, a K tail, one-hot sources (bit-exact)
+    monkeypatch.setenv("ZMI_WOQ_BLOCKS", "2")
+    _run(zo, 32, 256, 70, kind, "group", 4, x=_one_hot(256)[:32], dst_dt=capi.DT_F32, exact=True)
+    _run(zo, 16, 1000, 33, kind, "channel", bias=True)
+    _run(zo, 1, 512, 20, kind, "tensor", dst_dt=capi.DT_F32)
+    _run(zo, 9, 1024, 200, kind, "group", 8, calls=2)
+    _run(zo, 40, 512, 100, kind, "group", 8)          # more than 32 rows: the one-block form whatever the switch says
+
+
+def test_wide_decode_calls_take_two_column_blocks_by_themselves(zo):
+    _run(zo, 16, 1024, 12288, "s4", "group", 8, bias=True)
+    assert "two column blocks" in lowoha.last_kernel()
+    _run(zo, 16, 1024, 12360, "u4_bf16", "group", 8)      # 387 column blocks: the last workgroup has one
+    assert "two column blocks" in lowoha.last_kernel()
+    _run(zo, 4, 1024, 12288, "s4", "group", 8)
+    assert "two column blocks" not in lowoha.last_kernel()

@@ -17,6 +17,7 @@
 // loop after it).
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <type_traits>
 
 #include "../../include/zmi_lowoha.h"
@@ -156,20 +157,22 @@ template <int MT> struct WoqWaves { static constexpr int W = MT <= 2 ? 8 : 4; };
 // GENERAL = false: rows read 16 bytes at a time, one scale per 64-value chunk (scale groups are multiples of 64, or
 // there are none).  GENERAL = true: rows element by element (any stride, transposed sources, K not a multiple of 8),
 // scales looked up per 8 values.
-template <int MT, int Q, bool GENERAL>
-__global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1) void zmi_gemm_woq_kernel(ZmiWoqProblem p, ZmiEpilogue epi) {
+// NB: column blocks of 32 a workgroup multiplies with each row fragment (2: the rows cross L2 once per 64 columns)
+template <int MT, int Q, bool GENERAL, int NB = 1>
+__global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL && NB == 1) ? 4 : 1) void zmi_gemm_woq_kernel(ZmiWoqProblem p, ZmiEpilogue epi) {
   constexpr int W = WoqWaves<MT>::W, U = 8;
-  extern __shared__ float woq_red[];   // [W][MT * 16][64]
+  extern __shared__ float woq_red[];   // [W][NB][MT * 16][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nb = blockIdx.x, m0 = blockIdx.y * 32 * MT;
-  const int nc = min(nb * 32 + (lane & 31), p.N - 1), kh = lane >> 5;
+  const int m0 = blockIdx.y * 32 * MT, kh = lane >> 5, nblk = (p.N + 31) / 32;
   const int nkc = (p.K + 63) / 64;
 
-  woq_f32x16 acc[MT];
+  woq_f32x16 acc[NB][MT];
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
+  for (int b = 0; b < NB; ++b)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[b][i][r] = 0.0f;
 
   // Requests run ahead of their use: a wavefront's next 8 chunks of weights (the whole K up to 4096), and the rows and
   // scales of the chunk after the one being multiplied (loads come back in the order they were asked for, so a
@@ -177,12 +180,22 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1
   // in scalar registers) plus a 32-bit offset per lane that never changes.
   constexpr int RING = !GENERAL && MT <= 2 ? 2 : 1;
   constexpr int NS = GENERAL ? 4 : 1;
-  uint4 wq[U];
-  float sw[RING][NS], zw[RING][NS];
+  uint4 wq[NB][U];
+  float sw[RING][NS][NB], zw[RING][NS][NB];
   uint4 af[RING][4][MT];
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-  const char *wbase = (const char *)p.tiles + (int64_t)nb * nkc * 1024;
-  const uint32_t woff = lane * 16, noff = nc * 4;
+  // (a workgroup whose last block lies beyond N multiplies the last block that exists again and stores nothing of it)
+  const char *wbase[NB];
+  int nc[NB];
+  uint32_t noff[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int nb = min((int)blockIdx.x * NB + b, nblk - 1);
+    wbase[b] = (const char *)p.tiles + (int64_t)nb * nkc * 1024;
+    nc[b] = min(nb * 32 + (lane & 31), p.N - 1);
+    noff[b] = nc[b] * 4;
+  }
+  const uint32_t woff = lane * 16;
   uint32_t aoff[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
@@ -192,7 +205,7 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1
   }
   // the rows as a buffer of M * lda bf16 values (untyped, 32-bit offsets, range-checked)
   const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.A, 0, GENERAL ? 0 : p.M * (int)p.lda * 2, 0x00020000);
-  auto load_weights = [&](int kc) { return *(const uint4 *)(wbase + (int64_t)min(kc, nkc - 1) * 1024 + woff); };
+  auto load_weights = [&](int b, int kc) { return *(const uint4 *)(wbase[b] + (int64_t)min(kc, nkc - 1) * 1024 + woff); };
   // TAIL = false: every value of the chunk lies inside K
   auto load_rows = [&](auto tail, int slot, int kc) {
     constexpr bool TAIL = decltype(tail)::value;
@@ -217,14 +230,17 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1
       }
 #pragma unroll
     for (int t = 0; t < NS; ++t) {
-      if (GENERAL) {
-        const int64_t gi = (int64_t)min((kc * 64 + t * 16 + kh * 8) / p.group_size, p.n_groups - 1) * p.N + nc;
-        sw[slot][t] = p.sf[gi];
-        zw[slot][t] = Q == 0 ? 0.0f : p.zf[gi];
-      } else {
-        const int64_t go = (int64_t)min((kc * 64) / p.group_size, p.n_groups - 1) * p.N * 4;
-        sw[slot][t] = *(const float *)((const char *)p.sf + go + noff);
-        zw[slot][t] = Q == 0 ? 0.0f : *(const float *)((const char *)p.zf + go + noff);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (GENERAL) {
+          const int64_t gi = (int64_t)min((kc * 64 + t * 16 + kh * 8) / p.group_size, p.n_groups - 1) * p.N + nc[b];
+          sw[slot][t][b] = p.sf[gi];
+          zw[slot][t][b] = Q == 0 ? 0.0f : p.zf[gi];
+        } else {
+          const int64_t go = (int64_t)min((kc * 64) / p.group_size, p.n_groups - 1) * p.N * 4;
+          sw[slot][t][b] = *(const float *)((const char *)p.sf + go + noff[b]);
+          zw[slot][t][b] = Q == 0 ? 0.0f : *(const float *)((const char *)p.zf + go + noff[b]);
+        }
       }
     }
   };
@@ -236,22 +252,27 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1
       // (a chunk beyond K that a pass without the tail handling asks for ahead is never multiplied)
       if (RING == 1) load_rows(tail, 0, kc);
       else load_rows(tail, (u + 1) % RING, TAIL ? kc + W : min(kc + W, nkc - 1));
-      const uint4 w = wq[u];
-      wq[u] = load_weights(kc + U * W);
-      const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int ts = GENERAL ? t : 0;
-        const woq_bf16x8 b = woq_dequant<Q>(wd[t], sw[u % RING][ts], zw[u % RING][ts]);
+      for (int b = 0; b < NB; ++b) {
+        const uint4 w = wq[b][u];
+        wq[b][u] = load_weights(b, kc + U * W);
+        const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(woq_bf16x8, af[u % RING][t][i]), b, acc[i], 0, 0, 0);
+        for (int t = 0; t < 4; ++t) {
+          const int ts = GENERAL ? t : 0;
+          const woq_bf16x8 bv = woq_dequant<Q>(wd[t], sw[u % RING][ts][b], zw[u % RING][ts][b]);
+#pragma unroll
+          for (int i = 0; i < MT; ++i)
+            acc[b][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(woq_bf16x8, af[u % RING][t][i]), bv, acc[b][i], 0, 0, 0);
+        }
       }
     }
   };
   if (RING > 1) load_rows(std::true_type{}, 0, wave_s);
 #pragma unroll
-  for (int u = 0; u < U; ++u) wq[u] = load_weights(wave_s + u * W);
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) wq[b][u] = load_weights(b, wave_s + u * W);
   zmi_set_f32_flush();
   for (int kc0 = wave_s; kc0 < nkc; kc0 += U * W) {
     // a pass whose 8 chunks, and the chunk it asks for ahead, lie inside K (or beyond the last chunk) needs no tail handling
@@ -263,23 +284,26 @@ __global__ __launch_bounds__(WoqWaves<MT>::W * 64, (MT == 1 && !GENERAL) ? 4 : 1
   __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 3);
 
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
+  for (int b = 0; b < NB; ++b)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) woq_red[((wave * MT + i) * 16 + r) * 64 + lane] = acc[i][r];
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) woq_red[(((wave * NB + b) * MT + i) * 16 + r) * 64 + lane] = acc[b][i][r];
   __syncthreads();
-  for (int sidx = threadIdx.x; sidx < MT * 16 * 64; sidx += W * 64) {
-    const int ln = sidx & 63, r = (sidx >> 6) & 15, i = sidx >> 10;
+  for (int sidx = threadIdx.x; sidx < NB * MT * 16 * 64; sidx += W * 64) {
+    const int ln = sidx & 63, r = (sidx >> 6) & 15, i = (sidx >> 10) % MT, b = sidx / (MT * 1024);
+    const int nb = (int)blockIdx.x * NB + b;
     const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * (ln >> 5) + (r & 3), n = nb * 32 + (ln & 31);
-    if (m >= p.M || n >= p.N) continue;
+    if (m >= p.M || n >= p.N || nb >= nblk) continue;
     float y = woq_red[sidx];
 #pragma unroll
-    for (int w = 1; w < W; ++w) y = __fadd_rn(y, woq_red[w * MT * 16 * 64 + sidx]);
+    for (int w = 1; w < W; ++w) y = __fadd_rn(y, woq_red[w * NB * MT * 16 * 64 + sidx]);
     const int64_t o = (int64_t)m * p.ldc + n;
     if (epi.alpha != 1.0f) y = __fmul_rn(y, epi.alpha);
     if (epi.beta != 0.0f) y = __fadd_rn(y, __fmul_rn(zmi_ld_f32(p.dst, epi.dst_dt, o), epi.beta));
     // (-0 is the one value whose addition changes nothing, not even the sign of a zero)
-    const float b = p.bias ? zmi_ld_f32(p.bias, epi.bias_dt, n) : -0.0f;
-    zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_tail(epi, y, b, m, n));
+    const float bv = p.bias ? zmi_ld_f32(p.bias, epi.bias_dt, n) : -0.0f;
+    zmi_store(p.dst, epi.dst_dt, o, zmi_epilogue_tail(epi, y, bv, m, n));
   }
 }
 
@@ -301,11 +325,40 @@ static hipError_t woq_launch_q(const ZmiWoqProblem &p, const ZmiEpilogue &epi, i
   return hipGetLastError();
 }
 
+// two column blocks per workgroup: up to 32 rows on the fast build
+static hipError_t woq_launch_nb2(const ZmiWoqProblem &p, const ZmiEpilogue &epi, int q, hipStream_t stream) {
+  constexpr int W = WoqWaves<1>::W;
+  const int smem = W * 2 * 16 * 64 * 4;
+  const dim3 grid((unsigned)(((p.N + 31) / 32 + 1) / 2), 1);
+  const void *f = q == 0 ? (const void *)zmi_gemm_woq_kernel<1, 0, false, 2> : q == 1 ? (const void *)zmi_gemm_woq_kernel<1, 1, false, 2>
+                : q == 2 ? (const void *)zmi_gemm_woq_kernel<1, 2, false, 2> : (const void *)zmi_gemm_woq_kernel<1, 3, false, 2>;
+  hipError_t e = zmi_func_smem_once(f, smem);
+  if (e != hipSuccess) return e;
+  switch (q) {
+  case 0: hipLaunchKernelGGL((zmi_gemm_woq_kernel<1, 0, false, 2>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  case 1: hipLaunchKernelGGL((zmi_gemm_woq_kernel<1, 1, false, 2>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  case 2: hipLaunchKernelGGL((zmi_gemm_woq_kernel<1, 2, false, 2>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  default: hipLaunchKernelGGL((zmi_gemm_woq_kernel<1, 3, false, 2>), grid, dim3(W * 64), smem, stream, p, epi); break;
+  }
+  return hipGetLastError();
+}
+
 template <bool GENERAL>
 static hipError_t woq_launch_m(const ZmiWoqProblem &p, const ZmiEpilogue &epi, int q, hipStream_t stream) {
   if (p.M <= 32) return woq_launch_q<1, GENERAL>(p, epi, q, stream);
   if (p.M <= 64) return woq_launch_q<2, GENERAL>(p, epi, q, stream);
   return woq_launch_q<4, GENERAL>(p, epi, q, stream);
+}
+
+static bool woq_general(const ZmiWoqProblem &p) { return !p.a_fast || (p.n_groups > 1 && p.group_size % 64 != 0); }
+
+// Column blocks per workgroup.  More than a few rows and enough column blocks to give every CU a workgroup of two: the
+// rows cross L2 half as often (M = 16, K = 4096, N = 14336: 16.5 -> 13.5 us).  ZMI_WOQ_BLOCKS=1 / 2 forces the choice
+// where the two-block build exists (up to 32 rows, the fast build); the tests use it.
+int zmi_woq_blocks(const ZmiWoqProblem &p) {
+  if (woq_general(p) || p.M > 32) return 1;
+  if (const char *env = std::getenv("ZMI_WOQ_BLOCKS")) return std::atoi(env) == 2 ? 2 : 1;
+  return p.M > 4 && (p.N + 31) / 32 >= 384 ? 2 : 1;
 }
 
 hipError_t zmi_launch_gemm_woq(const ZmiWoqProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
@@ -317,6 +370,7 @@ hipError_t zmi_launch_gemm_woq(const ZmiWoqProblem &p, const ZmiEpilogue &epi, h
     return hipErrorInvalidValue;
   const int q = p.is_u4 ? (p.zp_float_domain ? 3 : 2) : (p.has_zp ? 1 : 0);
   if (p.is_u4 && !p.has_zp) return hipErrorInvalidValue;
-  const bool general = !p.a_fast || (p.n_groups > 1 && p.group_size % 64 != 0);
+  const bool general = woq_general(p);
+  if (zmi_woq_blocks(p) == 2) return woq_launch_nb2(p, epi, q, stream);
   return general ? woq_launch_m<true>(p, epi, q, stream) : woq_launch_m<false>(p, epi, q, stream);
 }

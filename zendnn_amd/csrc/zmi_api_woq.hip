@@ -117,7 +117,9 @@ int32_t matmul_woq(char layout, int32_t transA, int32_t transB, int32_t M, int32
   w.M = M; w.N = N; w.K = K;
   w.is_u4 = u4 ? 1 : 0;
   w.bias = bias;
-  set_kernel_name(u4 ? "woq_u4_dequant_mfma32x32x16_bf16" : "woq_s4_dequant_mfma32x32x16_bf16");
+  const bool two = zmi_woq_blocks(w) == 2;
+  set_kernel_name(u4 ? (two ? "woq_u4_dequant_mfma32x32x16_bf16 (two column blocks per workgroup)" : "woq_u4_dequant_mfma32x32x16_bf16")
+                     : (two ? "woq_s4_dequant_mfma32x32x16_bf16 (two column blocks per workgroup)" : "woq_s4_dequant_mfma32x32x16_bf16"));
   st = hip_ok(zmi_launch_gemm_woq(w, epi, stream()), "weight-only GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
   upload_fence();
   return st;

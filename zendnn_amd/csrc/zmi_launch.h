@@ -215,6 +215,8 @@ hipError_t zmi_launch_woq_tiles(const void *packed, int64_t K, int64_t N, int64_
                                 hipStream_t stream);
 // (of the epilogue descriptor only alpha, beta, bias_dt, the post-ops and dst_dt are read)
 hipError_t zmi_launch_gemm_woq(const ZmiWoqProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+// column blocks of 32 a workgroup of that launch multiplies with each row fragment (1 or 2)
+int zmi_woq_blocks(const ZmiWoqProblem &p);
 
 // 4-bit tiles of a blob of widened s4 weights (zmi_s4_tiles_bytes(K, N) bytes)
 hipError_t zmi_launch_s4_tiles(const uint8_t *blob, int64_t K, int64_t N, uint8_t *out, hipStream_t stream);
