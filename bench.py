@@ -31,7 +31,7 @@ INT8_PEAK_TOPS = 5000.0
 K_DEC, N_DEC = 4096, 14336
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
 # size), measured with the commands recorded in profiles/zmi_gemm_decode16_kernel_decode_M16_K4096_N14336.md
-DECODE_TRAFFIC_BYTES = 60345848
+DECODE_TRAFFIC_BYTES = 60346524
 
 
 def main():
