@@ -388,6 +388,11 @@ ZO_EXPORT float zo_eltwise(int32_t po, float x, float alpha, float beta) {
   case ZMI_PO_SQRT: return sqrtf(x);
   case ZMI_PO_EXP: return expf(x);
   case ZMI_PO_LOG: return logf(x);
+  /* mish_fwd, operators/matmul/matmul_ref_kernel.cpp:755-760 (std:: overloads on float: all float arithmetic) */
+  case ZMI_PO_MISH: {
+    const float softplus = fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x)));
+    return x * tanhf(softplus);
+  }
   default: return x;
   }
 }
@@ -624,6 +629,9 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
     double zd = round((double)(-lo) / (double)s);
     dyn_zp = zd < -2147483648.0 ? INT32_MIN : zd > 2147483647.0 ? INT32_MAX : (int32_t)zd;
     if (s < 1e-10f) s = 1e-10f;
+    /* a bf16 scale buffer: the parameters are stored first (narrowed, lowoha_reorder_utils.cpp:600-628, 810) and the
+     * codes are then made by the static reorder on what the buffer reads back as (lowoha_reorder.cpp:186-205) */
+    if (p->src_scale.dt == ZMI_DT_BF16) s = zo_bf16_to_f32(zo_f32_to_bf16_rne(s));
     qbuf = (int8_t *)malloc((size_t)M * K);
     sbuf = (float *)malloc(sizeof(float));
     for (int64_t m = 0; m < M; ++m)
@@ -639,7 +647,7 @@ ZO_EXPORT int32_t zo_matmul_int8(const zo_matmul_call *c) {
         }
         ((uint8_t *)qbuf)[m * K + k] = (uint8_t)q;
       }
-    sbuf[0] = p->src_scale.dt == ZMI_DT_BF16 ? zo_bf16_to_f32(zo_f32_to_bf16_rne(s)) : s;
+    sbuf[0] = s;
     if (c->scale_out) c->scale_out[0] = sbuf[0];
     if (c->zp_out) c->zp_out[0] = dyn_zp;
     pl.src_zp.buff = &dyn_zp; pl.src_zp.dt = ZMI_DT_S32;

@@ -85,8 +85,28 @@ def test_matmul_validation_status_codes():
     p = _int8_params()
     p.postop_ = [lowoha.PostOp(capi.PO_CLIP, alpha=float("nan"), beta=1.0)]
     assert _mm(p) == capi.FAILURE
+    # mish: refused with per-row source scales on s8 rows, with dynamic quantization and on W4A8
+    # (lowoha_matmul_utils.cpp:379-408); the static scale chain takes it (no GPU here: the call then
+    # fails later, for another reason)
+    p = _int8_params(dt_src=capi.DT_S8, dt_dst=capi.DT_BF16, src_scale=q((4, 1)), wei_scale=q((1, 8)))
     p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
-    assert _mm(p) == capi.FAILURE
+    assert _mm(p) == capi.FAILURE and "mish" in lowoha.last_error()
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (4, 1))
+    p.wei_scale = q((1, 8))
+    p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
+    assert _mm(p) == capi.FAILURE and "mish" in lowoha.last_error()
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S4, dst=capi.DT_BF16, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (4, 1))
+    p.wei_scale = q((1, 8))
+    p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
+    assert _mm(p) == capi.FAILURE and "mish" in lowoha.last_error()
+    p = _int8_params(src_scale=q((1,)), wei_scale=q((1, 8)))
+    p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
+    _mm(p)
+    assert "mish" not in lowoha.last_error()
     # outside the implemented path: status unimplemented, not failure
     assert _mm(lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_BF16, dst=capi.DT_BF16)) == capi.UNIMPLEMENTED
     # GGML-packed weights: transB = true is required (the packed layout is N x K), as in the reference

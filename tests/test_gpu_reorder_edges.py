@@ -181,10 +181,10 @@ def test_every_eltwise_post_op_f32(zo, po, M):
     H.check_f32(got, want, rtol=1e-5, atol=1e-6)
 
 
-@pytest.mark.parametrize("po", [capi.PO_ELU, capi.PO_SQUARE, capi.PO_ABS, capi.PO_SQRT, capi.PO_EXP, capi.PO_LOG])
+@pytest.mark.parametrize("po", [capi.PO_ELU, capi.PO_SQUARE, capi.PO_ABS, capi.PO_SQRT, capi.PO_EXP, capi.PO_LOG, capi.PO_MISH])
 @pytest.mark.parametrize("M,dst_dt", [(7, capi.DT_F32), (24, capi.DT_BF16), (200, capi.DT_F32), (200, capi.DT_BF16)])
 def test_remaining_eltwise_post_ops(zo, po, M, dst_dt):
-    """elu (alpha from the post-op) / square / abs / sqrt / exp / log through the interpreter of every kernel that can
+    """elu (alpha from the post-op) / square / abs / sqrt / exp / log / mish through the interpreter of every kernel that can
     take the call: f32 within 1e-5 relative, bf16 within one ulp.  sqrt and log see a chain whose result is positive
     (ReLU + a bias in front of them keeps them off the reference's NaN / -inf cases, which are compared too: NaN == NaN)."""
     rng = np.random.default_rng(po * 100 + M)
@@ -301,3 +301,29 @@ def test_weight_cache_modes_agree():
     for o in outs[1:]:
         assert torch.equal(o, outs[0])
     assert torch.equal(outs[0], (a.cpu().int() @ w.cpu().int()).to(H.DEV))
+
+
+def test_mish_refused_where_the_reference_refuses_it():
+    """mish with per-row source scales on s8 rows and with dynamic quantization: failure before any launch
+    (lowoha_matmul_utils.cpp:379-408); the static per-tensor chain above computes it."""
+    rng = np.random.default_rng(5)
+    M, K, N = 8, 64, 32
+    ws_d = H.to_dev(rng.uniform(0.001, 0.01, N).astype(np.float32))
+    ss_d = H.to_dev(rng.uniform(0.01, 0.02, M).astype(np.float32))
+    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+    w_d = H.to_dev(H.gen_weights(rng, K, N))
+    p = lowoha.MatmulParams(src=capi.DT_S8, wei=capi.DT_S8, dst=capi.DT_BF16)
+    p.src_scale = lowoha.QuantParam(ss_d, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
+    a_d = H.to_dev(rng.integers(-128, 128, (M, K), dtype=np.int8))
+    assert lowoha.matmul_direct("r", False, False, M, N, K, 1.0, a_d, K, w_d, N, None, 0.0, dst, N, True, p) == capi.FAILURE
+    assert "mish" in lowoha.last_error()
+    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+    p.dynamic_quant = True
+    p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (M, 1))
+    p.wei_scale = lowoha.QuantParam(ws_d, capi.DT_F32, (1, N))
+    p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
+    x_d = H.to_dev(H.gen_bf16_normal(rng, (M, K)))
+    assert lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x_d, K, w_d, N, None, 0.0, dst, N, True, p) == capi.FAILURE
+    assert "mish" in lowoha.last_error()

@@ -719,6 +719,24 @@ def test_remaining_eltwise_types_closed_forms_and_libm(zo):
 
 
 # ---------------------------------------------------- gated act / reduce
+def test_mish_against_libm_double_and_limits(zo):
+    """mish_fwd (matmul_ref_kernel.cpp:755-760) = x tanh(ln(1 + e^x)): libm in double on a grid, the limits the
+    mathematics fixes (mish(0) = 0, mish(x) -> x for large x, -> 0 from below for very negative x) and the identity
+    tanh(softplus(x)) = ((1 + e^x)^2 - 1) / ((1 + e^x)^2 + 1), which a dropped max(x, 0) or a wrong sign of |x| fails."""
+    xs = np.concatenate([np.linspace(-30, 30, 1201), [0.0, -0.0, 1e-6, -1e-6, 88.0, -88.0, 20.0]]).astype(np.float32)
+    got = zo.eltwise(capi.PO_MISH, xs)
+    for i, x in enumerate(xs.astype(np.float64)):
+        want = x * math.tanh(math.log1p(math.exp(x))) if x < 30 else x
+        n = (1.0 + math.exp(x)) ** 2 if x < 30 else float("inf")
+        alt = x * ((n - 1.0) / (n + 1.0)) if n != float("inf") else x
+        assert abs(want - alt) <= 1e-12 * max(1.0, abs(want)) + 1e-300
+        assert abs(float(got[i]) - want) <= 4 * float(np.spacing(np.float32(abs(want)))) + 1e-37, (x, got[i], want)
+    assert float(zo.eltwise(capi.PO_MISH, np.array([0.0], dtype=np.float32))[0]) == 0.0
+    assert float(zo.eltwise(capi.PO_MISH, np.array([50.0], dtype=np.float32))[0]) == 50.0
+    tail = float(zo.eltwise(capi.PO_MISH, np.array([-25.0], dtype=np.float32))[0])
+    assert -1e-9 < tail < 0.0
+
+
 def test_gated_act_brute_force(zo):
     rng = np.random.default_rng(13)
     M, dim = 5, 24
@@ -934,3 +952,23 @@ def test_dynamic_u8_dequantizes_to_the_source_within_half_a_step(zo):
     # identity weights: dst = (q - zp) * scale, the dequantized source
     assert np.abs(dst[:, :K] - x).max() <= 0.5 * scales[0] * (1 + 1e-5) + 1e-6
     assert scales[0] == (x.max() - x.min()) / np.float32(255.0)
+
+
+def test_dynamic_u8_with_a_bf16_scale_buffer_quantizes_with_the_narrowed_scale(zo):
+    """Range [0, 76.5]: scale 76.5 / 255 = 0.3 in f32, which a bf16 buffer stores as 0.30078125; the reference stores the
+    parameters and then quantizes with what the buffer reads back as (lowoha_reorder.cpp:186-205), so 76.5 becomes
+    code 254 (255 with the f32 scale) and 60 becomes 199 (200); the zero-point comes from the scale as computed."""
+    K = 64
+    x = np.zeros((1, K), dtype=np.float32)
+    x[0, :5] = [0.0, 30.0, 45.0, 60.0, 76.5]
+    eye = np.eye(K, dtype=np.int8)
+    zp = np.zeros(1, dtype=np.int32)
+    codes = {}
+    for sdt in (capi.DT_F32, capi.DT_BF16):
+        p = _params(dt_src=capi.DT_F32, dt_wei=capi.DT_S8, dt_dst=capi.DT_S32, dt_compute=capi.DT_U8, dynamic_quant=1,
+                    src_scale=capi.quant(None, sdt, (1, 1)), src_zp=capi.quant(None, capi.DT_S32, (1, 1)))
+        st, _, acc, scales = zo.matmul_int8(x, eye, p, 1, K, K, want_acc=True, want_scales=True, zp_out=zp)
+        assert st == capi.SUCCESS and zp[0] == 0
+        codes[sdt] = (acc[0, :5].tolist(), float(scales[0]))
+    assert codes[capi.DT_F32] == ([0, 100, 150, 200, 255], float(np.float32(76.5) / np.float32(255.0)))
+    assert codes[capi.DT_BF16] == ([0, 100, 150, 199, 254], 0.30078125)

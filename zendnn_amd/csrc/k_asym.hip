@@ -76,8 +76,16 @@ __global__ __launch_bounds__(256) void zmi_asym_tensor_params_kernel(const float
   const double zd = round((double)(-lo) / (double)s);
   *zp = zd < -2147483648.0 ? (int32_t)0x80000000 : zd > 2147483647.0 ? 0x7fffffff : (int32_t)zd;
   if (s < 1e-10f) s = 1e-10f;
+  // A bf16 scale buffer holds the narrowed value, and the codes are made with what that buffer reads back as: the
+  // reference computes the parameters, stores them, and then runs its static reorder on the stored parameters
+  // (lowoha_reorder.cpp:186-205 after compute_dynamic_quant_params, lowoha_reorder_utils.cpp:600-628, 810).  The
+  // zero-point above comes from the scale as computed, as there.
+  if (user_scale && user_dt == ZMI_DT_BF16) {
+    const uint16_t h = zmi_f32_to_bf16_rne(s);
+    *(uint16_t *)user_scale = h;
+    s = zmi_bf16_to_f32(h);
+  }
   *scale = s;
-  if (user_scale && user_dt == ZMI_DT_BF16) *(uint16_t *)user_scale = zmi_f32_to_bf16_rne(s);
 }
 
 template <bool BF16>
@@ -102,8 +110,8 @@ __global__ __launch_bounds__(256) void zmi_asym_tensor_quant_kernel(const void *
   }
 }
 
-// scale: the f32 the codes are made with (the caller's buffer when its type is f32, else scratch with the bf16 copy
-// going to user_scale); lohi: 2 * M floats of scratch
+// scale: the f32 the codes are made with (the caller's buffer when its type is f32; with a bf16 scale buffer scratch
+// that receives the narrowed value widened again, the bf16 itself going to user_scale); lohi: 2 * M floats of scratch
 hipError_t zmi_launch_quant_asym_tensor(const void *x, int32_t x_dt, int64_t M, int64_t K, int64_t ldx, uint8_t *q,
                                         int64_t ldq, float *lohi, float *scale, int32_t *zp, void *user_scale,
                                         int32_t user_dt, hipStream_t stream) {

@@ -873,11 +873,14 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
       forked = true;
     }
     e = ring_launch<256>(p, nullptr, 1, zmi_ring_items<256>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, stream);
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess && !forked) return e;
   }
-  e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, rem_stream, forked);
-  if (e != hipSuccess) return e;
-  e = ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, rem_stream, forked);
+  if (e == hipSuccess)
+    e = ring_launch<128>(p, nullptr, 1, zmi_ring_items<128>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, rem_stream, forked);
+  // (once forked, the join below runs whatever the launches returned: the caller's stream must stay ordered behind
+  // the side stream, and a capture must not be left with an unjoined fork)
+  if (e == hipSuccess)
+    e = ring_launch<64>(p, nullptr, 1, zmi_ring_items<64>(p.M, p.N, top, gated), true, nullptr, top, sp, epi, rem_stream, forked);
   if (forked) {
     hipError_t j = hipEventRecord(side->join, side->stream);
     if (j == hipSuccess) j = hipStreamWaitEvent(stream, side->join, 0);

@@ -9,6 +9,14 @@
 
 namespace zmi {
 
+bool is_dynamic_quant_config(const zmi_matmul_params_t &p);
+// elements the dims of a quantization parameter describe, buffer or not (1 without dims)
+static int64_t shape_elems(const zmi_quant_t &q) {
+  int64_t n = 1;
+  for (int i = 0; i < q.ndims; ++i) n *= q.dims[i];
+  return n;
+}
+
 // Mirrors validate_matmul_direct_inputs of the reference
 // (zendnnl/src/lowoha_operators/matmul/lowoha_matmul_utils.cpp:180-411) for the
 // rules that concern the int8 path.  Every failure is status failure.
@@ -81,9 +89,16 @@ int32_t validate_matmul(const void *src, const void *weight, const void *dst, in
       return ZMI_FAILURE;
     }
     if (po.po_type == ZMI_PO_MISH) {
-      // rejected on the int8 sym-quant / dynamic-quant paths, which is every path here
-      set_error("mish is not supported on the int8 paths");
-      return ZMI_FAILURE;
+      // refused where the reference refuses it (lowoha_matmul_utils.cpp:379-408): source scales per row or per
+      // K group on s8 rows (is_sym_quant_config, lowoha_matmul_utils.hpp:184-204), dynamic quantization, W4A8;
+      // the static scale chain computes it
+      const bool sym_quant = p.dt_src == ZMI_DT_S8 && p.dt_wei == ZMI_DT_S8 && !p.src_zp.buff &&
+                             (p.dt_dst == ZMI_DT_F32 || p.dt_dst == ZMI_DT_BF16) && shape_elems(p.src_scale) > 1;
+      const bool w4a8 = p.dt_wei == ZMI_DT_S4 && p.dynamic_quant;
+      if (sym_quant || is_dynamic_quant_config(p) || w4a8) {
+        set_error("mish is not supported with per-row / per-group source scales, dynamic quantization or W4A8");
+        return ZMI_FAILURE;
+      }
     }
   }
   return ZMI_SUCCESS;
@@ -227,6 +242,9 @@ int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, 
     // fault its validator already refuses mish for); here they compute what the reference's own kernel defines
     // (operators/matmul/matmul_ref_kernel.cpp:694-751; elu's alpha is the post-op's alpha).
     case ZMI_PO_ELU: case ZMI_PO_SQUARE: case ZMI_PO_ABS: case ZMI_PO_SQRT: case ZMI_PO_EXP: case ZMI_PO_LOG:
+      break;
+    // (the validator has refused it on the paths where the reference does)
+    case ZMI_PO_MISH:
       break;
     case ZMI_PO_CLIP:
       if (d.alpha > d.beta) { float t = d.alpha; d.alpha = d.beta; d.beta = t; }
@@ -457,6 +475,12 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     if (!src || !weight || !dst || M <= 0 || N <= 0 || K <= 0) { set_error("null pointer or non-positive dimension"); return ZMI_FAILURE; }
     int32_t st = validate_w4a8(p, M, N, K);
     if (st != ZMI_SUCCESS) return st;
+    // (the general validator's post-op rule, lowoha_matmul_utils.cpp:379-408, for this path)
+    for (int i = 0; i < p.n_postops; ++i)
+      if (p.postops[i].po_type == ZMI_PO_MISH) {
+        set_error("mish is not supported with per-row / per-group source scales, dynamic quantization or W4A8");
+        return ZMI_FAILURE;
+      }
     if (p.pack_format_b != 0 || p.mem_format_b == 'r') { set_error("s4 weights are passed as plain packed nibbles (mem_format_b 'n', no pack format)"); return ZMI_FAILURE; }
   } else if (diagnostics_enabled()) {
     int32_t st = validate_matmul(src, weight, dst, M, N, K, Batch_A, Batch_B, p, is_weights_const != 0);

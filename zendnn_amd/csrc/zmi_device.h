@@ -306,6 +306,8 @@ __device__ __forceinline__ float zmi_eltwise(int type, float x, float alpha, flo
   case ZMI_PO_SQRT: return __fsqrt_rn(x);
   case ZMI_PO_EXP: return zmi_expf(x);
   case ZMI_PO_LOG: return logf(x);
+  // mish_fwd, matmul_ref_kernel.cpp:755-760: x * tanh(softplus(x)), softplus = max(x, 0) + log1p(exp(-|x|))
+  case ZMI_PO_MISH: return x * tanhf(fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))));
   default: return x;
   }
 }
