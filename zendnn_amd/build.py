@@ -15,7 +15,7 @@ HOST = os.path.join(HERE, "host")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 
-HIP_SOURCES = ["k_prepack.hip", "k_quant.hip", "k_ring.hip", "k_smallm.hip", "k_decode.hip", "k_pergroup.hip", "k_moe.hip", "k_util.hip", "k_calib.hip", "k_group_decode.hip", "k_router.hip", "k_stream.hip", "k_pgring.hip", "k_woq.hip", "k_asym.hip",
+HIP_SOURCES = ["k_prepack.hip", "k_quant.hip", "k_ring.hip", "k_pring.hip", "k_smallm.hip", "k_decode.hip", "k_pergroup.hip", "k_moe.hip", "k_util.hip", "k_calib.hip", "k_group_decode.hip", "k_router.hip", "k_stream.hip", "k_pgring.hip", "k_woq.hip", "k_asym.hip",
                "zmi_host.hip", "zmi_api.hip", "zmi_api_group.hip", "zmi_api_noalloc.hip", "zmi_api_woq.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

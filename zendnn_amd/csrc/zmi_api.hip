@@ -329,6 +329,15 @@ ZmiRingPlan plan_ring_gemm(int M, int N, int K) {
   return zmi_ring_plan(M, N, K, top_hint, force);
 }
 
+// The persistent form of the large-M kernel (k_pring.hip): one problem whose (256-row band, 64-column unit) cells give
+// every compute unit at least three (a tile of 256 x 192 or more).  ZMI_PRING = 0 / 1 overrides the size rule.
+static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi) {
+  if (!zmi_pring_takes(prob, epi)) return false;
+  if (const char *env = std::getenv("ZMI_PRING")) return std::atoi(env) != 0;
+  const int64_t cells = (int64_t)((prob.M + 255) / 256) * (zmi_blob_npad(prob.N) / 64);
+  return prob.M >= 256 && cells >= 3 * (int64_t)zmi_cu_count();
+}
+
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
   if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
     set_kernel_name(zmi_decode_16row_kernel(prob, false) ? "decode16_dma_rows_mfma16x16x64" : "decode_lds_rows_mfma16x16x64");
@@ -356,6 +365,11 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
       // (null: a reduction launch finishes the elements -- also with a weight zero-point, whose per-row term only
       // the reduction's element-finishing code adds)
       split.arrivals = prob.row_comp ? nullptr : slice_arrivals(plan->tiles);
+    }
+    if (plan->slices == 1 && pring_wanted(prob, epi)) {
+      set_kernel_name("pring_mfma32x32x32_persistent");
+      if (!hip_ok(zmi_launch_gemm_pring(prob, epi, stream()), "persistent MFMA GEMM launch")) return ZMI_FAILURE;
+      return ZMI_SUCCESS;
     }
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")

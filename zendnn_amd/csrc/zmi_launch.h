@@ -93,6 +93,9 @@ struct ZmiRingSide {
 };
 hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int top, const ZmiRingSplit *split,
                                 hipStream_t stream, const ZmiRingSide *side = nullptr);
+// k_pring.hip: the persistent form for one problem (A in fragment-major order, bf16 destination, straight-line epilogue)
+bool zmi_pring_takes(const ZmiProblem &p, const ZmiEpilogue &epi);
+hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
                                       const ZmiEpilogue &epi, hipStream_t stream);
