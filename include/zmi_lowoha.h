@@ -382,6 +382,12 @@ ZMI_API int32_t zmi_moe_fused_device(const zmi_moe_device_t *d);
 ZMI_API int32_t zmi_calib_hbm_read(void *const *bufs, int32_t n_bufs, uint64_t bytes,
                            int32_t warm, int32_t launches, void *stream,
                            float *us_per_launch, float *span_us);
+/* The same read with the launch shape given: workgroups of `threads` threads (256, 512, 1024), `requests` requests
+ * of 16 bytes per lane (8, 14, 16), bytes / (threads * requests * 16) workgroups.  The best shape's figure is the
+ * ceiling a streaming kernel of this size can be held against. */
+ZMI_API int32_t zmi_calib_hbm_read_shape(void *const *bufs, int32_t n_bufs, uint64_t bytes,
+                           int32_t threads, int32_t requests, int32_t warm, int32_t launches,
+                           void *stream, float *us_per_launch, float *span_us);
 ZMI_API int32_t zmi_calib_mfma_i8(const void *operands, int32_t vary_operands,
                           int32_t wgs_per_cu, int32_t iters, void *stream,
                           float *tops, float *shader_mhz);

@@ -173,6 +173,8 @@ SIGNATURES = {
     "zmi_moe_fused_device": (C.c_int32, [C.POINTER(MoeDeviceT)]),
     "zmi_calib_hbm_read": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.c_uint64, C.c_int32, C.c_int32,
                                        C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "zmi_calib_hbm_read_shape": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.c_uint64, C.c_int32, C.c_int32, C.c_int32,
+                                             C.c_int32, C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "zmi_calib_mfma_i8": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                       C.POINTER(C.c_float), C.POINTER(C.c_float)]),
 }

@@ -44,6 +44,26 @@ __global__ __launch_bounds__(512) void zmi_calib_read_kernel(const v4i *__restri
   }
 }
 
+// The same read with the launch shape as a parameter: `grid` workgroups of THREADS threads, every lane REQ requests of
+// 16 bytes, all in flight (grid * THREADS * REQ * 16 bytes in all; workgroup b reads its own contiguous range).
+template <int THREADS, int REQ>
+__global__ __launch_bounds__(THREADS) void zmi_calib_read_shape_kernel(const v4i *__restrict__ p, int *sink) {
+  const unsigned long long t0 = wall_clock64();
+  const v4i *base = p + ((size_t)blockIdx.x * THREADS * REQ) + (threadIdx.x / 64) * 64 * REQ + threadIdx.x % 64;
+  v4i v[REQ];
+#pragma unroll
+  for (int i = 0; i < REQ; i++) v[i] = __builtin_nontemporal_load(base + (size_t)i * 64);
+  v4i acc = {0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < REQ; i++) { acc[0] ^= v[i][0]; acc[1] ^= v[i][1]; acc[2] ^= v[i][2]; acc[3] ^= v[i][3]; }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678) sink[0] = 1;   // (keeps the loads)
+  __syncthreads();
+  if (threadIdx.x == 0 && blockIdx.x < 8192) {
+    g_calib_ts[blockIdx.x * 2] = t0;
+    g_calib_ts[blockIdx.x * 2 + 1] = wall_clock64();
+  }
+}
+
 // 8 independent accumulators per wavefront; with VARY the operands of consecutive instructions differ
 template <bool VARY>
 __global__ __launch_bounds__(256) void zmi_calib_mfma_kernel(const v4i *__restrict__ operands, int iters, int *sink) {
@@ -95,6 +115,55 @@ CALIB_API int32_t zmi_calib_hbm_read(void *const *bufs, int32_t n_bufs, uint64_t
   ok = ok && hipStreamSynchronize(st) == hipSuccess && hipEventRecord(e0, st) == hipSuccess;
   for (int i = 0; ok && i < launches; ++i)
     hipLaunchKernelGGL(zmi_calib_read_kernel, dim3(grid), dim3(512), 0, st, (const v4i *)bufs[i % n_bufs], sink);
+  float ms = 0.0f;
+  ok = ok && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+       hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+  if (ok && us_per_launch) *us_per_launch = ms * 1e3f / launches;
+  if (ok && span_us) {
+    const int n = grid < 8192 ? grid : 8192;
+    std::vector<unsigned long long> ts(2 * (size_t)n);
+    ok = hipMemcpyFromSymbol(ts.data(), HIP_SYMBOL(g_calib_ts), ts.size() * 8) == hipSuccess;
+    double worst = 0.0;
+    for (int x = 0; ok && x < 8; ++x) {
+      unsigned long long a = ~0ull, b = 0;
+      for (int i = x; i < n; i += 8) { a = std::min(a, ts[i * 2]); b = std::max(b, ts[i * 2 + 1]); }
+      if (b > a) worst = std::max(worst, (double)(b - a) * 0.01);
+    }
+    *span_us = (float)worst;
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(sink);
+  return ok ? ZMI_SUCCESS : ZMI_FAILURE;
+}
+
+// zmi_calib_hbm_read with the launch shape given: threads per workgroup (256, 512 or 1024) and requests per lane
+// (8, 14 or 16); bytes must be a multiple of threads * requests * 16.  What the best shape reaches is the ceiling a
+// streaming kernel can be held against; the shape of the default entry point is the decode kernels' own.
+CALIB_API int32_t zmi_calib_hbm_read_shape(void *const *bufs, int32_t n_bufs, uint64_t bytes, int32_t threads, int32_t requests,
+                                           int32_t warm, int32_t launches, void *stream, float *us_per_launch, float *span_us) {
+  if (!bufs || n_bufs <= 0 || bytes == 0 || launches <= 0 || threads <= 0 || requests <= 0) return ZMI_FAILURE;
+  const uint64_t per_wg = (uint64_t)threads * requests * 16;
+  if (bytes % per_wg != 0) return ZMI_FAILURE;
+  hipStream_t st = (hipStream_t)stream;
+  const int grid = (int)(bytes / per_wg);
+  int *sink = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipMalloc(&sink, 256) != hipSuccess) return ZMI_FAILURE;
+  bool ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
+  bool known = true;
+  auto launch = [&](const void *buf) {
+    const v4i *p = (const v4i *)buf;
+#define ZMI_CALIB_SHAPE(T, R) \
+    if (threads == T && requests == R) { hipLaunchKernelGGL((zmi_calib_read_shape_kernel<T, R>), dim3(grid), dim3(T), 0, st, p, sink); return; }
+    ZMI_CALIB_SHAPE(256, 8) ZMI_CALIB_SHAPE(256, 14) ZMI_CALIB_SHAPE(256, 16) ZMI_CALIB_SHAPE(512, 8) ZMI_CALIB_SHAPE(512, 14)
+    ZMI_CALIB_SHAPE(512, 16) ZMI_CALIB_SHAPE(1024, 8) ZMI_CALIB_SHAPE(1024, 14) ZMI_CALIB_SHAPE(1024, 16)
+#undef ZMI_CALIB_SHAPE
+    known = false;
+  };
+  for (int i = 0; ok && known && i < warm; ++i) launch(bufs[i % n_bufs]);
+  ok = ok && known && hipStreamSynchronize(st) == hipSuccess && hipEventRecord(e0, st) == hipSuccess;
+  for (int i = 0; ok && i < launches; ++i) launch(bufs[i % n_bufs]);
   float ms = 0.0f;
   ok = ok && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
        hipEventElapsedTime(&ms, e0, e1) == hipSuccess;

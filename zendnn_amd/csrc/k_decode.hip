@@ -294,11 +294,17 @@ __global__ __launch_bounds__(DEC_THREADS, (RPW == 1 ? 4 : 2)) void zmi_gemm_deco
 // (Measured and dropped: the rows by helper wavefronts -- their requests end up behind the weights of
 // the whole compute unit; at most 2 .. 6 chunks of weights in flight per wavefront; neighbouring
 // workgroups starting at different slices of K; rows and weights requested alternately.)
+// The value is in a vector register at this point of the program, and later uses read that register.
+template <class T>
+__device__ __forceinline__ void zmi_pin_v(T &x) { asm volatile("" : "+v"(x)); }
 __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-#define D16_W_FIRST 2    // chunks of weights requested ahead of the rows
+// chunks of weights requested ahead of the rows (us per call with rows that are given, M = 16, N = 14336, whole-line
+// row requests: 0 chunks 12.12, 2 chunks 12.38, 4 chunks 12.20, all 8 12.50)
+#define D16_W_FIRST 0
 // ... ahead of the wait for rows that are quantized inside the launch (us per call at M = 16, N = 14336, one box:
 // 4 chunks 14.40, 5 chunks 14.17, 6 chunks 14.41, 7 chunks 14.68, all 8 14.67)
+// (with whole-line row requests: 3 chunks 13.77, 4 chunks 13.75, 5 chunks 13.51, 6 chunks 13.72, all 8 14.19)
 #define D16_FQ_FIRST 5
 
 // K beyond 4096 (n_slices > 1, blockIdx.y = slice): the workgroups of a column block take up to 64 chunks of K each
@@ -327,11 +333,40 @@ __device__ __forceinline__ void zmi_lds_barrier() { asm volatile("s_waitcnt lgkm
 // after they started against 9.7 us.  Sixteen copies of the flags on different memory channels bring the end of the
 // wait forward by 1.3 us, and with the rows then requested ahead of the last three chunks of weights the call takes
 // 14.2 us (either change alone: nothing, or 0.3 us).
-template <int FQ>
+#ifdef D16_TIMING
+// measurement build only: per workgroup, the constant-rate clock at its start, after its MFMAs and at its end
+__device__ unsigned long long d16_times[16 * 1024];
+extern "C" __attribute__((visibility("default"))) int zmi_debug_d16_times(unsigned long long *out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(d16_times), sizeof(d16_times));
+}
+#define D16_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 1024) d16_times[blockIdx.x * 16 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define D16_STAMPW(i) do { if (threadIdx.x % 64 == 0 && blockIdx.x < 1024) d16_times[blockIdx.x * 16 + (i) + threadIdx.x / 64] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define D16_STAMP(i)
+#define D16_STAMPW(i)
+#endif
+
+// PAIR (K a multiple of 1024, one slice): the rows are staged two chunks at a time, so that a request takes whole
+// 128-byte lines of eight rows instead of 64-byte halves of sixteen.  Every workgroup of the launch reads the same
+// rows at the same time, and it is the number of requests the L2 channels see in the launch's first microseconds,
+// not their bytes, that holds the weight stream back (M = 16 against M = 4: +1.3 us with half lines).  A pair of
+// chunks is 2 KiB of LDS: [rows 0..7 | rows 8..15][row][eight 16-byte slots], slot = (chunk % 2) * 4 + k group,
+// stored at position slot ^ ((row >> 1) & 7) (the MFMA's reads of sixteen rows then spread over the banks).
+template <int FQ, bool PAIR>
 __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiProblem p, ZmiEpilogue epi, ZmiFusedQuant fq,
                                                                            int n_slices, int32_t *partial,
                                                                            unsigned int *arrivals) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  D16_STAMP(0);
+  // Every argument word the straight-line path reads, requested here in one batch: the compiler otherwise fetches
+  // argument words where they are first used, one scalar load and one wait after the other -- two round trips ahead
+  // of the first weight request and five behind the last barrier, a microsecond of the launch in all.
+  // (one statement: the loads of all its operands are issued ahead of its one wait)
+  asm volatile("" ::"s"(p.A), "s"(p.lda), "s"(p.blob), "s"(p.dst), "s"(p.ldc), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.a_is_u8),
+               "s"(p.src_scale_ptr), "s"(p.wei_scale_ptr), "s"(p.src_zp_ptr), "s"(p.bias), "s"(p.src_scale_val),
+               "s"(p.wei_scale_val), "s"(p.src_zp_val), "s"(p.row_comp), "s"(epi.src_scale_mode), "s"(epi.src_scale_dt),
+               "s"(epi.wei_scale_mode), "s"(epi.wei_scale_dt), "s"(epi.has_zp), "s"(epi.bias_dt), "s"(epi.dst_dt),
+               "s"(epi.fast_kind), "s"(n_slices));
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int M = p.M, N = p.N, K = p.K;
@@ -346,8 +381,12 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     blk -= M;
   }
   const int slice = (int)blockIdx.y;
-  const int c0 = (int)((int64_t)slice * (K_pad / 64) / n_slices);               // this workgroup's chunks of 64 k
-  const int nchunks = (int)((int64_t)(slice + 1) * (K_pad / 64) / n_slices) - c0;
+  // this workgroup's chunks of 64 k (one slice: no division in front of the first request)
+  int c0 = 0, nchunks = K_pad / 64;
+  if (n_slices > 1) {
+    c0 = (int)((unsigned)slice * (unsigned)(K_pad / 64) / (unsigned)n_slices);
+    nchunks = (int)((unsigned)(slice + 1) * (unsigned)(K_pad / 64) / (unsigned)n_slices) - c0;
+  }
 
   // one chunk of rows -> LDS
   const int G = ((K + 15) & ~15) / 16;      // readable 16-byte granules per row
@@ -363,6 +402,26 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
 
   const int c_begin = c0 + wave * nchunks / DEC_WAVES;
   const int c_end = c0 + (wave + 1) * nchunks / DEC_WAVES;
+  // PAIR: chunks c_begin + 2 u and + 2 u + 1, rows 8 h .. 8 h + 7 (lane: row lane / 8, slot lane % 8)
+  const int p_r = lane / 8;
+  auto stage_pair = [&](int u, int h) {
+    const int row = h * 8 + p_r;
+    const int slot = (lane % 8) ^ ((row >> 1) & 7);
+    const uint32_t voff = (uint32_t)row * (uint32_t)p.lda + (uint32_t)(c_begin + 2 * u) * 64u + (uint32_t)slot * 16u;
+    if (row < M)
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"((c_begin - c0) * 1024 + u * 2048 + h * 1024), "v"(voff), "s"(p.A) : "memory", "m0");
+  };
+  auto stage_rows = [&]() {
+    if (PAIR) {
+      #pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (c_begin + 2 * u < c_end) { stage_pair(u, 0); stage_pair(u, 1); }
+    } else {
+      #pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (c_begin + u < c_end) stage_chunk(c_begin + u);
+    }
+  };
   const int c16 = lane % 16, g = lane / 16;
   const uint8_t *tiles = p.blob + zmi_blob_tiles_off(N);
   const uint8_t *bsrc[2];
@@ -380,9 +439,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   if (!FQ) {
     #pragma unroll
     for (int u = 0; u < D16_W_FIRST; ++u) load_b(u);
-    #pragma unroll
-    for (int u = 0; u < 8; ++u)
-      if (c_begin + u < c_end) stage_chunk(c_begin + u);
+    stage_rows();
     #pragma unroll
     for (int u = D16_W_FIRST; u < 8; ++u) load_b(u);
   } else {
@@ -391,11 +448,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     // (every wavefront for itself: there is no barrier before the MFMAs; the copies of the flags are ZMI_FQ_COPIES
     // pages apart, so that the waiting wavefronts of the device do not all read one memory channel)
     rows_ok = zmi_fq_wait_scalar(fq, M, fq.flags + (fq.n_copies > 1 ? ((blk * DEC_WAVES + wave) % fq.n_copies) * 1024 : 0));
-    if (rows_ok) {
-      #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (c_begin + u < c_end) stage_chunk(c_begin + u);
-    }
+    if (rows_ok) stage_rows();
     #pragma unroll
     for (int u = FQ; u < 8; ++u) load_b(u);
   }
@@ -418,14 +471,22 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   for (int u = 0; u < 8; ++u) {
     const bool live = c_begin + u < c_end;
     const int c = live ? c_begin + u : c_begin;
-    v4i a = *(const v4i *)(lds + (c - c0) * 1024 + (c16 * 4 + (g ^ ((c16 >> 2) & 3))) * 16);
+    v4i a;
+    if (PAIR) a = *(const v4i *)(lds + (c_begin - c0) * 1024 + (u / 2) * 2048 + (c16 / 8) * 1024 + (c16 % 8) * 128 +
+                                 ((((u % 2) * 4 + g) ^ ((c16 >> 1) & 7))) * 16);
+    else a = *(const v4i *)(lds + (c - c0) * 1024 + (c16 * 4 + (g ^ ((c16 >> 2) & 3))) * 16);
     a[0] ^= xm; a[1] ^= xm; a[2] ^= xm; a[3] ^= xm;   // u8 rows enter the MFMA as (a - 128)
     if (!live) a = (v4i){0, 0, 0, 0};   // whatever b holds then adds nothing
     acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][0], acc[0], 0, 0, 0);
     acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[u][1], acc[1], 0, 0, 0);
   }
 
+  // the element's constants, decoded while the slower wavefronts of the workgroup still multiply
+  ZmiColCtx cc0 = zmi_col_ctx_raw(epi, p, craw, zp_word, e_n, n_ok, N);
+  float rs0 = zmi_row_scale_from_raw(epi, p, rs_word, m_ok);
+  zmi_pin_v(cc0.wscale); zmi_pin_v(cc0.bias); zmi_pin_v(cc0.comp); zmi_pin_v(cc0.shift); zmi_pin_v(rs0);
   // ---- cross-wavefront reduction through LDS (reuses the operand area) ----
+  D16_STAMPW(1);
   zmi_lds_barrier();
   int32_t *red = (int32_t *)lds;
   #pragma unroll
@@ -448,6 +509,7 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
   int32_t s = 0;
   #pragma unroll
   for (int w = 0; w < DEC_WAVES; ++w) s += red[w * 512 + off];
+  D16_STAMP(9);
   if (n_slices > 1) {
     if (!arrivals) {
       if (e_live) partial[((int64_t)slice * 16 + e_row) * N + e_n] = s;
@@ -468,8 +530,8 @@ __global__ __launch_bounds__(DEC_THREADS, 4) void zmi_gemm_decode16_kernel(ZmiPr
     for (int sl = 0; sl < n_slices; ++sl)
       s += __hip_atomic_load(partial + ((int64_t)sl * 16 + e_row) * N + e_n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  const ZmiColCtx cc0 = zmi_col_ctx_raw(epi, p, craw, zp_word, e_n, n_ok, N);
-  zmi_finish_element(p, epi, cc0, zmi_row_scale_from_raw(epi, p, rs_word, m_ok), s, e_row, e_n);
+  zmi_finish_element(p, epi, cc0, rs0, s, e_row, e_n);
+  D16_STAMP(10);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -773,9 +835,9 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     if (n_blk <= 0) return hipSuccess;
     const int64_t per = (zmi_blob_kpad(p.K) / 64 + slices - 1) / slices + 1;   // chunks of the longest slice, rounded up
     const size_t op = (size_t)(per < 64 ? per : 64) * 1024;
-    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel<0>, 4096 * 16);
+    hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_decode16_kernel<0, false>, 4096 * 16);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(zmi_gemm_decode16_kernel<0>, dim3(n_blk, slices), dim3(DEC_THREADS),
+    hipLaunchKernelGGL((zmi_gemm_decode16_kernel<0, false>), dim3(n_blk, slices), dim3(DEC_THREADS),
                        op > DEC_RED_BYTES ? op : DEC_RED_BYTES, stream, p, epi, ZmiFusedQuant{}, slices, partial, arrivals);
     e = hipGetLastError();
     if (e != hipSuccess || arrivals) return e;
@@ -799,15 +861,18 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     // (the operand area, reused by the partial tiles, and with the quantization in the launch a word per wavefront)
     const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
     const size_t smem = (op > DEC_RED_BYTES ? op : DEC_RED_BYTES) + (fq ? 64 : 0);
-    const void *f = fq ? (const void *)zmi_gemm_decode16_kernel<D16_FQ_FIRST> : (const void *)zmi_gemm_decode16_kernel<0>;
+    // (whole lines of the rows per request where every wavefront's share of K is whole pairs of chunks)
+    const bool pair = p.K % 1024 == 0 && !getenv("ZMI_DECODE_NO_ROW_PAIRS");
+    const void *f = fq ? (pair ? (const void *)zmi_gemm_decode16_kernel<D16_FQ_FIRST, true> : (const void *)zmi_gemm_decode16_kernel<D16_FQ_FIRST, false>)
+                       : (pair ? (const void *)zmi_gemm_decode16_kernel<0, true> : (const void *)zmi_gemm_decode16_kernel<0, false>);
     hipError_t e = zmi_func_smem_once(f, 4096 * 16 + 64);
     if (e != hipSuccess) return e;
-    if (fq)
-      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<D16_FQ_FIRST>, dim3(n_blk + p.M), dim3(DEC_THREADS), smem, stream, p, epi, *fq,
-                         1, (int32_t *)nullptr, (unsigned int *)nullptr);
-    else
-      hipLaunchKernelGGL(zmi_gemm_decode16_kernel<0>, dim3(n_blk), dim3(DEC_THREADS), smem, stream, p, epi, ZmiFusedQuant{},
-                         1, (int32_t *)nullptr, (unsigned int *)nullptr);
+    const dim3 grid(n_blk + (fq ? p.M : 0)), block(DEC_THREADS);
+    const ZmiFusedQuant q = fq ? *fq : ZmiFusedQuant{};
+    if (fq && pair) hipLaunchKernelGGL((zmi_gemm_decode16_kernel<D16_FQ_FIRST, true>), grid, block, smem, stream, p, epi, q, 1, (int32_t *)nullptr, (unsigned int *)nullptr);
+    else if (fq) hipLaunchKernelGGL((zmi_gemm_decode16_kernel<D16_FQ_FIRST, false>), grid, block, smem, stream, p, epi, q, 1, (int32_t *)nullptr, (unsigned int *)nullptr);
+    else if (pair) hipLaunchKernelGGL((zmi_gemm_decode16_kernel<0, true>), grid, block, smem, stream, p, epi, q, 1, (int32_t *)nullptr, (unsigned int *)nullptr);
+    else hipLaunchKernelGGL((zmi_gemm_decode16_kernel<0, false>), grid, block, smem, stream, p, epi, q, 1, (int32_t *)nullptr, (unsigned int *)nullptr);
     return hipGetLastError();
   }
   // rows per workgroup: 16 up to 64 rows (more workgroups in flight: 12 / 17 us per call at
