@@ -310,6 +310,9 @@ ZMI_API void zmi_clear_weight_cache(void);
 /* Frees the calling thread's scratch arena (reference: clear_fused_moe_scratch,
  * group_matmul/group_matmul_direct.hpp:683). */
 ZMI_API void zmi_clear_scratch(void);
+/* The library reads its environment switches (ZMI_*, ZENDNNL_*) once per process; this reads them again.  Not while
+ * calls of other threads are in flight.  (No counterpart in the reference, whose switches are read per call.) */
+ZMI_API void zmi_reload_env(void);
 /* Library version string. */
 ZMI_API const char *zmi_version(void);
 

@@ -3,6 +3,9 @@ import sys
 
 import pytest
 
+# the library reads its environment switches once per process; the tests flip them between calls
+os.environ.setdefault("ZMI_ENV_LIVE", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -86,8 +86,7 @@ def test_matmul_validation_status_codes():
     p.postop_ = [lowoha.PostOp(capi.PO_CLIP, alpha=float("nan"), beta=1.0)]
     assert _mm(p) == capi.FAILURE
     # mish: refused with per-row source scales on s8 rows, with dynamic quantization and on W4A8
-    # (lowoha_matmul_utils.cpp:379-408); the static scale chain takes it (no GPU here: the call then
-    # fails later, for another reason)
+    # (lowoha_matmul_utils.cpp:379-408); the static scale chain takes it
     p = _int8_params(dt_src=capi.DT_S8, dt_dst=capi.DT_BF16, src_scale=q((4, 1)), wei_scale=q((1, 8)))
     p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
     assert _mm(p) == capi.FAILURE and "mish" in lowoha.last_error()
@@ -103,10 +102,12 @@ def test_matmul_validation_status_codes():
     p.wei_scale = q((1, 8))
     p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
     assert _mm(p) == capi.FAILURE and "mish" in lowoha.last_error()
+    # (the static chain accepts it: the call gets as far as the next check -- a leading dimension that is too small,
+    # so that this case, like every case of this file, is refused before anything touches the placeholder pointers)
     p = _int8_params(src_scale=q((1,)), wei_scale=q((1, 8)))
     p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
-    _mm(p)
-    assert "mish" not in lowoha.last_error()
+    assert lowoha.matmul_direct("r", False, False, 4, 8, 16, 1.0, FAKE, 8, FAKE, 8, None, 0.0, FAKE, 8, True, p) == capi.FAILURE
+    assert "mish" not in lowoha.last_error() and "leading dimension" in lowoha.last_error()
     # outside the implemented path: status unimplemented, not failure
     assert _mm(lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_BF16, dst=capi.DT_BF16)) == capi.UNIMPLEMENTED
     # GGML-packed weights: transB = true is required (the packed layout is N x K), as in the reference
@@ -262,3 +263,14 @@ def test_product_does_not_touch_the_oracle():
                     if re.search(r"zmi_oracle|libzmi_oracle|from oracle|import oracle|oracle/", text):
                         bad.append(os.path.join(dirpath, f))
     assert not bad, bad
+
+
+def test_environment_switches_are_read_once_and_reloadable(monkeypatch):
+    """The switches are cached per process (zmi_reload_env reads them again); under ZMI_ENV_LIVE, which the test
+    session sets, every look goes to the environment -- the diagnostics gate above relies on it."""
+    lib = capi.load()
+    assert os.environ.get("ZMI_ENV_LIVE") == "1"
+    lib.zmi_reload_env()
+    monkeypatch.setenv("ZENDNNL_DIAGNOSTICS_ENABLE", "0")
+    lib.zmi_reload_env()
+    assert _mm(_int8_params(), M=0) == capi.FAILURE

@@ -172,6 +172,31 @@ def test_fused_quantization_three_forms_bit_exact(zo, M, K, N, monkeypatch):
     assert np.all(np.isfinite(bad[0]))
 
 
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 2080), (13, 1000, 333)])
+def test_handoff_flags_in_ordinary_memory(zo, M, K, N, monkeypatch):
+    """ZMI_NO_UNCACHED_FLAGS: the hand-off words live in ordinary device memory, as on a device that refuses the
+    uncached kind; the launch that would wait through the scalar unit takes the row-group kernel's form, which waits
+    with device-scope vector loads.  Bit-identical to the oracle, and switching back works."""
+    rng = np.random.default_rng(M + K + N)
+    x, w, ws, p, dst, call, keep = _fused_call(M, K, N, rng)
+    ph = H.host_params(p, src_scale=None, wei_scale=ws)
+    ph.mem_format_b = "n"
+    hk = []
+    st, want, _, _ = zo.matmul_int8(x, w, ph.flat(hk), M, N, K)
+    assert st == capi.SUCCESS
+    monkeypatch.setenv("ZMI_NO_DECODE_SELFQ", "1")
+    for plain in (True, False, True):
+        if plain:
+            monkeypatch.setenv("ZMI_NO_UNCACHED_FLAGS", "1")
+        else:
+            monkeypatch.delenv("ZMI_NO_UNCACHED_FLAGS", raising=False)
+        for rep in range(2):
+            dst.fill_(12345.0)
+            assert call() == capi.SUCCESS, lowoha.last_error()
+            assert lowoha.last_kernel() == FUSED_NAMES["rowgroup" if plain else "handoff16"]
+            assert np.array_equal(H.to_host(dst), want), (plain, rep)
+
+
 def test_fused_quantization_default_form_by_width(zo, monkeypatch):
     """Which form a call takes by itself: up to 12 rows and an output wide enough for 64 two-block workgroups (at
     most one per compute unit) quantize in the workgroups, the others keep the hand-off."""

@@ -105,6 +105,38 @@ def test_plain_grouped_gemms_match_the_mfma_bound_kernel_bit_for_bit(zo, monkeyp
         H.check_bf16(got[e][:Ms[e]], want, max_frac=5e-3, atol=1e-6 if post == capi.PO_GELU_TANH else 0.0)
 
 
+@pytest.mark.parametrize("Ms", [[100, 0, 128, 70], [130, 40, 129], [20, 64, 33, 17, 50]])
+@pytest.mark.parametrize("dst_dt,post", [(capi.DT_BF16, None), (capi.DT_BF16, capi.PO_GELU_TANH), (capi.DT_F32, None)])
+def test_mfma_bound_kernel_in_k_slices_is_bit_identical(zo, monkeypatch, Ms, dst_dt, post):
+    """A grouped launch of the MFMA-bound kernel with few tiles and a long K goes out in K slices: the slice that
+    arrives last at its tile's word adds the others' int32 partial tiles and finishes the elements.  Bit-identical
+    to the unsliced launch (ZMI_NO_GROUP_RING_SLICES) on repeated calls -- the arrival words are zero again after
+    every launch -- and equal to the oracle.  Row counts: partly filled tiles, two row blocks per expert, experts
+    without rows, 64-row tiles (the last list)."""
+    rng = np.random.default_rng(sum(Ms) + (post or 0) + dst_dt)
+    K, N = 3200, 600                 # 50 stages of 64 k: two slices of 25; a column edge inside the third tile
+    run, host = _grouped(Ms, K, N, dst_dt, post=post, bias=True, rng=rng)
+    _with_kernel(monkeypatch, None)
+    monkeypatch.setenv("ZMI_NO_GROUP_RING_SLICES", "1")
+    ref, name_ref = run()
+    assert name_ref == "group: ring_mfma32x32x32"
+    monkeypatch.delenv("ZMI_NO_GROUP_RING_SLICES")
+    for rep in range(3):
+        got, name = run()
+        assert name == "group: ring_mfma32x32x32 (K slices)"
+        for e, m in enumerate(Ms):
+            assert np.array_equal(got[e], ref[e]), f"call {rep}, expert {e} ({m} rows)"
+    e = 0
+    keep = []
+    ph = H.host_params(host["params"][e], src_scale=None, wei_scale=host["wsc"][e])
+    st, want, _, _ = zo.matmul_int8(host["xs"][e][:Ms[e]], host["ws"][e], ph.flat(keep), Ms[e], N, K, bias=host["bs"][e])
+    assert st == capi.SUCCESS
+    if dst_dt == capi.DT_F32:
+        H.check_f32(got[e][:Ms[e]], want)
+    else:
+        H.check_bf16(got[e][:Ms[e]], want, max_frac=5e-3, atol=1e-6 if post == capi.PO_GELU_TANH else 0.0)
+
+
 @pytest.mark.parametrize("top", [TOP128, TOP256])
 def test_static_u8_rows_with_zero_point(zo, monkeypatch, top):
     """u8 rows with a source zero-point: the compensation term travels through the parked column constants."""

@@ -50,6 +50,48 @@ def test_noalloc_matches_matmul_direct_two_calls_in_a_row():
     _case(128, 4096, 512, rng, capi.DT_BF16, capi.PO_GELU_TANH, scale_buf=True, scale_dt=capi.DT_BF16)
     _case(40, 520, 96, rng, capi.DT_F32, None, per_tensor=True, scale_buf=True)
     _case(1, 4096, 1024, rng, capi.DT_BF16, capi.PO_SWISH)
+    # 13 .. 16 rows on the 16-row kernel with K that is no multiple of 16 (the rows' stride in the array is)
+    _case(16, 1000, 300, rng, capi.DT_BF16, capi.PO_SWISH)
+    _case(13, 4090, 200, rng, capi.DT_F32, None, scale_buf=True)
+
+
+def test_noalloc_calls_leave_the_free_device_memory_unchanged():
+    """The entry point's defining property: after a first call (which may load code objects), calls with new shapes
+    under its limits change neither the free device memory nor the caching allocator's reservation -- every buffer of
+    the calls below exists before the first measurement."""
+    rng = np.random.default_rng(99)
+    shapes = [(16, 4096, 2048), (3, 520, 96), (128, 4096, 512), (64, 1024, 300), (1, 256, 64)]
+    cases = []
+    for M, K, N in shapes:
+        x = H.to_dev(H.gen_bf16_normal(rng, (M, K)))
+        blob = H.prepack(H.to_dev(H.gen_weights(rng, K, N)), K, N)
+        ws = H.to_dev(rng.uniform(0.001, 0.01, N).astype(np.float32))
+        dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
+        p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, compute=capi.DT_S8)
+        p.dynamic_quant = True
+        p.src_scale = lowoha.QuantParam(None, capi.DT_F32, (M, 1))
+        p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
+        p.mem_format_b = "r"
+        p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
+        cases.append((M, K, N, x, blob, dst, p, ws))
+
+    def call(c):
+        M, K, N, x, blob, dst, p, _ = c
+        st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x, K, blob, N, None, 0.0, dst, N, True, p, noalloc=True)
+        assert st == capi.SUCCESS, lowoha.last_error()
+
+    for c in cases:        # first calls: code objects, the blob header checks
+        call(c)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0 = torch.cuda.memory_reserved()
+    for _ in range(3):
+        for c in cases:
+            call(c)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert torch.cuda.memory_reserved() == reserved0
 
 
 def test_noalloc_rejects_what_the_array_cannot_hold():

@@ -165,6 +165,7 @@ SIGNATURES = {
     "zmi_last_kernel": (C.c_char_p, []),
     "zmi_clear_weight_cache": (None, []),
     "zmi_clear_scratch": (None, []),
+    "zmi_reload_env": (None, []),
     "zmi_version": (C.c_char_p, []),
     "zmi_moe_route": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                   C.c_void_p, C.c_void_p]),

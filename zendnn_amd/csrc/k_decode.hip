@@ -789,7 +789,7 @@ bool zmi_decode_kernel_fits(const ZmiProblem &p) {
 // K slices of the 16-row kernel for K beyond 4096 (0: the shape is not its: more than 16 rows, or rows it cannot address)
 int zmi_decode16_slices(int M, int64_t K, int64_t lda) {
   const int64_t nchunks = zmi_blob_kpad(K) / 64;
-  if (M <= 0 || M > 16 || nchunks <= 64 || lda * 16 >= ((int64_t)1 << 31) || getenv("ZMI_DECODE_ROWGROUP_KERNEL")) return 0;
+  if (M <= 0 || M > 16 || nchunks <= 64 || lda * 16 >= ((int64_t)1 << 31) || zmi_env(ZE_DECODE_ROWGROUP_KERNEL)) return 0;
   return (int)((nchunks + 63) / 64);
 }
 size_t zmi_decode16_partial_bytes(int M, int N, int64_t K) {
@@ -801,7 +801,7 @@ size_t zmi_decode16_partial_bytes(int M, int N, int64_t K) {
 // (ZMI_DECODE_ROWGROUP_KERNEL: the tests reach the row-group kernel with few rows through it.)
 bool zmi_decode_16row_kernel(const ZmiProblem &p, bool fused_quant) {
   (void)fused_quant;
-  return p.M <= 16 && (int64_t)p.lda * 16 < ((int64_t)1 << 31) && !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
+  return p.M <= 16 && (int64_t)p.lda * 16 < ((int64_t)1 << 31) && !zmi_env(ZE_DECODE_ROWGROUP_KERNEL);
 }
 
 // bf16 rows quantized by the workgroups that use them (zmi_gemm_decode16_selfq_kernel): rows of whole 16-byte
@@ -818,10 +818,10 @@ bool zmi_decode_selfq_takes(const ZmiProblem &p, const ZmiFusedQuant *fq) {
   if (p.K % 8 != 0 || ((uintptr_t)fq->x % 16) != 0 || (fq->ldx * 2) % 16 != 0) return false;
   const int wgs = (zmi_decode_grid(p) + 1) / 2;
   int min_wgs = 64, max_m = 12;
-  if (const char *e = getenv("ZMI_DECODE_SELFQ_MIN_WGS")) min_wgs = atoi(e);
-  if (const char *e = getenv("ZMI_DECODE_SELFQ_MAX_M")) max_m = atoi(e);
-  return p.M <= max_m && wgs <= zmi_cu_count() && wgs >= min_wgs && !getenv("ZMI_NO_DECODE_SELFQ") &&
-         !getenv("ZMI_DECODE_ROWGROUP_KERNEL");
+  if (const char *e = zmi_env(ZE_DECODE_SELFQ_MIN_WGS)) min_wgs = atoi(e);
+  if (const char *e = zmi_env(ZE_DECODE_SELFQ_MAX_M)) max_m = atoi(e);
+  return p.M <= max_m && wgs <= zmi_cu_count() && wgs >= min_wgs && !zmi_env(ZE_NO_DECODE_SELFQ) &&
+         !zmi_env(ZE_DECODE_ROWGROUP_KERNEL);
 }
 
 hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
@@ -862,7 +862,7 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
     const size_t op = (size_t)zmi_blob_kpad(p.K) * 16;
     const size_t smem = (op > DEC_RED_BYTES ? op : DEC_RED_BYTES) + (fq ? 64 : 0);
     // (whole lines of the rows per request where every wavefront's share of K is whole pairs of chunks)
-    const bool pair = p.K % 1024 == 0 && !getenv("ZMI_DECODE_NO_ROW_PAIRS");
+    const bool pair = p.K % 1024 == 0 && !zmi_env(ZE_DECODE_NO_ROW_PAIRS);
     const void *f = fq ? (pair ? (const void *)zmi_gemm_decode16_kernel<D16_FQ_FIRST, true> : (const void *)zmi_gemm_decode16_kernel<D16_FQ_FIRST, false>)
                        : (pair ? (const void *)zmi_gemm_decode16_kernel<0, true> : (const void *)zmi_gemm_decode16_kernel<0, false>);
     hipError_t e = zmi_func_smem_once(f, 4096 * 16 + 64);
@@ -883,7 +883,7 @@ hipError_t zmi_launch_gemm_decode(const ZmiProblem &p, const ZmiEpilogue &epi, c
   // against 20.3 us; ZMI_DECODE_RPW = 1 | 4 overrides the choice above 16 rows)
   int rpw = p.M <= 64 ? 1 : 4;
   if (p.M > 32 && (int64_t)n_blk * ((p.M + 15) / 16) > 1000) rpw = 4;
-  if (const char *e = getenv("ZMI_DECODE_RPW")) { const int v = atoi(e); if ((v == 1 || v == 4) && p.M > 16) rpw = v; }
+  if (const char *e = zmi_env(ZE_DECODE_RPW)) { const int v = atoi(e); if ((v == 1 || v == 4) && p.M > 16) rpw = v; }
   const int n_rg = (p.M + 16 * rpw - 1) / (16 * rpw);
   // (several workgroups per column block: a multiple of 8, for the renumbering over the XCDs)
   const int grid = n_rg == 1 ? n_blk : (n_blk * n_rg + 7) / 8 * 8;

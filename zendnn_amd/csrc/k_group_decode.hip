@@ -136,7 +136,7 @@ bool zmi_group_decode_takes(const ZmiEpilogue &epi, int N) {
   // activation is the MFMA-bound kernel's interpreter's
   if (gated && ((N / 2) % 32 != 0 || epi.fast_kind != ZMI_EK_NONE)) return false;
   if (epi.n_groups > 0) return false;
-  return getenv("ZMI_NO_GROUP_DECODE") == nullptr;
+  return zmi_env(ZE_NO_GROUP_DECODE) == nullptr;
 }
 
 hipError_t zmi_launch_gemm_group_decode(const ZmiProblem *probs_dev, int n_prob, int max_out_cols, const ZmiEpilogue &epi,

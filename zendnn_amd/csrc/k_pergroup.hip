@@ -487,14 +487,14 @@ static bool pgd_fits(const ZmiProblem &p, int G, int *cpw, int *gpw) {
 
 bool zmi_pergroup_decode_shape(const ZmiProblem &p, int G) {
   int cpw, gpw;
-  return pgd_fits(p, G, &cpw, &gpw) && !getenv("ZMI_PERGROUP_GENERIC");
+  return pgd_fits(p, G, &cpw, &gpw) && !zmi_env(ZE_PERGROUP_GENERIC);
 }
 
 bool zmi_pergroup_group_size_ok(int64_t gs) { return gs > 0 && (gs % 64 == 0 || gs == 32 || gs == 16); }
 
 bool zmi_pergroup_s4_shape(const ZmiProblem &p, int G) {
   int cpw, gpw;
-  return pgd_fits(p, G, &cpw, &gpw) && cpw % 2 == 0 && !getenv("ZMI_PERGROUP_GENERIC") && !getenv("ZMI_NO_S4_STREAM");
+  return pgd_fits(p, G, &cpw, &gpw) && cpw % 2 == 0 && !zmi_env(ZE_PERGROUP_GENERIC) && !zmi_env(ZE_NO_S4_STREAM);
 }
 
 hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiFusedQuant *fq,
@@ -526,7 +526,7 @@ hipError_t zmi_launch_gemm_pergroup(const ZmiProblem &p, const ZmiEpilogue &epi,
     default: break;
     }
   }
-  if (pgd_fits(p, G, &cpw, &gpw) && !getenv("ZMI_PERGROUP_GENERIC")) {
+  if (pgd_fits(p, G, &cpw, &gpw) && !zmi_env(ZE_PERGROUP_GENERIC)) {
     switch (cpw * 16 + gpw) {
     case 8 * 16 + 8: return pgd_launch<8, 8>(p, epi, fq, stream);
     case 8 * 16 + 4: return pgd_launch<8, 4>(p, epi, fq, stream);

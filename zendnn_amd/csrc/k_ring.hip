@@ -141,7 +141,7 @@ __global__ __launch_bounds__(R_THREADS, (RingCfg<BM, DEEP>::OCC)) void zmi_gemm_
   // Grouped launches read the tile table made by zmi_ring_count_kernel: the real tile count
   // (the grid is only a bound when the row counts live on the device) and, per problem,
   // the index of its first tile.
-  if (tile_tab) n_items = tile_tab[bm_idx];
+  if (tile_tab) n_items = tile_tab[bm_idx] * split.slices;
   const int b = blockIdx.x;
   const int per_xcd = (n_items + 7) / 8;
   const int item = (b % 8) * per_xcd + b / 8;
@@ -901,9 +901,28 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
 // null (row counts known only on the device) worst_rows / worst_cols bound them and surplus
 // workgroups exit at once.  tab_dev is 4 + 3 * n_prob ints of scratch for the tile table
 // (tab_ready: already filled for this table, tile height and epilogue kind by an earlier kernel).
+// split (optional): K slices with arrival words (plain epilogues, padded 128- or 64-row tiles); its workspace holds
+// zmi_ring_group_items(...) * slices partial tiles.
+int zmi_ring_group_items(const ZmiProblem *probs_host, int n_prob, int top, int64_t worst_rows, int worst_cols, bool gated) {
+  const int th = top & 0xffff;
+  if (probs_host) {
+    int items = 0;
+    for (int e = 0; e < n_prob; ++e) {
+      const ZmiProblem &q = probs_host[e];
+      if (q.M <= 0) continue;
+      items += th == 256 ? zmi_ring_items<256>(q.M, q.N, top, gated) : th == 128 ? zmi_ring_items<128>(q.M, q.N, top, gated)
+                                                                                  : zmi_ring_items<64>(q.M, q.N, top, gated);
+    }
+    return items;
+  }
+  const int per = gated ? 128 : 256;
+  const int ncols = gated ? worst_cols / 2 : worst_cols;
+  return (int)(worst_rows / th + n_prob) * ((ncols + per - 1) / per);
+}
+
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
-                                      const ZmiEpilogue &epi, hipStream_t stream) {
+                                      const ZmiEpilogue &epi, hipStream_t stream, const ZmiRingSplit *split) {
   const bool gated = epi.gated_act != 0;
   if (!tab_dev) return hipErrorInvalidValue;
   int items[3] = {0, 0, 0};   // 256, 128, 64
@@ -932,7 +951,12 @@ hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiPro
     hipLaunchKernelGGL(zmi_ring_count_kernel, dim3(1), dim3(64), 0, stream, probs_dev, n_prob, top, gated ? 1 : 0, tab_dev);
   const bool exact = probs_host != nullptr;
   ZmiProblem dummy = {};
-  const ZmiRingSplit whole = {1, nullptr};
+  ZmiRingSplit whole = {1, nullptr, nullptr};
+  if (split && split->slices > 1) {
+    // (one launch of padded tiles, the slice that arrives last finishes the elements: no reduction launch here)
+    if (gated || !(top & ZMI_RING_PAD) || (top & 0xffff) == 256 || !split->partial || !split->arrivals) return hipErrorInvalidValue;
+    whole = *split;
+  }
   hipError_t e = hipSuccess;
   if ((top & 0xffff) == 256) {
     e = ring_launch<256>(dummy, probs_dev, n_prob, items[0], exact, tab_dev, top, whole, epi, stream);

@@ -454,7 +454,7 @@ bool zmi_group_stream_takes(const ZmiEpilogue &epi, int N, int top_flags) {
   if (!(top_flags & ZMI_RING_PAD) || (top != 128 && top != 256)) return false;
   if (epi.n_groups > 0) return false;
   if (epi.gated_act != 0 && ((N / 2) % 32 != 0 || epi.fast_kind != ZMI_EK_NONE)) return false;
-  return getenv("ZMI_NO_GROUP_STREAM") == nullptr;
+  return zmi_env(ZE_NO_GROUP_STREAM) == nullptr;
 }
 
 template <int MI, int D, int OCC, bool SPLIT>

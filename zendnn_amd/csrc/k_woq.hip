@@ -357,7 +357,7 @@ static bool woq_general(const ZmiWoqProblem &p) { return !p.a_fast || (p.n_group
 // where the two-block build exists (up to 32 rows, the fast build); the tests use it.
 int zmi_woq_blocks(const ZmiWoqProblem &p) {
   if (woq_general(p) || p.M > 32) return 1;
-  if (const char *env = std::getenv("ZMI_WOQ_BLOCKS")) return std::atoi(env) == 2 ? 2 : 1;
+  if (const char *env = zmi_env(ZE_WOQ_BLOCKS)) return std::atoi(env) == 2 ? 2 : 1;
   return p.M > 4 && (p.N + 31) / 32 >= 384 ? 2 : 1;
 }
 

@@ -299,8 +299,8 @@ static bool decode_kernel_allowed(int M, int N, int K) {
   // ZMI_DECODE_MAX_M (0 .. 128) caps the rows the decode kernel takes; the tests use it to
   // reach the other kernels with few rows
   int max_m = 128;
-  if (const char *env = std::getenv("ZMI_DECODE_MAX_M")) max_m = std::atoi(env);
-  if (std::getenv("ZMI_NO_DECODE_KERNEL")) max_m = 0;
+  if (const char *env = zmi_env(ZE_DECODE_MAX_M)) max_m = std::atoi(env);
+  if (zmi_env(ZE_NO_DECODE_KERNEL)) max_m = 0;
   if (M > max_m || M > 128 || zmi_blob_kpad(K) > 4096) return false;
   return M <= 64 || !wide_output(M, N);
 }
@@ -310,8 +310,8 @@ static bool decode_kernel_allowed(int M, int N, int K) {
 static bool decode_sliced_allowed(int M, int N, int K) {
   (void)N;
   int max_m = 16;
-  if (const char *env = std::getenv("ZMI_DECODE_MAX_M")) max_m = std::min(max_m, std::atoi(env));
-  if (std::getenv("ZMI_NO_DECODE_KERNEL") || std::getenv("ZMI_NO_DECODE_SLICED")) max_m = 0;
+  if (const char *env = zmi_env(ZE_DECODE_MAX_M)) max_m = std::min(max_m, std::atoi(env));
+  if (zmi_env(ZE_NO_DECODE_KERNEL) || zmi_env(ZE_NO_DECODE_SLICED)) max_m = 0;
   return M <= max_m && zmi_blob_kpad(K) > 4096 && zmi_decode16_slices(M, K, zmi_round_up(K, 16)) >= 2;
 }
 
@@ -320,25 +320,35 @@ static bool decode_sliced_allowed(int M, int N, int K) {
 // to reach every kernel configuration with small shapes.
 ZmiRingPlan plan_ring_gemm(int M, int N, int K) {
   int top_hint = 0, force = 0;
-  if (const char *env = std::getenv("ZMI_GEMM_TOP")) {
+  if (const char *env = zmi_env(ZE_GEMM_TOP)) {
     const int v = std::atoi(env);
     if (v == 128 || v == 256) top_hint = v;
     if (v == 64) top_hint = 64 | 0x10000;   // (ZMI_RING_PAD)
   }
-  if (const char *env = std::getenv("ZMI_RING_SPLITK")) force = std::atoi(env);
+  if (const char *env = zmi_env(ZE_RING_SPLITK)) force = std::atoi(env);
   return zmi_ring_plan(M, N, K, top_hint, force);
+}
+
+// Whether a launch may quantize its own rows and hand them over inside the launch.  Not under stream capture: the
+// hand-off names the launch by a per-thread number baked into the kernel arguments, and a replayed graph would find
+// the flags of its first run already stamped (the quantization is then a launch of its own, which replays correctly).
+static bool fused_quant_allowed() {
+  if (zmi_env(ZE_NO_FUSED_QUANT)) return false;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream(), &cs) != hipSuccess) { (void)hipGetLastError(); return true; }
+  return cs == hipStreamCaptureStatusNone;
 }
 
 // The persistent form of the large-M kernel (k_pring.hip): one problem whose (256-row band, 64-column unit) cells give
 // every compute unit at least three (a tile of 256 x 192 or more).  ZMI_PRING = 0 / 1 overrides the size rule.
 static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi) {
   if (!zmi_pring_takes(prob, epi)) return false;
-  if (const char *env = std::getenv("ZMI_PRING")) return std::atoi(env) != 0;
+  if (const char *env = zmi_env(ZE_PRING)) return std::atoi(env) != 0;
   const int64_t cells = (int64_t)((prob.M + 255) / 256) * (zmi_blob_npad(prob.N) / 64);
   return prob.M >= 256 && cells >= 3 * (int64_t)zmi_cu_count();
 }
 
-int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
+int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan, const ZmiPringQuant *pq) {
   if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
     set_kernel_name(zmi_decode_16row_kernel(prob, false) ? "decode16_dma_rows_mfma16x16x64" : "decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
@@ -367,10 +377,11 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
       split.arrivals = prob.row_comp ? nullptr : slice_arrivals(plan->tiles);
     }
     if (plan->slices == 1 && pring_wanted(prob, epi)) {
-      set_kernel_name("pring_mfma32x32x32_persistent");
-      if (!hip_ok(zmi_launch_gemm_pring(prob, epi, stream()), "persistent MFMA GEMM launch")) return ZMI_FAILURE;
+      set_kernel_name(pq ? "pring_mfma32x32x32_persistent (per-token quant in the launch)" : "pring_mfma32x32x32_persistent");
+      if (!hip_ok(zmi_launch_gemm_pring(prob, epi, stream(), pq), "persistent MFMA GEMM launch")) return ZMI_FAILURE;
       return ZMI_SUCCESS;
     }
+    if (pq) { set_error("in-launch quantization without the persistent kernel"); return ZMI_FAILURE; }
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")
                                      : (th == 256 ? "ring_mfma32x32x32_top256"
@@ -386,7 +397,7 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
 bool use_ring_kernel(int M, int N, int K) {
   if (decode_kernel_allowed(M, N, K) || decode_sliced_allowed(M, N, K)) return false;
   // ZMI_RING_MIN_M overrides the choice (the tests reach the 64-row tile through it)
-  if (const char *env = std::getenv("ZMI_RING_MIN_M")) {
+  if (const char *env = zmi_env(ZE_RING_MIN_M)) {
     const int min_m = std::atoi(env);
     if (min_m > 0) return M >= min_m;
   }
@@ -399,7 +410,7 @@ bool use_ring_kernel(int M, int N, int K) {
 
 // rows from which the per-group GEMM takes the MFMA-tiled kernel (ZMI_PGRING_MIN_M overrides; 0 turns it off)
 int pgring_min_rows() {
-  if (const char *env = std::getenv("ZMI_PGRING_MIN_M")) {
+  if (const char *env = zmi_env(ZE_PGRING_MIN_M)) {
     const int v = std::atoi(env);
     return v > 0 ? v : 0x7fffffff;
   }
@@ -712,6 +723,8 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
   ZmiFusedQuant fused;
   std::memset(&fused, 0, sizeof(fused));
   bool use_fused = false;
+  bool late_quant = false;    // the row quantization has not been launched yet (see below)
+  float *late_scales = nullptr;
   int8_t *a_frag = nullptr;   // per-group GEMM at large M: the rows in fragment order, once they exist
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
@@ -729,7 +742,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
     if (pg_groups && !bcast_src) {
       // reference: the per-group dynamic reorder in front of the sym-quant GEMM
       // (matmul/quantization/reorder_quantization.cpp:43-280 with {M,G} scale dims)
-      if (zmi_pergroup_decode_shape(prob, (int)pg_groups) && !std::getenv("ZMI_NO_FUSED_QUANT")) {
+      if (zmi_pergroup_decode_shape(prob, (int)pg_groups) && fused_quant_allowed()) {
         // decode shapes: the quantization is part of the GEMM launch (its first M workgroups)
         if (!fused_handoff(&fused)) return ZMI_FAILURE;
         fused.x = src; fused.ldx = lda; fused.x_dt = p.dt_src;
@@ -750,7 +763,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
     } else if (bcast_src && per_token && K % 4 == 0 && zmi_pergroup_decode_shape(prob, (int)pg_groups) &&
-               !std::getenv("ZMI_NO_FUSED_QUANT")) {
+               fused_quant_allowed()) {
       // W4A8 decode shapes with one scale per row: the per-token quantization is part of the per-group GEMM
       // launch, whose workgroups read the row's scale for every group (no broadcast copy)
       if (!fused_handoff(&fused)) return ZMI_FAILURE;
@@ -763,7 +776,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       ep.src_scale.dt = ZMI_DT_F32;
       ep.src_scale.ndims = 2; ep.src_scale.dims[0] = M; ep.src_scale.dims[1] = pg_groups;
     } else if (per_token && !bcast_src && !ring && M <= 128 && K % 4 == 0 && (decode_kernel || zmi_smallm_grid(prob) <= 512) &&
-               !decode_sliced_allowed(M, N, K) && !std::getenv("ZMI_NO_FUSED_QUANT")) {
+               !decode_sliced_allowed(M, N, K) && fused_quant_allowed()) {
       // (the K-sliced decode kernel takes quantized rows: with the quantization of 14336-element rows inside the
       // launch its workgroups wait longer than the separate launch costs -- 32 against 22 us)
       if (!fused_handoff(&fused)) return ZMI_FAILURE;
@@ -779,7 +792,15 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
       // (without a caller buffer the scales live in scratch, in the dtype the params name: the reference allocates
       // its own buffer of that dtype, reorder_quantization.cpp:103-117, and its GEMM reads the narrowed values back)
-      if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, frag_kpad, scale_out, sdt, stream()), "quant launch"))
+      // Rows for the large-M kernel whose persistent form can quantize them inside its own launch: the decision waits
+      // for the epilogue (below); either way the rows are quantized on this stream ahead of the first tile.
+      // (the scales of one 256-row band must not share a cache line with the next band's: a caller's buffer that is
+      // not 128-byte aligned takes the separate launch)
+      if (ring && M > 1 && sdt == ZMI_DT_F32 && plan.slices == 1 && zmi_pring_quant_ok(src, p.dt_src, lda, K) && fused_quant_allowed() &&
+          ((uintptr_t)scale_out) % 128 == 0 && !zmi_env(ZE_NO_PRING_QUANT)) {
+        late_quant = true;
+        late_scales = (float *)scale_out;
+      } else if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, frag_kpad, scale_out, sdt, stream()), "quant launch"))
         return ZMI_FAILURE;
       ep.src_scale.buff = scale_out;
       ep.src_scale.dt = sdt;
@@ -871,7 +892,19 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       st = hip_ok(zmi_launch_gemm_smallm_fused(prob, epi, fused, stream()), "fused small-M GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
     }
   } else {
-    st = run_single_gemm(prob, epi, ring ? &plan : nullptr);
+    ZmiPringQuant pq = {};
+    if (late_quant) {
+      ZmiFusedQuant ho;
+      unsigned int *words = pring_wanted(prob, epi) ? pring_sync_words(2 + (int64_t)(M + 7) / 8) : nullptr;
+      if (words && fused_handoff(&ho)) {   // (its launch number, time limit and error word)
+        pq.x = src; pq.ldx = lda; pq.scales = late_scales; pq.sync = words; pq.error = ho.error;
+        pq.epoch = ho.epoch; pq.wait_ticks = ho.wait_ticks; pq.n_chunks = (M + 7) / 8;
+      } else if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, (int8_t *)const_cast<void *>(prob.A), K16, frag_kpad,
+                                               late_scales, ZMI_DT_F32, stream()), "quant launch")) {
+        return ZMI_FAILURE;
+      }
+    }
+    st = run_single_gemm(prob, epi, ring ? &plan : nullptr, pq.x ? &pq : nullptr);
   }
   upload_fence();
   return st;

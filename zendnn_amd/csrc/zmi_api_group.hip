@@ -239,10 +239,11 @@ struct Stage {
   std::vector<ZmiProblem> probs;
   ZmiEpilogue epi;
   mutable bool streamed = false;   // set by launch_stage: the weight-traffic-bound kernel took the large experts
+  mutable bool ring_sliced = false;  // set by launch_stage: the MFMA-bound kernel's launch went out in K slices
 };
 
 int group_top(int64_t rows, int n_prob, int64_t K, int64_t N, bool gated) {
-  if (const char *env = std::getenv("ZMI_GROUP_TOP")) { int v = std::atoi(env); if (v > 0) return v; }
+  if (const char *env = zmi_env(ZE_GROUP_TOP)) { int v = std::atoi(env); if (v > 0) return v; }
   return zmi_ring_pick_top_group(rows, n_prob, K, N, gated);
 }
 
@@ -260,7 +261,7 @@ struct StreamPlan { int top, slices; };
 size_t stream_partial_bound() { return (size_t)zmi_cu_count() * 2 * 256 * 256 * sizeof(int32_t); }
 StreamPlan group_stream_plan(int max_rows, const ZmiEpilogue &epi, int N, int K, int64_t tiles) {
   StreamPlan plan = {0, 1};
-  if ((max_rows <= 16 || max_rows > 256) && !std::getenv("ZMI_GROUP_STREAM_TOP")) return plan;
+  if ((max_rows <= 16 || max_rows > 256) && !zmi_env(ZE_GROUP_STREAM_TOP)) return plan;
   const int th = max_rows <= 128 ? 128 : 256;
   const int64_t slots = th == 128 ? 2 * (int64_t)zmi_cu_count() : zmi_cu_count();   // workgroups the device holds at once
   const int nk = (int)(zmi_blob_kpad(K) / 64);
@@ -269,15 +270,40 @@ StreamPlan group_stream_plan(int max_rows, const ZmiEpilogue &epi, int N, int K,
   // MFMA-bound kernel's deep-ring build reaches the same end sooner: 115 + 35 us against 136 us on config 4's Op2)
   if (epi.gated_act == 0 && th == 128 && tiles > 0 && tiles * 2 <= slots) slices = (int)std::min<int64_t>(4, slots / tiles);
   while (slices > 1 && nk / slices < 16) --slices;
-  if (const char *env = std::getenv("ZMI_GROUP_STREAM_SLICES")) slices = std::max(1, std::atoi(env));
+  if (const char *env = zmi_env(ZE_GROUP_STREAM_SLICES)) slices = std::max(1, std::atoi(env));
   if (epi.gated_act != 0) slices = 1;
   int top = 0;
   if (tiles >= slots || slices > 1) top = th | ZMI_RING_PAD;
-  if (const char *env = std::getenv("ZMI_GROUP_STREAM_TOP")) top = std::atoi(env);   // (0 switches the kernel off)
+  if (const char *env = zmi_env(ZE_GROUP_STREAM_TOP)) top = std::atoi(env);   // (0 switches the kernel off)
   if (!top || !zmi_group_stream_takes(epi, N, top)) return plan;
   plan.top = top;
   plan.slices = slices;
   return plan;
+}
+
+// K slices for a grouped launch of the MFMA-bound kernel that leaves workgroup slots empty (the down projection of a
+// few hundred rows: 8 experts x ~128 rows, 14336 -> 4096, is 128 .. 256 tiles, and a tile's stream of 14336 k runs at
+// what one compute unit keeps in flight): 2 .. 4 slices per tile while tiles x slices fit the device's slots and a
+// slice keeps 24 stages of 64 k; the slice that arrives last at its tile's word adds the partial tiles and finishes
+// the elements (exact: int32).  The workspace comes out of the room reserved for sliced grouped launches.
+ZmiRingSplit ring_group_split(int top, int items, int K, bool gated) {
+  ZmiRingSplit rs = {1, nullptr, nullptr};
+  const int th = top & 0xffff;
+  if (gated || !(top & ZMI_RING_PAD) || th == 256 || items <= 0 || zmi_env(ZE_NO_GROUP_RING_SLICES)) return rs;
+  const int64_t slots = 2 * (int64_t)zmi_cu_count();
+  int slices = (int)std::min<int64_t>(4, slots / items);
+  const int nk = (int)(zmi_blob_kpad(K) / 64);
+  while (slices > 1 && nk / slices < 24) --slices;
+  if (slices < 2) return rs;
+  const size_t bytes = (size_t)items * slices * th * 256 * sizeof(int32_t);
+  if (bytes > stream_partial_bound()) return rs;
+  unsigned int *arr = slice_arrivals(items);
+  int32_t *partial = arr ? (int32_t *)arena().alloc(bytes) : nullptr;
+  if (!arr || !partial) return rs;
+  rs.slices = slices;
+  rs.partial = partial;
+  rs.arrivals = arr;
+  return rs;
 }
 
 // Every expert's activations are fragment-major.  Experts with more than 16 rows: one launch of the MFMA-bound
@@ -301,7 +327,7 @@ int32_t launch_stage(const Stage &st, const char *what) {
   // are most of the weight traffic (a decode step: 0.26 against 0.32 ms for 8 experts x 2 .. 6 rows of configuration
   // 4's block); a few small experts among large ones stream under the large ones' MFMA work inside the one launch
   // instead (configuration 5: 0.45 against 0.49 ms).  ZMI_GROUP_DECODE=1 forces the split (tests).
-  const bool force_split = getenv("ZMI_GROUP_DECODE") != nullptr;
+  const bool force_split = zmi_env(ZE_GROUP_DECODE) != nullptr;
   const bool split = small > 0 && small_ok && (small >= large || force_split);
   int top = group_top(rows, n, kmax, cols, gated);
   // experts of at most 256 rows are a stream of their weights: the kernel built for that takes the launch
@@ -326,8 +352,11 @@ int32_t launch_stage(const Stage &st, const char *what) {
       }
       if (!hip_ok(zmi_launch_ring_table(dev, n, top, gated, tab, stream()), what)) return ZMI_FAILURE;
       if (!hip_ok(zmi_launch_gemm_stream_group(st.probs.data(), dev, n, top, 0, 0, tab, &rs, st.epi, stream()), what)) return ZMI_FAILURE;
-    } else if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream()), what)) {
-      return ZMI_FAILURE;
+    } else {
+      const ZmiRingSplit rs = ring_group_split(top, zmi_ring_group_items(st.probs.data(), n, top, 0, 0, gated), kmax, gated);
+      st.ring_sliced = rs.slices > 1;
+      if (!hip_ok(zmi_launch_gemm_ring_group(st.probs.data(), dev, n, top, 0, 0, tab, false, st.epi, stream(), &rs), what))
+        return ZMI_FAILURE;
     }
   }
   if (split && !hip_ok(zmi_launch_gemm_group_decode(dev, n, gated ? cols / 2 : cols, st.epi, stream()), what)) return ZMI_FAILURE;
@@ -666,7 +695,8 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
     st = launch_stage(op1, "Op1 GEMM launch");
     if (st != ZMI_SUCCESS) return st;
     set_kernel_name(op1.streamed ? (fuse_act ? "group: stream_mfma32x32x32 (gated epilogue)" : "group: stream_mfma32x32x32")
-                                 : (fuse_act ? "group: ring_mfma32x32x32 (gated epilogue)" : "group: ring_mfma32x32x32"));
+                                 : (fuse_act ? "group: ring_mfma32x32x32 (gated epilogue)"
+                                             : op1.ring_sliced ? "group: ring_mfma32x32x32 (K slices)" : "group: ring_mfma32x32x32"));
 
     if (run_act && !fuse_act) {
       // reference: group_matmul_moe_act_execute, group_matmul/group_matmul_moe_act.cpp
@@ -875,7 +905,7 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   probe.fast_kind = ZMI_EK_NONE;
   // (worth a launch of its own only when small experts are most of the work: see launch_stage; the row counts live
   // on the device, so the average decides)
-  const bool decode_step = R <= 16 * (int64_t)E || getenv("ZMI_GROUP_DECODE") != nullptr;
+  const bool decode_step = R <= 16 * (int64_t)E || zmi_env(ZE_GROUP_DECODE) != nullptr;
   const bool small2 = decode_step && zmi_group_decode_takes(probe, H);
   probe.gated_act = d->gated_act;
   const bool small1 = decode_step && zmi_group_decode_takes(probe, 2 * I);
@@ -918,8 +948,10 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
       if (!rs.partial) rs.slices = 1;
     }
     if (!hip_ok(zmi_launch_gemm_stream_group(nullptr, op2, E, top2, R, H, tile_tab2, &rs, e2, s), "Op2 GEMM launch")) return ZMI_FAILURE;
-  } else if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s), "Op2 GEMM launch")) {
-    return ZMI_FAILURE;
+  } else {
+    const ZmiRingSplit rs = ring_group_split(top2, zmi_ring_group_items(nullptr, E, top2, R, H, false), I, false);
+    if (!hip_ok(zmi_launch_gemm_ring_group(nullptr, op2, E, top2, R, H, tile_tab2, true, e2, s, &rs), "Op2 GEMM launch"))
+      return ZMI_FAILURE;
   }
   if (small2 && !hip_ok(zmi_launch_gemm_group_decode(op2, E, H, e2, s), "Op2 decode-shaped GEMM launch")) return ZMI_FAILURE;
   if (!hip_ok(zmi_launch_moe_combine(nullptr, Y, H, slot_of, d->topk_weights, 0, T, topk, H, ZMI_DT_BF16, d->out, d->ldo, s), "moe combine launch")) return ZMI_FAILURE;

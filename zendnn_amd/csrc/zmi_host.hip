@@ -9,7 +9,74 @@
 #include <mutex>
 #include <tuple>
 #include <set>
+#include <string>
 #include <vector>
+
+// ---- environment switches (see zmi_launch.h) ----
+namespace {
+const char *const kEnvNames[ZE_COUNT] = {
+    "ZMI_DECODE_ROWGROUP_KERNEL",
+    "ZMI_DECODE_SELFQ_MIN_WGS",
+    "ZMI_DECODE_SELFQ_MAX_M",
+    "ZMI_NO_DECODE_SELFQ",
+    "ZMI_DECODE_NO_ROW_PAIRS",
+    "ZMI_DECODE_RPW",
+    "ZMI_NO_GROUP_DECODE",
+    "ZMI_PERGROUP_GENERIC",
+    "ZMI_NO_S4_STREAM",
+    "ZMI_PRING_GRID",
+    "ZMI_NO_GROUP_STREAM",
+    "ZMI_WOQ_BLOCKS",
+    "ZMI_DECODE_MAX_M",
+    "ZMI_NO_DECODE_KERNEL",
+    "ZMI_NO_DECODE_SLICED",
+    "ZMI_GEMM_TOP",
+    "ZMI_RING_SPLITK",
+    "ZMI_PRING",
+    "ZMI_RING_MIN_M",
+    "ZMI_PGRING_MIN_M",
+    "ZMI_NO_FUSED_QUANT",
+    "ZMI_GROUP_TOP",
+    "ZMI_GROUP_STREAM_TOP",
+    "ZMI_GROUP_STREAM_SLICES",
+    "ZMI_GROUP_DECODE",
+    "ZENDNNL_LRU_CACHE_CAPACITY",
+    "ZMI_NO_SLICE_ARRIVALS",
+    "ZMI_NO_SIDE_STREAM",
+    "ZMI_FUSED_WAIT_US",
+    "ZENDNNL_DIAGNOSTICS_ENABLE",
+    "ZENDNNL_MATMUL_WEIGHT_CACHE",
+    "ZMI_NO_UNCACHED_FLAGS",
+    "ZMI_NO_GROUP_RING_SLICES",
+    "ZMI_NO_PRING_QUANT"};
+struct EnvTable {
+  std::string val[ZE_COUNT];
+  bool set[ZE_COUNT] = {};
+  bool live = false;
+  void load() {
+    for (int i = 0; i < ZE_COUNT; ++i) {
+      const char *e = std::getenv(kEnvNames[i]);
+      set[i] = e != nullptr;
+      val[i] = e ? e : "";
+    }
+    const char *l = std::getenv("ZMI_ENV_LIVE");
+    live = l && l[0] && l[0] != '0';
+  }
+};
+EnvTable &env_table() {
+  static EnvTable t = [] { EnvTable x; x.load(); return x; }();
+  return t;
+}
+}  // namespace
+
+const char *zmi_env(ZmiEnvVar v) {
+  EnvTable &t = env_table();
+  if (t.live) return std::getenv(kEnvNames[v]);
+  return t.set[v] ? t.val[v].c_str() : nullptr;
+}
+
+// Reads the switches again (not while calls of other threads are in flight).
+extern "C" __attribute__((visibility("default"))) void zmi_reload_env(void) { env_table().load(); }
 
 namespace zmi {
 
@@ -30,7 +97,8 @@ struct ThreadCtx {
   int next = 0;
   // hand-off words of the launches that quantize their own rows (ZmiFusedQuant::sync / error)
   unsigned int *fq_flags = nullptr;      // device: one flag per row, holding the epoch of the launch that published it
-  bool fq_flags_uncached = false;
+  unsigned int *fq_flags_plain = nullptr;   // the same in ordinary device memory (uncached memory refused or switched off)
+  bool fq_uncached_refused = false;
   unsigned int fq_epoch = 0;             // name of this thread's latest launch of that kind
   unsigned int *fq_err_host = nullptr;   // pinned host word the kernels set when a wait ran out
   unsigned int *fq_err_dev = nullptr;    // the same word as the device addresses it
@@ -40,6 +108,9 @@ struct ThreadCtx {
   // arrival words of K-sliced launches (see slice_arrivals())
   unsigned int *arrivals = nullptr;
   int64_t n_arrivals = 0;
+  // (see pring_sync_words())
+  unsigned int *pring_sync = nullptr;
+  int64_t n_pring_sync = 0;
   // side stream (see side_stream())
   hipStream_t side = nullptr;
   hipEvent_t side_fork = nullptr, side_join = nullptr;
@@ -69,7 +140,7 @@ std::set<std::tuple<const void *, int64_t, int64_t>> g_checked_blobs;   // (blob
 size_t cache_capacity() {
   // same variable the reference reads for its weight caches
   static const size_t cap = [] {
-    const char *e = std::getenv("ZENDNNL_LRU_CACHE_CAPACITY");
+    const char *e = zmi_env(ZE_ZENDNNL_LRU_CACHE_CAPACITY);
     long v = e ? std::atol(e) : 0;
     return v > 0 ? (size_t)v : (size_t)1 << 30;
   }();
@@ -91,7 +162,7 @@ bool hip_ok(hipError_t e, const char *what) {
 
 unsigned int *slice_arrivals(int64_t n) {
   auto &c = tctx;
-  if (std::getenv("ZMI_NO_SLICE_ARRIVALS")) return nullptr;
+  if (zmi_env(ZE_NO_SLICE_ARRIVALS)) return nullptr;
   if (n > c.n_arrivals) {
     // (launches still in flight count in the old words)
     if (c.arrivals) {
@@ -113,11 +184,36 @@ unsigned int *slice_arrivals(int64_t n) {
   return c.arrivals;
 }
 
+// Words of the persistent large-M kernel's in-launch quantization (two counters that are zero between launches, then
+// one flag per chunk of eight rows that keeps the number of the launch that wrote it): zeroed once, grown on demand.
+unsigned int *pring_sync_words(int64_t n) {
+  auto &c = tctx;
+  if (n > c.n_pring_sync) {
+    if (c.pring_sync) {
+      if (hipStreamSynchronize(c.stream) != hipSuccess || hipFree(c.pring_sync) != hipSuccess) (void)hipGetLastError();
+      c.pring_sync = nullptr;
+      c.n_pring_sync = 0;
+    }
+    const int64_t want = n < 4096 ? 4096 : n * 2;
+    void *d = nullptr;
+    if (hipMalloc(&d, (size_t)want * sizeof(unsigned int)) != hipSuccess ||
+        hipMemset(d, 0, (size_t)want * sizeof(unsigned int)) != hipSuccess) {
+      (void)hipGetLastError();
+      if (d) (void)hipFree(d);
+      return nullptr;
+    }
+    (void)hipStreamSynchronize(nullptr);   // (the zeros are there before the first launch on any stream reads them)
+    c.pring_sync = (unsigned int *)d;
+    c.n_pring_sync = want;
+  }
+  return c.pring_sync;
+}
+
 ZmiRingSide side_stream() {
   auto &c = tctx;
   if (!c.side_tried) {
     c.side_tried = true;
-    if (!std::getenv("ZMI_NO_SIDE_STREAM")) {
+    if (!zmi_env(ZE_NO_SIDE_STREAM)) {
       bool ok = hipStreamCreateWithFlags(&c.side, hipStreamNonBlocking) == hipSuccess &&
                 hipEventCreateWithFlags(&c.side_fork, hipEventDisableTiming) == hipSuccess &&
                 hipEventCreateWithFlags(&c.side_join, hipEventDisableTiming) == hipSuccess;
@@ -254,37 +350,47 @@ constexpr int kFqCopies = 16;
 
 bool fused_handoff(ZmiFusedQuant *fq) {
   ThreadCtx &c = tctx;
-  if (!c.fq_flags) {
-    void *d = nullptr, *h = nullptr, *hd = nullptr;
-    // (uncached: the waiting side may read the flags through the scalar unit, which cannot ask for device scope;
-    // never freed -- memory of this kind that a kernel has read stays allocated until the process ends;
-    // a device that refuses the uncached kind gets ordinary memory and the waits that read it with device-scope loads)
-    if (hipExtMallocWithFlags(&d, kFqCopies * 4096, hipDeviceMallocUncached) != hipSuccess) {
-      (void)hipGetLastError();
-      d = nullptr;
-      if (!hip_ok(hipMalloc(&d, 512), "hipMalloc(hand-off words)")) return false;
-      c.fq_flags_uncached = false;
-    } else {
-      c.fq_flags_uncached = true;
-    }
-    if (!hip_ok(hipMemset(d, 0, c.fq_flags_uncached ? kFqCopies * 4096 : 512), "hipMemset(hand-off words)")) return false;
+  if (!c.fq_err_host) {
+    void *h = nullptr, *hd = nullptr;
     if (!hip_ok(hipHostMalloc(&h, 64, hipHostMallocMapped), "hipHostMalloc(error word)")) return false;
     std::memset(h, 0, 64);
     if (!hip_ok(hipHostGetDevicePointer(&hd, h, 0), "hipHostGetDevicePointer(error word)")) return false;
-    c.fq_flags = (unsigned int *)d;
     c.fq_err_host = (unsigned int *)h;
     c.fq_err_dev = (unsigned int *)hd;
   }
-  fq->flags = c.fq_flags;
-  fq->flags_uncached = c.fq_flags_uncached ? 1 : 0;
-  fq->n_copies = c.fq_flags_uncached ? kFqCopies : 1;
+  // Uncached device memory: the waiting side may read the flags through the scalar unit, which cannot ask for device
+  // scope.  Never freed -- memory of this kind that a kernel has read stays allocated until the process ends.  A
+  // device that refuses the uncached kind (or ZMI_NO_UNCACHED_FLAGS, which the tests use to reach that path) gets
+  // ordinary memory, and the kernels then wait with device-scope vector loads.
+  const bool want_plain = zmi_env(ZE_NO_UNCACHED_FLAGS) != nullptr;
+  if (!want_plain && !c.fq_flags && !c.fq_uncached_refused) {
+    void *d = nullptr;
+    if (hipExtMallocWithFlags(&d, kFqCopies * 4096, hipDeviceMallocUncached) != hipSuccess) {
+      (void)hipGetLastError();
+      c.fq_uncached_refused = true;
+    } else {
+      if (!hip_ok(hipMemset(d, 0, kFqCopies * 4096), "hipMemset(hand-off words)")) return false;
+      c.fq_flags = (unsigned int *)d;
+    }
+  }
+  const bool plain = want_plain || !c.fq_flags;
+  if (plain && !c.fq_flags_plain) {
+    void *d = nullptr;
+    if (!hip_ok(hipMalloc(&d, 512), "hipMalloc(hand-off words)")) return false;
+    if (!hip_ok(hipMemset(d, 0, 512), "hipMemset(hand-off words)")) return false;
+    c.fq_flags_plain = (unsigned int *)d;
+  }
+  // (the two sets of words share the epoch counter: a set that sat out some launches holds older epochs, never newer)
+  fq->flags = plain ? c.fq_flags_plain : c.fq_flags;
+  fq->flags_uncached = plain ? 0 : 1;
+  fq->n_copies = plain ? 1 : kFqCopies;
   if (++c.fq_epoch == 0) c.fq_epoch = 1;   // (0 is what the flags hold before the first launch)
   fq->epoch = c.fq_epoch;
   fq->error = c.fq_err_dev;
   // 100 ms unless ZMI_FUSED_WAIT_US says otherwise (0: every wait gives up at once; the tests of the
   // failure path use it)
   uint64_t us = 100000;
-  if (const char *e = std::getenv("ZMI_FUSED_WAIT_US")) us = (uint64_t)std::strtoull(e, nullptr, 10);
+  if (const char *e = zmi_env(ZE_FUSED_WAIT_US)) us = (uint64_t)std::strtoull(e, nullptr, 10);
   const uint64_t ticks = us * 100;
   fq->wait_ticks = ticks > 0xffffffffull ? 0xffffffffu : (uint32_t)ticks;
   return true;
@@ -548,12 +654,12 @@ int64_t nelems(const zmi_quant_t &q) {
 
 bool diagnostics_enabled() {
   // validation gate of the reference (ZENDNNL_DIAGNOSTICS_ENABLE, on unless "0")
-  const char *e = std::getenv("ZENDNNL_DIAGNOSTICS_ENABLE");
+  const char *e = zmi_env(ZE_ZENDNNL_DIAGNOSTICS_ENABLE);
   return !(e && e[0] == '0' && e[1] == 0);
 }
 
 int weight_cache_env() {
-  const char *e = std::getenv("ZENDNNL_MATMUL_WEIGHT_CACHE");
+  const char *e = zmi_env(ZE_ZENDNNL_MATMUL_WEIGHT_CACHE);
   if (!e) return 2;
   int v = std::atoi(e);
   return v < 0 ? 0 : (v > 2 ? 2 : v);

@@ -25,6 +25,48 @@ inline hipError_t zmi_func_smem_once(const void *func, int bytes) {
   return e;
 }
 
+// Environment switches.  The process reads each of them once, at the first call that asks for any (zmi_reload_env()
+// reads them again; with ZMI_ENV_LIVE=1 in the environment at that first call every look goes to the environment,
+// which is how the tests flip switches between calls).  zmi_env returns the value, or null when the variable is unset.
+enum ZmiEnvVar {
+  ZE_DECODE_ROWGROUP_KERNEL,
+  ZE_DECODE_SELFQ_MIN_WGS,
+  ZE_DECODE_SELFQ_MAX_M,
+  ZE_NO_DECODE_SELFQ,
+  ZE_DECODE_NO_ROW_PAIRS,
+  ZE_DECODE_RPW,
+  ZE_NO_GROUP_DECODE,
+  ZE_PERGROUP_GENERIC,
+  ZE_NO_S4_STREAM,
+  ZE_PRING_GRID,
+  ZE_NO_GROUP_STREAM,
+  ZE_WOQ_BLOCKS,
+  ZE_DECODE_MAX_M,
+  ZE_NO_DECODE_KERNEL,
+  ZE_NO_DECODE_SLICED,
+  ZE_GEMM_TOP,
+  ZE_RING_SPLITK,
+  ZE_PRING,
+  ZE_RING_MIN_M,
+  ZE_PGRING_MIN_M,
+  ZE_NO_FUSED_QUANT,
+  ZE_GROUP_TOP,
+  ZE_GROUP_STREAM_TOP,
+  ZE_GROUP_STREAM_SLICES,
+  ZE_GROUP_DECODE,
+  ZE_ZENDNNL_LRU_CACHE_CAPACITY,
+  ZE_NO_SLICE_ARRIVALS,
+  ZE_NO_SIDE_STREAM,
+  ZE_FUSED_WAIT_US,
+  ZE_ZENDNNL_DIAGNOSTICS_ENABLE,
+  ZE_ZENDNNL_MATMUL_WEIGHT_CACHE,
+  ZE_NO_UNCACHED_FLAGS,
+  ZE_NO_GROUP_RING_SLICES,
+  ZE_NO_PRING_QUANT,
+  ZE_COUNT
+};
+const char *zmi_env(ZmiEnvVar v);
+
 // One matrix of a (possibly grouped) per-token quantization launch; row_start is
 // the index of its first row in the launch's global row numbering.
 struct ZmiQuantMat {
@@ -95,10 +137,28 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
                                 hipStream_t stream, const ZmiRingSide *side = nullptr);
 // k_pring.hip: the persistent form for one problem (A in fragment-major order, bf16 destination, straight-line epilogue)
 bool zmi_pring_takes(const ZmiProblem &p, const ZmiEpilogue &epi);
-hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
+// Per-token quantization of the bf16 source inside that launch (q null or q->x null: the rows at p.A are there already).
+// The workgroups first quantize the rows, eight at a time, claiming chunks from a counter until none is left (so the
+// rows get done by whichever workgroups are running); a chunk's flag takes the launch's number once its bytes are
+// written through, and a workgroup waits for the 32 flags of a band before it starts a tile of that band -- for at
+// most wait_ticks of the 100 MHz clock, after which it sets *error and stores nothing more.
+struct ZmiPringQuant {
+  const void *x;            // bf16 rows, K a multiple of 16 up to 8192, 16-byte aligned rows
+  int64_t ldx;              // elements
+  float *scales;            // [M] f32, device memory: written here, read by the epilogue (= p.src_scale_ptr)
+  unsigned int *sync;       // [0] chunk counter, [1] exit counter (both zero between launches), [2 + c] flag of chunk c
+  unsigned int *error;      // pinned host word, as the device addresses it
+  uint32_t epoch;           // the launch's number (never 0)
+  uint32_t wait_ticks;
+  int32_t n_chunks;         // ceil(M / 8)
+};
+bool zmi_pring_quant_ok(const void *x, int32_t x_dt, int64_t ldx, int K);
+hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream, const ZmiPringQuant *q = nullptr);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
-                                      const ZmiEpilogue &epi, hipStream_t stream);
+                                      const ZmiEpilogue &epi, hipStream_t stream, const ZmiRingSplit *split = nullptr);
+// tiles of such a launch at tile height `top` (a bound when the row counts live on the device: probs_host null)
+int zmi_ring_group_items(const ZmiProblem *probs_host, int n_prob, int top, int64_t worst_rows, int worst_cols, bool gated);
 
 // k_group_decode.hip: the problems of a grouped launch that have 1 .. 16 rows (rows in fragment order), gated or not;
 // one workgroup per (problem, 32 output columns), max_out_cols = the widest problem's output columns

@@ -252,6 +252,14 @@ class FusedMoe:
 def group_matmul_direct(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc,
                         is_weights_const, params, moe_postop=None, gated_act=None, fused_moe=None):
     """All per-expert arguments are Python lists, as the reference's std::vector arguments."""
+    return prepared_group_matmul(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc,
+                                 is_weights_const, params, moe_postop, gated_act, fused_moe)[0]()
+
+
+def prepared_group_matmul(layout, transA, transB, M, N, K, alpha, src, lda, weight, ldb, bias, beta, dst, ldc,
+                          is_weights_const, params, moe_postop=None, gated_act=None, fused_moe=None):
+    """The flattened arguments of group_matmul_direct, marshalled once: returns (call, keep); call() is one foreign
+    call with the same argument block every time (what a C++ caller's vectors cost: nothing per call)."""
     lib = capi.load()
     keep = []
     g = capi.GroupArgsT()
@@ -324,8 +332,11 @@ def group_matmul_direct(layout, transA, transB, M, N, K, alpha, src, lda, weight
                 setattr(fm, name, arr)
         putf("dst_down", C.c_void_p, fused_moe.dst_down, _ptr)
         putf("ldc_down", C.c_int32, fused_moe.ldc_down)
-    return lib.zmi_group_matmul_direct(C.byref(g), C.byref(pp) if pp is not None else None,
-                                       int(gated_act or 0), C.byref(fm) if fm is not None else None)
+    keep.extend([g, pp, fm])
+    a_g, a_pp, a_fm, act = C.byref(g), (C.byref(pp) if pp is not None else None), (C.byref(fm) if fm is not None else None), int(gated_act or 0)
+    fn = lib.zmi_group_matmul_direct
+    # (the closure holds `keep`: the argument block points into buffers only that list owns)
+    return (lambda _keep=keep: fn(a_g, a_pp, act, a_fm)), keep
 
 
 def moe_route(topk_ids, E):
