@@ -17,6 +17,19 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 FAKE = 0x1000   # non-null placeholder; validation fails before anything dereferences it
 
 
+def _device_present():
+    try:
+        import torch
+        return torch.cuda.device_count() > 0
+    except Exception:
+        return False
+
+
+# The validation tests hand the library addresses that are no memory: they belong on a machine without a device,
+# where a case that slipped past the validators fails at the device check instead of launching on such an address.
+fake_pointers = pytest.mark.skipif(_device_present(), reason="placeholder addresses: run where no device can be launched on")
+
+
 def test_library_exports_every_declared_symbol():
     lib = capi.load()
     hdr = open(os.path.join(ROOT, "include", "zmi_lowoha.h")).read()
@@ -51,6 +64,7 @@ def _int8_params(**kw):
     return p
 
 
+@fake_pointers
 def test_matmul_validation_status_codes():
     one = np.ones(4, dtype=np.float32)
     q = lambda dims, dt=capi.DT_F32: lowoha.QuantParam(one.ctypes.data, dt, dims)
@@ -143,6 +157,7 @@ def _prepack_rp(**kw):
     return rp
 
 
+@fake_pointers
 def test_prepack_size_and_validation():
     rp = _prepack_rp()
     n = lowoha.weight_prepack_size(rp)
@@ -164,6 +179,7 @@ def test_prepack_size_and_validation():
     assert lowoha.reorder_direct(None, FAKE, _prepack_rp()) == capi.FAILURE
 
 
+@fake_pointers
 def test_reorder_dynamic_validation():
     rp = lowoha.ReorderParams()
     rp.dynamic_quant = True
@@ -205,6 +221,7 @@ def _group(E=3, **over):
                                       a["ldc"], a["is_weights_const"], a["params"], **extra)
 
 
+@fake_pointers
 def test_group_validation_status_codes():
     E = 3
     assert _group(M=[]) == capi.FAILURE

@@ -22,7 +22,10 @@ def env():
     def set_(**kv):
         for k, v in kv.items():
             saved.setdefault(k, os.environ.get(k))
-            os.environ[k] = str(v)
+            if v is None:
+                os.environ.pop(k, None)      # (the switches are on when the variable exists, whatever it holds)
+            else:
+                os.environ[k] = str(v)
 
     yield set_
     for k, v in saved.items():
@@ -153,7 +156,7 @@ def test_rows_quantized_inside_the_launch_match_the_separate_launch(env, M, K, N
     b = H.to_dev((rng.standard_normal(N) * 0.1).astype(np.float32))
     res = []
     for no_fuse in (1, 0, 0):
-        env(ZMI_NO_PRING_QUANT=no_fuse)
+        env(ZMI_NO_PRING_QUANT=1 if no_fuse else None)
         sbuf = torch.zeros(M, dtype=torch.float32, device=H.DEV)
         out, name = _dyn_call(x, blob, ws, b, M, K, N, sbuf)
         assert "pring" in name and (("quant in the launch" in name) == (not no_fuse)), name

@@ -387,20 +387,31 @@ __device__ __forceinline__ void pr_quant_chunk(const ZmiProblem &p, const ZmiPri
 }
 
 // All rows of the launch, then nothing: returns when no chunk is left to claim.
+// Every branch around the barriers of this loop is taken by whole wavefronts (the first wavefront claims and publishes,
+// all its lanes writing the same words; the chunk number is made a scalar).  With a one-thread branch at the loop's end
+// and the same branch at its start the compiler joined the two, let the other lanes run on to the next barrier without
+// that thread, and the loop never ended.
 __device__ __forceinline__ void pr_quant_rows(const ZmiProblem &p, const ZmiPringQuant &q) {
   float *red = reinterpret_cast<float *>(zmi_pring_smem);
   int *slot = reinterpret_cast<int *>(zmi_pring_smem + 256);
+  const int lane = threadIdx.x % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   for (;;) {
-    if (threadIdx.x == 0) *slot = (int)__hip_atomic_fetch_add(&q.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0) {
+      // (one lane adds one, the others nothing: every lane of the wavefront then holds a value of the counter from
+      // before that lane's own addition, and lane 0's is the chunk)
+      const unsigned int got = __hip_atomic_fetch_add(&q.sync[0], lane == 0 ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *slot = __builtin_amdgcn_readfirstlane((int)got);
+    }
     __syncthreads();
-    const int c = *slot;
+    const int c = __builtin_amdgcn_readfirstlane(*slot);
     __syncthreads();
     if (c >= q.n_chunks) return;
     pr_quant_chunk(p, q, c, red);
     // the chunk's flag, once every store of the workgroup has been acknowledged
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0) __hip_atomic_store(&q.sync[2 + c], q.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0) __hip_atomic_store(&q.sync[2 + c], q.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -445,9 +456,9 @@ __global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pring_kernel(ZmiProble
       int *votes = reinterpret_cast<int *>(zmi_pring_smem + 512);
       pr_wait_vm<0>();   // (the tile's counted waits below count its own requests only)
       __syncthreads();
-      if (threadIdx.x % 64 == 0) votes[threadIdx.x / 64] = mine ? 1 : 0;
+      votes[__builtin_amdgcn_readfirstlane(threadIdx.x / 64)] = mine ? 1 : 0;   // (every lane: no one-thread branch in this loop)
       __syncthreads();
-      rows_ok = (votes[0] & votes[1] & votes[2] & votes[3]) != 0;
+      rows_ok = __builtin_amdgcn_readfirstlane(votes[0] & votes[1] & votes[2] & votes[3]) != 0;   // (a scalar: see pr_quant_rows)
       __syncthreads();
       if (!rows_ok) break;
       band_ready = band;

@@ -281,16 +281,18 @@ StreamPlan group_stream_plan(int max_rows, const ZmiEpilogue &epi, int N, int K,
   return plan;
 }
 
-// K slices for a grouped launch of the MFMA-bound kernel that leaves workgroup slots empty (the down projection of a
-// few hundred rows: 8 experts x ~128 rows, 14336 -> 4096, is 128 .. 256 tiles, and a tile's stream of 14336 k runs at
-// what one compute unit keeps in flight): 2 .. 4 slices per tile while tiles x slices fit the device's slots and a
-// slice keeps 24 stages of 64 k; the slice that arrives last at its tile's word adds the partial tiles and finishes
-// the elements (exact: int32).  The workspace comes out of the room reserved for sliced grouped launches.
+// K slices for a grouped launch of the MFMA-bound kernel that leaves compute units empty (a down projection of a few
+// experts: 2 experts x ~128 rows, 14336 -> 4096, is 32 tiles): 2 .. 4 slices per tile while tiles x slices still fit one
+// workgroup per compute unit (the deep-ring build) and a slice keeps 24 stages of 64 k; the slice that arrives last at
+// its tile's word adds the partial tiles and finishes the elements (exact: int32).  Beyond one workgroup per compute
+// unit slices lose: 8 experts x 113 .. 142 rows, 14336 -> 4096 (192 tiles), two slices each as 384 workgroups of the
+// two-per-unit build took 182 us against 139 us for the 192 unsliced ones with the deep ring.  The workspace comes out
+// of the room reserved for sliced grouped launches.
 ZmiRingSplit ring_group_split(int top, int items, int K, bool gated) {
   ZmiRingSplit rs = {1, nullptr, nullptr};
   const int th = top & 0xffff;
   if (gated || !(top & ZMI_RING_PAD) || th == 256 || items <= 0 || zmi_env(ZE_NO_GROUP_RING_SLICES)) return rs;
-  const int64_t slots = 2 * (int64_t)zmi_cu_count();
+  const int64_t slots = zmi_cu_count();
   int slices = (int)std::min<int64_t>(4, slots / items);
   const int nk = (int)(zmi_blob_kpad(K) / 64);
   while (slices > 1 && nk / slices < 24) --slices;
