@@ -38,7 +38,8 @@ static void validate_only() {
   matmul_params q = p;
   q.postop_.resize(1);
   q.postop_[0].po_type = zendnnl::ops::post_op_type_t::mish;
-  CHECK(matmul_direct('r', false, false, 4, 8, 16, 1.f, fake, 16, fake, 8, nullptr, 0.f, fake, 8, true, b, q) == status_t::failure);
+  // (mish on the static scale chain is accepted: what stops this call is the leading dimension, before any launch)
+  CHECK(matmul_direct('r', false, false, 4, 8, 16, 1.f, fake, 8, fake, 8, nullptr, 0.f, fake, 8, true, b, q) == status_t::failure);
   matmul_params bf;
   bf.dtypes.src = bf.dtypes.wei = bf.dtypes.dst = data_type_t::bf16;
   CHECK(matmul_direct('r', false, false, 4, 8, 16, 1.f, fake, 16, fake, 8, nullptr, 0.f, fake, 8, true, b, bf) == status_t::unimplemented);
@@ -170,8 +171,10 @@ static void gpu_w4a8_example() {
 }
 
 int main(int argc, char **argv) {
-  validate_only();
-  if (!(argc > 1 && std::strcmp(argv[1], "--validate-only") == 0)) { gpu_example(); gpu_w4a8_example(); }
+  // The validation cases hand the library addresses that are no memory: they run where no device can be launched on
+  // (a case that slipped past the validators then stops at the device check), never in front of the GPU examples.
+  if (argc > 1 && std::strcmp(argv[1], "--validate-only") == 0) validate_only();
+  else { gpu_example(); gpu_w4a8_example(); }
   std::printf(fails ? "adapter example: %d check(s) failed\n" : "adapter example: ok\n", fails);
   return fails ? 1 : 0;
 }

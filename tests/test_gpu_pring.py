@@ -116,75 +116,3 @@ def test_dynamic_quant_rows_match_the_tiled_kernel_bit_for_bit(env):
         outs.append(H.to_host(dst))
     assert np.array_equal(outs[0], outs[1])
 
-
-def _dyn_call(x, blob, ws, b, M, K, N, sbuf, po=capi.PO_SWISH):
-    p = lowoha.MatmulParams(src=capi.DT_BF16, wei=capi.DT_S8, dst=capi.DT_BF16, bias=capi.DT_F32, compute=capi.DT_S8)
-    p.dynamic_quant = True
-    p.src_scale = lowoha.QuantParam(sbuf, capi.DT_F32, (M, 1))
-    p.wei_scale = lowoha.QuantParam(ws, capi.DT_F32, (1, N))
-    p.postop_ = [lowoha.PostOp(po)]
-    p.mem_format_b = "r"
-    p.lowoha_algo = capi.ALGO_AOCL_DLP_BLOCKED
-    dst = torch.zeros((M, N), dtype=torch.bfloat16, device=H.DEV)
-    st = lowoha.matmul_direct("r", False, False, M, N, K, 1.0, x, x.shape[1], blob, N, b, 0.0, dst, N, True, p)
-    assert st == capi.SUCCESS, lowoha.last_error()
-    return H.to_host(dst), lowoha.last_kernel()
-
-
-# bands that are partly filled, chunks of fewer than eight rows, K from one 16-value piece per row to the largest the
-# launch takes, a source with a row stride, the default grid at BASELINE config 3's row count
-@pytest.mark.parametrize("M,K,N,ldx,grid", [(1100, 512, 3584, 512, 64), (257, 4096, 1024, 4104, 8), (520, 8192, 512, 8192, 16),
-                                            (300, 16, 640, 16, 8), (2048, 4096, 2048, 4096, 0), (1027, 1008, 1536, 1008, 24)])
-def test_rows_quantized_inside_the_launch_match_the_separate_launch(env, M, K, N, ldx, grid):
-    """Per-token quantization inside the persistent kernel's launch against the quantization launch followed by the
-    same kernel: scales and outputs bit-identical, also on a repeated call (the flags then hold the numbers of earlier
-    launches) and after a call of another shape; the scales against their closed form amax / 127."""
-    env(ZMI_PRING=1, ZMI_RING_MIN_M=1, ZMI_NO_DECODE_KERNEL=1, ZMI_RING_SPLITK=1)
-    if grid:
-        env(ZMI_PRING_GRID=grid)
-    rng = np.random.default_rng(M * 7 + K)
-    xh = np.zeros((M, ldx), dtype=np.uint16)
-    xh[:, :K] = H.gen_bf16_normal(rng, (M, K))
-    xh[:, K:] = 0x7fc0                       # (a NaN pattern in the stride's gap: never read)
-    if M > 40:
-        xh[33, :K] = 0                        # an all-zero row: the floor of the scale
-        xh[34, 3 % K] = 0x7f80                # an infinity: left out of the maximum, saturates
-    x = H.to_dev(xh)
-    w = H.to_dev(H.gen_weights(rng, K, N))
-    blob = H.prepack(w, K, N)
-    ws = H.to_dev(rng.uniform(0.001, 0.01, N).astype(np.float32))
-    b = H.to_dev((rng.standard_normal(N) * 0.1).astype(np.float32))
-    res = []
-    for no_fuse in (1, 0, 0):
-        env(ZMI_NO_PRING_QUANT=1 if no_fuse else None)
-        sbuf = torch.zeros(M, dtype=torch.float32, device=H.DEV)
-        out, name = _dyn_call(x, blob, ws, b, M, K, N, sbuf)
-        assert "pring" in name and (("quant in the launch" in name) == (not no_fuse)), name
-        res.append((out, H.to_host(sbuf)))
-        if no_fuse == 0 and len(res) == 2:
-            # another shape in between: the words of the first chunks are reused with other launch numbers
-            x2 = H.to_dev(H.gen_bf16_normal(rng, (264, 64)))
-            w2 = H.to_dev(H.gen_weights(rng, 64, 512))
-            _dyn_call(x2, H.prepack(w2, 64, 512), ws[:512].contiguous(), b[:512].contiguous(), 264, 64, 512, None)
-    for out, sc in res[1:]:
-        assert np.array_equal(sc.view(np.uint32), res[0][1].view(np.uint32))
-        assert np.array_equal(out, res[0][0])
-    vals = (xh[:, :K].astype(np.uint32) << 16).view(np.float32)
-    amax = np.max(np.where(np.isfinite(vals), np.abs(vals), np.float32(0)), axis=1).astype(np.float32)
-    want = np.maximum(np.maximum(amax, np.float32(1e-10)) / np.float32(127.0), np.float32(1e-10)).astype(np.float32)
-    assert np.array_equal(res[1][1].view(np.uint32), want.view(np.uint32))
-
-
-def test_scale_buffer_that_shares_cache_lines_between_bands_takes_the_separate_launch(env):
-    env(ZMI_PRING=1, ZMI_PRING_GRID=8, ZMI_RING_MIN_M=1, ZMI_RING_SPLITK=1)
-    rng = np.random.default_rng(11)
-    M, K, N = 520, 256, 512
-    x = H.to_dev(H.gen_bf16_normal(rng, (M, K)))
-    blob = H.prepack(H.to_dev(H.gen_weights(rng, K, N)), K, N)
-    ws = H.to_dev(rng.uniform(0.001, 0.01, N).astype(np.float32))
-    b = H.to_dev(np.zeros(N, dtype=np.float32))
-    whole = torch.zeros(M + 8, dtype=torch.float32, device=H.DEV)
-    out_a, name_a = _dyn_call(x, blob, ws, b, M, K, N, whole[1:M + 1])
-    out_b, name_b = _dyn_call(x, blob, ws, b, M, K, N, whole[:M])
-    assert "quant in the launch" not in name_a and "quant in the launch" in name_b
-    assert np.array_equal(out_a, out_b)

@@ -306,135 +306,8 @@ __device__ __forceinline__ void pr_tile(const ZmiProblem &p, const ZmiEpilogue &
 // XCD walks the whole activation matrix and an eighth of the weights, through its own L2); its cells, band-major,
 // are split evenly over its compute units, and a compute unit covers its run with tiles of up to four units that
 // never cross a band.  Workgroup ids go round robin over the XCDs.
-// ---- the row quantization inside the launch (see ZmiPringQuant) -------------------------------------------------
-// One chunk = rows 8 c .. 8 c + 7.  Thread t: row t % 8, and of every 512 k the 16 values from (t / 8) * 16 -- one
-// 16-byte piece of the fragment layout, so that the eight threads of one t / 8 write 128 contiguous bytes.  The row's
-// values stay in registers between the maximum and the rounding (arithmetic of k_quant.hip: the maximum over the finite
-// values, scale = max(amax, 1e-10) / 127 floored at 1e-10, zmi_quant_elem).  Stores go through to device scope: the
-// other XCDs read these bytes in this same launch.
-#define PR_Q_STEPS 16   // K up to 16 * 512
-__device__ __forceinline__ void pr_store16_agent(void *ptr, v4i v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(ptr), "v"(v) : "memory");
-}
-__device__ __forceinline__ void pr_quant_chunk(const ZmiProblem &p, const ZmiPringQuant &q, int c, float *red) {
-  const int tid = threadIdx.x, r = tid % 8, qd = tid / 8, lane = tid % 64, wave = tid / 64;
-  const int M = p.M, K = p.K;
-  const int64_t K_pad = zmi_blob_kpad(K);
-  const int row = c * 8 + r;
-  const bool valid = row < M;
-  const uint16_t *src = (const uint16_t *)q.x + (int64_t)(valid ? row : M - 1) * q.ldx;
-  v4i raw[PR_Q_STEPS][2];
-  float amax = 0.0f;
-#pragma unroll
-  for (int s = 0; s < PR_Q_STEPS; ++s) {
-    const int k = (s * 32 + qd) * 16;
-    raw[s][0] = (v4i){0, 0, 0, 0};
-    raw[s][1] = (v4i){0, 0, 0, 0};
-    if (k < K && valid) {
-      raw[s][0] = *zmi_global<const v4i>(src + k);
-      raw[s][1] = *zmi_global<const v4i>(src + k + 8);
-    }
-  }
-#pragma unroll
-  for (int s = 0; s < PR_Q_STEPS; ++s)
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t w = (uint32_t)raw[s][h][j];
-        const float a0 = fabsf(__uint_as_float(w << 16)), a1 = fabsf(__uint_as_float(w & 0xffff0000u));
-        if ((__float_as_uint(a0) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a0);
-        if ((__float_as_uint(a1) & 0x7f800000u) != 0x7f800000u) amax = fmaxf(amax, a1);
-      }
-  // the row's maximum: the lanes of one row in a wavefront (l % 8 equal), then the four wavefronts
-  amax = fmaxf(amax, __shfl_xor(amax, 8));
-  amax = fmaxf(amax, __shfl_xor(amax, 16));
-  amax = fmaxf(amax, __shfl_xor(amax, 32));
-  if (lane < 8) red[wave * 8 + lane] = amax;
-  __syncthreads();
-  amax = fmaxf(fmaxf(red[r], red[8 + r]), fmaxf(red[16 + r], red[24 + r]));
-  __syncthreads();
-  if (amax < 1e-10f) amax = 1e-10f;
-  float sc = __fdiv_rn(amax, 127.0f);
-  if (sc < 1e-10f) sc = 1e-10f;
-  const float inv = __fdiv_rn(1.0f, sc);
-  if (valid && qd == 0)
-    __hip_atomic_store((unsigned int *)&q.scales[row], __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (!valid) return;
-  int8_t *dst = (int8_t *)const_cast<void *>(p.A);
-#pragma unroll
-  for (int s = 0; s < PR_Q_STEPS; ++s) {
-    const int k = (s * 32 + qd) * 16;
-    if (k < K) {
-      v4i o;
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-          uint32_t word = 0;
-#pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const uint32_t w = (uint32_t)raw[s][h][jj * 2 + e];
-            const int8_t q0 = zmi_quant_elem(__uint_as_float(w << 16), sc, inv);
-            const int8_t q1 = zmi_quant_elem(__uint_as_float(w & 0xffff0000u), sc, inv);
-            word |= ((uint32_t)(uint8_t)q0 | ((uint32_t)(uint8_t)q1 << 8)) << (16 * e);
-          }
-          o[h * 2 + jj] = (int)word;
-        }
-      pr_store16_agent(dst + zmi_afrag_off(row, k, K_pad), o);
-    }
-  }
-}
-
-// All rows of the launch, then nothing: returns when no chunk is left to claim.
-// Every branch around the barriers of this loop is taken by whole wavefronts (the first wavefront claims and publishes,
-// all its lanes writing the same words; the chunk number is made a scalar).  With a one-thread branch at the loop's end
-// and the same branch at its start the compiler joined the two, let the other lanes run on to the next barrier without
-// that thread, and the loop never ended.
-__device__ __forceinline__ void pr_quant_rows(const ZmiProblem &p, const ZmiPringQuant &q) {
-  float *red = reinterpret_cast<float *>(zmi_pring_smem);
-  int *slot = reinterpret_cast<int *>(zmi_pring_smem + 256);
-  const int lane = threadIdx.x % 64;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
-  for (;;) {
-    if (wave == 0) {
-      // (one lane adds one, the others nothing: every lane of the wavefront then holds a value of the counter from
-      // before that lane's own addition, and lane 0's is the chunk)
-      const unsigned int got = __hip_atomic_fetch_add(&q.sync[0], lane == 0 ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      *slot = __builtin_amdgcn_readfirstlane((int)got);
-    }
-    __syncthreads();
-    const int c = __builtin_amdgcn_readfirstlane(*slot);
-    __syncthreads();
-    if (c >= q.n_chunks) return;
-    pr_quant_chunk(p, q, c, red);
-    // the chunk's flag, once every store of the workgroup has been acknowledged
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (wave == 0) __hip_atomic_store(&q.sync[2 + c], q.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-}
-
-// Every wavefront for itself: the flags of the band's chunks carry the launch's number, or the time ran out.
-__device__ __forceinline__ bool pr_wait_band(const ZmiPringQuant &q, int band) {
-  const int lane = threadIdx.x % 64;
-  const int c = band * 32 + (lane % 32);
-  const unsigned int *f = &q.sync[2 + (c < q.n_chunks ? c : q.n_chunks - 1)];
-  const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
-  bool ok = false;
-  for (;;) {
-    const unsigned int v = __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (__all(v == q.epoch)) { ok = true; break; }
-    if (__builtin_amdgcn_s_memrealtime() - t0 > (uint64_t)q.wait_ticks) break;
-    __builtin_amdgcn_s_sleep(8);
-  }
-  if (!ok && lane == 0) __hip_atomic_store(q.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  return ok;
-}
-
 template <int EK>
-__global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pring_kernel(ZmiProblem p, ZmiEpilogue epi, ZmiPringQuant q) {
-  if (q.x) pr_quant_rows(p, q);
+__global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pring_kernel(ZmiProblem p, ZmiEpilogue epi) {
   const int np = (int)(zmi_blob_npad(p.N) / 64);
   const int bands = (p.M + 255) / 256;
   const int b = blockIdx.x, x = b % 8, j = b / 8, cpx = gridDim.x / 8;
@@ -446,23 +319,8 @@ __global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pring_kernel(ZmiProble
   zmi_set_f32_flush();
   bool first = true;
   int tile_no = 0;
-  int band_ready = -1;
-  bool rows_ok = true;
-  while (u < u1 && rows_ok) {
+  while (u < u1) {
     const int band = u / wx, pin = u % wx;
-    if (q.x && band != band_ready) {
-      // (uniform over the workgroup only after the exchange: every wavefront waits for itself)
-      const bool mine = pr_wait_band(q, band);
-      int *votes = reinterpret_cast<int *>(zmi_pring_smem + 512);
-      pr_wait_vm<0>();   // (the tile's counted waits below count its own requests only)
-      __syncthreads();
-      votes[__builtin_amdgcn_readfirstlane(threadIdx.x / 64)] = mine ? 1 : 0;   // (every lane: no one-thread branch in this loop)
-      __syncthreads();
-      rows_ok = __builtin_amdgcn_readfirstlane(votes[0] & votes[1] & votes[2] & votes[3]) != 0;   // (a scalar: see pr_quant_rows)
-      __syncthreads();
-      if (!rows_ok) break;
-      band_ready = band;
-    }
     const int band_end = (band + 1) * wx;
     const int n = (u1 < band_end ? u1 : band_end) - u;
     const int k = (n + 3) / 4;
@@ -478,17 +336,6 @@ __global__ __launch_bounds__(PR_THREADS, 1) void zmi_gemm_pring_kernel(ZmiProble
     ++tile_no;
     u += ni;
   }
-  if (q.x) {
-    // the workgroup that leaves last puts the two counters back to zero for the next launch
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const unsigned int before = __hip_atomic_fetch_add(&q.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (before == gridDim.x - 1) {
-        __hip_atomic_store(&q.sync[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&q.sync[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-  }
 }
 
 // One problem with a bf16 destination, a straight-line epilogue, 16-byte aligned rows and N a multiple of 4.
@@ -500,30 +347,16 @@ bool zmi_pring_takes(const ZmiProblem &p, const ZmiEpilogue &epi) {
 }
 
 template <int EK>
-static hipError_t pring_launch(const ZmiProblem &p, const ZmiEpilogue &epi, const ZmiPringQuant &q, int grid, hipStream_t stream) {
+static hipError_t pring_launch(const ZmiProblem &p, const ZmiEpilogue &epi, int grid, hipStream_t stream) {
   hipError_t e = zmi_func_smem_once((const void *)zmi_gemm_pring_kernel<EK>, PR_SMEM);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL((zmi_gemm_pring_kernel<EK>), dim3(grid), dim3(PR_THREADS), PR_SMEM, stream, p, epi, q);
+  hipLaunchKernelGGL((zmi_gemm_pring_kernel<EK>), dim3(grid), dim3(PR_THREADS), PR_SMEM, stream, p, epi);
   return hipGetLastError();
 }
 
-// What the quantization inside the launch takes: bf16 rows, 16-byte aligned, K a multiple of 16 up to 8192.
-bool zmi_pring_quant_ok(const void *x, int32_t x_dt, int64_t ldx, int K) {
-  return x && x_dt == ZMI_DT_BF16 && K % 16 == 0 && K <= PR_Q_STEPS * 512 && ((uintptr_t)x) % 16 == 0 && (ldx * 2) % 16 == 0 &&
-         ldx >= K;
-}
-
 // p.A in fragment-major order (zmi_afrag_off).  One workgroup per compute unit.
-hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream, const ZmiPringQuant *qp) {
+hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream) {
   if (!zmi_pring_takes(p, epi)) return hipErrorInvalidValue;
-  ZmiPringQuant q = {};
-  if (qp && qp->x) {
-    q = *qp;
-    if (!zmi_pring_quant_ok(q.x, ZMI_DT_BF16, q.ldx, p.K) || !q.scales || !q.sync || !q.error || q.epoch == 0 ||
-        q.n_chunks != (p.M + 7) / 8 || ((uintptr_t)q.scales) % 128 != 0 || (const void *)q.scales != p.src_scale_ptr || epi.src_scale_mode != ZMI_SS_TOKEN_PTR ||
-        epi.src_scale_dt != ZMI_DT_F32)
-      return hipErrorInvalidValue;
-  }
   int grid = zmi_cu_count() / 8 * 8;
   // (ZMI_PRING_GRID: fewer workgroups, so that small test shapes give every workgroup several tiles)
   if (const char *env = zmi_env(ZE_PRING_GRID)) {
@@ -532,9 +365,9 @@ hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hi
   }
   if (grid < 8) return hipErrorInvalidValue;
   switch (epi.fast_kind) {
-  case ZMI_EK_SWISH: return pring_launch<ZMI_EK_SWISH>(p, epi, q, grid, stream);
-  case ZMI_EK_GELU_TANH: return pring_launch<ZMI_EK_GELU_TANH>(p, epi, q, grid, stream);
-  case ZMI_EK_RELU: return pring_launch<ZMI_EK_RELU>(p, epi, q, grid, stream);
-  default: return pring_launch<ZMI_EK_NONE>(p, epi, q, grid, stream);
+  case ZMI_EK_SWISH: return pring_launch<ZMI_EK_SWISH>(p, epi, grid, stream);
+  case ZMI_EK_GELU_TANH: return pring_launch<ZMI_EK_GELU_TANH>(p, epi, grid, stream);
+  case ZMI_EK_RELU: return pring_launch<ZMI_EK_RELU>(p, epi, grid, stream);
+  default: return pring_launch<ZMI_EK_NONE>(p, epi, grid, stream);
   }
 }

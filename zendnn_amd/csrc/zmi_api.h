@@ -8,7 +8,7 @@ int32_t validate_matmul(const void *src, const void *weight, const void *dst, in
 bool is_dynamic_quant_config(const zmi_matmul_params_t &p);
 int32_t build_epilogue(const zmi_matmul_params_t &p, int M, int N, float alpha, float beta, const void *bias,
                        ZmiEpilogue *out, ZmiProblem *prob, bool allow_wei_zp = false);
-int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan, const ZmiPringQuant *pq = nullptr);
+int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan);
 bool a_needs_repack(const void *A, int64_t lda, int K, bool transA);
 bool use_ring_kernel(int M, int N, int K);
 // weight-only quantization (zmi_api_woq.hip): bf16 source, s4 / u4 weights, no dynamic_quant

@@ -339,16 +339,67 @@ static bool fused_quant_allowed() {
   return cs == hipStreamCaptureStatusNone;
 }
 
-// The persistent form of the large-M kernel (k_pring.hip): one problem whose (256-row band, 64-column unit) cells give
-// every compute unit at least three (a tile of 256 x 192 or more).  ZMI_PRING = 0 / 1 overrides the size rule.
-static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi) {
-  if (!zmi_pring_takes(prob, epi)) return false;
-  if (const char *env = zmi_env(ZE_PRING)) return std::atoi(env) != 0;
-  const int64_t cells = (int64_t)((prob.M + 255) / 256) * (zmi_blob_npad(prob.N) / 64);
-  return prob.M >= 256 && cells >= 3 * (int64_t)zmi_cu_count();
+// The persistent form of the large-M kernel (k_pring.hip) or the tiled one (k_ring.hip)?  Both last as long as their
+// busiest compute unit, so the two are priced in units of one 256 x 256 tile (main loop and epilogue, K = 4096:
+// 62 us) and the cheaper one takes the call; the persistent form also takes a tie when M fills its 256-row bands.
+//   persistent: the launch's own cell assignment is walked (k_pring.hip: XCDs by column, an XCD's cells split evenly
+//   over its compute units, tiles of 1 .. 4 cells that never cross a band) with a tile of 1 / 2 / 3 / 4 cells at
+//   0.40 / 0.57 / 0.78 / 1;
+//   tiled: 256-row tiles 1 per round of one tile per compute unit; 128-row tiles 0.57 while there is at most one per
+//   compute unit and 0.95 per round of two (the second workgroup on a unit hides the first one's epilogue, no more);
+//   64-row tiles 0.40 and 0.60.
+// The prices are from these measurements on MI355X (K = 4096, whole call in us, tiled / persistent): M x N =
+// 2048 x 4096 51.7 / 47.7, 1024 x 4096 39.1 / 35.1, 2048 x 2048 41.6 / 38.4, 512 x 14336 48.0 / 45.3, 768 x 14336
+// 68.8 / 62.5, 1300 x 14336 138.7 / 103.5, 1536 x 14336 130.7 / 106.7, 2048 x 14336 138.0 / 126.7, 4096 x 14336
+// 266.9 / 243.8, 2048 x 5000 69.4 / 61.0 (persistent cheaper or tie); 1536 x 4096 49.2 / 58.5, 1100 x 4096 42.7 / 53.5,
+// 600 x 8192 42.8 / 51.3, 1100 x 14336 78.0 / 87.4, 300 x 14336 41.7 / 42.7 (tiled cheaper, or a tie with a partly
+// filled band).  ZMI_PRING = 0 / 1 overrides the choice.
+static double pring_price(int M, int N) {
+  static const double tile_price[5] = {0.0, 0.40, 0.57, 0.78, 1.0};
+  const int np = (int)(zmi_blob_npad(N) / 64), bands = (M + 255) / 256;
+  const int cpx = std::max(1, zmi_cu_count() / 8);
+  double worst = 0.0;
+  for (int x = 0; x < 8; ++x) {
+    const int wx = (int)((int64_t)(x + 1) * np / 8) - (int)((int64_t)x * np / 8);
+    if (wx <= 0) continue;
+    const int64_t cells = (int64_t)wx * bands;
+    for (int j = 0; j < cpx; ++j) {
+      int u = (int)(cells * j / cpx);
+      const int u1 = (int)(cells * (j + 1) / cpx);
+      double price = 0.0;
+      while (u < u1) {
+        const int band_end = (u / wx + 1) * wx;
+        const int n = std::min(u1, band_end) - u;
+        const int k = (n + 3) / 4;
+        const int ni = (n + k - 1) / k;
+        price += tile_price[ni];
+        u += ni;
+      }
+      worst = std::max(worst, price);
+    }
+  }
+  return worst;
 }
 
-int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan, const ZmiPringQuant *pq) {
+static double ring_price(int M, int N, int top) {
+  const int th = top & 0xffff;
+  const int64_t n_cu = zmi_cu_count();
+  const int64_t tiles = (int64_t)((M + th - 1) / th) * ((N + 255) / 256);
+  if (th == 256) return (double)((tiles + n_cu - 1) / n_cu);
+  const double alone = th == 128 ? 0.57 : 0.40, paired = th == 128 ? 0.95 : 0.60;
+  if (tiles <= n_cu) return alone;
+  return (double)((tiles + 2 * n_cu - 1) / (2 * n_cu)) * paired;
+}
+
+static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi, int ring_top) {
+  if (!zmi_pring_takes(prob, epi)) return false;
+  if (const char *env = zmi_env(ZE_PRING)) return std::atoi(env) != 0;
+  if (prob.M < 256) return false;
+  const double mine = pring_price(prob.M, prob.N), other = ring_price(prob.M, prob.N, ring_top);
+  return mine < other - 1e-9 || (mine < other + 1e-9 && prob.M % 256 == 0);
+}
+
+int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
   if (decode_kernel_allowed(prob.M, prob.N, prob.K)) {
     set_kernel_name(zmi_decode_16row_kernel(prob, false) ? "decode16_dma_rows_mfma16x16x64" : "decode_lds_rows_mfma16x16x64");
     if (!hip_ok(zmi_launch_gemm_decode(prob, epi, nullptr, stream()), "decode GEMM launch")) return ZMI_FAILURE;
@@ -376,12 +427,11 @@ int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const Zm
       // the reduction's element-finishing code adds)
       split.arrivals = prob.row_comp ? nullptr : slice_arrivals(plan->tiles);
     }
-    if (plan->slices == 1 && pring_wanted(prob, epi)) {
-      set_kernel_name(pq ? "pring_mfma32x32x32_persistent (per-token quant in the launch)" : "pring_mfma32x32x32_persistent");
-      if (!hip_ok(zmi_launch_gemm_pring(prob, epi, stream(), pq), "persistent MFMA GEMM launch")) return ZMI_FAILURE;
+    if (plan->slices == 1 && pring_wanted(prob, epi, plan->top)) {
+      set_kernel_name("pring_mfma32x32x32_persistent");
+      if (!hip_ok(zmi_launch_gemm_pring(prob, epi, stream()), "persistent MFMA GEMM launch")) return ZMI_FAILURE;
       return ZMI_SUCCESS;
     }
-    if (pq) { set_error("in-launch quantization without the persistent kernel"); return ZMI_FAILURE; }
     const int th = plan->top & 0xffff;
     set_kernel_name(plan->slices > 1 ? (th == 64 ? "ring_mfma32x32x32_top64_ksliced" : "ring_mfma32x32x32_top128_ksliced")
                                      : (th == 256 ? "ring_mfma32x32x32_top256"
@@ -723,8 +773,6 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
   ZmiFusedQuant fused;
   std::memset(&fused, 0, sizeof(fused));
   bool use_fused = false;
-  bool late_quant = false;    // the row quantization has not been launched yet (see below)
-  float *late_scales = nullptr;
   int8_t *a_frag = nullptr;   // per-group GEMM at large M: the rows in fragment order, once they exist
   if (dyn) {
     // reference: reorder_quantization_wrapper, matmul/quantization/reorder_quantization.cpp:43-280
@@ -792,15 +840,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       void *scale_out = p.src_scale.buff ? (void *)p.src_scale.buff : (void *)sc;
       // (without a caller buffer the scales live in scratch, in the dtype the params name: the reference allocates
       // its own buffer of that dtype, reorder_quantization.cpp:103-117, and its GEMM reads the narrowed values back)
-      // Rows for the large-M kernel whose persistent form can quantize them inside its own launch: the decision waits
-      // for the epilogue (below); either way the rows are quantized on this stream ahead of the first tile.
-      // (the scales of one 256-row band must not share a cache line with the next band's: a caller's buffer that is
-      // not 128-byte aligned takes the separate launch)
-      if (ring && M > 1 && sdt == ZMI_DT_F32 && plan.slices == 1 && zmi_pring_quant_ok(src, p.dt_src, lda, K) && fused_quant_allowed() &&
-          ((uintptr_t)scale_out) % 128 == 0 && !zmi_env(ZE_NO_PRING_QUANT)) {
-        late_quant = true;
-        late_scales = (float *)scale_out;
-      } else if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, frag_kpad, scale_out, sdt, stream()), "quant launch"))
+      if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, q, K16, frag_kpad, scale_out, sdt, stream()), "quant launch"))
         return ZMI_FAILURE;
       ep.src_scale.buff = scale_out;
       ep.src_scale.dt = sdt;
@@ -892,19 +932,7 @@ static int32_t matmul_single(char layout, int32_t transA, int32_t transB, int32_
       st = hip_ok(zmi_launch_gemm_smallm_fused(prob, epi, fused, stream()), "fused small-M GEMM launch") ? ZMI_SUCCESS : ZMI_FAILURE;
     }
   } else {
-    ZmiPringQuant pq = {};
-    if (late_quant) {
-      ZmiFusedQuant ho;
-      unsigned int *words = pring_wanted(prob, epi) ? pring_sync_words(2 + (int64_t)(M + 7) / 8) : nullptr;
-      if (words && fused_handoff(&ho)) {   // (its launch number, time limit and error word)
-        pq.x = src; pq.ldx = lda; pq.scales = late_scales; pq.sync = words; pq.error = ho.error;
-        pq.epoch = ho.epoch; pq.wait_ticks = ho.wait_ticks; pq.n_chunks = (M + 7) / 8;
-      } else if (!hip_ok(zmi_launch_quant_rows(src, p.dt_src, M, K, lda, (int8_t *)const_cast<void *>(prob.A), K16, frag_kpad,
-                                               late_scales, ZMI_DT_F32, stream()), "quant launch")) {
-        return ZMI_FAILURE;
-      }
-    }
-    st = run_single_gemm(prob, epi, ring ? &plan : nullptr, pq.x ? &pq : nullptr);
+    st = run_single_gemm(prob, epi, ring ? &plan : nullptr);
   }
   upload_fence();
   return st;

@@ -26,7 +26,6 @@ bool ensure_device();
 // Zeroed device words (one per 32-column block, at least n of them) that K-sliced launches count their arrivals in and
 // leave zeroed; null when they cannot be had or ZMI_NO_SLICE_ARRIVALS is set (the launch then ends in a reduction kernel).
 unsigned int *slice_arrivals(int64_t n);
-unsigned int *pring_sync_words(int64_t n);
 
 // The calling thread's side stream (default priority, created on first use) with a fork and a join event, for work
 // that may run beside the stream's own; null fields when it cannot be had or ZMI_NO_SIDE_STREAM is set.

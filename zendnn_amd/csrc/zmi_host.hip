@@ -47,8 +47,7 @@ const char *const kEnvNames[ZE_COUNT] = {
     "ZENDNNL_DIAGNOSTICS_ENABLE",
     "ZENDNNL_MATMUL_WEIGHT_CACHE",
     "ZMI_NO_UNCACHED_FLAGS",
-    "ZMI_NO_GROUP_RING_SLICES",
-    "ZMI_NO_PRING_QUANT"};
+    "ZMI_NO_GROUP_RING_SLICES"};
 struct EnvTable {
   std::string val[ZE_COUNT];
   bool set[ZE_COUNT] = {};
@@ -108,9 +107,6 @@ struct ThreadCtx {
   // arrival words of K-sliced launches (see slice_arrivals())
   unsigned int *arrivals = nullptr;
   int64_t n_arrivals = 0;
-  // (see pring_sync_words())
-  unsigned int *pring_sync = nullptr;
-  int64_t n_pring_sync = 0;
   // side stream (see side_stream())
   hipStream_t side = nullptr;
   hipEvent_t side_fork = nullptr, side_join = nullptr;
@@ -186,29 +182,6 @@ unsigned int *slice_arrivals(int64_t n) {
 
 // Words of the persistent large-M kernel's in-launch quantization (two counters that are zero between launches, then
 // one flag per chunk of eight rows that keeps the number of the launch that wrote it): zeroed once, grown on demand.
-unsigned int *pring_sync_words(int64_t n) {
-  auto &c = tctx;
-  if (n > c.n_pring_sync) {
-    if (c.pring_sync) {
-      if (hipStreamSynchronize(c.stream) != hipSuccess || hipFree(c.pring_sync) != hipSuccess) (void)hipGetLastError();
-      c.pring_sync = nullptr;
-      c.n_pring_sync = 0;
-    }
-    const int64_t want = n < 4096 ? 4096 : n * 2;
-    void *d = nullptr;
-    if (hipMalloc(&d, (size_t)want * sizeof(unsigned int)) != hipSuccess ||
-        hipMemset(d, 0, (size_t)want * sizeof(unsigned int)) != hipSuccess) {
-      (void)hipGetLastError();
-      if (d) (void)hipFree(d);
-      return nullptr;
-    }
-    (void)hipStreamSynchronize(nullptr);   // (the zeros are there before the first launch on any stream reads them)
-    c.pring_sync = (unsigned int *)d;
-    c.n_pring_sync = want;
-  }
-  return c.pring_sync;
-}
-
 ZmiRingSide side_stream() {
   auto &c = tctx;
   if (!c.side_tried) {

@@ -62,7 +62,6 @@ enum ZmiEnvVar {
   ZE_ZENDNNL_MATMUL_WEIGHT_CACHE,
   ZE_NO_UNCACHED_FLAGS,
   ZE_NO_GROUP_RING_SLICES,
-  ZE_NO_PRING_QUANT,
   ZE_COUNT
 };
 const char *zmi_env(ZmiEnvVar v);
@@ -137,23 +136,7 @@ hipError_t zmi_launch_gemm_ring(const ZmiProblem &p, const ZmiEpilogue &epi, int
                                 hipStream_t stream, const ZmiRingSide *side = nullptr);
 // k_pring.hip: the persistent form for one problem (A in fragment-major order, bf16 destination, straight-line epilogue)
 bool zmi_pring_takes(const ZmiProblem &p, const ZmiEpilogue &epi);
-// Per-token quantization of the bf16 source inside that launch (q null or q->x null: the rows at p.A are there already).
-// The workgroups first quantize the rows, eight at a time, claiming chunks from a counter until none is left (so the
-// rows get done by whichever workgroups are running); a chunk's flag takes the launch's number once its bytes are
-// written through, and a workgroup waits for the 32 flags of a band before it starts a tile of that band -- for at
-// most wait_ticks of the 100 MHz clock, after which it sets *error and stores nothing more.
-struct ZmiPringQuant {
-  const void *x;            // bf16 rows, K a multiple of 16 up to 8192, 16-byte aligned rows
-  int64_t ldx;              // elements
-  float *scales;            // [M] f32, device memory: written here, read by the epilogue (= p.src_scale_ptr)
-  unsigned int *sync;       // [0] chunk counter, [1] exit counter (both zero between launches), [2 + c] flag of chunk c
-  unsigned int *error;      // pinned host word, as the device addresses it
-  uint32_t epoch;           // the launch's number (never 0)
-  uint32_t wait_ticks;
-  int32_t n_chunks;         // ceil(M / 8)
-};
-bool zmi_pring_quant_ok(const void *x, int32_t x_dt, int64_t ldx, int K);
-hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream, const ZmiPringQuant *q = nullptr);
+hipError_t zmi_launch_gemm_pring(const ZmiProblem &p, const ZmiEpilogue &epi, hipStream_t stream);
 hipError_t zmi_launch_gemm_ring_group(const ZmiProblem *probs_host, const ZmiProblem *probs_dev, int n_prob,
                                       int top, int64_t worst_rows, int worst_cols, int *tab_dev, bool tab_ready,
                                       const ZmiEpilogue &epi, hipStream_t stream, const ZmiRingSplit *split = nullptr);
