@@ -17,6 +17,15 @@ def _run(args):
     assert "adapter example: ok" in r.stdout
 
 
+def _device_present():
+    try:
+        import torch
+        return torch.cuda.device_count() > 0
+    except Exception:
+        return False
+
+
+@pytest.mark.skipif(_device_present(), reason="placeholder addresses: run where no device can be launched on")
 def test_cpp_adapter_validation_paths():
     _run(["--validate-only"])
 

@@ -383,6 +383,7 @@ static double pring_price(int M, int N) {
 
 static double ring_price(int M, int N, int top) {
   const int th = top & 0xffff;
+  if (th <= 0) return 1e30;
   const int64_t n_cu = zmi_cu_count();
   const int64_t tiles = (int64_t)((M + th - 1) / th) * ((N + 255) / 256);
   if (th == 256) return (double)((tiles + n_cu - 1) / n_cu);
@@ -394,7 +395,7 @@ static double ring_price(int M, int N, int top) {
 static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi, int ring_top) {
   if (!zmi_pring_takes(prob, epi)) return false;
   if (const char *env = zmi_env(ZE_PRING)) return std::atoi(env) != 0;
-  if (prob.M < 256) return false;
+  if (prob.M < 256 || zmi_env(ZE_GEMM_TOP)) return false;   // (a forced tile height asks for the tiled form)
   const double mine = pring_price(prob.M, prob.N), other = ring_price(prob.M, prob.N, ring_top);
   return mine < other - 1e-9 || (mine < other + 1e-9 && prob.M % 256 == 0);
 }
@@ -960,6 +961,7 @@ int32_t zmi_matmul_direct(char layout, int32_t transA, int32_t transB, int32_t M
                           const void *bias, float beta, void *dst, int32_t ldc, int32_t is_weights_const,
                           const zmi_batch_params_t *batch_params, const zmi_matmul_params_t *params) {
   clear_error();
+  note_operand(src); note_operand(weight); note_operand(dst); note_operand(bias);
   if (async_failure_pending()) return ZMI_FAILURE;
   if (!params) { set_error("null params"); return ZMI_FAILURE; }
   const zmi_matmul_params_t &p = *params;
@@ -1158,6 +1160,7 @@ static int32_t reorder_dynamic(const void *src, void *dst, zmi_reorder_params_t 
 
 int32_t zmi_reorder_direct(const void *src, void *dst, zmi_reorder_params_t *params) {
   clear_error();
+  note_operand(src); note_operand(dst);
   if (!params) { set_error("null params"); return ZMI_FAILURE; }
   if (params->is_prepack) {
     // reference: weight_prepack_into, reorder/prepack/lowoha_prepack.cpp:315-373
@@ -1183,6 +1186,7 @@ int32_t zmi_group_dynamic_quant(int32_t n, const void *const *src, const int32_t
   // reference: group_dynamic_quant, reorder/lowoha_reorder.cpp:279-404
   clear_error();
   if (!params || n <= 0 || !src || !M || !K || !dst || !scale) { set_error("group_dynamic_quant: bad arguments"); return ZMI_FAILURE; }
+  for (int32_t i = 0; i < n; ++i) { note_operand(src[i]); note_operand(dst[i]); note_operand(scale[i]); }
   if (!(params->src_dtype == ZMI_DT_BF16 || params->src_dtype == ZMI_DT_F32) || params->dst_dtype != ZMI_DT_S8) {
     set_error("group_dynamic_quant: only bf16/f32 -> s8");
     return ZMI_FAILURE;

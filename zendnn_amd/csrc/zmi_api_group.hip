@@ -374,6 +374,16 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
   clear_error();
   if (!args) { set_error("null args"); return ZMI_FAILURE; }
   const zmi_group_args_t &a = *args;
+  for (int32_t i = 0; a.src && i < a.n_src; ++i) note_operand(a.src[i]);
+  for (int32_t i = 0; a.weight && i < a.n_weight; ++i) note_operand(a.weight[i]);
+  for (int32_t i = 0; a.bias && i < a.n_bias; ++i) note_operand(a.bias[i]);
+  for (int32_t i = 0; a.dst && i < a.n_dst; ++i) note_operand(a.dst[i]);
+  if (fused_moe) {
+    for (int32_t i = 0; fused_moe->down_weight && i < fused_moe->n_down_weight; ++i) note_operand(fused_moe->down_weight[i]);
+    for (int32_t i = 0; fused_moe->bias_down && i < fused_moe->n_bias_down; ++i) note_operand(fused_moe->bias_down[i]);
+    for (int32_t i = 0; fused_moe->dst_down && i < fused_moe->n_dst_down; ++i) note_operand(fused_moe->dst_down[i]);
+  }
+  if (moe_postop) { note_operand(moe_postop->output); note_operand(moe_postop->topk_weights); }
   size_t num_ops = 0;
   bool op1_internal = false, op2_internal = false;
   int32_t st = validate_group(a, moe_postop, gated_act, fused_moe, &num_ops, &op1_internal, &op2_internal);
@@ -836,6 +846,8 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
     set_error("moe_fused_device: null argument");
     return ZMI_FAILURE;
   }
+  note_operand(d->x); note_operand(d->topk_ids); note_operand(d->topk_weights); note_operand(d->w13_blob);
+  note_operand(d->w2_blob); note_operand(d->w13_scale); note_operand(d->w2_scale); note_operand(d->out);
   const int T = d->T, H = d->H, I = d->I, E = d->E, topk = d->topk;
   if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0 || d->ldx < H || d->ldo < H) { set_error("moe_fused_device: bad shape"); return ZMI_FAILURE; }
   if (H % 16 != 0 || I % 32 != 0) { set_error("moe_fused_device: H must be a multiple of 16 and I of 32"); return ZMI_UNIMPLEMENTED; }

@@ -55,6 +55,7 @@ extern "C" int32_t zmi_matmul_direct_noalloc(char layout, int32_t transA, int32_
                                              const zmi_batch_params_t *batch_params, const zmi_matmul_params_t *params) {
   clear_error();
   (void)ldb;
+  note_operand(src); note_operand(weight); note_operand(dst); note_operand(bias);
   // a hand-off of an earlier launch on this thread that gave up is reported here, as zmi_matmul_direct does
   if (async_failure_pending()) return ZMI_FAILURE;
   if (!params) { set_error("null params"); return ZMI_FAILURE; }

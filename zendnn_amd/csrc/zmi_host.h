@@ -20,8 +20,10 @@ hipStream_t stream();
 // Returns false (and records the error) when a HIP call failed.
 bool hip_ok(hipError_t e, const char *what);
 
-// Makes sure a GPU is usable and the per-device state exists.
+// Makes sure a GPU is usable and the per-device state exists; refuses the call when one of the operands noted since
+// clear_error() lies in the first 64 KiB of the address space (no memory: a placeholder or an offset).
 bool ensure_device();
+void note_operand(const void *p);
 
 // Zeroed device words (one per 32-column block, at least n of them) that K-sliced launches count their arrivals in and
 // leave zeroed; null when they cannot be had or ZMI_NO_SLICE_ARRIVALS is set (the launch then ends in a reduction kernel).

@@ -103,6 +103,7 @@ struct ThreadCtx {
   unsigned int *fq_err_dev = nullptr;    // the same word as the device addresses it
   // stream hand-over (zmi_set_stream): work of this thread may still be queued on `stream`
   bool enqueued = false;
+  bool low_operand = false;   // (see note_operand())
   hipEvent_t handover = nullptr;
   // arrival words of K-sliced launches (see slice_arrivals())
   unsigned int *arrivals = nullptr;
@@ -145,7 +146,13 @@ size_t cache_capacity() {
 }  // namespace
 
 void set_error(const std::string &msg) { tctx.error = msg; }
-void clear_error() { tctx.error.clear(); }
+void clear_error() { tctx.error.clear(); tctx.low_operand = false; }
+// An operand address in the first 64 KiB is no memory (a placeholder, an offset taken for a pointer): the entry points
+// note their operands here and ensure_device() refuses the call before anything is queued, instead of a kernel
+// faulting on it.  No more than that: whether an address above is device memory is the caller's business.
+void note_operand(const void *p) {
+  if (p && (uintptr_t)p < 65536) tctx.low_operand = true;
+}
 void set_kernel_name(const char *name) { tctx.kernel = name; }
 hipStream_t stream() { return tctx.stream; }
 
@@ -200,8 +207,7 @@ ZmiRingSide side_stream() {
   return s;
 }
 
-bool ensure_device() {
-  tctx.enqueued = true;   // every entry point passes here before it queues work
+static bool device_present() {
   static std::atomic<bool> ready{false};
   if (ready.load(std::memory_order_acquire)) return true;
   std::lock_guard<std::mutex> lk(g_mu);
@@ -215,6 +221,16 @@ bool ensure_device() {
   }
   g_device_ready = true;
   ready.store(true, std::memory_order_release);
+  return true;
+}
+
+bool ensure_device() {
+  tctx.enqueued = true;   // every entry point passes here before it queues work
+  if (!device_present()) return false;
+  if (tctx.low_operand) {
+    set_error("an operand address lies in the first 64 KiB: that is no memory a kernel can be launched on");
+    return false;
+  }
   return true;
 }
 
