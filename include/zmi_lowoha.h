@@ -391,6 +391,13 @@ ZMI_API int32_t zmi_calib_hbm_read(void *const *bufs, int32_t n_bufs, uint64_t b
 ZMI_API int32_t zmi_calib_hbm_read_shape(void *const *bufs, int32_t n_bufs, uint64_t bytes,
                            int32_t threads, int32_t requests, int32_t warm, int32_t launches,
                            void *stream, float *us_per_launch, float *span_us);
+/* No counterpart in the reference (its planner is internal: matmul/partitioning).  Which large-M kernel a single
+ * problem of this shape gets when its destination is bf16, its rows 16-byte aligned and its epilogue one of the
+ * straight-line ones: tile_rows 0 = none of them (a decode-shaped kernel takes the call), else the tile height
+ * (64 / 128 / 256); k_slices >= 1; persistent 1 = the persistent form (k_pring.hip), 0 = the tiled one (k_ring.hip).
+ * Needs no device (256 compute units are assumed without one); honours the ZMI_* overrides. */
+ZMI_API int32_t zmi_large_m_plan(int32_t M, int32_t N, int32_t K, int32_t *tile_rows, int32_t *k_slices,
+                         int32_t *persistent);
 ZMI_API int32_t zmi_calib_mfma_i8(const void *operands, int32_t vary_operands,
                           int32_t wgs_per_cu, int32_t iters, void *stream,
                           float *tops, float *shader_mhz);

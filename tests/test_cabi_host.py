@@ -291,3 +291,47 @@ def test_environment_switches_are_read_once_and_reloadable(monkeypatch):
     monkeypatch.setenv("ZENDNNL_DIAGNOSTICS_ENABLE", "0")
     lib.zmi_reload_env()
     assert _mm(_int8_params(), M=0) == capi.FAILURE
+
+
+def _plan(lib, M, N, K):
+    t, s, p = C.c_int32(), C.c_int32(), C.c_int32()
+    assert lib.zmi_large_m_plan(M, N, K, C.byref(t), C.byref(s), C.byref(p)) == capi.SUCCESS
+    return t.value, s.value, p.value
+
+
+def test_large_m_plan_follows_the_measurements(monkeypatch):
+    """Which form of the large-M kernel takes a call is decided on the host from prices that came out of measurements
+    on MI355X (whole call, tiled / persistent, K = 4096): the shapes below are those measurements, and the plan must
+    pick the faster form for each -- except 900 x 14336 (71.8 / 67.8 us), which the prices are known to get wrong.
+    Without a device the planner assumes 256 compute units, the MI355X figure."""
+    for v in ("ZMI_PRING", "ZMI_GEMM_TOP", "ZMI_RING_SPLITK", "ZMI_RING_MIN_M", "ZMI_DECODE_MAX_M", "ZMI_NO_DECODE_KERNEL"):
+        monkeypatch.delenv(v, raising=False)
+    lib = capi.load()
+    lib.zmi_reload_env()
+    persistent_wins = [(2048, 4096), (1024, 4096), (1024, 8192), (2048, 2048), (512, 14336), (768, 14336), (1300, 14336),
+                       (1536, 14336), (1792, 14336), (2048, 14336), (4096, 14336), (2048, 5000), (256, 14336), (4096, 4096),
+                       (1024, 14336), (2048, 8192)]
+    tiled_wins = [(1536, 4096), (1100, 4096), (600, 8192), (1100, 14336), (300, 14336)]
+    for M, N in persistent_wins:
+        assert _plan(lib, M, N, 4096) == (256, 1, 1), (M, N)
+    for M, N in tiled_wins:
+        t, s, p = _plan(lib, M, N, 4096)
+        assert p == 0 and t in (64, 128, 256) and s == 1, (M, N, t, s, p)
+    # the decode-shaped kernels keep their calls; few rows against many columns go out in K slices of 64-row tiles
+    assert _plan(lib, 16, 14336, 4096) == (0, 0, 0)
+    t, s, p = _plan(lib, 128, 14336, 4096)
+    assert (t, p) == (64, 0) and s >= 2
+    # the overrides
+    monkeypatch.setenv("ZMI_PRING", "0")
+    lib.zmi_reload_env()
+    assert _plan(lib, 2048, 14336, 4096)[2] == 0
+    monkeypatch.setenv("ZMI_PRING", "1")
+    lib.zmi_reload_env()
+    assert _plan(lib, 1100, 4096, 4096)[2] == 1
+    monkeypatch.delenv("ZMI_PRING")
+    monkeypatch.setenv("ZMI_GEMM_TOP", "256")
+    lib.zmi_reload_env()
+    assert _plan(lib, 2048, 14336, 4096) == (256, 1, 0)
+    monkeypatch.delenv("ZMI_GEMM_TOP")
+    lib.zmi_reload_env()
+    assert lib.zmi_large_m_plan(0, 8, 8, None, None, None) == capi.FAILURE

@@ -176,6 +176,8 @@ SIGNATURES = {
                                        C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "zmi_calib_hbm_read_shape": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.c_uint64, C.c_int32, C.c_int32, C.c_int32,
                                              C.c_int32, C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "zmi_large_m_plan": (C.c_int32, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                     C.POINTER(C.c_int32)]),
     "zmi_calib_mfma_i8": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                       C.POINTER(C.c_float), C.POINTER(C.c_float)]),
 }

@@ -392,12 +392,16 @@ static double ring_price(int M, int N, int top) {
   return (double)((tiles + 2 * n_cu - 1) / (2 * n_cu)) * paired;
 }
 
-static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi, int ring_top) {
-  if (!zmi_pring_takes(prob, epi)) return false;
+// (shape only: what the call's epilogue and alignment allow is zmi_pring_takes)
+static bool pring_cheaper(int M, int N, int ring_top) {
   if (const char *env = zmi_env(ZE_PRING)) return std::atoi(env) != 0;
-  if (prob.M < 256 || zmi_env(ZE_GEMM_TOP)) return false;   // (a forced tile height asks for the tiled form)
-  const double mine = pring_price(prob.M, prob.N), other = ring_price(prob.M, prob.N, ring_top);
-  return mine < other - 1e-9 || (mine < other + 1e-9 && prob.M % 256 == 0);
+  if (M < 256 || zmi_env(ZE_GEMM_TOP)) return false;   // (a forced tile height asks for the tiled form)
+  const double mine = pring_price(M, N), other = ring_price(M, N, ring_top);
+  return mine < other - 1e-9 || (mine < other + 1e-9 && M % 256 == 0);
+}
+
+static bool pring_wanted(const ZmiProblem &prob, const ZmiEpilogue &epi, int ring_top) {
+  return zmi_pring_takes(prob, epi) && pring_cheaper(prob.M, prob.N, ring_top);
 }
 
 int32_t run_single_gemm(const ZmiProblem &prob, const ZmiEpilogue &epi, const ZmiRingPlan *plan) {
@@ -1036,6 +1040,19 @@ static int32_t validate_prepack(const zmi_prepack_params_t &pp) {
   if (pp.ldb < min_ld) { set_error("prepack: ldb too small"); return ZMI_FAILURE; }
   if (pp.algo != ZMI_ALGO_AOCL_DLP_BLOCKED) { set_error("prepack: only aocl_dlp_blocked is supported"); return ZMI_UNIMPLEMENTED; }
   if (pp.wei_dtype != ZMI_DT_S8) { set_error("prepack: only s8 weights are implemented"); return ZMI_UNIMPLEMENTED; }
+  return ZMI_SUCCESS;
+}
+
+int32_t zmi_large_m_plan(int32_t M, int32_t N, int32_t K, int32_t *tile_rows, int32_t *k_slices, int32_t *persistent) {
+  clear_error();
+  if (M <= 0 || N <= 0 || K <= 0 || !tile_rows || !k_slices || !persistent) { set_error("large_m_plan: bad arguments"); return ZMI_FAILURE; }
+  *tile_rows = 0; *k_slices = 0; *persistent = 0;
+  if (!use_ring_kernel(M, N, K)) return ZMI_SUCCESS;   // (the decode-shaped kernels take the call)
+  const ZmiRingPlan plan = plan_ring_gemm(M, N, K);
+  *tile_rows = plan.top & 0xffff;
+  *k_slices = plan.slices;
+  *persistent = plan.slices == 1 && N >= 64 && N % 4 == 0 && pring_cheaper(M, N, plan.top) ? 1 : 0;
+  if (*persistent) *tile_rows = 256;
   return ZMI_SUCCESS;
 }
 
