@@ -335,3 +335,22 @@ def test_large_m_plan_follows_the_measurements(monkeypatch):
     monkeypatch.delenv("ZMI_GEMM_TOP")
     lib.zmi_reload_env()
     assert lib.zmi_large_m_plan(0, 8, 8, None, None, None) == capi.FAILURE
+
+
+def test_environment_table_names_follow_the_enum():
+    """The switches are looked up by position: the enum in zmi_launch.h and the name table in zmi_host.hip must list
+    the same switches in the same order, and nothing else in the sources may read the environment itself."""
+    src = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "zendnn_amd", "csrc")
+    head = open(os.path.join(src, "zmi_launch.h")).read()
+    enum = head[head.index("enum ZmiEnvVar {"):head.index("ZE_COUNT")]
+    enums = re.findall(r"\bZE_[A-Z0-9_]+", enum)
+    host = open(os.path.join(src, "zmi_host.hip")).read()
+    table = host[host.index("kEnvNames"):]
+    names = re.findall(r'"([A-Z0-9_]+)"', table[:table.index("};")])
+    assert len(enums) == len(names) > 20
+    for e, n in zip(enums, names):
+        assert e[3:] == (n[4:] if n.startswith("ZMI_") else n), (e, n)
+    for f in os.listdir(src):
+        text = open(os.path.join(src, f)).read()
+        if f != "zmi_host.hip":
+            assert "getenv(" not in text, f
