@@ -26,7 +26,8 @@
  *                                product of the shifted operands in Python integers (u8 / s8, transposed A)
  *   dequant chain / bias         special cases (unit scales, equal per-channel
  *                                scales == per-tensor), op order from source
- *   post-ops                     libm double evaluation within 2 f32 ulp
+ *   post-ops                     libm double evaluation within 2 f32 ulp (mish = x * tanh(softplus(x)) included: double
+ *                                evaluation, the limits for large |x|, mish(0) = 0)
  *   per-group scales             closed form (all-ones operands, power-of-two scales: every step exact),
  *                                equal power-of-two group scales == per-token chain bit for bit,
  *                                numpy float32 brute force on small random cases
@@ -50,7 +51,9 @@
  *                                parity unpinned, the comparison of products is to a tolerance.
  *   dynamic u8 (per tensor)      closed forms (values k / 4: scale 0.25, zero-point 100, codes and product known exactly;
  *                                constant and non-finite tensors; the 2.5 * 255 tie), identity weights dequantize to the
- *                                source within half a step; the AVX-512 kernels' reciprocal form: parity unpinned on ties
+ *                                source within half a step; with a bf16 scale buffer the codes are made with the narrowed
+ *                                scale and the zero-point with the un-narrowed one (closed form: scale 0.3 -> 0.30078125,
+ *                                codes known exactly); the AVX-512 kernels' reciprocal form: parity unpinned on ties
  *   zo_gated_act, zo_moe_reduce  brute force + the reference example's closed form
  *   prepack layout, weight_prepack_size values: parity unpinned (opaque by the
  *     reference's contract; only the round trip matmul(prepack(B)) == matmul(B)
