@@ -179,19 +179,6 @@ int32_t validate_group(const zmi_group_args_t &a, const zmi_moe_postop_t *postop
   return ZMI_SUCCESS;
 }
 
-bool same_quant_shape(const zmi_quant_t &x, const zmi_quant_t &y, int Mx, int My, int Nx, int Ny) {
-  // same granularity class: absent / one element / per row / per column
-  auto cls = [](const zmi_quant_t &q, int M, int N, bool has) {
-    if (!has) return 0;
-    const int64_t n = nelems(q);
-    if (n == 1) return 1;
-    if (n == M) return 2;
-    if (n == N) return 3;
-    return 4;
-  };
-  return x.dt == y.dt && cls(x, Mx, Nx, x.buff != nullptr || x.ndims > 0) == cls(y, My, Ny, y.buff != nullptr || y.ndims > 0);
-}
-
 // One epilogue descriptor serves a grouped launch only if every expert asks for
 // the same arithmetic.
 bool params_uniform(const zmi_group_args_t &a, size_t num_ops) {
@@ -581,10 +568,8 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
 
     // ---- scratch plan ----
     size_t need = 0;
-    int64_t rows = 0;
     for (size_t i = 0; i < num_ops; ++i) {
       if (a.M[i] <= 0) continue;
-      rows += a.M[i];
       if (dyn) need += Arena::padded((size_t)zmi_afrag_bytes(a.M[i], a.K[i])) + Arena::padded(sizeof(float) * (size_t)a.M[i]);
       else need += Arena::padded((size_t)zmi_afrag_bytes(a.M[i], a.K[i]));
       const bool cache = a.params[i].mem_format_b != 'r' && a.is_weights_const[i] &&
