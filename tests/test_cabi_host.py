@@ -321,6 +321,12 @@ def test_large_m_plan_follows_the_measurements(monkeypatch):
     assert _plan(lib, 16, 14336, 4096) == (0, 0, 0)
     t, s, p = _plan(lib, 128, 14336, 4096)
     assert (t, p) == (64, 0) and s >= 2
+    # few rows: 64-row tiles in as many K slices as leave a slice 24 stages and fit one workgroup per compute unit
+    # (the shapes of the planner's own measurements)
+    assert _plan(lib, 96, 14336, 4096) == (64, 2, 0)
+    assert _plan(lib, 128, 8192, 8192) == (64, 4, 0)
+    assert _plan(lib, 128, 4096, 14336) == (64, 4, 0)
+    assert _plan(lib, 256, 4096, 4096) == (64, 2, 0)
     # the overrides
     monkeypatch.setenv("ZMI_PRING", "0")
     lib.zmi_reload_env()
