@@ -591,7 +591,22 @@ int32_t zmi_group_matmul_direct(const zmi_group_args_t *args, const zmi_moe_post
       need += Arena::padded(tbl);
     }
     need += 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * num_ops));
-    need += 2 * Arena::padded(stream_partial_bound());   // K-sliced grouped launches (one workspace per GEMM stage)
+    // Room for the partial tiles of a K-sliced stage, only where a stage can go out in slices: a plain epilogue and,
+    // among the experts of more than 16 rows, at most one 128-row tile per compute unit (the least group_stream_plan and
+    // ring_group_split ask for), or a forced slice count.  (A stage that finds no room runs unsliced.)
+    {
+      const int64_t n_cu = zmi_cu_count();
+      const bool forced = zmi_env(ZE_GROUP_STREAM_SLICES) != nullptr;
+      int64_t t1 = 0, t2 = 0;
+      for (size_t i = 0; i < num_ops; ++i) {
+        if (a.M[i] <= 16) continue;
+        const int64_t row_blocks = (a.M[i] + 127) / 128;
+        t1 += row_blocks * ((a.N[i] + 255) / 256);
+        if (fused_moe) t2 += row_blocks * ((fused_moe->N_down[i] + 255) / 256);
+      }
+      const int sliced_stages = ((forced || (!fuse_act && t1 <= n_cu)) ? 1 : 0) + ((fused_moe && (forced || t2 <= n_cu)) ? 1 : 0);
+      need += (size_t)sliced_stages * Arena::padded(stream_partial_bound());
+    }
     if (!arena().begin(need)) return ZMI_FAILURE;
 
     // ---- stage 1: sources (dynamic per-token quantization of every expert in one launch)
@@ -851,7 +866,9 @@ int32_t zmi_moe_fused_device(const zmi_moe_device_t *d) {
   need += Arena::padded((size_t)Rp * kpI) + Arena::padded(sizeof(float) * Rp);       // A2, s2
   need += Arena::padded((size_t)Rp * H * 2);                                         // Y bf16
   need += 2 * Arena::padded(sizeof(ZmiProblem) * E) + 4096 + 2 * Arena::padded(sizeof(int) * (4 + 3 * (size_t)E));
-  need += Arena::padded(stream_partial_bound());   // Op2 in K slices
+  // Op2 in K slices: only where its planners can ask for them (at most one 128-row tile per compute unit, or forced)
+  if (zmi_env(ZE_GROUP_STREAM_SLICES) || (R / 128) * (int64_t)((H + 255) / 256) <= (int64_t)zmi_cu_count())
+    need += Arena::padded(stream_partial_bound());
   const size_t hist_ints = zmi_moe_route_scratch_ints(R, E);
   need += Arena::padded(hist_ints * sizeof(int32_t));
   if (!arena().begin(need)) return ZMI_FAILURE;
