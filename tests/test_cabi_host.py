@@ -360,3 +360,16 @@ def test_environment_table_names_follow_the_enum():
         text = open(os.path.join(src, f)).read()
         if f != "zmi_host.hip":
             assert "getenv(" not in text, f
+
+
+@fake_pointers
+def test_placeholder_addresses_are_refused_before_anything_is_queued():
+    """A call that passes every validator with an operand address in the first 64 KiB (here the accepted form of the
+    mish post-op on the static scale chain) is refused by the library itself, with or without a device: such an
+    address is no memory, and a kernel launched on it faults the device."""
+    p = _int8_params()
+    p.postop_ = [lowoha.PostOp(capi.PO_MISH)]
+    st = lowoha.matmul_direct("r", False, False, 4, 8, 16, 1.0, FAKE, 16, FAKE, 8, None, 0.0, FAKE, 8, True, p)
+    assert st == capi.FAILURE and "first 64 KiB" in lowoha.last_error(), lowoha.last_error()
+    rp = _prepack_rp()
+    assert lowoha.reorder_direct(FAKE, FAKE, rp) == capi.FAILURE and "first 64 KiB" in lowoha.last_error()

@@ -226,12 +226,11 @@ static bool device_present() {
 
 bool ensure_device() {
   tctx.enqueued = true;   // every entry point passes here before it queues work
-  if (!device_present()) return false;
   if (tctx.low_operand) {
     set_error("an operand address lies in the first 64 KiB: that is no memory a kernel can be launched on");
     return false;
   }
-  return true;
+  return device_present();
 }
 
 void note_enqueue() { tctx.enqueued = true; }
